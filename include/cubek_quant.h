@@ -1,0 +1,178 @@
+/*
+ * cubek_quant.h — C ABI of the MI355X (gfx950) quantize / dequantize library.
+ *
+ * Every entry point is what a foreign-function binding of the reference crate
+ * `cubek-quant` would bind for its quantize/dequantize path.  The reference
+ * interface each one replaces is cited next to it (paths are relative to the
+ * reference tree, crates/cubek-quant/...).
+ *
+ * Conventions
+ *   - plain pointers and sizes only; `ptr` fields are DEVICE pointers;
+ *   - the caller owns every buffer (inputs, outputs, scales, workspace);
+ *   - calls are asynchronous and ordered on the given HIP stream (NULL = the
+ *     default stream); nothing here synchronises the device;
+ *   - every function returns a cq_status (0 = success) and never aborts;
+ *   - the library keeps no mutable global state, calls are re-entrant.
+ */
+#ifndef CUBEK_QUANT_H
+#define CUBEK_QUANT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CQ_ABI_VERSION 1
+#define CQ_MAX_RANK 8       /* tensors of rank 1..8                               */
+#define CQ_MAX_BLOCK_DIMS 5 /* same bound as the reference's BlockSize storage    */
+
+/* Status codes. Conditions the reference answers with panic!/assert! are
+ * reported as distinct codes instead (src/quantize.rs:203-206,218,273,324;
+ * src/lib.rs:28-31); launch failures map to CQ_ERR_HIP (LaunchError). */
+typedef enum cq_status {
+    CQ_OK = 0,
+    CQ_ERR_INVALID_ARGUMENT = 1,    /* NULL pointer, bad rank, bad enum value            */
+    CQ_ERR_UNSUPPORTED_SCHEME = 2,  /* value/store/param combination not implemented     */
+    CQ_ERR_BLOCK_NOT_DIVISIBLE = 3, /* check_block_size_compat failed (src/lib.rs:20-33) */
+    CQ_ERR_SHAPE_MISMATCH = 4,      /* packed/unpacked/scales shapes do not agree        */
+    CQ_ERR_NON_CONTIGUOUS = 5,      /* value tensors must be contiguous row-major        */
+    CQ_ERR_WORKSPACE_TOO_SMALL = 6,
+    CQ_ERR_HIP = 7,                 /* a HIP runtime call failed; see cq_last_hip_error  */
+    CQ_ERR_TOO_LARGE = 8            /* more elements than an entry point accepts         */
+} cq_status;
+
+/* Float element types of value tensors and scale parameters
+ * (the reference passes ElemType / StorageType: src/quantize.rs:181,
+ * src/dequantize.rs:177). */
+typedef enum cq_dtype {
+    CQ_F32 = 0,
+    CQ_F16 = 1,
+    CQ_BF16 = 2
+} cq_dtype;
+
+/* QuantValue (re-exported at src/lib.rs:14). Integer ranges used by the
+ * kernels: Q8F [-128,127], Q8S [-127,127], Q4F [-8,7], Q4S [-7,7],
+ * Q2F [-2,1], Q2S [-1,1], E2M1 [-6,6], E4M3 [-448,448], E5M2 [-57344,57344]. */
+typedef enum cq_value {
+    CQ_VALUE_Q8F = 0,
+    CQ_VALUE_Q8S = 1,
+    CQ_VALUE_Q4F = 2,
+    CQ_VALUE_Q4S = 3,
+    CQ_VALUE_Q2F = 4,
+    CQ_VALUE_Q2S = 5,
+    CQ_VALUE_E2M1 = 6,
+    CQ_VALUE_E4M3 = 7,
+    CQ_VALUE_E5M2 = 8
+} cq_value;
+
+typedef enum cq_param { /* QuantParam: dtype of the stored scales */
+    CQ_PARAM_F32 = 0,
+    CQ_PARAM_F16 = 1,
+    CQ_PARAM_BF16 = 2
+} cq_param;
+
+typedef enum cq_store { /* QuantStore */
+    CQ_STORE_U32 = 0,   /* 32/size_bits codes per u32 word, element 0 in the low bits */
+    CQ_STORE_NATIVE = 1 /* i8 / fp8 bytes, or two e2m1 nibbles per byte               */
+} cq_store;
+
+typedef enum cq_level { /* QuantLevel */
+    CQ_LEVEL_TENSOR = 0,
+    CQ_LEVEL_BLOCK = 1
+} cq_level;
+
+typedef enum cq_mode { /* QuantMode */
+    CQ_MODE_SYMMETRIC = 0
+} cq_mode;
+
+/* QuantScheme.  `block` holds the block size per trailing dimension exactly as
+ * the reference's QuantLevel::block([..]) does (u8 entries, at most 5); it is
+ * left-padded with 1s up to the tensor rank (src/layout/scales.rs:239). */
+typedef struct cq_scheme {
+    uint8_t value;      /* cq_value */
+    uint8_t param;      /* cq_param */
+    uint8_t store;      /* cq_store */
+    uint8_t level;      /* cq_level */
+    uint8_t mode;       /* cq_mode  */
+    uint8_t block_rank; /* number of valid entries in block[] (0 for per-tensor) */
+    uint8_t block[CQ_MAX_BLOCK_DIMS];
+    uint8_t reserved;   /* must be 0 */
+} cq_scheme;
+
+/* Borrowed tensor handle = the fields of the reference's TensorHandleRef
+ * (handle, shape, strides, elem_size).  Strides are in elements. */
+typedef struct cq_tensor {
+    void* ptr;
+    const uint64_t* shape;
+    const uint64_t* strides;
+    uint32_t rank;
+    uint32_t elem_size; /* bytes per element */
+} cq_tensor;
+
+typedef struct ihipStream_t* cq_stream_t; /* == hipStream_t */
+
+/* ---- scheme helpers (QuantScheme / QuantValue methods used by the path) ---- */
+
+/* QuantValue::size_bits (call sites src/quantize.rs:62, src/dequantize.rs:91). */
+uint32_t cq_value_size_bits(uint8_t value);
+/* QuantScheme::num_quants = stored bits / value bits
+ * (call sites src/quantize.rs:144,290; src/dequantize.rs:67,248). */
+uint32_t cq_scheme_num_quants(const cq_scheme* scheme);
+/* QuantValue::range (call sites src/quantize.rs:243,296). */
+cq_status cq_value_range(uint8_t value, float* range_min, float* range_max);
+
+/* ---- the path ---- */
+
+/* Replaces cubek_quant::quantize::launch_ref (src/quantize.rs:174-221).
+ *   input      : float tensor of dtype `input_dtype`, contiguous
+ *   output     : U32 store -> u32 tensor, shape = input shape with the last
+ *                dimension divided by num_quants (tests/suite/symmetric.rs:68-69);
+ *                NATIVE store -> 1-byte tensor (E2M1: last dimension / 2)
+ *   scale      : scales typed as `input_dtype`, shape [1] (per-tensor) or one
+ *                entry per block; its strides are honoured
+ *   out_scale  : same shape as `scale`, typed as scheme->param; receives the
+ *                scale of every block */
+cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                      const cq_tensor* scale, const cq_tensor* out_scale,
+                      const cq_scheme* scheme, cq_dtype input_dtype);
+
+/* Replaces cubek_quant::dequantize::launch_ref (src/dequantize.rs:171-229).
+ *   values : quantized tensor as written by cq_quantize
+ *   output : float tensor of dtype `output_dtype`, unpacked shape
+ *   params : scales typed as scheme->param */
+cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_tensor* output,
+                        const cq_tensor* params, const cq_scheme* scheme,
+                        cq_dtype output_dtype);
+
+/* Scale production.  The reference crate leaves this to its caller; the rule is
+ * the one its tests apply on the host, scale = 2*max|x| / (q_max - q_min) in f32
+ * (tests/suite/symmetric.rs:35-38,156-179), with NaN elements ignored.
+ *   scales : typed as `input_dtype` (what cq_quantize expects as `scale`),
+ *            contiguous, shape [1] or one entry per block
+ *   workspace : cq_workspace_bytes() bytes of device memory, 256-byte aligned;
+ *               only per-tensor schemes use it, may be NULL for block schemes */
+cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq_tensor* scales,
+                            const cq_scheme* scheme, cq_dtype input_dtype,
+                            void* workspace, size_t workspace_bytes);
+
+/* Fused abs-max + scale + quantize: same results as cq_compute_scales followed
+ * by cq_quantize, without materialising the input-typed scales. */
+cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                              const cq_tensor* out_scale, const cq_scheme* scheme,
+                              cq_dtype input_dtype, void* workspace, size_t workspace_bytes);
+
+/* Device bytes the two entry points above need for `num_elements` inputs. */
+size_t cq_workspace_bytes(const cq_scheme* scheme, uint64_t num_elements);
+
+/* ---- diagnostics ---- */
+const char* cq_strerror(cq_status status);
+/* hipError_t of the most recent failed HIP call on the calling thread (0 if none). */
+int cq_last_hip_error(void);
+uint32_t cq_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUBEK_QUANT_H */
