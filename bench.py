@@ -1,0 +1,300 @@
+#!/usr/bin/env python3
+"""Throughput of the quantize/dequantize path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg5] [--no-sweep] [--no-cpu]
+
+A step = one pass of the hot path over one synthetic tensor that is already
+resident in HBM: fused dynamic quantize (abs-max, scale, round, clamp, pack)
+followed by dequantize of the result.  The headline workload is the largest
+configuration (cfg5: e2m1 block 32, bf16 [28672, 8192]); the other four
+configurations are measured in short loops and reported under "per_config".
+
+value      = algorithmic bytes of one step / wall time per step  (GB/s, 1e9)
+             algorithmic bytes = input once + codes once + scales once, per direction
+roofline   = the quantize kernel alone: algorithmic bytes / its mean HIP-event duration,
+             against the 8 TB/s HBM peak
+cpu_baseline = the CPU oracle (oracle/cq_oracle.c, the scalar restatement of the
+             reference algorithm) on a bounded row sample of the same tensor
+
+Prints ONE JSON line on stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+# name -> (rows, cols, elem, value, block, generator)
+WORKLOADS = {
+    "cfg1": dict(shape=(1024, 1024), elem="F32", value="Q8S", block=None, dist="normal1", seed=1,
+                 desc="per-tensor symmetric q8, f32 [1024,1024] ~N(0,1)"),
+    "cfg2": dict(shape=(4096, 4096), elem="BF16", value="Q8S", block=32, dist="normal_outliers", seed=2,
+                 desc="per-block(32) symmetric q8, bf16 [4096,4096] ~N(0,0.02) + 0.1% x50 outliers"),
+    "cfg3": dict(shape=(14336, 4096), elem="BF16", value="Q4S", block=32, dist="normal", seed=3,
+                 desc="per-block(32) symmetric q4, bf16 [14336,4096] ~N(0,0.02)"),
+    "cfg4": dict(shape=(8192, 8192), elem="F32", value="Q2S", block=64, dist="laplace", seed=4,
+                 desc="per-block(64) symmetric q2, f32 [8192,8192] ~Laplace(0,0.01)"),
+    "cfg5": dict(shape=(28672, 8192), elem="BF16", value="E2M1", block=32, dist="normal_t3", seed=5,
+                 desc="per-block(32) e2m1 (4-bit fields), bf16 [28672,8192] ~N(0,0.02) + 1% Student-t(3)"),
+}
+
+# HBM bytes per launch of the quantize kernel measured with rocprofv3 --pmc
+# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); filled from
+# the summaries under profiles/.  None = not measured for that workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(w) -> int:
+    rows, cols = w["shape"]
+    n = rows * cols
+    elem_bytes = 4 if w["elem"] == "F32" else 2
+    bits = {"Q8S": 8, "Q4S": 4, "Q2S": 2, "E2M1": 4}[w["value"]]
+    scales = 1 if w["block"] is None else n // w["block"]
+    return n * elem_bytes + n * bits // 8 + scales * 4
+
+
+def make_input(torch, w):
+    """Seeded synthetic tensor generated on the device, chunked to bound memory."""
+    rows, cols = w["shape"]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(w["seed"])
+    dt = torch.float32 if w["elem"] == "F32" else torch.bfloat16
+    out = torch.empty((rows, cols), dtype=dt, device="cuda")
+    step = max(1, (64 << 20) // (cols * 4))
+    for r0 in range(0, rows, step):
+        r1 = min(rows, r0 + step)
+        shp = (r1 - r0, cols)
+        dist = w["dist"]
+        if dist == "normal1":
+            x = torch.randn(shp, generator=g, device="cuda")
+        elif dist == "normal":
+            x = torch.randn(shp, generator=g, device="cuda") * 0.02
+        elif dist == "normal_outliers":
+            x = torch.randn(shp, generator=g, device="cuda") * 0.02
+            m = torch.rand(shp, generator=g, device="cuda") < 0.001
+            x = torch.where(m, x * 50.0, x)
+        elif dist == "laplace":
+            u = torch.rand(shp, generator=g, device="cuda") - 0.5
+            x = -0.01 * torch.sign(u) * torch.log1p(-2.0 * u.abs().clamp(max=0.4999999))
+        elif dist == "normal_t3":
+            x = torch.randn(shp, generator=g, device="cuda") * 0.02
+            m = torch.rand(shp, generator=g, device="cuda") < 0.01
+            z = torch.randn(shp, generator=g, device="cuda")
+            chi = (torch.randn((3,) + shp, generator=g, device="cuda") ** 2).sum(0) / 3.0
+            x = torch.where(m, 0.02 * z / chi.sqrt(), x)
+        else:
+            raise ValueError(dist)
+        out[r0:r1] = x.to(dt)
+    return out
+
+
+class Path:
+    """Buffers + launches of one workload (quantize_dynamic, quantize, dequantize)."""
+
+    def __init__(self, torch, w, x):
+        from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantScheme, QuantValue,
+                               TensorHandleRef)
+        from cubek_amd import dequantize as dq, quantize as qz
+
+        self.torch, self.qz, self.dq = torch, qz, dq
+        self.elem = ElemType[w["elem"]]
+        level = QuantLevel.Tensor if w["block"] is None else QuantLevel.block([w["block"]])
+        self.scheme = QuantScheme.default().with_value(QuantValue[w["value"]]).with_level(level)
+        shape = tuple(x.shape)
+        self.x = x
+        self.codes = torch.empty(self.scheme.packed_shape(shape), dtype=torch.int32, device="cuda")
+        self.scales = torch.empty(self.scheme.scales_shape(shape), dtype=torch.float32, device="cuda")
+        self.in_scales = torch.empty(self.scheme.scales_shape(shape), dtype=x.dtype, device="cuda")
+        self.y = torch.empty_like(x)
+        nbytes = qz.workspace_bytes(self.scheme, x.numel())
+        self.ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device="cuda")
+        self.ws_bytes = nbytes
+        self.client = ComputeClient.current()
+        h = TensorHandleRef.from_torch
+        self.hx, self.hc, self.hs, self.hy, self.his = h(x), h(self.codes), h(self.scales), h(self.y), h(self.in_scales)
+
+    def quantize_dynamic(self):
+        self.qz.launch_dynamic(self.client, self.hx, self.hc, self.hs, self.scheme, self.elem,
+                               self.ws.data_ptr(), self.ws_bytes)
+
+    def compute_scales(self):
+        self.qz.compute_scales(self.client, self.hx, self.his, self.scheme, self.elem,
+                               self.ws.data_ptr(), self.ws_bytes)
+
+    def quantize_given(self):
+        self.qz.launch_ref(self.client, self.hx, self.hc, self.his, self.hs, self.scheme, self.elem)
+
+    def dequantize(self):
+        self.dq.launch_ref(self.client, self.hc, self.hy, self.hs, self.scheme, self.elem)
+
+
+def time_kernel(torch, fn, iters, warmup=3):
+    """Mean duration (ms) of one launch, HIP events on the launch stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in evs)
+    return sum(ts) / len(ts), ts[len(ts) // 2]
+
+
+def cpu_baseline(torch, w, path, budget_s=12.0):
+    """The CPU oracle on a bounded sample of rows: quantize (given scales) + dequantize."""
+    import numpy as np
+
+    from oracle import oracle
+
+    rows, cols = w["shape"]
+    threads = min(16, len(os.sched_getaffinity(0)))
+    elem = path.elem
+
+    def host_rows(nrows):
+        xs = path.x[:nrows].contiguous()
+        if xs.dtype == torch.float32:
+            return xs.cpu().numpy()
+        return xs.view(torch.int16).cpu().numpy().view(np.uint16)
+
+    def run(nrows):
+        xs = host_rows(nrows)
+        shape = (nrows, cols)
+        scales = oracle.compute_scales(xs, elem, shape, path.scheme)  # not timed: the reference takes scales as input
+        t0 = time.perf_counter()
+        words, out_scale = oracle.quantize(xs, elem, shape, scales, path.scheme, threads=threads)
+        oracle.dequantize(words, shape, out_scale, elem, path.scheme, threads=threads)
+        return time.perf_counter() - t0
+
+    probe_rows = max(threads, min(rows, (1 << 21) // cols))
+    t_probe = run(probe_rows)
+    nrows = int(min(rows, max(probe_rows, probe_rows * budget_s / max(t_probe, 1e-3))))
+    nrows = max(threads, nrows // threads * threads)
+    t = run(nrows)
+    sample_bytes = 2 * algorithmic_bytes(dict(w, shape=(nrows, cols)))
+    return {
+        "value": sample_bytes / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"first {nrows} of {rows} rows of the headline tensor ({nrows * cols} elements), "
+                  f"quantize with given scales + dequantize, {t:.2f} s on {threads} threads",
+        "elements_per_s": nrows * cols / t,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg5", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-sweep", action="store_true", help="skip the per-config table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py measures one GPU: this path has no multi-GPU part (per-block quantization "
+                 "shards by rows without communication); run with --gpus 1")
+
+    import torch
+
+    from cubek_amd import _ffi
+
+    _ffi.lib()  # fail loudly if the HIP library is not built
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+
+    w = WORKLOADS[args.workload]
+    x = make_input(torch, w)
+    path = Path(torch, w, x)
+    q_bytes = algorithmic_bytes(w)
+    step_bytes = 2 * q_bytes
+    n = x.numel()
+
+    def step(events=None):
+        if events is not None:
+            events[0].record()
+        path.quantize_dynamic()
+        if events is not None:
+            events[1].record()
+        path.dequantize()
+        if events is not None:
+            events[2].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(evs[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    q_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
+    d_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
+
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    q_gbps = q_bytes / (q_ms * 1e-3) / 1e9
+    d_gbps = q_bytes / (d_ms * 1e-3) / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES.get(args.workload)
+
+    result = {
+        "metric": "quant/dequant GB/s (bytes read+written) and % of MI355X HBM peak, 1 GPU",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if w["elem"] == "BF16" else "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {w['desc']}; step = fused dynamic quantize + dequantize",
+                   "shape": list(w["shape"]), "block": w["block"], "value": w["value"], "store": "U32",
+                   "param": "F32", "algorithmic_bytes_per_step": step_bytes},
+        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 1),
+        "elements_per_s": round(2 * n / (ms_per_step * 1e-3)),
+        "roofline": {"bound": "hbm", "kernel": "quantize_flat_kernel (fused abs-max+scale+quantize+pack)",
+                     "achieved": round(q_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(q_gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "algorithmic_bytes_per_launch": q_bytes, "avg_launch_ms": round(q_ms, 4)},
+        "roofline_dequantize": {"bound": "hbm", "kernel": "dequantize_flat_kernel", "achieved": round(d_gbps, 1),
+                                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(d_gbps / HBM_PEAK_GBPS, 4),
+                                "algorithmic_bytes_per_launch": q_bytes, "avg_launch_ms": round(d_ms, 4)},
+    }
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, w, path)
+        result["cpu_baseline"]["value"] = round(result["cpu_baseline"]["value"], 3)
+        result["cpu_baseline"]["elements_per_s"] = round(result["cpu_baseline"]["elements_per_s"])
+
+    if not args.no_sweep:
+        table = []
+        del path, x
+        torch.cuda.empty_cache()
+        for name, wk in WORKLOADS.items():
+            xi = make_input(torch, wk)
+            p = Path(torch, wk, xi)
+            b = algorithmic_bytes(wk)
+            p.compute_scales()
+            row = {"workload": name, "algorithmic_bytes": b,
+                   # working sets under 256 MB stay in the Infinity Cache between launches:
+                   # such rows are not HBM-bound and are reported, not gated
+                   "cache_resident": 2 * b < (256 << 20)}
+            for label, fn in (("quantize_dynamic", p.quantize_dynamic), ("quantize_given_scales", p.quantize_given),
+                              ("dequantize", p.dequantize)):
+                mean_ms, med_ms = time_kernel(torch, fn, 30)
+                row[label] = {"ms": round(med_ms, 4), "GBps": round(b / (med_ms * 1e-3) / 1e9, 1),
+                              "frac_hbm_peak": round(b / (med_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+            table.append(row)
+            del p, xi
+            torch.cuda.empty_cache()
+        result["per_config"] = table
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,478 @@
+// C ABI of the library: argument validation, path selection, launches.
+// Mirrors the host side of the reference's launch functions
+// (crates/cubek-quant/src/quantize.rs:174-326, src/dequantize.rs:171-332):
+// the reference's panics become status codes, its JIT launch becomes a
+// precompiled gfx950 kernel launch on the caller's stream.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "../../include/cubek_quant.h"
+#include "cq_internal.hpp"
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+
+cq_status hip_status(hipError_t e) {
+    if (e == hipSuccess) return CQ_OK;
+    g_last_hip_error = static_cast<int>(e);
+    return CQ_ERR_HIP;
+}
+
+uint32_t dtype_size(int dtype) { return dtype == CQ_F32 ? 4u : 2u; }
+bool valid_dtype(int dtype) { return dtype == CQ_F32 || dtype == CQ_F16 || dtype == CQ_BF16; }
+int param_to_dtype(uint8_t p) { return p == CQ_PARAM_F32 ? CQ_F32 : (p == CQ_PARAM_F16 ? CQ_F16 : CQ_BF16); }
+
+uint32_t value_bits(uint8_t v) {
+    switch (v) {
+        case CQ_VALUE_Q8F: case CQ_VALUE_Q8S: case CQ_VALUE_E4M3: case CQ_VALUE_E5M2: return 8;
+        case CQ_VALUE_Q4F: case CQ_VALUE_Q4S: case CQ_VALUE_E2M1: return 4;
+        case CQ_VALUE_Q2F: case CQ_VALUE_Q2S: return 2;
+        default: return 0;
+    }
+}
+
+cq_status check_scheme(const cq_scheme* s) {
+    if (!s) return CQ_ERR_INVALID_ARGUMENT;
+    if (value_bits(s->value) == 0 || s->param > CQ_PARAM_BF16 || s->store > CQ_STORE_NATIVE ||
+        s->level > CQ_LEVEL_BLOCK || s->reserved != 0)
+        return CQ_ERR_INVALID_ARGUMENT;
+    if (s->mode != CQ_MODE_SYMMETRIC) return CQ_ERR_UNSUPPORTED_SCHEME;
+    if (s->level == CQ_LEVEL_BLOCK) {
+        if (s->block_rank < 1 || s->block_rank > CQ_MAX_BLOCK_DIMS) return CQ_ERR_INVALID_ARGUMENT;
+        for (uint32_t i = 0; i < s->block_rank; i++)
+            if (s->block[i] == 0) return CQ_ERR_INVALID_ARGUMENT;
+    }
+    if (s->store == CQ_STORE_NATIVE) {
+        // the native arm of launch_ref accepts only these values (src/quantize.rs:192-219)
+        switch (s->value) {
+            case CQ_VALUE_Q8F: case CQ_VALUE_Q8S: case CQ_VALUE_E4M3: case CQ_VALUE_E5M2:
+            case CQ_VALUE_E2M1: break;
+            default: return CQ_ERR_UNSUPPORTED_SCHEME;
+        }
+    }
+    return CQ_OK;
+}
+
+bool tensor_ok(const cq_tensor* t) {
+    return t && t->ptr && t->shape && t->strides && t->rank >= 1 && t->rank <= CQ_MAX_RANK;
+}
+
+uint64_t numel(const cq_tensor* t) {
+    uint64_t n = 1;
+    for (uint32_t i = 0; i < t->rank; i++) n *= t->shape[i];
+    return n;
+}
+
+bool is_contiguous(const cq_tensor* t) {
+    uint64_t expect = 1;
+    for (int d = static_cast<int>(t->rank) - 1; d >= 0; d--) {
+        if (t->shape[d] != 1 && t->strides[d] != expect) return false;
+        expect *= t->shape[d];
+    }
+    return true;
+}
+
+bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// Everything the launches need to know about one (values, scales) pair.
+struct Plan {
+    uint32_t rank;
+    uint64_t shape[CQ_MAX_RANK];  // unpacked shape
+    uint64_t n;                   // elements
+    uint32_t bits, nq;            // bits per value; values per stored element
+    cq::Range range;
+    cq::Layout layout;
+    bool tensor_level;
+    bool last_dim_blocks;   // block extents are 1 everywhere but the last dimension
+    uint32_t block_last;
+    uint64_t num_blocks;
+};
+
+uint32_t stored_nq(const cq_scheme* s) {
+    if (s->store == CQ_STORE_U32) return 32u / value_bits(s->value);
+    return s->value == CQ_VALUE_E2M1 ? 2u : 1u;
+}
+
+// Line size the reference would pick for the native kernels: the widest of
+// 16 bytes / elem_size, halving until it divides the last dimension
+// (src/quantize.rs:235-240).  Only used for its block-size assertion.
+uint32_t native_line_size(uint32_t elem_size, uint64_t last_dim) {
+    uint32_t l = 16u / elem_size;
+    while (l > 1 && last_dim % l) l /= 2;
+    return l;
+}
+
+// `values` is the stored tensor, `floats` the float tensor (input of quantize,
+// output of dequantize); both must be contiguous and agree in shape.
+cq_status make_plan(const cq_scheme* s, const cq_tensor* floats, int dtype, const cq_tensor* values,
+                    const cq_tensor* scale_a, uint32_t scale_a_size, const cq_tensor* scale_b,
+                    uint32_t scale_b_size, Plan* p) {
+    if (!tensor_ok(floats) || !tensor_ok(values) || !tensor_ok(scale_a) || (scale_b && !tensor_ok(scale_b)))
+        return CQ_ERR_INVALID_ARGUMENT;
+    if (!valid_dtype(dtype)) return CQ_ERR_INVALID_ARGUMENT;
+    p->bits = value_bits(s->value);
+    p->nq = stored_nq(s);
+    if (cq_value_range(s->value, &p->range.lo, &p->range.hi) != CQ_OK) return CQ_ERR_INVALID_ARGUMENT;
+    if (floats->elem_size != dtype_size(dtype)) return CQ_ERR_SHAPE_MISMATCH;
+    if (values->elem_size != (s->store == CQ_STORE_U32 ? 4u : 1u)) return CQ_ERR_SHAPE_MISMATCH;
+    if (scale_a->elem_size != scale_a_size || (scale_b && scale_b->elem_size != scale_b_size))
+        return CQ_ERR_SHAPE_MISMATCH;
+    if (floats->rank != values->rank) return CQ_ERR_SHAPE_MISMATCH;
+    p->rank = floats->rank;
+    for (uint32_t d = 0; d < p->rank; d++) {
+        p->shape[d] = floats->shape[d];
+        uint64_t want = d + 1 == p->rank ? values->shape[d] * p->nq : values->shape[d];
+        if (floats->shape[d] != want) return CQ_ERR_SHAPE_MISMATCH;
+        if (floats->shape[d] == 0 || floats->shape[d] > 0xffffffffull) return CQ_ERR_TOO_LARGE;
+    }
+    p->n = numel(floats);
+    if (!is_contiguous(floats) || !is_contiguous(values)) return CQ_ERR_NON_CONTIGUOUS;
+
+    std::memset(&p->layout, 0, sizeof(p->layout));
+    p->tensor_level = s->level == CQ_LEVEL_TENSOR;
+    p->last_dim_blocks = false;
+    p->block_last = 0;
+    p->num_blocks = 1;
+    if (p->tensor_level) {
+        if (numel(scale_a) < 1 || (scale_b && numel(scale_b) < 1)) return CQ_ERR_SHAPE_MISMATCH;
+        return CQ_OK;
+    }
+    if (s->block_rank > p->rank) return CQ_ERR_SHAPE_MISMATCH;
+    // check_block_size_compat (src/lib.rs:20-33): the last block extent must be a
+    // multiple of num_quants (packed) or of the line size (native)
+    uint32_t last_block = s->block[s->block_rank - 1];
+    uint32_t div = s->store == CQ_STORE_U32 ? p->nq
+                                            : native_line_size(floats->elem_size, p->shape[p->rank - 1]);
+    if (last_block % div) return CQ_ERR_BLOCK_NOT_DIVISIBLE;
+    if (scale_a->rank != p->rank || (scale_b && scale_b->rank != p->rank)) return CQ_ERR_SHAPE_MISMATCH;
+    p->layout.rank = p->rank;
+    p->last_dim_blocks = true;
+    uint32_t pad = p->rank - s->block_rank;
+    for (uint32_t d = 0; d < p->rank; d++) {
+        uint32_t b = d < pad ? 1u : s->block[d - pad];
+        if (p->shape[d] % b) return CQ_ERR_SHAPE_MISMATCH;
+        uint64_t nb = p->shape[d] / b;
+        if (scale_a->shape[d] != nb || (scale_b && scale_b->shape[d] != nb)) return CQ_ERR_SHAPE_MISMATCH;
+        p->layout.shape[d] = static_cast<uint32_t>(p->shape[d]);
+        p->layout.block[d] = b;
+        p->layout.stride_a[d] = scale_a->strides[d];
+        p->layout.stride_b[d] = scale_b ? scale_b->strides[d] : scale_a->strides[d];
+        p->num_blocks *= nb;
+        if (d + 1 < p->rank && b != 1) p->last_dim_blocks = false;
+    }
+    p->block_last = last_block;
+    return CQ_OK;
+}
+
+// Can the flat kernels take this launch?  (contiguous scales, 1-D blocks along
+// the last axis that map onto lane groups, 16-byte aligned float tensor)
+bool flat_ok(const Plan& p, int dtype, const cq_tensor* floats, const cq_tensor* values,
+             const cq_tensor* scale_a, const cq_tensor* scale_b) {
+    if (!aligned(floats->ptr, 16) || !aligned(values->ptr, 8)) return false;
+    if (p.tensor_level) return true;
+    if (!p.last_dim_blocks) return false;
+    if (!is_contiguous(scale_a) || (scale_b && !is_contiguous(scale_b))) return false;
+    return cq::flat_block_supported(dtype, p.block_last);
+}
+
+cq::GenericArgs generic_args(const Plan& p, const cq_scheme* s) {
+    cq::GenericArgs g;
+    std::memset(&g, 0, sizeof(g));
+    g.param_dtype = param_to_dtype(s->param);
+    g.value = s->value;
+    g.range = p.range;
+    g.layout = p.layout;
+    return g;
+}
+
+}  // namespace
+
+extern "C" {
+
+uint32_t cq_abi_version(void) { return CQ_ABI_VERSION; }
+
+int cq_last_hip_error(void) { return g_last_hip_error; }
+
+const char* cq_strerror(cq_status st) {
+    switch (st) {
+        case CQ_OK: return "success";
+        case CQ_ERR_INVALID_ARGUMENT: return "invalid argument";
+        case CQ_ERR_UNSUPPORTED_SCHEME: return "unsupported quantization scheme";
+        case CQ_ERR_BLOCK_NOT_DIVISIBLE: return "block size must be divisible by the number of values per stored element";
+        case CQ_ERR_SHAPE_MISMATCH: return "tensor shapes or element sizes do not agree with the scheme";
+        case CQ_ERR_NON_CONTIGUOUS: return "value tensors must be contiguous";
+        case CQ_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
+        case CQ_ERR_HIP: return "HIP runtime error";
+        case CQ_ERR_TOO_LARGE: return "tensor too large";
+        default: return "unknown status";
+    }
+}
+
+uint32_t cq_value_size_bits(uint8_t value) { return value_bits(value); }
+
+uint32_t cq_scheme_num_quants(const cq_scheme* s) {
+    if (!s || value_bits(s->value) == 0) return 0;
+    return stored_nq(s);
+}
+
+cq_status cq_value_range(uint8_t value, float* lo, float* hi) {
+    if (!lo || !hi) return CQ_ERR_INVALID_ARGUMENT;
+    switch (value) {
+        case CQ_VALUE_Q8F: *lo = -128.f; *hi = 127.f; break;
+        case CQ_VALUE_Q8S: *lo = -127.f; *hi = 127.f; break;
+        case CQ_VALUE_Q4F: *lo = -8.f; *hi = 7.f; break;
+        case CQ_VALUE_Q4S: *lo = -7.f; *hi = 7.f; break;
+        case CQ_VALUE_Q2F: *lo = -2.f; *hi = 1.f; break;
+        case CQ_VALUE_Q2S: *lo = -1.f; *hi = 1.f; break;
+        case CQ_VALUE_E2M1: *lo = -6.f; *hi = 6.f; break;
+        case CQ_VALUE_E4M3: *lo = -448.f; *hi = 448.f; break;
+        case CQ_VALUE_E5M2: *lo = -57344.f; *hi = 57344.f; break;
+        default: return CQ_ERR_INVALID_ARGUMENT;
+    }
+    return CQ_OK;
+}
+
+size_t cq_workspace_bytes(const cq_scheme* s, uint64_t /*num_elements*/) {
+    if (!s || s->level != CQ_LEVEL_TENSOR) return 0;
+    return cq::kMaxPartials * sizeof(float);  // abs-max partials of the grid reduction
+}
+
+cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                      const cq_tensor* scale, const cq_tensor* out_scale, const cq_scheme* scheme,
+                      cq_dtype input_dtype) {
+    cq_status st = check_scheme(scheme);
+    if (st != CQ_OK) return st;
+    Plan p;
+    int pd = param_to_dtype(scheme->param);
+    st = make_plan(scheme, input, input_dtype, output, scale, dtype_size(input_dtype), out_scale,
+                   dtype_size(pd), &p);
+    if (st != CQ_OK) return st;
+    if (!out_scale) return CQ_ERR_INVALID_ARGUMENT;
+
+    if (scheme->store == CQ_STORE_NATIVE) {
+        cq::GenericArgs g = generic_args(p, scheme);
+        g.input = input->ptr;
+        g.output = output->ptr;
+        g.scale_in = scale->ptr;
+        g.scale_in_dtype = input_dtype;
+        g.scale_out = out_scale->ptr;
+        g.word_begin = 0;
+        g.word_end = p.n / p.nq;
+        return hip_status(cq::launch_quantize_native(stream, input_dtype, g));
+    }
+
+    const uint64_t per_chunk = 16 / dtype_size(input_dtype);
+    uint64_t flat_words = 0;
+    if (flat_ok(p, input_dtype, input, output, scale, out_scale)) {
+        cq::FlatArgs a{};
+        a.input = input->ptr;
+        a.output = output->ptr;
+        a.scale_in = scale->ptr;
+        a.scale_in_dtype = input_dtype;
+        a.scale_out = out_scale->ptr;
+        // whole chunks that also end on a word boundary
+        uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+        a.num_chunks = (p.n / chunk_elems) * chunk_elems / per_chunk;
+        a.block = p.tensor_level ? 0 : p.block_last;
+        a.param_dtype = pd;
+        a.range = p.range;
+        st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, a));
+        if (st != CQ_OK) return st;
+        flat_words = a.num_chunks * per_chunk / p.nq;
+    }
+    if (flat_words < p.n / p.nq) {
+        cq::GenericArgs g = generic_args(p, scheme);
+        g.input = input->ptr;
+        g.output = output->ptr;
+        g.scale_in = scale->ptr;
+        g.scale_in_dtype = input_dtype;
+        g.scale_out = out_scale->ptr;
+        g.word_begin = flat_words;
+        g.word_end = p.n / p.nq;
+        st = hip_status(cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
+    }
+    return st;
+}
+
+cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_tensor* output,
+                        const cq_tensor* params, const cq_scheme* scheme, cq_dtype output_dtype) {
+    cq_status st = check_scheme(scheme);
+    if (st != CQ_OK) return st;
+    Plan p;
+    int pd = param_to_dtype(scheme->param);
+    st = make_plan(scheme, output, output_dtype, values, params, dtype_size(pd), nullptr, 0, &p);
+    if (st != CQ_OK) return st;
+
+    if (scheme->store == CQ_STORE_NATIVE) {
+        cq::GenericArgs g = generic_args(p, scheme);
+        g.input = values->ptr;
+        g.output = output->ptr;
+        g.scale_in = params->ptr;
+        g.word_begin = 0;
+        g.word_end = p.n / p.nq;
+        return hip_status(cq::launch_dequantize_native(stream, output_dtype, g));
+    }
+
+    const uint64_t per_chunk = 16 / dtype_size(output_dtype);
+    uint64_t flat_words = 0;
+    if (flat_ok(p, output_dtype, output, values, params, nullptr)) {
+        cq::FlatArgs a{};
+        a.input = values->ptr;
+        a.output = output->ptr;
+        a.scale_in = params->ptr;
+        uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+        a.num_chunks = (p.n / chunk_elems) * chunk_elems / per_chunk;
+        a.block = p.tensor_level ? 0 : p.block_last;
+        a.param_dtype = pd;
+        a.range = p.range;
+        st = hip_status(cq::launch_dequantize_flat(stream, output_dtype, p.bits, a));
+        if (st != CQ_OK) return st;
+        flat_words = a.num_chunks * per_chunk / p.nq;
+    }
+    if (flat_words < p.n / p.nq) {
+        cq::GenericArgs g = generic_args(p, scheme);
+        g.input = values->ptr;
+        g.output = output->ptr;
+        g.scale_in = params->ptr;
+        g.word_begin = flat_words;
+        g.word_end = p.n / p.nq;
+        st = hip_status(cq::launch_dequantize_generic(stream, output_dtype, p.bits, g));
+    }
+    return st;
+}
+
+// Shared by cq_compute_scales and cq_quantize_dynamic: scale of every block (or
+// of the tensor) as out_dtype(F(2*absmax/(hi-lo))), written into `scales`.
+static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_scheme* scheme,
+                                const cq_tensor* input, int input_dtype, const cq_tensor* scales,
+                                int out_dtype, void* workspace, size_t workspace_bytes) {
+    if (p.tensor_level) {
+        if (!workspace || workspace_bytes < cq::kMaxPartials * sizeof(float))
+            return CQ_ERR_WORKSPACE_TOO_SMALL;
+        if (!aligned(input->ptr, 16) || !aligned(workspace, 4)) return CQ_ERR_INVALID_ARGUMENT;
+        uint32_t num_partials = 0;
+        cq_status st = hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n,
+                                                             static_cast<float*>(workspace), &num_partials));
+        if (st != CQ_OK) return st;
+        return hip_status(cq::launch_tensor_scale(stream, input_dtype, out_dtype,
+                                                  static_cast<const float*>(workspace), num_partials,
+                                                  p.range, scales->ptr));
+    }
+    cq::GenericArgs g = generic_args(p, scheme);
+    g.input = input->ptr;
+    g.scale_out = scales->ptr;
+    return hip_status(cq::launch_scales_generic(stream, input_dtype, out_dtype, g, p.num_blocks));
+}
+
+cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq_tensor* scales,
+                            const cq_scheme* scheme, cq_dtype input_dtype, void* workspace,
+                            size_t workspace_bytes) {
+    cq_status st = check_scheme(scheme);
+    if (st != CQ_OK) return st;
+    if (!tensor_ok(input) || !tensor_ok(scales) || !valid_dtype(input_dtype)) return CQ_ERR_INVALID_ARGUMENT;
+    // build the plan against a synthetic stored tensor of the right shape
+    uint64_t vshape[CQ_MAX_RANK], vstrides[CQ_MAX_RANK];
+    uint32_t nq = stored_nq(scheme);
+    if (input->shape[input->rank - 1] % nq) return CQ_ERR_SHAPE_MISMATCH;
+    uint64_t acc = 1;
+    for (int d = static_cast<int>(input->rank) - 1; d >= 0; d--) {
+        vshape[d] = d + 1 == static_cast<int>(input->rank) ? input->shape[d] / nq : input->shape[d];
+        vstrides[d] = acc;
+        acc *= vshape[d];
+    }
+    cq_tensor values{input->ptr, vshape, vstrides, input->rank, scheme->store == CQ_STORE_U32 ? 4u : 1u};
+    Plan p;
+    st = make_plan(scheme, input, input_dtype, &values, scales, dtype_size(input_dtype), nullptr, 0, &p);
+    if (st != CQ_OK) return st;
+
+    if (!p.tensor_level && p.last_dim_blocks && is_contiguous(scales) && aligned(input->ptr, 16) &&
+        cq::flat_block_supported(input_dtype, p.block_last)) {
+        cq::FlatArgs a{};
+        a.input = input->ptr;
+        a.scale_out = scales->ptr;
+        a.num_chunks = p.n / (16 / dtype_size(input_dtype));
+        a.block = p.block_last;
+        a.range = p.range;
+        return hip_status(cq::launch_scales_flat(stream, input_dtype, a));
+    }
+    return produce_scales(stream, p, scheme, input, input_dtype, scales, input_dtype, workspace, workspace_bytes);
+}
+
+cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                              const cq_tensor* out_scale, const cq_scheme* scheme, cq_dtype input_dtype,
+                              void* workspace, size_t workspace_bytes) {
+    cq_status st = check_scheme(scheme);
+    if (st != CQ_OK) return st;
+    if (!out_scale) return CQ_ERR_INVALID_ARGUMENT;
+    Plan p;
+    int pd = param_to_dtype(scheme->param);
+    st = make_plan(scheme, input, input_dtype, output, out_scale, dtype_size(pd), nullptr, 0, &p);
+    if (st != CQ_OK) return st;
+
+    const uint64_t per_chunk = 16 / dtype_size(input_dtype);
+    const bool flat = scheme->store == CQ_STORE_U32 && flat_ok(p, input_dtype, input, output, out_scale, nullptr);
+
+    // fused single pass: abs-max, scale, quantize, pack in registers
+    if (flat && !p.tensor_level) {
+        cq::FlatArgs a{};
+        a.input = input->ptr;
+        a.output = output->ptr;
+        a.scale_out = out_scale->ptr;
+        a.num_chunks = p.n / per_chunk;
+        a.block = p.block_last;
+        a.param_dtype = pd;
+        a.range = p.range;
+        return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
+    }
+
+    // two passes: scales as FS(F(scale)) into out_scale, then quantize reading
+    // them back (the divisor F(FS(scale)) is the same either way)
+    st = produce_scales(stream, p, scheme, input, input_dtype, out_scale, pd, workspace, workspace_bytes);
+    if (st != CQ_OK) return st;
+
+    if (scheme->store == CQ_STORE_NATIVE) {
+        cq::GenericArgs g = generic_args(p, scheme);
+        g.input = input->ptr;
+        g.output = output->ptr;
+        g.scale_in = out_scale->ptr;
+        g.scale_in_dtype = pd;
+        g.scale_out = nullptr;
+        g.word_begin = 0;
+        g.word_end = p.n / p.nq;
+        return hip_status(cq::launch_quantize_native(stream, input_dtype, g));
+    }
+
+    uint64_t flat_words = 0;
+    if (flat) {  // per-tensor
+        cq::FlatArgs a{};
+        a.input = input->ptr;
+        a.output = output->ptr;
+        a.scale_in = out_scale->ptr;
+        a.scale_in_dtype = pd;
+        a.scale_out = nullptr;
+        uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+        a.num_chunks = (p.n / chunk_elems) * chunk_elems / per_chunk;
+        a.block = 0;
+        a.param_dtype = pd;
+        a.range = p.range;
+        st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, a));
+        if (st != CQ_OK) return st;
+        flat_words = a.num_chunks * per_chunk / p.nq;
+    }
+    if (flat_words < p.n / p.nq) {
+        cq::GenericArgs g = generic_args(p, scheme);
+        g.input = input->ptr;
+        g.output = output->ptr;
+        g.scale_in = out_scale->ptr;
+        g.scale_in_dtype = pd;
+        g.scale_out = nullptr;
+        g.word_begin = flat_words;
+        g.word_end = p.n / p.nq;
+        st = hip_status(cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
+    }
+    return st;
+}
+
+}  // extern "C"

@@ -1,0 +1,270 @@
+// Device-side building blocks shared by the gfx950 quantize/dequantize kernels.
+//
+// Arithmetic contract (what the reference's kernels compute, restated for one
+// wave): every operation on the tensor's float type F is the f32 operation on
+// the widened operands followed by ONE round-to-nearest-even to F.
+//   quantize  : code = clamp(rint(F(x / d)), lo, hi)      crates/cubek-quant/src/quantize.rs:19-31
+//   pack      : field i at bits [i*bits,(i+1)*bits)        src/quantize.rs:61-81
+//   dequantize: y = F(F(scale) * F(code))                  src/dequantize.rs:22-25,86-118
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/cubek_quant.h"
+
+namespace cq {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float bits_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// ---- element types -------------------------------------------------------
+// A "chunk" is 16 bytes of a float tensor: the unit one lane loads or stores.
+
+struct F32 {
+    static constexpr int kDtype = CQ_F32;
+    static constexpr int kBytes = 4;
+    static constexpr int kPerChunk = 4;
+    __device__ static __forceinline__ float round(float v) { return v; }
+    __device__ static __forceinline__ float load(const void* p, uint64_t i) {
+        return static_cast<const float*>(p)[i];
+    }
+    __device__ static __forceinline__ void store(void* p, uint64_t i, float v) {
+        static_cast<float*>(p)[i] = v;
+    }
+    __device__ static __forceinline__ void unpack(u32x4 raw, float* v) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = bits_f32(raw[j]);
+    }
+    // values already rounded to F
+    __device__ static __forceinline__ u32x4 pack(const float* v) {
+        u32x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; j++) r[j] = f32_bits(v[j]);
+        return r;
+    }
+};
+
+struct BF16 {
+    static constexpr int kDtype = CQ_BF16;
+    static constexpr int kBytes = 2;
+    static constexpr int kPerChunk = 8;
+    __device__ static __forceinline__ uint32_t pack2(float a, float b) {
+        f32x2 v = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, RNE
+    }
+    __device__ static __forceinline__ float round(float v) {
+        return bits_f32(pack2(v, 0.0f) << 16);
+    }
+    __device__ static __forceinline__ float load(const void* p, uint64_t i) {
+        return bits_f32(static_cast<uint32_t>(static_cast<const uint16_t*>(p)[i]) << 16);
+    }
+    __device__ static __forceinline__ void store(void* p, uint64_t i, float v) {
+        static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(pack2(v, 0.0f) & 0xffffu);
+    }
+    __device__ static __forceinline__ void unpack(u32x4 raw, float* v) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v[2 * j] = bits_f32(raw[j] << 16);
+            v[2 * j + 1] = bits_f32(raw[j] & 0xffff0000u);
+        }
+    }
+    __device__ static __forceinline__ u32x4 pack(const float* v) {
+        u32x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; j++) r[j] = pack2(v[2 * j], v[2 * j + 1]);
+        return r;
+    }
+};
+
+struct F16 {
+    static constexpr int kDtype = CQ_F16;
+    static constexpr int kBytes = 2;
+    static constexpr int kPerChunk = 8;
+    __device__ static __forceinline__ float round(float v) {
+        return static_cast<float>(static_cast<_Float16>(v));  // v_cvt_f16_f32 (RNE), widen back
+    }
+    __device__ static __forceinline__ float load(const void* p, uint64_t i) {
+        return static_cast<float>(static_cast<const _Float16*>(p)[i]);
+    }
+    __device__ static __forceinline__ void store(void* p, uint64_t i, float v) {
+        static_cast<_Float16*>(p)[i] = static_cast<_Float16>(v);
+    }
+    __device__ static __forceinline__ void unpack(u32x4 raw, float* v) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t w = raw[j];  // copy first: bit-casting the vector element in place reads lane 0
+            f16x2 h = __builtin_bit_cast(f16x2, w);
+            v[2 * j] = static_cast<float>(h[0]);
+            v[2 * j + 1] = static_cast<float>(h[1]);
+        }
+    }
+    __device__ static __forceinline__ u32x4 pack(const float* v) {
+        u32x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            f16x2 h = {static_cast<_Float16>(v[2 * j]), static_cast<_Float16>(v[2 * j + 1])};
+            r[j] = __builtin_bit_cast(uint32_t, h);
+        }
+        return r;
+    }
+};
+
+// Round an f32 value to a runtime-selected dtype (scale parameters), widened back.
+__device__ __forceinline__ float round_to_dtype(int dtype, float v) {
+    if (dtype == CQ_F32) return v;
+    if (dtype == CQ_BF16) return BF16::round(v);
+    return F16::round(v);
+}
+__device__ __forceinline__ float load_dtype(int dtype, const void* p, uint64_t i) {
+    if (dtype == CQ_F32) return F32::load(p, i);
+    if (dtype == CQ_BF16) return BF16::load(p, i);
+    return F16::load(p, i);
+}
+__device__ __forceinline__ void store_dtype(int dtype, void* p, uint64_t i, float v) {
+    if (dtype == CQ_F32)
+        F32::store(p, i, v);
+    else if (dtype == CQ_BF16)
+        BF16::store(p, i, v);
+    else
+        F16::store(p, i, v);
+}
+
+// ---- cross-lane helpers (64-wide wave, DPP where the pattern allows) -----
+
+template <int kCtrl>
+__device__ __forceinline__ uint32_t dpp(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(
+        static_cast<int>(v), static_cast<int>(v), kCtrl, 0xf, 0xf, false));
+}
+constexpr int kDppXor1 = 0xB1;         // quad_perm:[1,0,3,2]
+constexpr int kDppXor2 = 0x4E;         // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7-i inside each 8 lanes
+constexpr int kDppMirror = 0x140;      // lane i <-> 15-i inside each 16 lanes
+
+// max over aligned groups of kGroup lanes (kGroup a power of two, 1..64); every
+// lane of the group receives the result.  Inputs must be non-negative and not
+// NaN: their bit patterns then order like unsigned integers, which keeps the
+// butterfly free of float canonicalisation.
+template <int kGroup>
+__device__ __forceinline__ float group_max(float v) {
+    uint32_t b = f32_bits(v);
+    if constexpr (kGroup >= 2) b = max(b, dpp<kDppXor1>(b));
+    if constexpr (kGroup >= 4) b = max(b, dpp<kDppXor2>(b));
+    if constexpr (kGroup >= 8) b = max(b, dpp<kDppHalfMirror>(b));
+    if constexpr (kGroup >= 16) b = max(b, dpp<kDppMirror>(b));
+    if constexpr (kGroup >= 32) b = max(b, static_cast<uint32_t>(__shfl_xor(static_cast<int>(b), 16, kWave)));
+    if constexpr (kGroup >= 64) b = max(b, static_cast<uint32_t>(__shfl_xor(static_cast<int>(b), 32, kWave)));
+    return bits_f32(b);
+}
+
+// OR over aligned groups of 2 or 4 lanes (bit-field assembly across lanes).
+template <int kGroup>
+__device__ __forceinline__ uint32_t group_or(uint32_t v) {
+    if constexpr (kGroup >= 2) v |= dpp<kDppXor1>(v);
+    if constexpr (kGroup >= 4) v |= dpp<kDppXor2>(v);
+    return v;
+}
+
+// ---- quantize arithmetic -------------------------------------------------
+
+// Divisors for which x * rcp(d) stays within 2^-21 relative error of x / d:
+// finite, normal and far from the ends of the exponent range (false for NaN).
+__device__ __forceinline__ bool divisor_is_tame(float d) {
+    float a = fabsf(d);
+    return a >= 0x1p-100f && a <= 0x1p100f;
+}
+
+__device__ __forceinline__ float clamp_code(float r, float lo, float hi) {
+    return fmaxf(lo, fminf(r, hi));  // minNum/maxNum: NaN -> hi
+}
+
+// Reference formula, one element, IEEE division.
+template <class F>
+__device__ __forceinline__ float quantize_exact(float x, float d, float lo, float hi) {
+    return clamp_code(__builtin_rintf(F::round(x / d)), lo, hi);
+}
+
+// Quantize kN values of one block (common divisor d) to integer-valued floats.
+//
+// bf16: the correctly rounded bf16 quotient of two bf16 numbers is at least
+//   2^-17 (relative) away from every bf16 rounding boundary, so rounding
+//   x * rcp(d) (error < 2^-21) to bf16 gives the same bits as rounding x / d.
+//   Values far outside [lo,hi] or below 1/4 in magnitude land on the same code
+//   either way, so overflow/underflow of the product is harmless.
+// f32 : rint(x * rcp(d)) can differ from rint(fl(x / d)) only when the product
+//   is within 2^-21 relative of a half-integer; such lanes redo the chunk with
+//   IEEE division.  Clamping to [lo-1/4, hi+1/4] first removes the ties that
+//   clamp anyway and bounds the window by a per-range constant.
+// f16 : IEEE division (the f16 boundaries are too close for the shortcut).
+template <class F, int kN>
+__device__ __forceinline__ void quantize_values(const float* x, float d, float lo, float hi,
+                                                float* q) {
+    if constexpr (F::kDtype == CQ_BF16) {
+        if (divisor_is_tame(d)) {
+            float r = __builtin_amdgcn_rcpf(d);
+#pragma unroll
+            for (int i = 0; i < kN; i += 2) {
+                float a = clamp_code(x[i] * r, lo, hi);
+                float b = clamp_code(x[i + 1] * r, lo, hi);
+                uint32_t p = BF16::pack2(a, b);
+                q[i] = __builtin_rintf(bits_f32(p << 16));
+                q[i + 1] = __builtin_rintf(bits_f32(p & 0xffff0000u));
+            }
+            return;
+        }
+    } else if constexpr (F::kDtype == CQ_F32) {
+        if (divisor_is_tame(d)) {
+            float r = __builtin_amdgcn_rcpf(d);
+            float lo_q = lo - 0.25f, hi_q = hi + 0.25f;
+            float worst = 0.0f;
+#pragma unroll
+            for (int i = 0; i < kN; i++) {
+                float t = clamp_code(x[i] * r, lo_q, hi_q);
+                q[i] = __builtin_rintf(t);
+                worst = fmaxf(worst, fabsf(t - q[i]));
+            }
+            float window = (fmaxf(fabsf(lo), fabsf(hi)) + 1.0f) * 0x1p-21f;
+            if (worst < 0.5f - window) return;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kN; i++) q[i] = quantize_exact<F>(x[i], d, lo, hi);
+}
+
+// Two's-complement bit fields: kN integer-valued floats -> kN*kBits bits,
+// element 0 in the low bits (kN*kBits <= 32).
+template <int kBits, int kN>
+__device__ __forceinline__ uint32_t pack_fields(const float* q) {
+    static_assert(kN * kBits <= 32, "fields must fit one word");
+    constexpr uint32_t kMask = (1u << kBits) - 1u;
+    uint32_t w = 0;
+#pragma unroll
+    for (int i = 0; i < kN; i++) {
+        uint32_t f = static_cast<uint32_t>(static_cast<int32_t>(q[i])) & kMask;
+        w |= f << (i * kBits);
+    }
+    return w;
+}
+
+// Sign-extended field i of a word (v_bfe_i32).
+template <int kBits>
+__device__ __forceinline__ float unpack_field(uint32_t w, int i) {
+    int32_t s = static_cast<int32_t>(w << (32 - kBits - i * kBits)) >> (32 - kBits);
+    return static_cast<float>(s);
+}
+
+// scale = 2*absmax / (hi - lo) in f32 (crates/cubek-quant/tests/suite/symmetric.rs:35-38,176-177)
+__device__ __forceinline__ float scale_from_absmax(float amax, float range_width) {
+    return (2.0f * amax) / range_width;
+}
+
+}  // namespace cq

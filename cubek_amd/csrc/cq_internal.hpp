@@ -1,0 +1,79 @@
+// Host-side interface between the C ABI (cq_abi.hip) and the kernel launchers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/cubek_quant.h"
+
+namespace cq {
+
+// Scale addressing of one launch, the data of the reference's
+// ScalesLayout::{PerTensor,BlockScaled} (crates/cubek-quant/src/layout/scales.rs:15-195).
+struct Layout {
+    uint32_t rank;                   // 0 = per-tensor
+    uint32_t shape[CQ_MAX_RANK];     // unpacked element shape
+    uint32_t block[CQ_MAX_RANK];     // block extents left-padded with 1
+    uint64_t stride_a[CQ_MAX_RANK];  // strides (elements) of `scale` / `params`
+    uint64_t stride_b[CQ_MAX_RANK];  // strides (elements) of `out_scale`
+};
+
+struct Range {
+    float lo, hi;
+};
+
+// Flat fast path: contiguous tensors, scales contiguous, blocks are runs of
+// `block` consecutive elements (block == 0: one scale for the whole tensor).
+struct FlatArgs {
+    const void* input;    // float tensor (quantize) / u32 words (dequantize)
+    void* output;         // u32 words (quantize) / float tensor (dequantize)
+    const void* scale_in; // quantize with given scales (typed scale_in_dtype); dequantize: params
+    int scale_in_dtype;   // cq_dtype of scale_in (quantize only)
+    void* scale_out;      // quantize: out_scale typed as param dtype, NULL = do not write;
+                          // launch_scales_flat: scales typed like the input
+    uint64_t num_chunks;  // 16-byte chunks of the float tensor handled by this launch
+    uint32_t block;       // elements per block, 0 = per-tensor
+    int param_dtype;      // cq_dtype of the stored scales
+    Range range;
+};
+
+enum class ScaleSource { Given, Dynamic };
+
+// every launcher returns hipGetLastError() of its launch
+hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource src, const FlatArgs& a);
+hipError_t launch_dequantize_flat(hipStream_t s, int dtype, int bits, const FlatArgs& a);
+hipError_t launch_scales_flat(hipStream_t s, int dtype, const FlatArgs& a);  // block abs-max -> scales typed like input
+bool flat_block_supported(int dtype, uint32_t block);
+
+// Per-tensor abs-max, pass 1: writes `*num_partials` f32 partial maxima.
+constexpr uint32_t kMaxPartials = 256;
+hipError_t launch_absmax_partials(hipStream_t s, int dtype, const void* input, uint64_t num_elems,
+                                  float* partials, uint32_t* num_partials);
+// Per-tensor scale from the partials: out_dtype(f_dtype(2*absmax/(hi-lo))) stored at out[0].
+hipError_t launch_tensor_scale(hipStream_t s, int f_dtype, int out_dtype, const float* partials,
+                               uint32_t num_partials, Range range, void* out);
+
+// Generic path: any rank, N-D blocks, strided scales; one thread per stored word.
+struct GenericArgs {
+    const void* input;
+    void* output;
+    const void* scale_in;
+    int scale_in_dtype;     // cq_dtype of scale_in (quantize); dequantize reads param_dtype
+    void* scale_out;        // NULL = do not write out_scale
+    uint64_t word_begin, word_end;  // packed words (U32 store) or stored bytes (native store)
+    int param_dtype;
+    int value;  // cq_value
+    Range range;
+    Layout layout;
+};
+hipError_t launch_quantize_generic(hipStream_t s, int dtype, int bits, const GenericArgs& a);
+hipError_t launch_dequantize_generic(hipStream_t s, int dtype, int bits, const GenericArgs& a);
+// one thread per block: abs-max over the N-D block box; stores
+// out_dtype(dtype(2*absmax/(hi-lo))) through layout.stride_b into scale_out
+hipError_t launch_scales_generic(hipStream_t s, int dtype, int out_dtype, const GenericArgs& a,
+                                 uint64_t num_blocks);
+// native store (i8 / e4m3 / e5m2 / e2m1x2), one thread per stored byte
+hipError_t launch_quantize_native(hipStream_t s, int dtype, const GenericArgs& a);
+hipError_t launch_dequantize_native(hipStream_t s, int dtype, const GenericArgs& a);
+
+}  // namespace cq

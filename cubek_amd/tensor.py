@@ -1,0 +1,39 @@
+"""Borrowed tensor handles and the client object of the reference API.
+
+``TensorHandleRef`` carries what the reference's ``TensorHandleRef`` carries —
+device buffer, shape, strides (in elements), element size — and nothing else
+(crates/cubek-quant/src/quantize.rs:234-239, src/layout/scales.rs:213-215).
+``ComputeClient`` stands for ``ComputeClient<R>``: here it is just the HIP
+stream launches are ordered on.  torch is used only to own device memory.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Tuple
+
+
+@dataclass(frozen=True)
+class TensorHandleRef:
+    handle: int                 # device pointer
+    shape: Tuple[int, ...]
+    strides: Tuple[int, ...]    # in elements
+    elem_size: int
+
+    @staticmethod
+    def from_torch(t) -> "TensorHandleRef":
+        """Borrow a torch tensor living on the GPU (no copy, no ownership)."""
+        if not t.is_cuda:
+            raise ValueError("tensor handles must point at device memory")
+        return TensorHandleRef(t.data_ptr(), tuple(t.shape), tuple(t.stride()), t.element_size())
+
+
+@dataclass(frozen=True)
+class ComputeClient:
+    stream: int = 0  # hipStream_t as an integer; 0 = default stream
+
+    @staticmethod
+    def current() -> "ComputeClient":
+        """Client bound to torch's current HIP stream."""
+        import torch
+
+        return ComputeClient(torch.cuda.current_stream().cuda_stream)

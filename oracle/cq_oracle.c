@@ -288,12 +288,15 @@ static inline float quantize_one(float x, float d, int dtype, float lo, float hi
  * Returns the divisor F(FS(scale)) widened to f32. */
 static inline float write_scale(const cq_scheme* s, uint32_t rank, const uint64_t* shape,
                                 const void* scale, const uint64_t* strides, void* out_scale,
-                                int dtype, uint64_t elem) {
+                                const uint64_t* out_strides, int dtype, uint64_t elem) {
     int pd = param_dtype(s->param);
     uint64_t si = cqo_scale_index(s, rank, shape, strides, elem);
     float s_f = load_f(scale, dtype, si);
     float s_fs = round_to(pd, s_f);
-    if (cqo_is_block_start(s, rank, shape, elem)) store_f(out_scale, pd, si, s_fs);
+    /* out_scale is a view of its own: same mapping, its own strides
+     * (scales_view(.., out_scale, ..) at src/quantize.rs:317) */
+    if (cqo_is_block_start(s, rank, shape, elem))
+        store_f(out_scale, pd, cqo_scale_index(s, rank, shape, out_strides, elem), s_fs);
     return round_to(dtype, s_fs);
 }
 
@@ -308,14 +311,15 @@ static uint64_t num_elements(uint32_t rank, const uint64_t* shape) {
 /* quantize_symmetric_packed_kernel (src/quantize.rs:128-171), one word per step */
 int cqo_quantize_packed(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
                         const void* scale, const uint64_t* scale_strides, void* out_scale,
-                        uint32_t* output, const cq_scheme* s, uint64_t word_begin,
-                        uint64_t word_end) {
+                        const uint64_t* out_scale_strides, uint32_t* output, const cq_scheme* s,
+                        uint64_t word_begin, uint64_t word_end) {
     float lo, hi;
     if (s->store != CQ_STORE_U32 || cqo_value_range(s->value, &lo, &hi)) return -1;
     uint32_t bits = cqo_value_size_bits(s->value), nq = 32u / bits;
     for (uint64_t p = word_begin; p < word_end; p++) {
         uint64_t packed_pos = p * nq;
-        float d = write_scale(s, rank, shape, scale, scale_strides, out_scale, dtype, packed_pos);
+        float d = write_scale(s, rank, shape, scale, scale_strides, out_scale, out_scale_strides,
+                              dtype, packed_pos);
         int32_t codes[16];
         for (uint32_t i = 0; i < nq; i++)
             codes[i] = (int32_t)quantize_one(load_f(input, dtype, packed_pos + i), d, dtype, lo, hi);
@@ -353,12 +357,13 @@ int cqo_dequantize_packed(const uint32_t* values, uint32_t rank, const uint64_t*
 /* quantize_symmetric_native_kernel (src/quantize.rs:100-126) */
 int cqo_quantize_native(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
                         const void* scale, const uint64_t* scale_strides, void* out_scale,
-                        uint8_t* output, const cq_scheme* s, uint64_t elem_begin,
-                        uint64_t elem_end) {
+                        const uint64_t* out_scale_strides, uint8_t* output, const cq_scheme* s,
+                        uint64_t elem_begin, uint64_t elem_end) {
     float lo, hi;
     if (s->store != CQ_STORE_NATIVE || cqo_value_range(s->value, &lo, &hi)) return -1;
     for (uint64_t e = elem_begin; e < elem_end; e++) {
-        float d = write_scale(s, rank, shape, scale, scale_strides, out_scale, dtype, e);
+        float d = write_scale(s, rank, shape, scale, scale_strides, out_scale, out_scale_strides,
+                              dtype, e);
         float c = quantize_one(load_f(input, dtype, e), d, dtype, lo, hi);
         switch (s->value) {
             case CQ_VALUE_Q8F: case CQ_VALUE_Q8S: output[e] = (uint8_t)(int8_t)(int32_t)c; break;
@@ -448,6 +453,7 @@ typedef struct {
     const void* scale;
     const uint64_t* strides;
     void* out_scale;
+    const uint64_t* out_strides;
     void* out;
     const cq_scheme* s;
     uint64_t wb, we;
@@ -458,7 +464,8 @@ static void* run_job(void* arg) {
     job_t* j = (job_t*)arg;
     if (j->kind == 0)
         j->rc = cqo_quantize_packed(j->a, j->dtype, j->rank, j->shape, j->scale, j->strides,
-                                    j->out_scale, (uint32_t*)j->out, j->s, j->wb, j->we);
+                                    j->out_scale, j->out_strides, (uint32_t*)j->out, j->s, j->wb,
+                                    j->we);
     else
         j->rc = cqo_dequantize_packed((const uint32_t*)j->a, j->rank, j->shape, j->scale,
                                       j->strides, j->out, j->dtype, j->s, j->wb, j->we);
@@ -494,10 +501,10 @@ static int run_mt(job_t base, int threads) {
 
 int cqo_quantize_packed_mt(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
                            const void* scale, const uint64_t* scale_strides, void* out_scale,
-                           uint32_t* output, const cq_scheme* s, uint64_t word_begin,
-                           uint64_t word_end, int threads) {
-    job_t j = {0, input, dtype, rank, shape, scale, scale_strides, out_scale, output, s,
-               word_begin, word_end, 0};
+                           const uint64_t* out_scale_strides, uint32_t* output, const cq_scheme* s,
+                           uint64_t word_begin, uint64_t word_end, int threads) {
+    job_t j = {0, input, dtype, rank, shape, scale, scale_strides, out_scale, out_scale_strides,
+               output, s, word_begin, word_end, 0};
     return run_mt(j, threads);
 }
 
@@ -505,7 +512,7 @@ int cqo_dequantize_packed_mt(const uint32_t* values, uint32_t rank, const uint64
                              const void* params, const uint64_t* scale_strides, void* output,
                              int dtype, const cq_scheme* s, uint64_t word_begin,
                              uint64_t word_end, int threads) {
-    job_t j = {1, values, dtype, rank, shape, params, scale_strides, NULL, output, s,
+    job_t j = {1, values, dtype, rank, shape, params, scale_strides, NULL, NULL, output, s,
                word_begin, word_end, 0};
     return run_mt(j, threads);
 }

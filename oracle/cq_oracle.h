@@ -43,8 +43,8 @@ void cqo_unpack_word(uint32_t word, uint32_t bits, int32_t* codes);
 /* packed-u32 path; words [word_begin, word_end) only (whole tensor: 0, N/nq) */
 int cqo_quantize_packed(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
                         const void* scale, const uint64_t* scale_strides, void* out_scale,
-                        uint32_t* output, const cq_scheme* scheme, uint64_t word_begin,
-                        uint64_t word_end);
+                        const uint64_t* out_scale_strides, uint32_t* output,
+                        const cq_scheme* scheme, uint64_t word_begin, uint64_t word_end);
 int cqo_dequantize_packed(const uint32_t* values, uint32_t rank, const uint64_t* shape,
                           const void* params, const uint64_t* scale_strides, void* output,
                           int dtype, const cq_scheme* scheme, uint64_t word_begin,
@@ -54,8 +54,8 @@ int cqo_dequantize_packed(const uint32_t* values, uint32_t rank, const uint64_t*
  * elements [elem_begin, elem_end), both even for E2M1 */
 int cqo_quantize_native(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
                         const void* scale, const uint64_t* scale_strides, void* out_scale,
-                        uint8_t* output, const cq_scheme* scheme, uint64_t elem_begin,
-                        uint64_t elem_end);
+                        const uint64_t* out_scale_strides, uint8_t* output,
+                        const cq_scheme* scheme, uint64_t elem_begin, uint64_t elem_end);
 int cqo_dequantize_native(const uint8_t* values, uint32_t rank, const uint64_t* shape,
                           const void* params, const uint64_t* scale_strides, void* output,
                           int dtype, const cq_scheme* scheme, uint64_t elem_begin,
@@ -77,8 +77,9 @@ int cqo_compute_scales(const void* input, int dtype, uint32_t rank, const uint64
 /* threaded drivers used for the CPU baseline timing (split the word range) */
 int cqo_quantize_packed_mt(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
                            const void* scale, const uint64_t* scale_strides, void* out_scale,
-                           uint32_t* output, const cq_scheme* scheme, uint64_t word_begin,
-                           uint64_t word_end, int threads);
+                           const uint64_t* out_scale_strides, uint32_t* output,
+                           const cq_scheme* scheme, uint64_t word_begin, uint64_t word_end,
+                           int threads);
 int cqo_dequantize_packed_mt(const uint32_t* values, uint32_t rank, const uint64_t* shape,
                              const void* params, const uint64_t* scale_strides, void* output,
                              int dtype, const cq_scheme* scheme, uint64_t word_begin,

@@ -72,7 +72,7 @@ def _declare(L):
     L.cqo_pack_word.argtypes = [ctypes.POINTER(ctypes.c_int32), ctypes.c_uint32]
     L.cqo_unpack_word.restype = None
     L.cqo_unpack_word.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(ctypes.c_int32)]
-    q_args = [_vp, ctypes.c_int, ctypes.c_uint32, _u64p, _vp, _u64p, _vp, _vp, _sp,
+    q_args = [_vp, ctypes.c_int, ctypes.c_uint32, _u64p, _vp, _u64p, _vp, _u64p, _vp, _sp,
               ctypes.c_uint64, ctypes.c_uint64]
     d_args = [_vp, ctypes.c_uint32, _u64p, _vp, _u64p, _vp, ctypes.c_int, _sp,
               ctypes.c_uint64, ctypes.c_uint64]
@@ -138,6 +138,15 @@ def from_bits(a: np.ndarray, elem: ElemType) -> np.ndarray:
     return (a.astype(np.uint32) << 16).view(np.float32)
 
 
+def _check_footprint(scheme: QuantScheme, shape, strides, available: int) -> None:
+    """The C side trusts its pointers: refuse scale buffers smaller than the layout reaches."""
+    if scheme.level.is_tensor:
+        assert available >= 1
+        return
+    reach = 1 + sum((n - 1) * st for n, st in zip(scheme.scales_shape(shape), strides))
+    assert reach <= available, f"scale buffer of {available} entries, layout reaches {reach}"
+
+
 # ---------------------------------------------------------------- entry points
 
 def scale_index(scheme: QuantScheme, shape, scale_strides, elem: int) -> int:
@@ -165,9 +174,10 @@ def compute_scales(x: np.ndarray, elem: ElemType, shape, scheme: QuantScheme) ->
 
 
 def quantize(x: np.ndarray, elem: ElemType, shape, scale: np.ndarray, scheme: QuantScheme,
-             scale_strides=None, threads: int = 0):
+             scale_strides=None, threads: int = 0, out_scale_strides=None):
     """Returns (stored values, out_scale).  ``scale`` is typed ``elem``; out_scale
-    is typed scheme.param and has the same (possibly strided) footprint."""
+    is typed scheme.param, as large as ``scale``, addressed with
+    ``out_scale_strides`` (default: the strides of ``scale``)."""
     from cubek_amd.scheme import QuantStore
 
     c = scheme.to_c()
@@ -177,6 +187,11 @@ def quantize(x: np.ndarray, elem: ElemType, shape, scale: np.ndarray, scheme: Qu
         scale_strides = (1,) if scheme.level.is_tensor else contiguous_strides(scheme.scales_shape(shape))
     if scheme.level.is_tensor:
         scale_strides = (0,) * len(shape)
+    if out_scale_strides is None or scheme.level.is_tensor:
+        out_scale_strides = scale_strides
+    _check_footprint(scheme, shape, scale_strides, scale.size)
+    _check_footprint(scheme, shape, out_scale_strides, scale.size)
+    assert x.size == n and x.dtype == np_dtype(elem), "input array does not match shape/dtype"
     out_scale = np.zeros(scale.size, dtype=np_dtype(param_elem(scheme.param)))
     nq = scheme.num_quants()
     if scheme.store == QuantStore.U32:
@@ -184,17 +199,19 @@ def quantize(x: np.ndarray, elem: ElemType, shape, scale: np.ndarray, scheme: Qu
         if threads > 0:
             rc = lib().cqo_quantize_packed_mt(_ptr(x), int(elem), len(shape), _u64(shape),
                                               _ptr(scale), _u64(scale_strides), _ptr(out_scale),
-                                              _ptr(out), ctypes.byref(c), 0, n // nq, threads)
+                                              _u64(out_scale_strides), _ptr(out), ctypes.byref(c),
+                                              0, n // nq, threads)
         else:
             rc = lib().cqo_quantize_packed(_ptr(x), int(elem), len(shape), _u64(shape),
                                            _ptr(scale), _u64(scale_strides), _ptr(out_scale),
-                                           _ptr(out), ctypes.byref(c), 0, n // nq)
+                                           _u64(out_scale_strides), _ptr(out), ctypes.byref(c),
+                                           0, n // nq)
         out = out.reshape(scheme.packed_shape(shape))
     else:
         out = np.zeros(n // nq, dtype=np.uint8)
         rc = lib().cqo_quantize_native(_ptr(x), int(elem), len(shape), _u64(shape), _ptr(scale),
-                                       _u64(scale_strides), _ptr(out_scale), _ptr(out),
-                                       ctypes.byref(c), 0, n)
+                                       _u64(scale_strides), _ptr(out_scale),
+                                       _u64(out_scale_strides), _ptr(out), ctypes.byref(c), 0, n)
         out = out.reshape(scheme.packed_shape(shape))
     if rc:
         raise RuntimeError(f"oracle quantize failed: {rc}")
@@ -213,8 +230,10 @@ def dequantize(values: np.ndarray, shape, params: np.ndarray, elem: ElemType,
         scale_strides = (1,) if scheme.level.is_tensor else contiguous_strides(scheme.scales_shape(shape))
     if scheme.level.is_tensor:
         scale_strides = (0,) * len(shape)
+    _check_footprint(scheme, shape, scale_strides, params.size)
     out = np.zeros(n, dtype=np_dtype(elem))
     nq = scheme.num_quants()
+    assert values.size == n // nq, "stored array does not match shape"
     if scheme.store == QuantStore.U32:
         args = (_ptr(values), len(shape), _u64(shape), _ptr(params), _u64(scale_strides),
                 _ptr(out), int(elem), ctypes.byref(c), 0, n // nq)
