@@ -11,8 +11,9 @@ configurations are measured in short loops and reported under "per_config".
 
 value      = algorithmic bytes of one step / wall time per step  (GB/s, 1e9)
              algorithmic bytes = input once + codes once + scales once, per direction
-roofline   = the quantize kernel alone: algorithmic bytes / its mean HIP-event duration,
-             against the 8 TB/s HBM peak
+roofline   = the quantize kernel alone: algorithmic bytes / its average launch duration
+             over a region of K back-to-back launches between two HIP events on the
+             launch stream, against the 8 TB/s HBM peak
 cpu_baseline = the CPU oracle (oracle/cq_oracle.c, the scalar restatement of the
              reference algorithm) on a bounded row sample of the same tensor
 
@@ -138,19 +139,23 @@ class Path:
         self.dq.launch_ref(self.client, self.hc, self.hy, self.hs, self.scheme, self.elem)
 
 
-def time_kernel(torch, fn, iters, warmup=3):
-    """Mean duration (ms) of one launch, HIP events on the launch stream."""
+def timed_region(torch, fn, launches, warmup=3):
+    """Runs `launches` back-to-back calls of fn between two HIP events on the launch
+    stream (and a host clock bracketed by synchronize).  Returns (event ms per call,
+    wall ms per call).  Timing the region as a whole keeps the ~2.5 us an event pair
+    adds around a single launch out of the per-kernel figure."""
     for _ in range(warmup):
         fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
-    for a, b in evs:
-        a.record()
+    t0 = time.perf_counter()
+    a.record()
+    for _ in range(launches):
         fn()
-        b.record()
+    b.record()
     torch.cuda.synchronize()
-    ts = sorted(a.elapsed_time(b) for a, b in evs)
-    return sum(ts) / len(ts), ts[len(ts) // 2]
+    wall = time.perf_counter() - t0
+    return a.elapsed_time(b) / launches, wall * 1e3 / launches
 
 
 def cpu_baseline(torch, w, path, budget_s=12.0):
@@ -222,29 +227,15 @@ def main():
     step_bytes = 2 * q_bytes
     n = x.numel()
 
-    def step(events=None):
-        if events is not None:
-            events[0].record()
+    def step():
         path.quantize_dynamic()
-        if events is not None:
-            events[1].record()
         path.dequantize()
-        if events is not None:
-            events[2].record()
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        step(evs[k])
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall / args.steps * 1e3
-    q_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
-    d_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
+    # timed region: exactly K steps between synchronize() calls
+    ev_ms, ms_per_step = timed_region(torch, step, args.steps, warmup=args.warmup)
+    # the two kernels of the step, each as its own region of K back-to-back launches
+    q_ms, _ = timed_region(torch, path.quantize_dynamic, args.steps)
+    d_ms, _ = timed_region(torch, path.dequantize, args.steps)
 
     if args.copy_probe:
         for _ in range(3):
@@ -295,7 +286,7 @@ def main():
                    "cache_resident": 2 * b < (256 << 20)}
             for label, fn in (("quantize_dynamic", p.quantize_dynamic), ("quantize_given_scales", p.quantize_given),
                               ("dequantize", p.dequantize)):
-                mean_ms, med_ms = time_kernel(torch, fn, 30)
+                med_ms = sorted(timed_region(torch, fn, 30)[0] for _ in range(3))[1]
                 row[label] = {"ms": round(med_ms, 4), "GBps": round(b / (med_ms * 1e-3) / 1e9, 1),
                               "frac_hbm_peak": round(b / (med_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
             table.append(row)

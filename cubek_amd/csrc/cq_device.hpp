@@ -140,10 +140,14 @@ __device__ __forceinline__ void store_dtype(int dtype, void* p, uint64_t i, floa
 
 // ---- cross-lane helpers (64-wide wave, DPP where the pattern allows) -----
 
+// Reads the lane selected by the DPP control.  bound_ctrl with a zero `old`
+// lets the compiler fold the move into the consuming ALU instruction
+// (v_max_u32_dpp, v_or_b32_dpp); every pattern used here maps active lanes
+// onto active lanes, so the zero is never observed.
 template <int kCtrl>
 __device__ __forceinline__ uint32_t dpp(uint32_t v) {
-    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(
-        static_cast<int>(v), static_cast<int>(v), kCtrl, 0xf, 0xf, false));
+    return static_cast<uint32_t>(
+        __builtin_amdgcn_update_dpp(0, static_cast<int>(v), kCtrl, 0xf, 0xf, true));
 }
 constexpr int kDppXor1 = 0xB1;         // quad_perm:[1,0,3,2]
 constexpr int kDppXor2 = 0x4E;         // quad_perm:[2,3,0,1]
@@ -176,15 +180,36 @@ __device__ __forceinline__ uint32_t group_or(uint32_t v) {
 
 // ---- quantize arithmetic -------------------------------------------------
 
+// Per-launch constants of the value type.
+struct QuantParams {
+    float lo, hi;         // q_min, q_max
+    float width, rwidth;  // q_max - q_min and its correctly rounded reciprocal
+};
+
 // Divisors for which x * rcp(d) stays within 2^-21 relative error of x / d:
 // finite, normal and far from the ends of the exponent range (false for NaN).
 __device__ __forceinline__ bool divisor_is_tame(float d) {
-    float a = fabsf(d);
-    return a >= 0x1p-100f && a <= 0x1p100f;
+    // exponent field in [27, 227): 2^-100 <= |d| < 2^100
+    return ((f32_bits(d) & 0x7fffffffu) - 0x0d800000u) < (0x71800000u - 0x0d800000u);
+}
+// abs-max values for which the scale 2*amax/width (width <= 2^17) and its
+// divisor are tame: 2^-80 <= amax < 2^80.
+__device__ __forceinline__ bool absmax_is_tame(float amax) {
+    return (f32_bits(amax) - 0x17800000u) < (0x67800000u - 0x17800000u);
 }
 
+// Reference clamp: max(lo, min(x, hi)) with minNum/maxNum, so NaN -> hi.
 __device__ __forceinline__ float clamp_code(float r, float lo, float hi) {
-    return fmaxf(lo, fminf(r, hi));  // minNum/maxNum: NaN -> hi
+    return fmaxf(lo, fminf(r, hi));
+}
+// The same function in one instruction, on NEGATED operands: v_med3_f32 returns
+// min3 when an operand is NaN, so med3(-x, -hi, -lo) = -clamp(x) for numbers and
+// -hi for NaN.  Inline asm, because the compiler folds the surrounding negations
+// through the intrinsic (valid for numbers only), which would turn NaN into lo.
+__device__ __forceinline__ float neg_clamp_of_neg(float neg_x, float neg_hi, float neg_lo) {
+    float r;
+    asm("v_med3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(neg_x), "v"(neg_hi), "v"(neg_lo));
+    return r;
 }
 
 // Reference formula, one element, IEEE division.
@@ -193,66 +218,142 @@ __device__ __forceinline__ float quantize_exact(float x, float d, float lo, floa
     return clamp_code(__builtin_rintf(F::round(x / d)), lo, hi);
 }
 
-// Quantize kN values of one block (common divisor d) to integer-valued floats.
+// scale = 2*absmax / (q_max - q_min) in f32
+// (crates/cubek-quant/tests/suite/symmetric.rs:35-38,176-177), IEEE division.
+__device__ __forceinline__ float scale_from_absmax(float amax, float width) {
+    return (2.0f * amax) / width;
+}
+// The same quotient for tame abs-max values without dividing: q = t*(1/w),
+// one FMA for the exact residual t - q*w and one to apply it.  For the nine
+// widths in use (2, 3, 12, 14, 15, 254, 255, 896, 114688) the result equals the
+// IEEE quotient for every f32 significand (checked exhaustively by the tests).
+__device__ __forceinline__ float scale_from_absmax_tame(float amax, const QuantParams& p) {
+    const float t = amax + amax;
+    const float q = t * p.rwidth;
+    const float e = __builtin_fmaf(-q, p.width, t);
+    return __builtin_fmaf(e, p.rwidth, q);
+}
+
+// Quantize kN values of one block (common divisor d).  The result is the
+// NEGATED code of each value as an integer-valued float in [-hi, -lo]
+// (bit-identical to -quantize_exact); the packing step undoes the sign for free.
 //
 // bf16: the correctly rounded bf16 quotient of two bf16 numbers is at least
 //   2^-17 (relative) away from every bf16 rounding boundary, so rounding
 //   x * rcp(d) (error < 2^-21) to bf16 gives the same bits as rounding x / d.
 //   Values far outside [lo,hi] or below 1/4 in magnitude land on the same code
-//   either way, so overflow/underflow of the product is harmless.
+//   either way, so overflow/underflow of the product is harmless.  Clamping
+//   before the bf16 rounding is legal: rounding is monotone, lo and hi are bf16.
 // f32 : rint(x * rcp(d)) can differ from rint(fl(x / d)) only when the product
 //   is within 2^-21 relative of a half-integer; such lanes redo the chunk with
 //   IEEE division.  Clamping to [lo-1/4, hi+1/4] first removes the ties that
 //   clamp anyway and bounds the window by a per-range constant.
 // f16 : IEEE division (the f16 boundaries are too close for the shortcut).
+// Negation commutes with every step (multiply, RNE rounding to bf16, rint).
 template <class F, int kN>
-__device__ __forceinline__ void quantize_values(const float* x, float d, float lo, float hi,
-                                                float* q) {
+__device__ __forceinline__ void quantize_values_neg(const float* x, float d, bool d_tame, float lo,
+                                                    float hi, float* qn) {
     if constexpr (F::kDtype == CQ_BF16) {
-        if (divisor_is_tame(d)) {
-            float r = __builtin_amdgcn_rcpf(d);
+        if (d_tame) {
+            const float nr = -__builtin_amdgcn_rcpf(d);
+            const float nhi = -hi, nlo = -lo;
 #pragma unroll
             for (int i = 0; i < kN; i += 2) {
-                float a = clamp_code(x[i] * r, lo, hi);
-                float b = clamp_code(x[i + 1] * r, lo, hi);
-                uint32_t p = BF16::pack2(a, b);
-                q[i] = __builtin_rintf(bits_f32(p << 16));
-                q[i + 1] = __builtin_rintf(bits_f32(p & 0xffff0000u));
+                const float a = neg_clamp_of_neg(x[i] * nr, nhi, nlo);
+                const float b = neg_clamp_of_neg(x[i + 1] * nr, nhi, nlo);
+                const uint32_t p = BF16::pack2(a, b);
+                qn[i] = __builtin_rintf(bits_f32(p << 16));
+                qn[i + 1] = __builtin_rintf(bits_f32(p & 0xffff0000u));
             }
             return;
         }
     } else if constexpr (F::kDtype == CQ_F32) {
-        if (divisor_is_tame(d)) {
-            float r = __builtin_amdgcn_rcpf(d);
-            float lo_q = lo - 0.25f, hi_q = hi + 0.25f;
+        if (d_tame) {
+            const float nr = -__builtin_amdgcn_rcpf(d);
+            const float nhi_q = -(hi + 0.25f), nlo_q = -(lo - 0.25f);
             float worst = 0.0f;
 #pragma unroll
-            for (int i = 0; i < kN; i++) {
-                float t = clamp_code(x[i] * r, lo_q, hi_q);
-                q[i] = __builtin_rintf(t);
-                worst = fmaxf(worst, fabsf(t - q[i]));
+            for (int i = 0; i < kN; i += 2) {
+                const float t0 = neg_clamp_of_neg(x[i] * nr, nhi_q, nlo_q);
+                const float t1 = neg_clamp_of_neg(x[i + 1] * nr, nhi_q, nlo_q);
+                qn[i] = __builtin_rintf(t0);
+                qn[i + 1] = __builtin_rintf(t1);
+                worst = fmaxf(worst, fmaxf(fabsf(t0 - qn[i]), fabsf(t1 - qn[i + 1])));
             }
-            float window = (fmaxf(fabsf(lo), fabsf(hi)) + 1.0f) * 0x1p-21f;
+            const float window = (fmaxf(fabsf(lo), fabsf(hi)) + 1.0f) * 0x1p-21f;
             if (worst < 0.5f - window) return;
         }
     }
 #pragma unroll
-    for (int i = 0; i < kN; i++) q[i] = quantize_exact<F>(x[i], d, lo, hi);
+    for (int i = 0; i < kN; i++) qn[i] = -quantize_exact<F>(x[i], d, lo, hi);
 }
 
-// Two's-complement bit fields: kN integer-valued floats -> kN*kBits bits,
-// element 0 in the low bits (kN*kBits <= 32).
+// ---- bit packing -----------------------------------------------------------
+
+// Two's-complement bit fields by mask and shift: kN NEGATED integer-valued
+// floats -> kN*kBits bits, element 0 in the low bits.  Values outside the field range
+// wrap, as `i32 & mask` does in the reference (src/quantize.rs:75).
 template <int kBits, int kN>
-__device__ __forceinline__ uint32_t pack_fields(const float* q) {
+__device__ __forceinline__ uint32_t pack_fields_neg(const float* qn) {
     static_assert(kN * kBits <= 32, "fields must fit one word");
     constexpr uint32_t kMask = (1u << kBits) - 1u;
     uint32_t w = 0;
 #pragma unroll
     for (int i = 0; i < kN; i++) {
-        uint32_t f = static_cast<uint32_t>(static_cast<int32_t>(q[i])) & kMask;
+        uint32_t f = static_cast<uint32_t>(-static_cast<int32_t>(qn[i])) & kMask;
         w |= f << (i * kBits);
     }
     return w;
+}
+
+// bias pattern: the digit 2^(kBits-1) repeated over `bits` bits (0x8888.., 0x8080.., 0xAAAA..)
+template <int kBits>
+__host__ __device__ constexpr uint32_t field_bias(int bits) {
+    uint32_t b = 0;
+    for (int i = 0; i < bits; i += kBits) b |= (1u << (kBits - 1)) << i;
+    return b;
+}
+
+// kCount NEGATED integer-valued floats, each code inside the field range
+// [-2^(kBits-1), 2^(kBits-1)-1], -> kCount*kBits (<= 16) bits of BIASED digits
+// (code + 2^(kBits-1)), element 0 lowest, in the low bits of the result; the bits
+// above are garbage.  Horner in f32 is exact (all partial sums are integers below
+// 2^16) and subtracting from 2^23 + bias leaves the integer in the low mantissa
+// bits.  XOR with field_bias turns biased digits into two's-complement fields.
+template <int kBits, int kCount>
+__device__ __forceinline__ uint32_t pack_biased_neg(const float* cn) {
+    static_assert(kBits * kCount <= 16, "exactness needs at most 16 bits per float");
+    float u = cn[kCount - 1];
+#pragma unroll
+    for (int i = kCount - 2; i >= 0; i--) u = __builtin_fmaf(u, static_cast<float>(1 << kBits), cn[i]);
+    constexpr float kMagic = 8388608.0f + static_cast<float>(field_bias<kBits>(kBits * kCount));
+    return f32_bits(kMagic - u);
+}
+
+// The codes of one 16-byte chunk (given negated) as two's-complement fields.  kChunkBits = kN*kBits:
+//   64 -> w[0], w[1]; 32 -> w[0]; 16 / 8 -> low bits of w[0], upper bits zero.
+// kWide: the value range exceeds the field (E4M3/E5M2 in 8-bit fields), fields wrap.
+template <int kBits, int kN, bool kWide>
+__device__ __forceinline__ void pack_chunk_neg(const float* c, uint32_t* w) {
+    constexpr int kChunkBits = kN * kBits;
+    if constexpr (kWide) {
+        if constexpr (kChunkBits == 64) {
+            w[0] = pack_fields_neg<kBits, 4>(c);
+            w[1] = pack_fields_neg<kBits, 4>(c + 4);
+        } else {
+            w[0] = pack_fields_neg<kBits, kN>(c);
+        }
+    } else if constexpr (kChunkBits >= 32) {
+        constexpr int kPerHalf = 16 / kBits;
+#pragma unroll
+        for (int j = 0; j < kChunkBits / 32; j++) {
+            const uint32_t lo16 = pack_biased_neg<kBits, kPerHalf>(c + 2 * j * kPerHalf);
+            const uint32_t hi16 = pack_biased_neg<kBits, kPerHalf>(c + (2 * j + 1) * kPerHalf);
+            w[j] = __builtin_amdgcn_perm(hi16, lo16, 0x05040100u) ^ field_bias<kBits>(32);
+        }
+    } else {
+        w[0] = (pack_biased_neg<kBits, kN>(c) & ((1u << kChunkBits) - 1u)) ^ field_bias<kBits>(kChunkBits);
+    }
 }
 
 // Sign-extended field i of a word (v_bfe_i32).
@@ -260,11 +361,6 @@ template <int kBits>
 __device__ __forceinline__ float unpack_field(uint32_t w, int i) {
     int32_t s = static_cast<int32_t>(w << (32 - kBits - i * kBits)) >> (32 - kBits);
     return static_cast<float>(s);
-}
-
-// scale = 2*absmax / (hi - lo) in f32 (crates/cubek-quant/tests/suite/symmetric.rs:35-38,176-177)
-__device__ __forceinline__ float scale_from_absmax(float amax, float range_width) {
-    return (2.0f * amax) / range_width;
 }
 
 }  // namespace cq

@@ -1,8 +1,6 @@
 """``cubek_quant::dequantize`` for MI355X (crates/cubek-quant/src/dequantize.rs:171-178)."""
 from __future__ import annotations
 
-import ctypes
-
 from . import _ffi
 from .scheme import ElemType, QuantScheme
 from .tensor import ComputeClient, TensorHandleRef
@@ -12,10 +10,7 @@ def launch_ref(client: ComputeClient, values: TensorHandleRef, output: TensorHan
                params: TensorHandleRef, scheme: QuantScheme, input_dtype: ElemType) -> None:
     """Convert the quantized ``values`` back to floats of type ``input_dtype``
     (the reference names the output float type ``input_dtype``)."""
-    L = _ffi.lib()
-    cv, k1 = _ffi.make_tensor(values.handle, values.shape, values.strides, values.elem_size)
-    co, k2 = _ffi.make_tensor(output.handle, output.shape, output.strides, output.elem_size)
-    cp, k3 = _ffi.make_tensor(params.handle, params.shape, params.strides, params.elem_size)
-    cs = scheme.to_c()
-    _ffi.check(L.cq_dequantize(ctypes.c_void_p(client.stream), ctypes.byref(cv), ctypes.byref(co),
-                               ctypes.byref(cp), ctypes.byref(cs), int(input_dtype)))
+    rc = _ffi.lib().cq_dequantize(client.stream, values.as_c(), output.as_c(), params.as_c(),
+                                  scheme.to_c(), int(input_dtype))
+    if rc:
+        _ffi.check(rc)

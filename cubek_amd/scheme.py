@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import enum
+import functools
 from dataclasses import dataclass, replace
 from typing import Sequence, Tuple
 
@@ -201,6 +202,10 @@ class QuantScheme:
         return self.native_packing()
 
     def to_c(self) -> _CScheme:
+        """The ``cq_scheme`` struct (cached per scheme value; treat it as read-only)."""
+        return _scheme_to_c(self)
+
+    def _build_c(self) -> _CScheme:
         c = _CScheme()
         c.value, c.param, c.store = int(self.value), int(self.param), int(self.store)
         c.level = 0 if self.level.is_tensor else 1
@@ -213,6 +218,7 @@ class QuantScheme:
         return c
 
     # ---- host-side shape helpers used by callers and tests ----
+
 
     def packed_shape(self, shape: Sequence[int]) -> Tuple[int, ...]:
         """Shape of the quantized tensor in stored elements: last dim / num_quants."""
@@ -232,3 +238,8 @@ class QuantScheme:
                 raise ValueError(f"dimension {s} is not a multiple of its block size {b}")
             out.append(s // b)
         return tuple(out)
+
+
+@functools.lru_cache(maxsize=256)
+def _scheme_to_c(scheme: QuantScheme) -> _CScheme:
+    return scheme._build_c()

@@ -8,7 +8,7 @@ stream launches are ordered on.  torch is used only to own device memory.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Tuple
 
 
@@ -18,6 +18,15 @@ class TensorHandleRef:
     shape: Tuple[int, ...]
     strides: Tuple[int, ...]    # in elements
     elem_size: int
+    _c: list = field(default_factory=list, repr=False, compare=False)  # cached cq_tensor + its arrays
+
+    def as_c(self):
+        """The ``cq_tensor`` view of this handle (built once, reused by every launch)."""
+        if not self._c:
+            from . import _ffi
+
+            self._c.extend(_ffi.make_tensor(self.handle, self.shape, self.strides, self.elem_size))
+        return self._c[0]
 
     @staticmethod
     def from_torch(t) -> "TensorHandleRef":

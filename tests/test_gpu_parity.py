@@ -395,3 +395,43 @@ def test_error_codes(gpu):
     # wrong element size for the declared dtype
     assert status(lambda: qz.launch_ref(client, h(x), h(out), h(sc), h(sc.clone()), ok, ElemType.BF16)) \
         == _ffi.ERR_SHAPE_MISMATCH
+
+
+def test_scale_division_all_significands(gpu):
+    """The kernels divide 2*absmax by the range width with a reciprocal and one
+    residual correction.  Every f32 significand, at three exponents, for every
+    value type, against numpy's IEEE division."""
+    import torch
+    from cubek_amd import ComputeClient, TensorHandleRef
+    from cubek_amd import quantize as qz
+
+    client = ComputeClient.current()
+    sig = np.arange(1 << 23, dtype=np.uint32)
+    for value in ALL_VALUES:
+        lo, hi = value.range()
+        width = np.float32(hi - lo)
+        nq = 32 // value.size_bits()
+        scheme = QuantScheme.default().with_value(value).with_level(QuantLevel.block([nq]))
+        for exp_field in (127, 100, 140):
+            amax = (sig | np.uint32(exp_field << 23)).view(np.float32)
+            want = (amax + amax) / width
+            slices = nq // 4
+            per = (1 << 23) // slices
+            for k in range(slices):
+                a = torch.from_numpy(amax[k * per:(k + 1) * per]).cuda()
+                x = torch.zeros((per, nq), dtype=torch.float32, device="cuda")
+                x[:, 1] = a            # the block's abs-max ...
+                x[:, nq - 1] = -a / 2  # ... and a smaller negative value
+                scales = torch.zeros((per, 1), dtype=torch.float32, device="cuda")
+                qz.compute_scales(client, TensorHandleRef.from_torch(x), TensorHandleRef.from_torch(scales),
+                                  scheme, ElemType.F32)
+                codes = torch.zeros((per, 1), dtype=torch.int32, device="cuda")
+                out_scale = torch.zeros((per, 1), dtype=torch.float32, device="cuda")
+                qz.launch_dynamic(client, TensorHandleRef.from_torch(x), TensorHandleRef.from_torch(codes),
+                                  TensorHandleRef.from_torch(out_scale), scheme, ElemType.F32)
+                torch.cuda.synchronize()
+                ref = want[k * per:(k + 1) * per]
+                assert np.array_equal(scales.cpu().numpy().reshape(-1).view(np.uint32), ref.view(np.uint32)), \
+                    (value, exp_field, k)
+                assert np.array_equal(out_scale.cpu().numpy().reshape(-1).view(np.uint32), ref.view(np.uint32)), \
+                    (value, exp_field, k)
