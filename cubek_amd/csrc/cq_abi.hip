@@ -177,6 +177,17 @@ bool flat_ok(const Plan& p, int dtype, const cq_tensor* floats, const cq_tensor*
     return cq::flat_block_supported(dtype, p.block_last);
 }
 
+// Stored encoding of the flat kernels (cq::Encoding) and the field width they see.
+int flat_encoding(const cq_scheme* s) {
+    if (s->store == CQ_STORE_U32) return 0;
+    switch (s->value) {
+        case CQ_VALUE_E4M3: return 1;
+        case CQ_VALUE_E5M2: return 2;
+        case CQ_VALUE_E2M1: return 3;
+        default: return 0;  // native i8: the bytes of 8-bit two's-complement fields
+    }
+}
+
 cq::GenericArgs generic_args(const Plan& p, const cq_scheme* s) {
     cq::GenericArgs g;
     std::memset(&g, 0, sizeof(g));
@@ -251,18 +262,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     if (st != CQ_OK) return st;
     if (!out_scale) return CQ_ERR_INVALID_ARGUMENT;
 
-    if (scheme->store == CQ_STORE_NATIVE) {
-        cq::GenericArgs g = generic_args(p, scheme);
-        g.input = input->ptr;
-        g.output = output->ptr;
-        g.scale_in = scale->ptr;
-        g.scale_in_dtype = input_dtype;
-        g.scale_out = out_scale->ptr;
-        g.word_begin = 0;
-        g.word_end = p.n / p.nq;
-        return hip_status(cq::launch_quantize_native(stream, input_dtype, g));
-    }
-
+    const bool native = scheme->store == CQ_STORE_NATIVE;
     const uint64_t per_chunk = 16 / dtype_size(input_dtype);
     uint64_t flat_words = 0;
     if (flat_ok(p, input_dtype, input, output, scale, out_scale)) {
@@ -272,11 +272,12 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         a.scale_in = scale->ptr;
         a.scale_in_dtype = input_dtype;
         a.scale_out = out_scale->ptr;
-        // whole chunks that also end on a word boundary
+        // whole chunks that also end on a stored-element boundary
         uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
         a.num_chunks = (p.n / chunk_elems) * chunk_elems / per_chunk;
         a.block = p.tensor_level ? 0 : p.block_last;
         a.param_dtype = pd;
+        a.encoding = flat_encoding(scheme);
         a.range = p.range;
         st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, a));
         if (st != CQ_OK) return st;
@@ -291,7 +292,8 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         g.scale_out = out_scale->ptr;
         g.word_begin = flat_words;
         g.word_end = p.n / p.nq;
-        st = hip_status(cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
+        st = hip_status(native ? cq::launch_quantize_native(stream, input_dtype, g)
+                               : cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
     }
     return st;
 }
@@ -305,16 +307,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
     st = make_plan(scheme, output, output_dtype, values, params, dtype_size(pd), nullptr, 0, &p);
     if (st != CQ_OK) return st;
 
-    if (scheme->store == CQ_STORE_NATIVE) {
-        cq::GenericArgs g = generic_args(p, scheme);
-        g.input = values->ptr;
-        g.output = output->ptr;
-        g.scale_in = params->ptr;
-        g.word_begin = 0;
-        g.word_end = p.n / p.nq;
-        return hip_status(cq::launch_dequantize_native(stream, output_dtype, g));
-    }
-
+    const bool native = scheme->store == CQ_STORE_NATIVE;
     const uint64_t per_chunk = 16 / dtype_size(output_dtype);
     uint64_t flat_words = 0;
     if (flat_ok(p, output_dtype, output, values, params, nullptr)) {
@@ -326,6 +319,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         a.num_chunks = (p.n / chunk_elems) * chunk_elems / per_chunk;
         a.block = p.tensor_level ? 0 : p.block_last;
         a.param_dtype = pd;
+        a.encoding = flat_encoding(scheme);
         a.range = p.range;
         st = hip_status(cq::launch_dequantize_flat(stream, output_dtype, p.bits, a));
         if (st != CQ_OK) return st;
@@ -338,7 +332,8 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         g.scale_in = params->ptr;
         g.word_begin = flat_words;
         g.word_end = p.n / p.nq;
-        st = hip_status(cq::launch_dequantize_generic(stream, output_dtype, p.bits, g));
+        st = hip_status(native ? cq::launch_dequantize_native(stream, output_dtype, g)
+                               : cq::launch_dequantize_generic(stream, output_dtype, p.bits, g));
     }
     return st;
 }
@@ -412,7 +407,8 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
     if (st != CQ_OK) return st;
 
     const uint64_t per_chunk = 16 / dtype_size(input_dtype);
-    const bool flat = scheme->store == CQ_STORE_U32 && flat_ok(p, input_dtype, input, output, out_scale, nullptr);
+    const bool native = scheme->store == CQ_STORE_NATIVE;
+    const bool flat = flat_ok(p, input_dtype, input, output, out_scale, nullptr);
 
     // fused single pass: abs-max, scale, quantize, pack in registers
     if (flat && !p.tensor_level) {
@@ -423,6 +419,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         a.num_chunks = p.n / per_chunk;
         a.block = p.block_last;
         a.param_dtype = pd;
+        a.encoding = flat_encoding(scheme);
         a.range = p.range;
         return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
     }
@@ -431,18 +428,6 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
     // them back (the divisor F(FS(scale)) is the same either way)
     st = produce_scales(stream, p, scheme, input, input_dtype, out_scale, pd, workspace, workspace_bytes);
     if (st != CQ_OK) return st;
-
-    if (scheme->store == CQ_STORE_NATIVE) {
-        cq::GenericArgs g = generic_args(p, scheme);
-        g.input = input->ptr;
-        g.output = output->ptr;
-        g.scale_in = out_scale->ptr;
-        g.scale_in_dtype = pd;
-        g.scale_out = nullptr;
-        g.word_begin = 0;
-        g.word_end = p.n / p.nq;
-        return hip_status(cq::launch_quantize_native(stream, input_dtype, g));
-    }
 
     uint64_t flat_words = 0;
     if (flat) {  // per-tensor
@@ -456,6 +441,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         a.num_chunks = (p.n / chunk_elems) * chunk_elems / per_chunk;
         a.block = 0;
         a.param_dtype = pd;
+        a.encoding = flat_encoding(scheme);
         a.range = p.range;
         st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, a));
         if (st != CQ_OK) return st;
@@ -470,7 +456,8 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         g.scale_out = nullptr;
         g.word_begin = flat_words;
         g.word_end = p.n / p.nq;
-        st = hip_status(cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
+        st = hip_status(native ? cq::launch_quantize_native(stream, input_dtype, g)
+                               : cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
     }
     return st;
 }

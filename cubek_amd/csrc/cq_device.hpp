@@ -11,6 +11,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/cubek_quant.h"
 
 namespace cq {
@@ -22,6 +24,16 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kWave = 64;
+
+// Compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(<kCount-1>) — for
+// builtins whose selector operands must be constants.
+template <int kBegin, int kCount, class Fn>
+__device__ __forceinline__ void static_for(Fn&& f) {
+    if constexpr (kCount > 0) {
+        f(std::integral_constant<int, kBegin>{});
+        static_for<kBegin + 1, kCount - 1>(f);
+    }
+}
 
 __device__ __forceinline__ float bits_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
@@ -361,6 +373,65 @@ template <int kBits>
 __device__ __forceinline__ float unpack_field(uint32_t w, int i) {
     int32_t s = static_cast<int32_t>(w << (32 - kBits - i * kBits)) >> (32 - kBits);
     return static_cast<float>(s);
+}
+
+// ---- stored encodings --------------------------------------------------------
+// How one quantized value is stored.  kEncInt: two's-complement field (the U32
+// store of every value type, and the native i8 store, whose bytes coincide with
+// 8-bit fields).  The float encodings are the native store's e4m3 / e5m2 bytes
+// and e2m1 nibbles (element 2k in the low nibble), produced by the gfx950
+// conversion instructions from the already rounded and clamped integer, as the
+// reference's `Q::cast_from(clamp(round(x/scale)))` does (src/quantize.rs:33-43).
+enum Encoding : int { kEncInt = 0, kEncE4M3 = 1, kEncE5M2 = 2, kEncE2M1 = 3 };
+
+template <int kEnc>
+constexpr int encoding_bits(int int_bits) {
+    return kEnc == kEncInt ? int_bits : (kEnc == kEncE2M1 ? 4 : 8);
+}
+
+// kN negated integer-valued floats -> kN stored values, same word layout as pack_chunk_neg.
+template <int kEnc, int kN>
+__device__ __forceinline__ void encode_chunk_neg(const float* qn, uint32_t* w) {
+    if constexpr (kEnc == kEncE2M1) {
+        uint32_t r = 0;
+        static_for<0, kN / 2>([&](auto byte) {
+            constexpr int b = decltype(byte)::value;
+            r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, -qn[2 * b], -qn[2 * b + 1], 1.0f, b);
+        });
+        w[0] = r;
+    } else {
+#pragma unroll
+        for (int j = 0; j < kN / 4; j++) {
+            int r = 0;
+            if constexpr (kEnc == kEncE4M3) {
+                r = __builtin_amdgcn_cvt_pk_fp8_f32(-qn[4 * j], -qn[4 * j + 1], r, false);
+                r = __builtin_amdgcn_cvt_pk_fp8_f32(-qn[4 * j + 2], -qn[4 * j + 3], r, true);
+            } else {
+                r = __builtin_amdgcn_cvt_pk_bf8_f32(-qn[4 * j], -qn[4 * j + 1], r, false);
+                r = __builtin_amdgcn_cvt_pk_bf8_f32(-qn[4 * j + 2], -qn[4 * j + 3], r, true);
+            }
+            w[j] = static_cast<uint32_t>(r);
+        }
+    }
+}
+
+// Stored values 0..kCount-1 of a word as floats.
+template <int kEnc, int kBits, int kCount>
+__device__ __forceinline__ void decode_fields(uint32_t w, float* v) {
+    static_for<0, kCount>([&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        if constexpr (kEnc == kEncInt) {
+            v[i] = unpack_field<kBits>(w, i);
+        } else if constexpr (kEnc == kEncE4M3) {
+            v[i] = __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(w), i);
+        } else if constexpr (kEnc == kEncE5M2) {
+            v[i] = __builtin_amdgcn_cvt_f32_bf8(static_cast<int>(w), i);
+        } else if constexpr ((i & 1) == 0) {
+            f32x2 p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, i / 2);
+            v[i] = p[0];
+            v[i + 1] = p[1];
+        }
+    });
 }
 
 }  // namespace cq

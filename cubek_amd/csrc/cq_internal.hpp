@@ -34,6 +34,7 @@ struct FlatArgs {
     uint64_t num_chunks;  // 16-byte chunks of the float tensor handled by this launch
     uint32_t block;       // elements per block, 0 = per-tensor
     int param_dtype;      // cq_dtype of the stored scales
+    int encoding;         // 0 two's-complement fields (U32 store, native i8); 1 e4m3, 2 e5m2 bytes; 3 e2m1 nibbles
     Range range;
 };
 

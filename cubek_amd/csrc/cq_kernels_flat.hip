@@ -58,60 +58,92 @@ hipError_t launch_tiles(uint64_t num_chunks, int unroll, LaunchFn launch) {
     return hipSuccess;
 }
 
-template <class F, int kBits, int kGroup, int kSrc, bool kWide>
+template <class F, int kBits, int kGroup, int kSrc, bool kWide, int kEnc>
 hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
-    auto in = static_cast<const u32x4*>(a.input);
-    auto out = static_cast<uint32_t*>(a.output);
-    const QuantParams qp = quant_params(a.range);
-    const bool p32 = a.param_dtype == CQ_F32;
-    return launch_tiles(a.num_chunks, kUnrollQ, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
-        auto kernel =
-            checked ? (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, true>
-                           : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, true>)
-                    : (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false>
-                           : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false>);
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
-                           a.param_dtype, begin, end, qp);
-    });
+    // scale sources that exist: per-block launches compute the scale or read the
+    // input-typed tensor; per-tensor launches read one scale of either type
+    if constexpr ((kGroup == 0 && kSrc == kScaleDynamic) || (kGroup != 0 && kSrc == kScaleGivenParam)) {
+        return hipErrorInvalidValue;
+    } else {
+        auto in = static_cast<const u32x4*>(a.input);
+        auto out = static_cast<uint32_t*>(a.output);
+        const QuantParams qp = quant_params(a.range);
+        const bool p32 = a.param_dtype == CQ_F32;
+        return launch_tiles(a.num_chunks, kUnrollQ, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
+            auto kernel =
+                checked ? (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, true, kEnc>
+                               : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, true, kEnc>)
+                        : (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false, kEnc>
+                               : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false, kEnc>);
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
+                               a.param_dtype, begin, end, qp);
+        });
+    }
 }
 
-template <class F, int kBits, int kGroup>
-hipError_t quantize_launch(hipStream_t s, ScaleSource src, const FlatArgs& a) {
-    // only 8-bit fields can be narrower than their value range (E4M3, E5M2)
-    const bool wide = kBits == 8 && (a.range.hi > 127.0f || a.range.lo < -128.0f);
-    if (src == ScaleSource::Dynamic) {
-        if constexpr (kGroup > 0) {
-            if constexpr (kBits == 8)
-                if (wide) return quantize_launch_src<F, kBits, kGroup, kScaleDynamic, true>(s, a);
-            return quantize_launch_src<F, kBits, kGroup, kScaleDynamic, false>(s, a);
-        } else {
-            return hipErrorInvalidValue;
-        }
-    } else if (a.scale_in_dtype == F::kDtype) {
-        if constexpr (kBits == 8)
-            if (wide) return quantize_launch_src<F, kBits, kGroup, kScaleGivenF, true>(s, a);
-        return quantize_launch_src<F, kBits, kGroup, kScaleGivenF, false>(s, a);
-    } else if (a.scale_in_dtype == a.param_dtype) {
-        if constexpr (kBits == 8)
-            if (wide) return quantize_launch_src<F, kBits, kGroup, kScaleGivenParam, true>(s, a);
-        return quantize_launch_src<F, kBits, kGroup, kScaleGivenParam, false>(s, a);
-    }
+template <class F, int kBits, int kGroup, bool kWide, int kEnc>
+hipError_t quantize_launch_enc(hipStream_t s, ScaleSource src, const FlatArgs& a) {
+    if (src == ScaleSource::Dynamic) return quantize_launch_src<F, kBits, kGroup, kScaleDynamic, kWide, kEnc>(s, a);
+    // a scale typed like the input is read as such (identical to the param reading when both types agree)
+    if (a.scale_in_dtype == F::kDtype) return quantize_launch_src<F, kBits, kGroup, kScaleGivenF, kWide, kEnc>(s, a);
+    if (a.scale_in_dtype == a.param_dtype)
+        return quantize_launch_src<F, kBits, kGroup, kScaleGivenParam, kWide, kEnc>(s, a);
     return hipErrorInvalidValue;
 }
 
 template <class F, int kBits, int kGroup>
-hipError_t dequantize_launch(hipStream_t s, const FlatArgs& a) {
+hipError_t quantize_launch(hipStream_t s, ScaleSource src, const FlatArgs& a) {
+    switch (a.encoding) {
+        case kEncInt: {
+            // only 8-bit fields can be narrower than their value range (E4M3, E5M2)
+            const bool wide = kBits == 8 && (a.range.hi > 127.0f || a.range.lo < -128.0f);
+            if constexpr (kBits == 8)
+                if (wide) return quantize_launch_enc<F, kBits, kGroup, true, kEncInt>(s, src, a);
+            return quantize_launch_enc<F, kBits, kGroup, false, kEncInt>(s, src, a);
+        }
+        case kEncE4M3:
+            if constexpr (kBits == 8) return quantize_launch_enc<F, 8, kGroup, false, kEncE4M3>(s, src, a);
+            break;
+        case kEncE5M2:
+            if constexpr (kBits == 8) return quantize_launch_enc<F, 8, kGroup, false, kEncE5M2>(s, src, a);
+            break;
+        case kEncE2M1:
+            if constexpr (kBits == 4) return quantize_launch_enc<F, 4, kGroup, false, kEncE2M1>(s, src, a);
+            break;
+    }
+    return hipErrorInvalidValue;
+}
+
+template <class F, int kBits, int kGroup, int kEnc>
+hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
     auto in = static_cast<const uint32_t*>(a.input);
     auto out = static_cast<u32x4*>(a.output);
     const bool p32 = a.param_dtype == CQ_F32;
     return launch_tiles(a.num_chunks, kUnrollD<F>, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
         auto kernel =
-            checked ? (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F>, kThreads, true>
-                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F>, kThreads, true>)
-                    : (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F>, kThreads, false>
-                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F>, kThreads, false>);
+            checked ? (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F>, kThreads, true, kEnc>
+                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F>, kThreads, true, kEnc>)
+                    : (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F>, kThreads, false, kEnc>
+                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F>, kThreads, false, kEnc>);
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, begin, end);
     });
+}
+
+template <class F, int kBits, int kGroup>
+hipError_t dequantize_launch(hipStream_t s, const FlatArgs& a) {
+    switch (a.encoding) {
+        case kEncInt: return dequantize_launch_enc<F, kBits, kGroup, kEncInt>(s, a);
+        case kEncE4M3:
+            if constexpr (kBits == 8) return dequantize_launch_enc<F, 8, kGroup, kEncE4M3>(s, a);
+            break;
+        case kEncE5M2:
+            if constexpr (kBits == 8) return dequantize_launch_enc<F, 8, kGroup, kEncE5M2>(s, a);
+            break;
+        case kEncE2M1:
+            if constexpr (kBits == 4) return dequantize_launch_enc<F, 4, kGroup, kEncE2M1>(s, a);
+            break;
+    }
+    return hipErrorInvalidValue;
 }
 
 template <class F, int kGroup>

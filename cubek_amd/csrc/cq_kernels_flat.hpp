@@ -30,8 +30,10 @@ enum ScaleSrc : int {
 // kWide    : the value range does not fit its field (E4M3 / E5M2 in 8 bits).
 // kChecked : the launch may run past `chunk_end` (ragged last tile): addresses
 //            are clamped and stores masked.  Full tiles use the unchecked variant.
+// kEnc     : stored encoding (kEncInt for the U32 store and native i8; e4m3 / e5m2 /
+//            e2m1 for the native float stores, where kBits is the stored width).
 template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
-          int kThreads, bool kChecked>
+          int kThreads, bool kChecked, int kEnc = kEncInt>
 __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
     void* __restrict__ scale_out, int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end,
@@ -98,7 +100,10 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
         float qn[kN];  // negated codes
         quantize_values_neg<F, kN>(v, d, tame, qp.lo, qp.hi, qn);
         uint32_t w[2];
-        pack_chunk_neg<kBits, kN, kWide>(qn, w);
+        if constexpr (kEnc == kEncInt)
+            pack_chunk_neg<kBits, kN, kWide>(qn, w);
+        else
+            encode_chunk_neg<kEnc, kN>(qn, w);
 
         if constexpr (kChunkBits == 64) {
             if (live) __builtin_nontemporal_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(out) + c);
@@ -113,7 +118,8 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
     }
 }
 
-template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked>
+template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked,
+          int kEnc = kEncInt>
 __global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
     const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params,
     int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end) {
@@ -150,15 +156,13 @@ __global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
         const uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
         float y[kN];
         if constexpr (kChunkBits == 64) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                y[i] = sc[u] * unpack_field<kBits>(w0[u], i);
-                y[i + 4] = sc[u] * unpack_field<kBits>(w1[u], i);
-            }
+            decode_fields<kEnc, kBits, 4>(w0[u], y);
+            decode_fields<kEnc, kBits, 4>(w1[u], y + 4);
         } else {
-#pragma unroll
-            for (int i = 0; i < kN; i++) y[i] = sc[u] * unpack_field<kBits>(w0[u], i);
+            decode_fields<kEnc, kBits, kN>(w0[u], y);
         }
+#pragma unroll
+        for (int i = 0; i < kN; i++) y[i] = sc[u] * y[i];
         if (!kChecked || c < chunk_end) __builtin_nontemporal_store(F::pack(y), out + c);  // pack rounds to F
     }
 }
