@@ -424,28 +424,38 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
     }
 
-    // two passes: scales as FS(F(scale)) into out_scale, then quantize reading
-    // them back (the divisor F(FS(scale)) is the same either way)
-    st = produce_scales(stream, p, scheme, input, input_dtype, out_scale, pd, workspace, workspace_bytes);
-    if (st != CQ_OK) return st;
-
     uint64_t flat_words = 0;
-    if (flat) {  // per-tensor
+    const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+    const uint64_t flat_chunks = flat ? (p.n / chunk_elems) * chunk_elems / per_chunk : 0;
+    if (p.tensor_level && flat_chunks > 0) {
+        // per tensor, two-pass grid reduction: pass 1 leaves one abs-max per workgroup in
+        // the workspace; pass 2 (the quantize kernel) reduces those, derives the scale,
+        // writes out_scale[0] and quantizes
+        if (!workspace || workspace_bytes < cq::kMaxPartials * sizeof(float)) return CQ_ERR_WORKSPACE_TOO_SMALL;
+        if (!aligned(workspace, 4)) return CQ_ERR_INVALID_ARGUMENT;
+        uint32_t num_partials = 0;
+        st = hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n,
+                                                   static_cast<float*>(workspace), &num_partials));
+        if (st != CQ_OK) return st;
         cq::FlatArgs a{};
         a.input = input->ptr;
         a.output = output->ptr;
-        a.scale_in = out_scale->ptr;
-        a.scale_in_dtype = pd;
-        a.scale_out = nullptr;
-        uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
-        a.num_chunks = (p.n / chunk_elems) * chunk_elems / per_chunk;
+        a.scale_in = workspace;
+        a.num_partials = num_partials;
+        a.scale_out = out_scale->ptr;
+        a.num_chunks = flat_chunks;
         a.block = 0;
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
         a.range = p.range;
-        st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, a));
+        st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, a));
         if (st != CQ_OK) return st;
-        flat_words = a.num_chunks * per_chunk / p.nq;
+        flat_words = flat_chunks * per_chunk / p.nq;
+    } else {
+        // scales as FS(F(scale)) into out_scale first, then quantize reading them back
+        // (the divisor F(FS(scale)) is the same either way)
+        st = produce_scales(stream, p, scheme, input, input_dtype, out_scale, pd, workspace, workspace_bytes);
+        if (st != CQ_OK) return st;
     }
     if (flat_words < p.n / p.nq) {
         cq::GenericArgs g = generic_args(p, scheme);

@@ -27,7 +27,9 @@ struct Range {
 struct FlatArgs {
     const void* input;    // float tensor (quantize) / u32 words (dequantize)
     void* output;         // u32 words (quantize) / float tensor (dequantize)
-    const void* scale_in; // quantize with given scales (typed scale_in_dtype); dequantize: params
+    const void* scale_in; // quantize with given scales (typed scale_in_dtype); dequantize: params;
+                          // ScaleSource::Partials: the f32 abs-max partials of pass 1
+    uint32_t num_partials;
     int scale_in_dtype;   // cq_dtype of scale_in (quantize only)
     void* scale_out;      // quantize: out_scale typed as param dtype, NULL = do not write;
                           // launch_scales_flat: scales typed like the input
@@ -38,7 +40,7 @@ struct FlatArgs {
     Range range;
 };
 
-enum class ScaleSource { Given, Dynamic };
+enum class ScaleSource { Given, Dynamic, Partials };
 
 // every launcher returns hipGetLastError() of its launch
 hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource src, const FlatArgs& a);

@@ -61,8 +61,8 @@ hipError_t launch_tiles(uint64_t num_chunks, int unroll, LaunchFn launch) {
 template <class F, int kBits, int kGroup, int kSrc, bool kWide, int kEnc>
 hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
     // scale sources that exist: per-block launches compute the scale or read the
-    // input-typed tensor; per-tensor launches read one scale of either type
-    if constexpr ((kGroup == 0 && kSrc == kScaleDynamic) || (kGroup != 0 && kSrc == kScaleGivenParam)) {
+    // input-typed tensor; per-tensor launches read it or finish the grid reduction
+    if constexpr ((kGroup == 0 && kSrc == kScaleDynamic) || (kGroup != 0 && kSrc == kScalePartials)) {
         return hipErrorInvalidValue;
     } else {
         auto in = static_cast<const u32x4*>(a.input);
@@ -76,7 +76,7 @@ hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
                         : (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false, kEnc>
                                : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false, kEnc>);
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
-                               a.param_dtype, begin, end, qp);
+                               a.param_dtype, begin, end, qp, a.num_partials);
         });
     }
 }
@@ -84,11 +84,9 @@ hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
 template <class F, int kBits, int kGroup, bool kWide, int kEnc>
 hipError_t quantize_launch_enc(hipStream_t s, ScaleSource src, const FlatArgs& a) {
     if (src == ScaleSource::Dynamic) return quantize_launch_src<F, kBits, kGroup, kScaleDynamic, kWide, kEnc>(s, a);
-    // a scale typed like the input is read as such (identical to the param reading when both types agree)
+    if (src == ScaleSource::Partials) return quantize_launch_src<F, kBits, kGroup, kScalePartials, kWide, kEnc>(s, a);
     if (a.scale_in_dtype == F::kDtype) return quantize_launch_src<F, kBits, kGroup, kScaleGivenF, kWide, kEnc>(s, a);
-    if (a.scale_in_dtype == a.param_dtype)
-        return quantize_launch_src<F, kBits, kGroup, kScaleGivenParam, kWide, kEnc>(s, a);
-    return hipErrorInvalidValue;
+    return hipErrorInvalidValue;  // given scales are typed like the input
 }
 
 template <class F, int kBits, int kGroup>

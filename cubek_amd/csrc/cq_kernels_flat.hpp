@@ -22,7 +22,8 @@ namespace cq {
 enum ScaleSrc : int {
     kScaleDynamic = 0,     // abs-max of the block, computed here
     kScaleGivenF = 1,      // `scale_in`, typed like the input (the reference's `scale` argument)
-    kScaleGivenParam = 2,  // `scale_in`, typed as the param dtype (second pass of the per-tensor path)
+    kScalePartials = 2,    // per tensor: `scale_in` holds the f32 abs-max partials of pass 1; this
+                           // kernel (pass 2) finishes the reduction, derives the scale and quantizes
 };
 
 // kParamF32: the stored scales are f32 (the common case, resolved at compile
@@ -37,15 +38,14 @@ template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kW
 __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
     void* __restrict__ scale_out, int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end,
-    QuantParams qp) {
+    QuantParams qp, uint32_t num_partials) {
     constexpr bool kDynamic = kScaleSrc == kScaleDynamic;
+    static_assert(kScaleSrc != kScalePartials || kGroup == 0, "partials feed the per-tensor scale only");
     constexpr int kDiv = kGroup == 0 ? 1 : kGroup;
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;  // 64, 32, 16 or 8
     const int param_dtype = kParamF32 ? static_cast<int>(CQ_F32) : param_dtype_rt;
-    const auto load_scale = [&](uint64_t i) {
-        return kScaleSrc == kScaleGivenF ? F::load(scale_in, i) : load_dtype(param_dtype, scale_in, i);
-    };
+    const auto load_scale = [&](uint64_t i) { return F::load(scale_in, i); };
     const uint64_t first =
         chunk_begin + static_cast<uint64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
 
@@ -58,9 +58,25 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
         uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
         if (kChecked) c = c < chunk_end ? c : chunk_end - 1;
         raw[u] = __builtin_nontemporal_load(in + c);
-        if constexpr (!kDynamic && kGroup != 0) s_given[u] = load_scale(c / kDiv);
+        if constexpr (!kDynamic && kGroup != 0 && kScaleSrc != kScalePartials) s_given[u] = load_scale(c / kDiv);
     }
-    if constexpr (!kDynamic && kGroup == 0) {
+    if constexpr (kScaleSrc == kScalePartials) {
+        // second pass of the grid reduction: every workgroup reduces the (<= a few
+        // hundred) partial maxima again — max is exact, so all agree bit for bit
+        const float* partials = static_cast<const float*>(scale_in);
+        float amax = 0.0f;
+        for (uint32_t i = threadIdx.x; i < num_partials; i += kThreads) amax = fmaxf(amax, partials[i]);
+        amax = group_max<64>(amax);
+        __shared__ float wave_max[kThreads / kWave];
+        if ((threadIdx.x & (kWave - 1)) == 0) wave_max[threadIdx.x / kWave] = amax;
+        __syncthreads();
+        amax = wave_max[0];
+#pragma unroll
+        for (int w = 1; w < kThreads / kWave; w++) amax = fmaxf(amax, wave_max[w]);
+        const float s = F::round(scale_from_absmax(amax, qp.width));
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) s_given[u] = s;
+    } else if constexpr (!kDynamic && kGroup == 0) {
         const float s = load_scale(0);  // one scale for the whole tensor
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) s_given[u] = s;
@@ -92,9 +108,9 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
         const uint64_t si = kGroup == 0 ? 0 : c / kDiv;
         const bool block_start = kGroup == 0 ? c == 0 : (c % kDiv) == 0;
         if (scale_out != nullptr && live && block_start) store_dtype(param_dtype, scale_out, si, s_fs);
-        // divisor F(FS(scale)); s_f is already an F value when it came from F-typed data
+        // divisor F(FS(scale)); s_f is an F value, so f32 params leave it unchanged
         float d = s_fs;
-        if constexpr (!(kParamF32 && kScaleSrc != kScaleGivenParam)) d = F::round(s_fs);
+        if constexpr (!kParamF32) d = F::round(s_fs);
         if constexpr (!(kDynamic && kParamF32 && F::kDtype != CQ_F16)) tame = divisor_is_tame(d);
 
         float qn[kN];  // negated codes
