@@ -38,6 +38,25 @@ __device__ __forceinline__ void static_for(Fn&& f) {
 __device__ __forceinline__ float bits_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
 
+// Streaming accesses: every byte is touched once, so loads and stores carry the
+// non-temporal hint.  (CQ_PLAIN_STORES / CQ_PLAIN_LOADS exist for experiments.)
+template <class T>
+__device__ __forceinline__ T stream_load(const T* p) {
+#ifdef CQ_PLAIN_LOADS
+    return *p;
+#else
+    return __builtin_nontemporal_load(p);
+#endif
+}
+template <class T>
+__device__ __forceinline__ void stream_store(T v, T* p) {
+#ifdef CQ_PLAIN_STORES
+    *p = v;
+#else
+    __builtin_nontemporal_store(v, p);
+#endif
+}
+
 // ---- element types -------------------------------------------------------
 // A "chunk" is 16 bytes of a float tensor: the unit one lane loads or stores.
 

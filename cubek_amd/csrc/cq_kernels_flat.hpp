@@ -57,7 +57,7 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
     for (int u = 0; u < kUnroll; u++) {
         uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
         if (kChecked) c = c < chunk_end ? c : chunk_end - 1;
-        raw[u] = __builtin_nontemporal_load(in + c);
+        raw[u] = stream_load(in + c);
         if constexpr (!kDynamic && kGroup != 0 && kScaleSrc != kScalePartials) s_given[u] = load_scale(c / kDiv);
     }
     if constexpr (kScaleSrc == kScalePartials) {
@@ -122,14 +122,14 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
             encode_chunk_neg<kEnc, kN>(qn, w);
 
         if constexpr (kChunkBits == 64) {
-            if (live) __builtin_nontemporal_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(out) + c);
+            if (live) stream_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(out) + c);
         } else if constexpr (kChunkBits == 32) {
-            if (live) __builtin_nontemporal_store(w[0], out + c);
+            if (live) stream_store(w[0], out + c);
         } else {
             constexpr int kLanesPerWord = 32 / kChunkBits;  // 2 or 4
             const uint32_t sub = static_cast<uint32_t>(c) & (kLanesPerWord - 1);
             const uint32_t word = group_or<kLanesPerWord>(w[0] << (sub * kChunkBits));
-            if (live && sub == 0) __builtin_nontemporal_store(word, out + c / kLanesPerWord);
+            if (live && sub == 0) stream_store(word, out + c / kLanesPerWord);
         }
     }
 }
@@ -153,11 +153,11 @@ __global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
         if (kChecked) c = c < chunk_end ? c : chunk_end - 1;  // clamp instead of branching
         w1[u] = 0;
         if constexpr (kChunkBits == 64) {
-            u32x2 w = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(in) + c);
+            u32x2 w = stream_load(reinterpret_cast<const u32x2*>(in) + c);
             w0[u] = w[0];
             w1[u] = w[1];
         } else if constexpr (kChunkBits == 32) {
-            w0[u] = __builtin_nontemporal_load(in + c);
+            w0[u] = stream_load(in + c);
         } else {
             constexpr int kLanesPerWord = 32 / kChunkBits;
             uint32_t w = in[c / kLanesPerWord];  // neighbouring lanes share the word
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
         }
 #pragma unroll
         for (int i = 0; i < kN; i++) y[i] = sc[u] * y[i];
-        if (!kChecked || c < chunk_end) __builtin_nontemporal_store(F::pack(y), out + c);  // pack rounds to F
+        if (!kChecked || c < chunk_end) stream_store(F::pack(y), out + c);  // pack rounds to F
     }
 }
 
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(kThreads) void scales_flat_kernel(const u32x4* __re
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
-        raw[u] = __builtin_nontemporal_load(in + (c < num_chunks ? c : last));
+        raw[u] = stream_load(in + (c < num_chunks ? c : last));
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
