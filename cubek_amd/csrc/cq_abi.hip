@@ -346,7 +346,7 @@ static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_sche
     if (p.tensor_level) {
         if (!workspace || workspace_bytes < cq::kMaxPartials * sizeof(float))
             return CQ_ERR_WORKSPACE_TOO_SMALL;
-        if (!aligned(input->ptr, 16) || !aligned(workspace, 4)) return CQ_ERR_INVALID_ARGUMENT;
+        if (!aligned(workspace, 4)) return CQ_ERR_INVALID_ARGUMENT;
         uint32_t num_partials = 0;
         cq_status st = hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n,
                                                              static_cast<float*>(workspace), &num_partials));

@@ -206,13 +206,20 @@ hipError_t launch_scales_flat(hipStream_t s, int dtype, const FlatArgs& a) {
 
 hipError_t launch_absmax_partials(hipStream_t s, int dtype, const void* input, uint64_t num_elems,
                                   float* partials, uint32_t* num_partials) {
-    uint64_t per_chunk = dtype == CQ_F32 ? 4 : 8;
-    uint64_t chunks = num_elems / per_chunk;
-    uint64_t want = (chunks + kThreads * 4 - 1) / (kThreads * 4);
-    uint32_t grid = static_cast<uint32_t>(want < 1 ? 1 : (want > kMaxPartials ? kMaxPartials : want));
+    // At most kMaxPartials workgroups (pass 2 re-reads every partial in every
+    // workgroup), so they are fat: 1024 lanes x 4 loads = 64 KiB in flight each.
+    constexpr int kReduceThreads = 1024, kReduceUnroll = 4;
+    const uint64_t per_chunk = dtype == CQ_F32 ? 4 : 8;
+    const uint64_t chunks = num_elems / per_chunk;
+    const uint64_t per_group = static_cast<uint64_t>(kReduceThreads) * kReduceUnroll;
+    const uint64_t want = (chunks + per_group - 1) / per_group;
+    const uint32_t grid = static_cast<uint32_t>(want < 1 ? 1 : (want > kMaxPartials ? kMaxPartials : want));
+    const bool is_aligned = (reinterpret_cast<uintptr_t>(input) & 15u) == 0;
     *num_partials = grid;
-    CQ_SWITCH_DTYPE(dtype, hipLaunchKernelGGL((absmax_partials_kernel<kF, kThreads>), dim3(grid), dim3(kThreads), 0, s,
-                                              input, num_elems, partials);
+    CQ_SWITCH_DTYPE(dtype,
+                    auto kernel = is_aligned ? absmax_partials_kernel<kF, kReduceThreads, kReduceUnroll, true>
+                                             : absmax_partials_kernel<kF, kReduceThreads, kReduceUnroll, false>;
+                    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kReduceThreads), 0, s, input, num_elems, partials);
                     return hipGetLastError())
 }
 

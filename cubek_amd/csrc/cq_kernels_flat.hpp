@@ -213,26 +213,43 @@ __global__ __launch_bounds__(kThreads) void scales_flat_kernel(const u32x4* __re
     }
 }
 
-// Per-tensor abs-max, pass 1: grid-stride over chunks, one partial per workgroup.
-template <class F, int kThreads>
+// Per-tensor abs-max, pass 1: grid-stride over chunks with kUnroll 16-byte loads
+// in flight per lane, one partial per workgroup.  Lanes past the end re-read the
+// last chunk (harmless for a maximum).  kAligned = false: element-wise loads for
+// tensors that do not start on a 16-byte boundary.
+template <class F, int kThreads, int kUnroll, bool kAligned>
 __global__ __launch_bounds__(kThreads) void absmax_partials_kernel(const void* __restrict__ input,
                                                                    uint64_t num_elems,
                                                                    float* __restrict__ partials) {
     constexpr int kN = F::kPerChunk;
-    const u32x4* in = static_cast<const u32x4*>(input);
-    const uint64_t num_chunks = num_elems / kN;
-    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * kThreads;
+    const uint64_t gid = static_cast<uint64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const uint64_t total = static_cast<uint64_t>(gridDim.x) * kThreads;
     float amax = 0.0f;
-    for (uint64_t c = static_cast<uint64_t>(blockIdx.x) * kThreads + threadIdx.x; c < num_chunks;
-         c += stride) {
-        float v[kN];
-        F::unpack(in[c], v);
+    if constexpr (kAligned) {
+        const u32x4* in = static_cast<const u32x4*>(input);
+        const uint64_t num_chunks = num_elems / kN;
+        if (num_chunks > 0) {
+            for (uint64_t c0 = gid; c0 < num_chunks; c0 += total * kUnroll) {
+                u32x4 raw[kUnroll];
 #pragma unroll
-        for (int i = 0; i < kN; i++) amax = fmaxf(amax, fabsf(v[i]));
-    }
-    if (blockIdx.x == 0 && threadIdx.x == 0) {  // ragged tail, fewer than one chunk
-        for (uint64_t e = num_chunks * kN; e < num_elems; e++)
-            amax = fmaxf(amax, fabsf(F::load(input, e)));
+                for (int u = 0; u < kUnroll; u++) {
+                    const uint64_t c = c0 + static_cast<uint64_t>(u) * total;
+                    raw[u] = stream_load(in + (c < num_chunks ? c : num_chunks - 1));
+                }
+#pragma unroll
+                for (int u = 0; u < kUnroll; u++) {
+                    float v[kN];
+                    F::unpack(raw[u], v);
+#pragma unroll
+                    for (int i = 0; i < kN; i++) amax = fmaxf(amax, fabsf(v[i]));
+                }
+            }
+        }
+        if (gid == 0) {  // ragged tail, fewer than one chunk
+            for (uint64_t e = num_chunks * kN; e < num_elems; e++) amax = fmaxf(amax, fabsf(F::load(input, e)));
+        }
+    } else {
+        for (uint64_t e = gid; e < num_elems; e += total) amax = fmaxf(amax, fabsf(F::load(input, e)));
     }
     amax = group_max<64>(amax);
     __shared__ float wave_max[kThreads / kWave];

@@ -306,6 +306,21 @@ def test_unaligned_base_pointers(gpu, oracle):
     torch.cuda.synchronize()
     d_ref = oracle.dequantize(w_ref, shape, os_ref, ElemType.F32, scheme)
     assert np.array_equal(back[1:].cpu().numpy().reshape(shape), d_ref)
+    # per tensor on the same unaligned view: the grid abs-max must not assume alignment
+    pt = QuantScheme.default().with_value(QuantValue.Q8S)
+    s_t = oracle.compute_scales(x, ElemType.F32, shape, pt)
+    wt, ost = oracle.quantize(x, ElemType.F32, shape, s_t, pt)
+    out_t = torch.zeros(pt.packed_shape(shape), dtype=torch.int32, device="cuda")
+    os_t = torch.zeros((1,), dtype=torch.float32, device="cuda")
+    ws = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    qz.launch_dynamic(client, TensorHandleRef.from_torch(view), TensorHandleRef.from_torch(out_t),
+                      TensorHandleRef.from_torch(os_t), pt, ElemType.F32, ws.data_ptr(), 1024)
+    sc_t = torch.zeros((1,), dtype=torch.float32, device="cuda")
+    qz.compute_scales(client, TensorHandleRef.from_torch(view), TensorHandleRef.from_torch(sc_t), pt, ElemType.F32,
+                      ws.data_ptr(), 1024)
+    torch.cuda.synchronize()
+    assert np.array_equal(out_t.cpu().numpy().view(np.uint32), wt)
+    assert os_t.cpu().numpy()[0] == ost.reshape(-1)[0] == sc_t.cpu().numpy()[0]
 
 
 # ---------------------------------------------------------------- native store
