@@ -19,7 +19,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libc
 EXPORTED_SYMBOLS = (
     "cq_value_size_bits", "cq_scheme_num_quants", "cq_value_range", "cq_quantize", "cq_dequantize",
     "cq_compute_scales", "cq_quantize_dynamic", "cq_workspace_bytes", "cq_strerror",
-    "cq_last_hip_error", "cq_abi_version",
+    "cq_last_hip_error", "cq_abi_version", "cq_reduce_max_abs", "cq_reduce_workspace_bytes",
 )
 
 
@@ -45,7 +45,7 @@ class QuantError(RuntimeError):
 
 # status codes (mirrors enum cq_status)
 OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED_SCHEME, ERR_BLOCK_NOT_DIVISIBLE, ERR_SHAPE_MISMATCH, \
-    ERR_NON_CONTIGUOUS, ERR_WORKSPACE_TOO_SMALL, ERR_HIP, ERR_TOO_LARGE = range(9)
+    ERR_NON_CONTIGUOUS, ERR_WORKSPACE_TOO_SMALL, ERR_HIP, ERR_TOO_LARGE, ERR_INVALID_AXIS = range(10)
 
 _lib = None
 
@@ -83,6 +83,11 @@ def lib() -> ctypes.CDLL:
     L.cq_compute_scales.argtypes = [ctypes.c_void_p, tp, tp, sp, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
     L.cq_quantize_dynamic.restype = ctypes.c_int
     L.cq_quantize_dynamic.argtypes = [ctypes.c_void_p, tp, tp, tp, sp, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
+    L.cq_reduce_max_abs.restype = ctypes.c_int
+    L.cq_reduce_max_abs.argtypes = [ctypes.c_void_p, tp, tp, ctypes.c_uint32, ctypes.c_int, ctypes.c_void_p,
+                                    ctypes.c_size_t]
+    L.cq_reduce_workspace_bytes.restype = ctypes.c_size_t
+    L.cq_reduce_workspace_bytes.argtypes = [tp, ctypes.c_uint32, ctypes.c_int]
     _lib = L
     return L
 

@@ -217,6 +217,7 @@ const char* cq_strerror(cq_status st) {
         case CQ_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
         case CQ_ERR_HIP: return "HIP runtime error";
         case CQ_ERR_TOO_LARGE: return "tensor too large";
+        case CQ_ERR_INVALID_AXIS: return "the reduction axis must be smaller than the tensor rank";
         default: return "unknown status";
     }
 }
@@ -470,6 +471,48 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
                                : cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
     }
     return st;
+}
+
+static bool reduce_view(const cq_tensor* input, uint32_t axis, uint64_t* outer, uint64_t* len, uint64_t* inner) {
+    *outer = *inner = 1;
+    for (uint32_t d = 0; d < axis; d++) *outer *= input->shape[d];
+    for (uint32_t d = axis + 1; d < input->rank; d++) *inner *= input->shape[d];
+    *len = input->shape[axis];
+    return true;
+}
+
+size_t cq_reduce_workspace_bytes(const cq_tensor* input, uint32_t axis, cq_dtype dtype) {
+    if (!tensor_ok(input) || axis >= input->rank || !valid_dtype(dtype)) return 0;
+    uint64_t outer, len, inner;
+    reduce_view(input, axis, &outer, &len, &inner);
+    if (outer == 0 || inner == 0) return 0;
+    return cq::reduce_workspace_bytes(outer, len, inner, dtype);
+}
+
+cq_status cq_reduce_max_abs(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output, uint32_t axis,
+                            cq_dtype dtype, void* workspace, size_t workspace_bytes) {
+    if (!tensor_ok(input) || !tensor_ok(output) || !valid_dtype(dtype)) return CQ_ERR_INVALID_ARGUMENT;
+    if (axis >= input->rank) return CQ_ERR_INVALID_AXIS;
+    if (input->elem_size != dtype_size(dtype) || output->elem_size != dtype_size(dtype)) return CQ_ERR_SHAPE_MISMATCH;
+    if (output->rank != input->rank) return CQ_ERR_SHAPE_MISMATCH;
+    cq::ReduceArgs a{};
+    for (uint32_t d = 0; d < input->rank; d++) {
+        if (output->shape[d] != (d == axis ? 1 : input->shape[d])) return CQ_ERR_SHAPE_MISMATCH;
+        if (input->shape[d] > 0xffffffffull) return CQ_ERR_TOO_LARGE;
+        a.shape[d] = input->shape[d];
+        a.in_strides[d] = input->strides[d];
+        a.out_strides[d] = output->strides[d];
+    }
+    a.input = input->ptr;
+    a.output = output->ptr;
+    a.workspace = aligned(workspace, 16) ? workspace : nullptr;
+    a.workspace_bytes = a.workspace ? workspace_bytes : 0;
+    a.rank = input->rank;
+    a.axis = axis;
+    a.contiguous = is_contiguous(input) && is_contiguous(output);
+    reduce_view(input, axis, &a.outer, &a.len, &a.inner);
+    if (a.outer == 0 || a.inner == 0) return CQ_OK;  // no outputs
+    return hip_status(cq::launch_reduce_max_abs(stream, dtype, a));
 }
 
 }  // extern "C"

@@ -79,4 +79,19 @@ hipError_t launch_scales_generic(hipStream_t s, int dtype, int out_dtype, const 
 hipError_t launch_quantize_native(hipStream_t s, int dtype, const GenericArgs& a);
 hipError_t launch_dequantize_native(hipStream_t s, int dtype, const GenericArgs& a);
 
+// Abs-max along one axis (cq_reduce_max_abs).
+struct ReduceArgs {
+    const void* input;
+    void* output;
+    void* workspace;         // f32 partials, may be NULL
+    size_t workspace_bytes;
+    uint32_t rank, axis;
+    uint64_t shape[CQ_MAX_RANK];
+    uint64_t in_strides[CQ_MAX_RANK], out_strides[CQ_MAX_RANK];
+    bool contiguous;         // input and output are contiguous row-major
+    uint64_t outer, len, inner;  // the contiguous view [outer, len, inner] around the axis
+};
+hipError_t launch_reduce_max_abs(hipStream_t s, int dtype, const ReduceArgs& a);
+uint64_t reduce_workspace_bytes(uint64_t outer, uint64_t len, uint64_t inner, int dtype);
+
 }  // namespace cq

@@ -40,7 +40,8 @@ typedef enum cq_status {
     CQ_ERR_NON_CONTIGUOUS = 5,      /* value tensors must be contiguous row-major        */
     CQ_ERR_WORKSPACE_TOO_SMALL = 6,
     CQ_ERR_HIP = 7,                 /* a HIP runtime call failed; see cq_last_hip_error  */
-    CQ_ERR_TOO_LARGE = 8            /* more elements than an entry point accepts         */
+    CQ_ERR_TOO_LARGE = 8,           /* more elements than an entry point accepts         */
+    CQ_ERR_INVALID_AXIS = 9         /* reduction axis >= rank (ReduceError::InvalidAxis) */
 } cq_status;
 
 /* Float element types of value tensors and scale parameters
@@ -165,6 +166,21 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
 
 /* Device bytes the two entry points above need for `num_elements` inputs. */
 size_t cq_workspace_bytes(const cq_scheme* scheme, uint64_t num_elements);
+
+/* ---- abs-max along an axis (the step in front of the path) ---- */
+
+/* Replaces cubek_reduce::reduce::<R, MaxAbs> (crates/cubek-reduce/src/lib.rs:93-131 with
+ * src/instructions/maxabs.rs:10-96), the reduction a caller runs to obtain per-row /
+ * per-channel abs-max values before dividing them into scales.
+ *   input  : float tensor of dtype `dtype`, any strides
+ *   output : same dtype, same shape except extent 1 on `axis`
+ *            (anything else: CQ_ERR_SHAPE_MISMATCH, ReduceError::MismatchShape)
+ *   workspace : optional device scratch of cq_reduce_workspace_bytes() bytes; lets
+ *            reductions with few outputs spread one output over many workgroups
+ * NaN elements are ignored; an axis of extent 0 yields 0. */
+cq_status cq_reduce_max_abs(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                            uint32_t axis, cq_dtype dtype, void* workspace, size_t workspace_bytes);
+size_t cq_reduce_workspace_bytes(const cq_tensor* input, uint32_t axis, cq_dtype dtype);
 
 /* ---- diagnostics ---- */
 const char* cq_strerror(cq_status status);

@@ -218,4 +218,39 @@ inline void launch_ref(const ComputeClient& client, const TensorHandleRef& value
 }
 }  // namespace dequantize
 
+namespace reduce {
+// cubek_reduce::ReduceError (crates/cubek-reduce/src/error.rs:6-36), the variants this path can raise.
+struct ReduceError : std::runtime_error {
+    enum Kind { InvalidAxis, MismatchShape, Launch } kind;
+    ReduceError(Kind k, const std::string& what) : std::runtime_error(what), kind(k) {}
+};
+
+inline size_t workspace_bytes(const TensorHandleRef& input, size_t axis, ElemType dtype) {
+    cq_tensor i = input.as_c();
+    return cq_reduce_workspace_bytes(&i, static_cast<uint32_t>(axis), static_cast<cq_dtype>(dtype));
+}
+
+// cubek_reduce::reduce::<R, MaxAbs> (crates/cubek-reduce/src/lib.rs:93-131): `output` has the
+// shape of `input` with extent 1 on `axis`.  The reference returns Err(ReduceError); here it is thrown.
+inline void max_abs(const ComputeClient& client, const TensorHandleRef& input, const TensorHandleRef& output,
+                    size_t axis, ElemType dtype, void* workspace = nullptr, size_t workspace_size = 0) {
+    cq_tensor i = input.as_c(), o = output.as_c();
+    const cq_status st = cq_reduce_max_abs(client.stream, &i, &o, static_cast<uint32_t>(axis),
+                                           static_cast<cq_dtype>(dtype), workspace, workspace_size);
+    switch (st) {
+        case CQ_OK: return;
+        case CQ_ERR_INVALID_AXIS:
+            throw ReduceError(ReduceError::InvalidAxis, "The provided axis (" + std::to_string(axis) +
+                                                            ") must be smaller than the input tensor rank (" +
+                                                            std::to_string(input.shape.size()) + ").");
+        case CQ_ERR_SHAPE_MISMATCH:
+            throw ReduceError(ReduceError::MismatchShape, "The output shape is not the input shape with 1 on the axis.");
+        case CQ_ERR_HIP:
+            throw ReduceError(ReduceError::Launch, std::string(cq_strerror(st)) + " (hipError_t " +
+                                                       std::to_string(cq_last_hip_error()) + ")");
+        default: throw std::invalid_argument(cq_strerror(st));
+    }
+}
+}  // namespace reduce
+
 }  // namespace cubek_quant

@@ -442,6 +442,33 @@ int cqo_compute_scales(const void* input, int dtype, uint32_t rank, const uint64
     return 0;
 }
 
+/* MaxAbs along one axis (crates/cubek-reduce/src/instructions/maxabs.rs:47-96:
+ * identity 0, keep the larger of accumulator and |item|); NaN items are ignored.
+ * Any strides; output has extent 1 on `axis`. */
+int cqo_reduce_max_abs(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
+                       const uint64_t* in_strides, uint32_t axis, void* output,
+                       const uint64_t* out_strides) {
+    if (axis >= rank) return -1;
+    uint64_t num_out = 1;
+    for (uint32_t d = 0; d < rank; d++)
+        if (d != axis) num_out *= shape[d];
+    for (uint64_t i = 0; i < num_out; i++) {
+        uint64_t rem = i, in_off = 0, out_off = 0;
+        for (int d = (int)rank - 1; d >= 0; d--) {
+            if ((uint32_t)d == axis) continue;
+            uint64_t c = rem % shape[d];
+            rem /= shape[d];
+            in_off += c * in_strides[d];
+            out_off += c * out_strides[d];
+        }
+        float m = 0.0f;
+        for (uint64_t k = 0; k < shape[axis]; k++)
+            m = fmaxf(m, fabsf(load_f(input, dtype, in_off + k * in_strides[axis])));
+        store_f(output, dtype, out_off, m);
+    }
+    return 0;
+}
+
 /* --------------------------------------------------------- threaded drivers */
 
 typedef struct {

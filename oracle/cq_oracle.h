@@ -74,6 +74,11 @@ float cqo_e2m1_to_f32(uint8_t nibble);
 int cqo_compute_scales(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
                        void* scales, const cq_scheme* scheme);
 
+/* abs-max along one axis, any strides (crates/cubek-reduce/src/instructions/maxabs.rs) */
+int cqo_reduce_max_abs(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
+                       const uint64_t* in_strides, uint32_t axis, void* output,
+                       const uint64_t* out_strides);
+
 /* threaded drivers used for the CPU baseline timing (split the word range) */
 int cqo_quantize_packed_mt(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
                            const void* scale, const uint64_t* scale_strides, void* out_scale,

@@ -84,6 +84,8 @@ def _declare(L):
     L.cqo_quantize_packed_mt.argtypes = q_args + [ctypes.c_int]
     L.cqo_dequantize_packed_mt.restype = ctypes.c_int
     L.cqo_dequantize_packed_mt.argtypes = d_args + [ctypes.c_int]
+    L.cqo_reduce_max_abs.restype = ctypes.c_int
+    L.cqo_reduce_max_abs.argtypes = [_vp, ctypes.c_int, ctypes.c_uint32, _u64p, _u64p, ctypes.c_uint32, _vp, _u64p]
     L.cqo_compute_scales.restype = ctypes.c_int
     L.cqo_compute_scales.argtypes = [_vp, ctypes.c_int, ctypes.c_uint32, _u64p, _vp, _sp]
 
@@ -246,3 +248,17 @@ def dequantize(values: np.ndarray, shape, params: np.ndarray, elem: ElemType,
     if rc:
         raise RuntimeError(f"oracle dequantize failed: {rc}")
     return out.reshape(shape)
+
+
+def reduce_max_abs(x: np.ndarray, elem: ElemType, shape, axis: int, in_strides=None) -> np.ndarray:
+    """max |x| along ``axis`` (kept with extent 1); ``x`` is the raw buffer when strides are given."""
+    x = np.ascontiguousarray(x)
+    if in_strides is None:
+        in_strides = contiguous_strides(shape)
+    out_shape = tuple(1 if d == axis else s for d, s in enumerate(shape))
+    out = np.zeros(out_shape, dtype=np_dtype(elem))
+    rc = lib().cqo_reduce_max_abs(_ptr(x), int(elem), len(shape), _u64(shape), _u64(in_strides), axis,
+                                  _ptr(out), _u64(contiguous_strides(out_shape)))
+    if rc:
+        raise RuntimeError(f"cqo_reduce_max_abs failed: {rc}")
+    return out

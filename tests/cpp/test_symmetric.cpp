@@ -208,6 +208,39 @@ static void test_error_behaviour() {
     }
 }
 
+// MaxAbs along an axis feeding the test's scale rule: per-row abs-max of an [m, n] ramp,
+// and the error variants of cubek_reduce::reduce (crates/cubek-reduce/src/lib.rs:101-102).
+static void test_reduce_max_abs() {
+    ComputeClient client;
+    const size_t m = 16, n = 64;
+    std::vector<float> data(m * n);
+    for (size_t i = 0; i < m * n; i++) data[i] = (i % 2 ? -1.0f : 1.0f) * static_cast<float>(i) / 8.0f;
+    DeviceBuffer<float> x(data), rows(m), cols(n);
+    auto t_x = TensorHandleRef::contiguous(x.ptr, {m, n}, 4);
+    auto t_rows = TensorHandleRef::contiguous(rows.ptr, {m, 1}, 4);
+    auto t_cols = TensorHandleRef::contiguous(cols.ptr, {1, n}, 4);
+    reduce::max_abs(client, t_x, t_rows, 1, ElemType::F32);
+    reduce::max_abs(client, t_x, t_cols, 0, ElemType::F32);
+    HIP_OK(hipDeviceSynchronize());
+    bool ok = true;
+    auto got_rows = rows.read(), got_cols = cols.read();
+    for (size_t r = 0; r < m; r++) ok = ok && got_rows[r] == static_cast<float>(r * n + n - 1) / 8.0f;
+    for (size_t c = 0; c < n; c++) ok = ok && got_cols[c] == static_cast<float>((m - 1) * n + c) / 8.0f;
+    report("reduce::max_abs_rows_and_columns", ok);
+    bool bad_axis = false, bad_shape = false;
+    try {
+        reduce::max_abs(client, t_x, t_rows, 2, ElemType::F32);
+    } catch (const reduce::ReduceError& e) {
+        bad_axis = e.kind == reduce::ReduceError::InvalidAxis;
+    }
+    try {
+        reduce::max_abs(client, t_x, t_cols, 1, ElemType::F32);
+    } catch (const reduce::ReduceError& e) {
+        bad_shape = e.kind == reduce::ReduceError::MismatchShape;
+    }
+    report("reduce::invalid_axis_and_mismatch_shape", bad_axis && bad_shape);
+}
+
 int main() {
     int devices = 0;
     if (hipGetDeviceCount(&devices) != hipSuccess || devices == 0) {
@@ -225,6 +258,7 @@ int main() {
             test_quantization_block_symmetric(sz.x, sz.y, v.v, sz.x /* Shape x as block_size */, name);
         }
     test_error_behaviour();
+    test_reduce_max_abs();
     std::printf("%d failure(s)\n", failures);
     return failures == 0 ? 0 : 1;
 }

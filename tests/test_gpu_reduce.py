@@ -1,0 +1,135 @@
+"""cq_reduce_max_abs (through the C ABI) against the CPU oracle: every kernel
+variant (lane groups, wave per row, sliced rows, columns, sliced columns,
+strided fallback), bit for bit, plus the reference's error cases."""
+import numpy as np
+import pytest
+
+from cubek_amd import ComputeClient, ElemType, QuantError, TensorHandleRef, _ffi
+from cubek_amd import reduce as cq_reduce
+
+pytestmark = pytest.mark.gpu
+ELEMS = [ElemType.F32, ElemType.BF16, ElemType.F16]
+
+
+def run(torch, gpu, x_np, elem, shape, axis, use_workspace=True, in_strides=None, out_strides=None):
+    dx = gpu.to_dev(x_np.reshape(-1))
+    out_shape = tuple(1 if d == axis else s for d, s in enumerate(shape))
+    n_out = int(np.prod(out_shape))
+    hin = gpu.handle(dx, shape, in_strides if in_strides is not None else gpu.contiguous_strides(shape))
+    ostr = out_strides if out_strides is not None else gpu.contiguous_strides(out_shape)
+    reach = 1 + sum((n - 1) * st for n, st in zip(out_shape, ostr))
+    dout = torch.zeros(max(reach, 1), dtype=gpu.storage_dtype(elem), device="cuda")
+    hout = gpu.handle(dout, out_shape, ostr)
+    nbytes = cq_reduce.workspace_bytes(hin, axis, elem) if use_workspace else 0
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+    cq_reduce.max_abs(ComputeClient.current(), hin, hout, axis, elem, ws.data_ptr() if nbytes else 0, nbytes)
+    torch.cuda.synchronize()
+    return gpu.to_host(dout), n_out
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import gpu_harness
+
+    return gpu_harness
+
+
+@pytest.mark.parametrize("elem", ELEMS, ids=lambda e: e.name)
+def test_reduce_contiguous_all_paths(gpu, oracle, elem):
+    import torch
+
+    rng = np.random.default_rng(int(elem) + 7)
+    cases = [
+        ((64, 32), 1), ((300, 8), 1), ((33, 512), 1),          # lane groups (1..64 chunks per row)
+        ((40, 4096), 1), ((3, 100000), 1), ((1, 1 << 20), 1),  # wave per row, sliced rows
+        ((5000, 1000), 1),                                      # odd chunk count per row
+        ((512, 256), 0), ((4096, 64), 0), ((20000, 16), 0),     # columns, sliced columns
+        ((6, 50, 128), 1), ((4, 3, 8, 64), 2), ((2, 7, 24), 0),
+        ((10, 7), 1), ((10, 7), 0), ((5, 3, 2), 1),             # not chunk-aligned: fallback
+        ((8, 1, 64), 1),
+        ((100000, 64), 0), ((3000, 24), 0), ((2, 4000, 40), 1), ((1, 300, 1024), 1),  # tiles of chunk columns
+        ((3, 600, 520), 1), ((70000, 8), 0), ((5, 9, 16), 1),
+        ((300, 1001), 1), ((1001, 300), 0), ((9, 4097), 1),     # long odd axes: wave per output
+    ]
+    for shape, axis in cases:
+        x32 = rng.normal(0, 2, shape).astype(np.float32)
+        x32[rng.random(shape) < 0.01] = np.nan
+        x = oracle.to_bits(x32, elem)
+        want = oracle.reduce_max_abs(x, elem, shape, axis).reshape(-1)
+        for use_ws in (True, False):
+            got, n_out = run(torch, gpu, x, elem, shape, axis, use_workspace=use_ws)
+            assert np.array_equal(got[:n_out].view(np.uint8), want.view(np.uint8)), (shape, axis, use_ws)
+
+
+def test_reduce_strided_views_and_errors(gpu, oracle):
+    import torch
+
+    rng = np.random.default_rng(11)
+    base = rng.normal(0, 1, (48, 40)).astype(np.float32)
+    # transposed view [40, 48] (strides 1, 40), both axes; output written with a padded stride
+    for axis in (0, 1):
+        want = oracle.reduce_max_abs(base.reshape(-1), ElemType.F32, (40, 48), axis, in_strides=(1, 40)).reshape(-1)
+        out_shape = (1, 48) if axis == 0 else (40, 1)
+        ostr = (0, 2) if axis == 0 else (3, 0)
+        got, n_out = run(torch, gpu, base, ElemType.F32, (40, 48), axis, in_strides=(1, 40), out_strides=ostr)
+        step = 2 if axis == 0 else 3
+        assert np.array_equal(got[::step][:n_out], want)
+    x = torch.zeros((4, 8), dtype=torch.float32, device="cuda")
+    h = TensorHandleRef.from_torch
+    client = ComputeClient.current()
+
+    def status(fn):
+        with pytest.raises(QuantError) as e:
+            fn()
+        return e.value.status
+
+    good = torch.zeros((4, 1), dtype=torch.float32, device="cuda")
+    bad = torch.zeros((4, 2), dtype=torch.float32, device="cuda")
+    assert status(lambda: cq_reduce.max_abs(client, h(x), h(good), 2, ElemType.F32)) == _ffi.ERR_INVALID_AXIS
+    assert status(lambda: cq_reduce.max_abs(client, h(x), h(bad), 1, ElemType.F32)) == _ffi.ERR_SHAPE_MISMATCH
+    assert status(lambda: cq_reduce.max_abs(client, h(x), h(good), 1, ElemType.BF16)) == _ffi.ERR_SHAPE_MISMATCH
+
+
+def test_reduce_feeds_per_channel_scales(gpu, oracle):
+    """The use the reference's callers make of MaxAbs: per-row abs-max -> scale by the
+    test's rule -> quantize with those scales.  A [rows, 128] tensor with block [128]
+    has exactly one block per row, so the two routes must agree."""
+    import torch
+    from cubek_amd import QuantLevel, QuantScheme, QuantValue
+
+    rng = np.random.default_rng(5)
+    shape = (256, 128)
+    x = rng.normal(0, 1, shape).astype(np.float32)
+    amax, _ = run(torch, gpu, x, ElemType.F32, shape, 1)
+    scheme = QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([128]))
+    s_blocks = gpu.compute_scales(x, ElemType.F32, shape, scheme).reshape(-1)
+    assert np.array_equal((2 * amax[:256]) / np.float32(254.0), s_blocks)
+
+
+# shape / strides / axis of the reference's reduce suite
+# (crates/cubek-reduce/tests/suite/mod.rs:134-230); it runs Sum/Mean/Prod/ArgMax/ArgMin
+# over this matrix, here it is MaxAbs.
+REFERENCE_MATRIX = [
+    ((22,), (1,), 0), ((1024,), (1,), 0),
+    ((4, 8), (8, 1), 1), ((4, 8), (8, 1), 0),
+    ((8, 256), (256, 1), 1), ((8, 256), (256, 1), 0),
+    ((16, 16, 16), (1, 256, 16), 0), ((16, 16, 16), (1, 256, 16), 1),
+    ((11, 12, 13), (156, 13, 1), 2),
+    ((4, 4, 4, 4), (1, 16, 64, 4), 0), ((4, 4, 4, 4), (1, 16, 64, 4), 1),
+    ((4, 4, 4, 4), (64, 16, 4, 1), 3),
+    ((8, 8), (64, 1), 1), ((8, 8), (64, 1), 0),
+    ((4, 32), (0, 1), 0),
+]
+
+
+@pytest.mark.parametrize("elem", ELEMS, ids=lambda e: e.name)
+def test_reduce_reference_matrix(gpu, oracle, elem):
+    import torch
+
+    rng = np.random.default_rng(int(elem) + 91)
+    for shape, strides, axis in REFERENCE_MATRIX:
+        reach = 1 + sum((n - 1) * st for n, st in zip(shape, strides))
+        x = oracle.to_bits(rng.uniform(-1, 1, reach).astype(np.float32), elem)
+        want = oracle.reduce_max_abs(x, elem, shape, axis, in_strides=strides).reshape(-1)
+        got, n_out = run(torch, gpu, x, elem, shape, axis, in_strides=strides)
+        assert np.array_equal(got[:n_out].view(np.uint8), want.view(np.uint8)), (shape, strides, axis)
