@@ -84,6 +84,7 @@ struct Plan {
     uint32_t bits, nq;            // bits per value; values per stored element
     cq::Range range;
     cq::Layout layout;
+    cq::ValueStrides vs;    // vs.on: a value tensor is not contiguous row-major
     bool tensor_level;
     bool last_dim_blocks;   // block extents are 1 everywhere but the last dimension
     uint32_t block_last;
@@ -105,7 +106,7 @@ uint32_t native_line_size(uint32_t elem_size, uint64_t last_dim) {
 }
 
 // `values` is the stored tensor, `floats` the float tensor (input of quantize,
-// output of dequantize); both must be contiguous and agree in shape.
+// output of dequantize); they must agree in shape and may have any strides.
 cq_status make_plan(const cq_scheme* s, const cq_tensor* floats, int dtype, const cq_tensor* values,
                     const cq_tensor* scale_a, uint32_t scale_a_size, const cq_tensor* scale_b,
                     uint32_t scale_b_size, Plan* p) {
@@ -128,7 +129,14 @@ cq_status make_plan(const cq_scheme* s, const cq_tensor* floats, int dtype, cons
         if (floats->shape[d] == 0 || floats->shape[d] > 0xffffffffull) return CQ_ERR_TOO_LARGE;
     }
     p->n = numel(floats);
-    if (!is_contiguous(floats) || !is_contiguous(values)) return CQ_ERR_NON_CONTIGUOUS;
+    std::memset(&p->vs, 0, sizeof(p->vs));
+    p->vs.on = !is_contiguous(floats) || !is_contiguous(values);
+    p->vs.rank = p->rank;
+    for (uint32_t d = 0; d < p->rank; d++) {
+        p->vs.shape[d] = static_cast<uint32_t>(p->shape[d]);
+        p->vs.floats[d] = floats->strides[d];
+        p->vs.stored[d] = values->strides[d];
+    }
 
     std::memset(&p->layout, 0, sizeof(p->layout));
     p->tensor_level = s->level == CQ_LEVEL_TENSOR;
@@ -170,7 +178,7 @@ cq_status make_plan(const cq_scheme* s, const cq_tensor* floats, int dtype, cons
 // the last axis that map onto lane groups, 16-byte aligned float tensor)
 bool flat_ok(const Plan& p, int dtype, const cq_tensor* floats, const cq_tensor* values,
              const cq_tensor* scale_a, const cq_tensor* scale_b) {
-    if (!aligned(floats->ptr, 16) || !aligned(values->ptr, 8)) return false;
+    if (p.vs.on || !aligned(floats->ptr, 16) || !aligned(values->ptr, 8)) return false;
     if (p.tensor_level) return true;
     if (!p.last_dim_blocks) return false;
     if (!is_contiguous(scale_a) || (scale_b && !is_contiguous(scale_b))) return false;
@@ -195,6 +203,7 @@ cq::GenericArgs generic_args(const Plan& p, const cq_scheme* s) {
     g.value = s->value;
     g.range = p.range;
     g.layout = p.layout;
+    g.vs = p.vs;
     return g;
 }
 
@@ -213,7 +222,7 @@ const char* cq_strerror(cq_status st) {
         case CQ_ERR_UNSUPPORTED_SCHEME: return "unsupported quantization scheme";
         case CQ_ERR_BLOCK_NOT_DIVISIBLE: return "block size must be divisible by the number of values per stored element";
         case CQ_ERR_SHAPE_MISMATCH: return "tensor shapes or element sizes do not agree with the scheme";
-        case CQ_ERR_NON_CONTIGUOUS: return "value tensors must be contiguous";
+        case CQ_ERR_NON_CONTIGUOUS: return "tensor must be contiguous";
         case CQ_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
         case CQ_ERR_HIP: return "HIP runtime error";
         case CQ_ERR_TOO_LARGE: return "tensor too large";
@@ -349,8 +358,16 @@ static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_sche
             return CQ_ERR_WORKSPACE_TOO_SMALL;
         if (!aligned(workspace, 4)) return CQ_ERR_INVALID_ARGUMENT;
         uint32_t num_partials = 0;
-        cq_status st = hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n,
-                                                             static_cast<float*>(workspace), &num_partials));
+        cq_status st;
+        if (p.vs.on) {
+            cq::GenericArgs g = generic_args(p, scheme);
+            g.input = input->ptr;
+            st = hip_status(cq::launch_absmax_partials_strided(stream, input_dtype, g, p.n,
+                                                               static_cast<float*>(workspace), &num_partials));
+        } else {
+            st = hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n,
+                                                       static_cast<float*>(workspace), &num_partials));
+        }
         if (st != CQ_OK) return st;
         return hip_status(cq::launch_tensor_scale(stream, input_dtype, out_dtype,
                                                   static_cast<const float*>(workspace), num_partials,
@@ -383,7 +400,7 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
     st = make_plan(scheme, input, input_dtype, &values, scales, dtype_size(input_dtype), nullptr, 0, &p);
     if (st != CQ_OK) return st;
 
-    if (!p.tensor_level && p.last_dim_blocks && is_contiguous(scales) && aligned(input->ptr, 16) &&
+    if (!p.vs.on && !p.tensor_level && p.last_dim_blocks && is_contiguous(scales) && aligned(input->ptr, 16) &&
         cq::flat_block_supported(input_dtype, p.block_last)) {
         cq::FlatArgs a{};
         a.input = input->ptr;

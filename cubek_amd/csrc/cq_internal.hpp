@@ -56,7 +56,18 @@ hipError_t launch_absmax_partials(hipStream_t s, int dtype, const void* input, u
 hipError_t launch_tensor_scale(hipStream_t s, int f_dtype, int out_dtype, const float* partials,
                                uint32_t num_partials, Range range, void* out);
 
-// Generic path: any rank, N-D blocks, strided scales; one thread per stored word.
+// Addressing of the two value tensors of a launch when they are not contiguous
+// row-major (the reference reads and writes them through linear views built from
+// shape and strides: crates/cubek-quant/src/quantize.rs:309-317, src/dequantize.rs:261-270).
+struct ValueStrides {
+    uint32_t on;                   // 0: both contiguous, offsets are the logical indices
+    uint32_t rank;
+    uint32_t shape[CQ_MAX_RANK];   // unpacked element shape
+    uint64_t floats[CQ_MAX_RANK];  // strides (elements) of the float tensor
+    uint64_t stored[CQ_MAX_RANK];  // strides (stored elements) of the quantized tensor
+};
+
+// Generic path: any rank, any strides, N-D blocks, strided scales; one thread per stored word.
 struct GenericArgs {
     const void* input;
     void* output;
@@ -68,6 +79,7 @@ struct GenericArgs {
     int value;  // cq_value
     Range range;
     Layout layout;
+    ValueStrides vs;
 };
 hipError_t launch_quantize_generic(hipStream_t s, int dtype, int bits, const GenericArgs& a);
 hipError_t launch_dequantize_generic(hipStream_t s, int dtype, int bits, const GenericArgs& a);
@@ -75,6 +87,10 @@ hipError_t launch_dequantize_generic(hipStream_t s, int dtype, int bits, const G
 // out_dtype(dtype(2*absmax/(hi-lo))) through layout.stride_b into scale_out
 hipError_t launch_scales_generic(hipStream_t s, int dtype, int out_dtype, const GenericArgs& a,
                                  uint64_t num_blocks);
+// per-tensor abs-max partials of a strided float tensor (`a.vs`, `a.input`); same
+// contract as launch_absmax_partials
+hipError_t launch_absmax_partials_strided(hipStream_t s, int dtype, const GenericArgs& a, uint64_t num_elems,
+                                          float* partials, uint32_t* num_partials);
 // native store (i8 / e4m3 / e5m2 / e2m1x2), one thread per stored byte
 hipError_t launch_quantize_native(hipStream_t s, int dtype, const GenericArgs& a);
 hipError_t launch_dequantize_native(hipStream_t s, int dtype, const GenericArgs& a);

@@ -1,5 +1,5 @@
-// Generic quantize / dequantize kernels: any rank, N-D blocks, strided scale
-// tensors, ragged tails, native (byte) store.  One thread per stored element,
+// Generic quantize / dequantize kernels: any rank, any strides, N-D blocks, strided
+// scale tensors, ragged tails, native (byte) store.  One thread per stored element,
 // scale addressing exactly as the reference's BlockScaledLayout
 // (crates/cubek-quant/src/layout/scales.rs:144-160, :179-194).  These kernels
 // are the fallback and tail path; the streaming shapes take the flat kernels.
@@ -35,6 +35,28 @@ __device__ __forceinline__ ScalePos scale_pos(const Layout& L, uint64_t elem) {
     return r;
 }
 
+// Memory offsets of stored element `p` (logical, row-major over the packed shape) and
+// of the first of its `per` float elements; `step` is the float tensor's stride along
+// the last dimension.
+struct ValuePos {
+    uint64_t f, v, step;
+};
+
+__device__ __forceinline__ ValuePos value_pos(const ValueStrides& S, uint64_t p, uint32_t per) {
+    if (!S.on) return ValuePos{p * per, p, 1};
+    const int last = static_cast<int>(S.rank) - 1;
+    ValuePos r{0, 0, S.floats[last]};
+    uint64_t rem = p;
+    for (int d = last; d >= 0; d--) {
+        const uint32_t n = d == last ? S.shape[d] / per : S.shape[d];
+        const uint64_t c = rem % n;
+        rem /= n;
+        r.f += c * (d == last ? per : 1u) * S.floats[d];
+        r.v += c * S.stored[d];
+    }
+    return r;
+}
+
 // write_scale (src/quantize.rs:83-98); returns the divisor F(FS(scale)).
 template <class F>
 __device__ __forceinline__ float fetch_divisor(const GenericArgs& a, uint64_t elem) {
@@ -52,12 +74,13 @@ __global__ __launch_bounds__(kThreads) void quantize_generic_kernel(GenericArgs 
     const uint32_t nq = 32u / bits, mask = (1u << bits) - 1u;
     const uint64_t e0 = p * nq;
     const float d = fetch_divisor<F>(a, e0);
+    const ValuePos vp = value_pos(a.vs, p, nq);
     uint32_t w = 0;
     for (uint32_t i = 0; i < nq; i++) {
-        float q = quantize_exact<F>(F::load(a.input, e0 + i), d, a.range.lo, a.range.hi);
+        float q = quantize_exact<F>(F::load(a.input, vp.f + i * vp.step), d, a.range.lo, a.range.hi);
         w |= (static_cast<uint32_t>(static_cast<int32_t>(q)) & mask) << (i * bits);
     }
-    static_cast<uint32_t*>(a.output)[p] = w;
+    static_cast<uint32_t*>(a.output)[vp.v] = w;
 }
 
 template <class F>
@@ -68,10 +91,11 @@ __global__ __launch_bounds__(kThreads) void dequantize_generic_kernel(GenericArg
     const uint64_t e0 = p * nq;
     ScalePos sp = scale_pos(a.layout, e0);
     const float s = F::round(load_dtype(a.param_dtype, a.scale_in, sp.a));
-    const uint32_t w = static_cast<const uint32_t*>(a.input)[p];
+    const ValuePos vp = value_pos(a.vs, p, nq);
+    const uint32_t w = static_cast<const uint32_t*>(a.input)[vp.v];
     for (uint32_t i = 0; i < nq; i++) {
         int32_t v = static_cast<int32_t>(w << (32 - bits - i * bits)) >> (32 - bits);
-        F::store(a.output, e0 + i, s * static_cast<float>(v));
+        F::store(a.output, vp.f + i * vp.step, s * static_cast<float>(v));
     }
 }
 
@@ -99,7 +123,7 @@ __global__ __launch_bounds__(kThreads) void scales_generic_kernel(GenericArgs a,
         for (int d = static_cast<int>(L.rank) - 1; d >= 0; d--) {
             uint32_t o = static_cast<uint32_t>(kr % L.block[d]);
             kr /= L.block[d];
-            lin += static_cast<uint64_t>(origin[d] + o) * mul;
+            lin += static_cast<uint64_t>(origin[d] + o) * (a.vs.on ? a.vs.floats[d] : mul);
             mul *= L.shape[d];
         }
         amax = fmaxf(amax, fabsf(F::load(a.input, lin)));
@@ -147,18 +171,19 @@ __global__ __launch_bounds__(kThreads) void quantize_native_kernel(GenericArgs a
     if (j >= a.word_end) return;
     uint8_t* out = static_cast<uint8_t*>(a.output);
     if (a.value == CQ_VALUE_E2M1) {
+        const ValuePos vp = value_pos(a.vs, j, 2);
         uint32_t byte = 0;
         for (uint32_t h = 0; h < 2; h++) {
-            uint64_t e = 2 * j + h;
-            float d = fetch_divisor<F>(a, e);
-            float c = quantize_exact<F>(F::load(a.input, e), d, a.range.lo, a.range.hi);
+            float d = fetch_divisor<F>(a, 2 * j + h);
+            float c = quantize_exact<F>(F::load(a.input, vp.f + h * vp.step), d, a.range.lo, a.range.hi);
             byte |= encode_native(a.value, c) << (4 * h);
         }
-        out[j] = static_cast<uint8_t>(byte);
+        out[vp.v] = static_cast<uint8_t>(byte);
     } else {
+        const ValuePos vp = value_pos(a.vs, j, 1);
         float d = fetch_divisor<F>(a, j);
-        float c = quantize_exact<F>(F::load(a.input, j), d, a.range.lo, a.range.hi);
-        out[j] = static_cast<uint8_t>(encode_native(a.value, c));
+        float c = quantize_exact<F>(F::load(a.input, vp.f), d, a.range.lo, a.range.hi);
+        out[vp.v] = static_cast<uint8_t>(encode_native(a.value, c));
     }
 }
 
@@ -167,14 +192,33 @@ template <class F>
 __global__ __launch_bounds__(kThreads) void dequantize_native_kernel(GenericArgs a) {
     uint64_t j = a.word_begin + static_cast<uint64_t>(blockIdx.x) * kThreads + threadIdx.x;
     if (j >= a.word_end) return;
-    const uint8_t b = static_cast<const uint8_t*>(a.input)[j];
     const uint32_t per = a.value == CQ_VALUE_E2M1 ? 2u : 1u;
+    const ValuePos vp = value_pos(a.vs, j, per);
+    const uint8_t b = static_cast<const uint8_t*>(a.input)[vp.v];
     for (uint32_t h = 0; h < per; h++) {
-        uint64_t e = per * j + h;
-        ScalePos sp = scale_pos(a.layout, e);
+        ScalePos sp = scale_pos(a.layout, per * j + h);
         float s = F::round(load_dtype(a.param_dtype, a.scale_in, sp.a));
         float v = decode_native(a.value, per == 2 ? (b >> (4 * h)) & 0xfu : b);
-        F::store(a.output, e, s * F::round(v));
+        F::store(a.output, vp.f + h * vp.step, s * F::round(v));
+    }
+}
+
+// Per-tensor abs-max of a strided float tensor, pass 1: grid-stride over the logical
+// elements, one f32 partial per workgroup.
+template <class F>
+__global__ __launch_bounds__(kThreads) void absmax_partials_strided_kernel(GenericArgs a, uint64_t num_elems,
+                                                                           float* __restrict__ partials) {
+    float m = 0.0f;
+    for (uint64_t e = static_cast<uint64_t>(blockIdx.x) * kThreads + threadIdx.x; e < num_elems;
+         e += static_cast<uint64_t>(gridDim.x) * kThreads)
+        m = fmaxf(m, fabsf(F::load(a.input, value_pos(a.vs, e, 1).f)));
+    m = group_max<kWave>(m);
+    __shared__ float lds[kThreads / kWave];
+    if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kThreads / kWave; w++) m = fmaxf(m, lds[w]);
+        partials[blockIdx.x] = m;
     }
 }
 
@@ -209,6 +253,16 @@ hipError_t launch_scales_generic(hipStream_t s, int dtype, int out_dtype, const 
     if (num_blocks == 0) return hipSuccess;
     CQ_SWITCH_DTYPE(dtype, hipLaunchKernelGGL((scales_generic_kernel<kF>), grid_for(num_blocks), dim3(kThreads), 0, s,
                                               a, out_dtype, num_blocks);
+                    return hipGetLastError())
+}
+
+hipError_t launch_absmax_partials_strided(hipStream_t s, int dtype, const GenericArgs& a, uint64_t num_elems,
+                                          float* partials, uint32_t* num_partials) {
+    const uint64_t want = (num_elems + kThreads * 8 - 1) / (kThreads * 8);
+    const uint32_t grid = static_cast<uint32_t>(want < 1 ? 1 : (want > kMaxPartials ? kMaxPartials : want));
+    *num_partials = grid;
+    CQ_SWITCH_DTYPE(dtype, hipLaunchKernelGGL((absmax_partials_strided_kernel<kF>), dim3(grid), dim3(kThreads), 0, s, a,
+                                              num_elems, partials);
                     return hipGetLastError())
 }
 

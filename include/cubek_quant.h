@@ -37,7 +37,7 @@ typedef enum cq_status {
     CQ_ERR_UNSUPPORTED_SCHEME = 2,  /* value/store/param combination not implemented     */
     CQ_ERR_BLOCK_NOT_DIVISIBLE = 3, /* check_block_size_compat failed (src/lib.rs:20-33) */
     CQ_ERR_SHAPE_MISMATCH = 4,      /* packed/unpacked/scales shapes do not agree        */
-    CQ_ERR_NON_CONTIGUOUS = 5,      /* value tensors must be contiguous row-major        */
+    CQ_ERR_NON_CONTIGUOUS = 5,      /* kept for ABI stability; no entry point returns it  */
     CQ_ERR_WORKSPACE_TOO_SMALL = 6,
     CQ_ERR_HIP = 7,                 /* a HIP runtime call failed; see cq_last_hip_error  */
     CQ_ERR_TOO_LARGE = 8,           /* more elements than an entry point accepts         */
@@ -127,10 +127,12 @@ cq_status cq_value_range(uint8_t value, float* range_min, float* range_max);
 /* ---- the path ---- */
 
 /* Replaces cubek_quant::quantize::launch_ref (src/quantize.rs:174-221).
- *   input      : float tensor of dtype `input_dtype`, contiguous
+ *   input      : float tensor of dtype `input_dtype`, any strides (contiguous row-major
+ *                tensors take the streaming kernels, anything else a per-element path)
  *   output     : U32 store -> u32 tensor, shape = input shape with the last
  *                dimension divided by num_quants (tests/suite/symmetric.rs:68-69);
- *                NATIVE store -> 1-byte tensor (E2M1: last dimension / 2)
+ *                NATIVE store -> 1-byte tensor (E2M1: last dimension / 2);
+ *                any strides that do not make two stored elements overlap
  *   scale      : scales typed as `input_dtype`, shape [1] (per-tensor) or one
  *                entry per block; its strides are honoured
  *   out_scale  : same shape as `scale`, typed as scheme->param; receives the
@@ -140,8 +142,8 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
                       const cq_scheme* scheme, cq_dtype input_dtype);
 
 /* Replaces cubek_quant::dequantize::launch_ref (src/dequantize.rs:171-229).
- *   values : quantized tensor as written by cq_quantize
- *   output : float tensor of dtype `output_dtype`, unpacked shape
+ *   values : quantized tensor as written by cq_quantize, any strides
+ *   output : float tensor of dtype `output_dtype`, unpacked shape, any strides
  *   params : scales typed as scheme->param */
 cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_tensor* output,
                         const cq_tensor* params, const cq_scheme* scheme,

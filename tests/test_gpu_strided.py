@@ -1,0 +1,153 @@
+"""Non-contiguous value tensors through the C ABI.  The reference addresses its
+tensors through linear views built from shape and strides
+(crates/cubek-quant/src/quantize.rs:309-317, src/dequantize.rs:261-270), so a
+strided tensor must give what its contiguous copy gives: the oracle runs on the
+copy, the GPU on the strided buffers, and the logical views are compared bit
+for bit.  Elements of the destination buffers outside the views must stay untouched."""
+import zlib
+
+import zlib
+
+import numpy as np
+import pytest
+from numpy.lib.stride_tricks import as_strided
+
+from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantScheme, QuantStore, QuantValue)
+from cubek_amd import dequantize as dq
+from cubek_amd import quantize as qz
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import gpu_harness
+
+    return gpu_harness
+
+
+def reach(shape, strides):
+    return 1 + sum((n - 1) * st for n, st in zip(shape, strides))
+
+
+def view(buf, shape, strides):
+    assert reach(shape, strides) <= buf.size
+    return as_strided(buf, shape, tuple(st * buf.itemsize for st in strides))
+
+
+def layouts(shape, per):
+    """(name, float strides, stored strides) for logical `shape`, `per` values per stored element."""
+    pshape = shape[:-1] + (shape[-1] // per,)
+    rank = len(shape)
+
+    def contiguous(sh, pad=0):
+        st, acc = [], 1
+        for i, n in enumerate(reversed(sh)):
+            st.append(acc)
+            acc *= n + (pad if i == 0 else 0)
+        return tuple(reversed(st))
+
+    def permuted(sh):
+        # memory order = reversed logical order (a transposed tensor)
+        st, acc = [], 1
+        for n in sh:
+            st.append(acc)
+            acc *= n
+        return tuple(st)
+
+    out = [("pitched", contiguous(shape, 5), contiguous(pshape, 3)),
+           ("transposed_floats", permuted(shape), contiguous(pshape)),
+           ("transposed_stored", contiguous(shape), permuted(pshape)),
+           ("both", permuted(shape), permuted(pshape))]
+    if rank >= 2:
+        out.append(("every_other_row", tuple(s * (2 if d == 0 else 1) for d, s in enumerate(contiguous(shape))),
+                    tuple(s * (2 if d == 0 else 1) for d, s in enumerate(contiguous(pshape)))))
+    return pshape, out
+
+
+SCHEMES = [
+    ("q8s_tensor", QuantScheme.default().with_value(QuantValue.Q8S)),
+    ("q4s_block32", QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([32]))),
+    ("q2f_block_2x16", QuantScheme.default().with_value(QuantValue.Q2F).with_level(QuantLevel.block([2, 16]))),
+    ("e2m1_u32_block16", QuantScheme.default().with_value(QuantValue.E2M1).with_level(QuantLevel.block([16]))),
+    ("q8f_native_block16", QuantScheme.default().with_value(QuantValue.Q8F).with_store(QuantStore.Native)
+     .with_level(QuantLevel.block([16]))),
+    ("e4m3_native_tensor", QuantScheme.default().with_value(QuantValue.E4M3).with_store(QuantStore.Native)),
+    ("e2m1_native_block32", QuantScheme.default().with_value(QuantValue.E2M1).with_store(QuantStore.Native)
+     .with_level(QuantLevel.block([32]))),
+]
+
+
+@pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
+@pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
+def test_strided_value_tensors(gpu, oracle, elem, name, scheme):
+    import torch
+
+    rng = np.random.default_rng(zlib.crc32(name.encode()) % 1000 + int(elem))
+    client = ComputeClient.current()
+    per = scheme.num_quants()
+    stored_np = np.uint32 if scheme.store == QuantStore.U32 else np.uint8
+    pe = gpu.param_elem(scheme)
+    for shape in ((6, 64), (2, 4, 96)):
+        pshape, cases = layouts(shape, per)
+        sshape = scheme.scales_shape(shape)
+        for case, fstr, vstr in cases:
+            fbuf = oracle.to_bits(rng.normal(0, 1, reach(shape, fstr)).astype(np.float32), elem)
+            xc = np.ascontiguousarray(view(fbuf, shape, fstr))
+            s_ref = oracle.compute_scales(xc, elem, shape, scheme)
+            w_ref, os_ref = oracle.quantize(xc, elem, shape, s_ref, scheme)
+            y_ref = oracle.dequantize(w_ref, shape, os_ref, elem, scheme)
+            tag = (name, elem.name, shape, case)
+
+            d_f = gpu.to_dev(fbuf)
+            h_f = gpu.handle(d_f, shape, fstr)
+            sentinel = 0xA5 if stored_np == np.uint8 else 0xA5A5A5A5
+            vbuf0 = np.full(reach(pshape, vstr), sentinel, dtype=stored_np)
+
+            def stored_handle():
+                d = gpu.to_dev(vbuf0)
+                return d, gpu.handle(d, pshape, vstr)
+
+            def check_stored(d_v, what):
+                got = gpu.to_host(d_v).view(stored_np)
+                assert np.array_equal(view(got, pshape, vstr), w_ref.reshape(pshape)), tag + (what,)
+                mask = np.ones(got.size, dtype=bool)
+                view(mask, pshape, vstr)[...] = False
+                assert np.all(got[mask] == sentinel), tag + (what, "wrote outside the view")
+
+            # scales from the strided floats
+            d_s = torch.zeros(sshape, dtype=gpu.storage_dtype(elem), device="cuda")
+            ws, nbytes = gpu.workspace(scheme, int(np.prod(shape)))
+            qz.compute_scales(client, h_f, gpu.handle(d_s), scheme, elem, ws.data_ptr(), nbytes)
+            assert np.array_equal(gpu.to_host(d_s).reshape(-1), s_ref.reshape(-1)), tag + ("scales",)
+
+            # quantize with given scales
+            d_v, h_v = stored_handle()
+            d_os = torch.zeros(sshape, dtype=gpu.storage_dtype(pe), device="cuda")
+            qz.launch_ref(client, h_f, h_v, gpu.handle(d_s), gpu.handle(d_os), scheme, elem)
+            torch.cuda.synchronize()
+            check_stored(d_v, "quantize")
+            assert np.array_equal(gpu.to_host(d_os).reshape(-1), os_ref.reshape(-1)), tag + ("out_scale",)
+
+            # fused dynamic quantize
+            d_v2, h_v2 = stored_handle()
+            d_os2 = torch.zeros(sshape, dtype=gpu.storage_dtype(pe), device="cuda")
+            qz.launch_dynamic(client, h_f, h_v2, gpu.handle(d_os2), scheme, elem, ws.data_ptr(), nbytes)
+            torch.cuda.synchronize()
+            check_stored(d_v2, "dynamic")
+            assert np.array_equal(gpu.to_host(d_os2).reshape(-1), os_ref.reshape(-1)), tag + ("dynamic out_scale",)
+
+            # dequantize strided stored -> strided floats
+            fill = np.float32(777.0) if elem == ElemType.F32 else np.uint16(0x7777)
+            ybuf0 = np.full(fbuf.size, fill, dtype=fbuf.dtype)
+            d_y = gpu.to_dev(ybuf0)
+            dq.launch_ref(client, h_v, gpu.handle(d_y, shape, fstr), gpu.handle(d_os), scheme, elem)
+            torch.cuda.synchronize()
+            got = gpu.to_host(d_y).view(fbuf.dtype)
+            lhs, rhs = view(got, shape, fstr), y_ref.reshape(shape)
+            if elem == ElemType.F32:
+                lhs, rhs = lhs.view(np.uint32), rhs.view(np.uint32)
+            assert np.array_equal(lhs, rhs), tag + ("dequantize",)
+            mask = np.ones(got.size, dtype=bool)
+            view(mask, shape, fstr)[...] = False
+            assert np.all(got[mask] == fill), tag + ("dequantize wrote outside the view",)
