@@ -6,8 +6,6 @@ copy, the GPU on the strided buffers, and the logical views are compared bit
 for bit.  Elements of the destination buffers outside the views must stay untouched."""
 import zlib
 
-import zlib
-
 import numpy as np
 import pytest
 from numpy.lib.stride_tricks import as_strided
