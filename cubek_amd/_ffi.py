@@ -20,6 +20,7 @@ EXPORTED_SYMBOLS = (
     "cq_value_size_bits", "cq_scheme_num_quants", "cq_value_range", "cq_quantize", "cq_dequantize",
     "cq_compute_scales", "cq_quantize_dynamic", "cq_workspace_bytes", "cq_strerror",
     "cq_last_hip_error", "cq_abi_version", "cq_reduce_max_abs", "cq_reduce_workspace_bytes",
+    "cq_into_contiguous_packed",
 )
 
 
@@ -88,6 +89,9 @@ def lib() -> ctypes.CDLL:
                                     ctypes.c_size_t]
     L.cq_reduce_workspace_bytes.restype = ctypes.c_size_t
     L.cq_reduce_workspace_bytes.argtypes = [tp, ctypes.c_uint32, ctypes.c_int]
+    L.cq_into_contiguous_packed.restype = ctypes.c_int
+    L.cq_into_contiguous_packed.argtypes = [ctypes.c_void_p, tp, tp, ctypes.POINTER(ctypes.c_uint64), ctypes.c_uint32,
+                                            ctypes.c_uint32]
     _lib = L
     return L
 

@@ -490,6 +490,42 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
     return st;
 }
 
+cq_status cq_into_contiguous_packed(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                                    const uint64_t* shape, uint32_t rank, uint32_t packing) {
+    if (!tensor_ok(input) || !tensor_ok(output) || !shape) return CQ_ERR_INVALID_ARGUMENT;
+    if (input->rank != rank || output->rank != rank) return CQ_ERR_SHAPE_MISMATCH;
+    const uint32_t elem = input->elem_size;
+    if ((elem != 4 && elem != 1) || output->elem_size != elem) return CQ_ERR_SHAPE_MISMATCH;
+    if (packing == 0 || (8 * elem) % packing) return CQ_ERR_INVALID_ARGUMENT;
+    cq::RepackArgs a;
+    std::memset(&a, 0, sizeof(a));
+    // packed along the rightmost dimension of stride 1
+    a.packed_dim = rank - 1;
+    for (int d = static_cast<int>(rank) - 1; d >= 0; d--)
+        if (input->strides[d] == 1) {
+            a.packed_dim = static_cast<uint32_t>(d);
+            break;
+        }
+    if (shape[rank - 1] % packing || shape[a.packed_dim] % packing) return CQ_ERR_SHAPE_MISMATCH;
+    a.num_out = 1;
+    for (uint32_t d = 0; d < rank; d++) {
+        if (shape[d] > 0xffffffffull) return CQ_ERR_TOO_LARGE;
+        if (input->shape[d] != (d == a.packed_dim ? shape[d] / packing : shape[d])) return CQ_ERR_SHAPE_MISMATCH;
+        if (output->shape[d] != (d + 1 == rank ? shape[d] / packing : shape[d])) return CQ_ERR_SHAPE_MISMATCH;
+        a.shape[d] = static_cast<uint32_t>(shape[d]);
+        a.strides[d] = input->strides[d];
+        a.num_out *= output->shape[d];
+    }
+    if (!is_contiguous(output)) return CQ_ERR_NON_CONTIGUOUS;
+    a.input = input->ptr;
+    a.output = output->ptr;
+    a.elem_bytes = elem;
+    a.packing = packing;
+    a.bits = 8 * elem / packing;
+    a.rank = rank;
+    return hip_status(cq::launch_repack(stream, a));
+}
+
 static bool reduce_view(const cq_tensor* input, uint32_t axis, uint64_t* outer, uint64_t* len, uint64_t* inner) {
     *outer = *inner = 1;
     for (uint32_t d = 0; d < axis; d++) *outer *= input->shape[d];

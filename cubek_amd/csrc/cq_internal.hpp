@@ -110,4 +110,18 @@ struct ReduceArgs {
 hipError_t launch_reduce_max_abs(hipStream_t s, int dtype, const ReduceArgs& a);
 uint64_t reduce_workspace_bytes(uint64_t outer, uint64_t len, uint64_t inner, int dtype);
 
+
+// Re-packing of a strided quantized tensor (cq_into_contiguous_packed).
+struct RepackArgs {
+    const void* input;
+    void* output;
+    uint32_t elem_bytes;          // 4 (u32 words) or 1 (bytes)
+    uint32_t packing, bits;       // values per stored element, bits per value
+    uint32_t rank, packed_dim;
+    uint32_t shape[CQ_MAX_RANK];  // logical (unpacked) shape
+    uint64_t strides[CQ_MAX_RANK];  // input strides, in stored elements
+    uint64_t num_out;             // stored elements of the output
+};
+hipError_t launch_repack(hipStream_t s, const RepackArgs& a);
+
 }  // namespace cq

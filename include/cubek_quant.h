@@ -37,7 +37,7 @@ typedef enum cq_status {
     CQ_ERR_UNSUPPORTED_SCHEME = 2,  /* value/store/param combination not implemented     */
     CQ_ERR_BLOCK_NOT_DIVISIBLE = 3, /* check_block_size_compat failed (src/lib.rs:20-33) */
     CQ_ERR_SHAPE_MISMATCH = 4,      /* packed/unpacked/scales shapes do not agree        */
-    CQ_ERR_NON_CONTIGUOUS = 5,      /* kept for ABI stability; no entry point returns it  */
+    CQ_ERR_NON_CONTIGUOUS = 5,      /* an output that must be contiguous row-major is not */
     CQ_ERR_WORKSPACE_TOO_SMALL = 6,
     CQ_ERR_HIP = 7,                 /* a HIP runtime call failed; see cq_last_hip_error  */
     CQ_ERR_TOO_LARGE = 8,           /* more elements than an entry point accepts         */
@@ -183,6 +183,22 @@ size_t cq_workspace_bytes(const cq_scheme* scheme, uint64_t num_elements);
 cq_status cq_reduce_max_abs(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
                             uint32_t axis, cq_dtype dtype, void* workspace, size_t workspace_bytes);
 size_t cq_reduce_workspace_bytes(const cq_tensor* input, uint32_t axis, cq_dtype dtype);
+
+/* ---- re-packing of strided quantized tensors (the step behind the path) ---- */
+
+/* Replaces cubecl_std::tensor::into_contiguous_packed as cubek-matmul calls it on a
+ * quantized operand (crates/cubek-matmul/src/base.rs:505-529): a quantized tensor with
+ * any strides (e.g. a transposed view) becomes a contiguous one packed along the last
+ * dimension of the logical shape.
+ *   input   : u32 (elem_size 4) or u8 (elem_size 1) tensor holding `packing` values per
+ *             element, value 0 in the low bits, packed along the rightmost dimension
+ *             whose stride is 1 (the last one if there is none); its shape is `shape`
+ *             with that dimension divided by `packing`
+ *   shape   : logical (unpacked) shape, `rank` entries; the last dimension and the
+ *             packed dimension must be multiples of `packing`
+ *   output  : contiguous, same element type, `shape` with the last dimension / packing */
+cq_status cq_into_contiguous_packed(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                                    const uint64_t* shape, uint32_t rank, uint32_t packing);
 
 /* ---- diagnostics ---- */
 const char* cq_strerror(cq_status status);

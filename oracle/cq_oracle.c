@@ -469,6 +469,47 @@ int cqo_reduce_max_abs(const void* input, int dtype, uint32_t rank, const uint64
     return 0;
 }
 
+/* Re-pack a strided quantized tensor into a contiguous one packed along the last
+ * dimension: what cubek-matmul asks of cubecl-std's into_contiguous_packed
+ * (crates/cubek-matmul/src/base.rs:505-529).  `shape` is the logical (unpacked)
+ * shape; the input stores `packing` values per element along `packed_dim`, value 0
+ * in the low bits, and is addressed through `in_strides`; output element `pos`
+ * gathers the logical values pos*packing .. pos*packing+packing-1.
+ * parity unpinned: cubecl-std is not vendored with the reference. */
+int cqo_into_contiguous_packed(const void* input, uint32_t elem_bytes, uint32_t packing, uint32_t rank,
+                               const uint64_t* shape, const uint64_t* in_strides, uint32_t packed_dim,
+                               void* output) {
+    if ((elem_bytes != 1 && elem_bytes != 4) || packing == 0 || (8 * elem_bytes) % packing || rank == 0 ||
+        packed_dim >= rank || shape[rank - 1] % packing || shape[packed_dim] % packing)
+        return -1;
+    const uint32_t bits = 8 * elem_bytes / packing;
+    const uint32_t mask = bits == 32 ? 0xffffffffu : (1u << bits) - 1u;
+    uint64_t n = 1;
+    for (uint32_t d = 0; d < rank; d++) n *= shape[d];
+    for (uint64_t pos = 0; pos < n / packing; pos++) {
+        uint32_t out = 0;
+        for (uint32_t k = 0; k < packing; k++) {
+            uint64_t rem = pos * packing + k, off = 0, sub = 0;
+            for (int d = (int)rank - 1; d >= 0; d--) {
+                uint64_t c = rem % shape[d];
+                rem /= shape[d];
+                if ((uint32_t)d == packed_dim) {
+                    sub = c % packing;
+                    c /= packing;
+                }
+                off += c * in_strides[d];
+            }
+            uint32_t word = elem_bytes == 4 ? ((const uint32_t*)input)[off] : ((const uint8_t*)input)[off];
+            out |= ((word >> (sub * bits)) & mask) << (k * bits);
+        }
+        if (elem_bytes == 4)
+            ((uint32_t*)output)[pos] = out;
+        else
+            ((uint8_t*)output)[pos] = (uint8_t)out;
+    }
+    return 0;
+}
+
 /* --------------------------------------------------------- threaded drivers */
 
 typedef struct {

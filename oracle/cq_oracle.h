@@ -79,6 +79,12 @@ int cqo_reduce_max_abs(const void* input, int dtype, uint32_t rank, const uint64
                        const uint64_t* in_strides, uint32_t axis, void* output,
                        const uint64_t* out_strides);
 
+/* strided quantized tensor -> contiguous, packed along the last dimension
+ * (cubecl-std into_contiguous_packed as called at crates/cubek-matmul/src/base.rs:505-529) */
+int cqo_into_contiguous_packed(const void* input, uint32_t elem_bytes, uint32_t packing, uint32_t rank,
+                               const uint64_t* shape, const uint64_t* in_strides, uint32_t packed_dim,
+                               void* output);
+
 /* threaded drivers used for the CPU baseline timing (split the word range) */
 int cqo_quantize_packed_mt(const void* input, int dtype, uint32_t rank, const uint64_t* shape,
                            const void* scale, const uint64_t* scale_strides, void* out_scale,

@@ -86,6 +86,9 @@ def _declare(L):
     L.cqo_dequantize_packed_mt.argtypes = d_args + [ctypes.c_int]
     L.cqo_reduce_max_abs.restype = ctypes.c_int
     L.cqo_reduce_max_abs.argtypes = [_vp, ctypes.c_int, ctypes.c_uint32, _u64p, _u64p, ctypes.c_uint32, _vp, _u64p]
+    L.cqo_into_contiguous_packed.restype = ctypes.c_int
+    L.cqo_into_contiguous_packed.argtypes = [_vp, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, _u64p, _u64p,
+                                             ctypes.c_uint32, _vp]
     L.cqo_compute_scales.restype = ctypes.c_int
     L.cqo_compute_scales.argtypes = [_vp, ctypes.c_int, ctypes.c_uint32, _u64p, _vp, _sp]
 
@@ -261,4 +264,20 @@ def reduce_max_abs(x: np.ndarray, elem: ElemType, shape, axis: int, in_strides=N
                                   _ptr(out), _u64(contiguous_strides(out_shape)))
     if rc:
         raise RuntimeError(f"cqo_reduce_max_abs failed: {rc}")
+    return out
+
+
+def into_contiguous_packed(buf: np.ndarray, packing: int, shape, in_strides, packed_dim: int) -> np.ndarray:
+    """Strided stored tensor (``buf`` uint32 or uint8, ``packing`` values per element along
+    ``packed_dim``) -> contiguous tensor packed along the last dimension of the logical ``shape``."""
+    buf = np.ascontiguousarray(buf)
+    assert buf.dtype in (np.uint32, np.uint8)
+    in_shape = tuple(s // packing if d == packed_dim else s for d, s in enumerate(shape))
+    assert 1 + sum((n - 1) * st for n, st in zip(in_shape, in_strides)) <= buf.size
+    out_shape = tuple(shape[:-1]) + (shape[-1] // packing,)
+    out = np.zeros(out_shape, dtype=buf.dtype)
+    rc = lib().cqo_into_contiguous_packed(_ptr(buf), buf.itemsize, packing, len(shape), _u64(shape),
+                                          _u64(in_strides), packed_dim, _ptr(out))
+    if rc:
+        raise RuntimeError(f"cqo_into_contiguous_packed failed: {rc}")
     return out
