@@ -7,6 +7,8 @@
 #include "cq_device.hpp"
 #include "cq_internal.hpp"
 
+#include <cstring>
+
 namespace cq {
 namespace {
 
@@ -48,10 +50,157 @@ __global__ __launch_bounds__(kThreads) void repack_generic_kernel(RepackArgs a) 
     static_cast<W*>(a.output)[pos] = static_cast<W>(out);
 }
 
+// ---- tiled transposition: packed along a stride-1 dimension that is not the last ----
+// In the plane of (packed dim p, last dim l) the input is [l][p / P] words and the
+// output [p][l / P] words.  A block of P input words (P consecutive l, one word
+// column) holds a P x P matrix of fields whose transpose is P output words (P
+// consecutive p, one word column).  A workgroup moves a tile of 32*P input rows x
+// 32 or 64 word columns: every thread loads four such blocks with 16-byte loads,
+// transposes them in registers, scatters the words into LDS laid out as the output
+// tile (word columns * P rows x 32 words), and the workgroup streams that out in 16-byte stores.
+struct TileArgs {
+    const uint32_t* in;
+    uint32_t* out;
+    uint32_t wp, wl;        // input words along p, output words along l
+    uint64_t in_l_stride;   // input stride of the last dimension, in words
+    uint64_t out_p_stride;  // output stride of the packed dimension, in words
+    uint32_t num_batch_dims;
+    uint32_t batch_shape[CQ_MAX_RANK];
+    uint64_t batch_in[CQ_MAX_RANK], batch_out[CQ_MAX_RANK];
+};
+
+// Transpose the kP x kP matrix of (32/kP)-bit fields held in kP words: field s of word
+// i <-> field i of word s.  Recursive off-diagonal block swaps.
+template <int kP>
+__device__ __forceinline__ void transpose_fields(uint32_t (&a)[kP]) {
+    constexpr int kBits = 32 / kP;
+#pragma unroll
+    for (int b = 1; b < kP; b <<= 1) {
+        uint32_t mask = 0;  // fields whose index has bit `b` clear
+#pragma unroll
+        for (int f = 0; f < kP; f++)
+            if (!(f & b)) mask |= ((kBits == 32 ? 0u : (1u << kBits)) - 1u) << (f * kBits);
+#pragma unroll
+        for (int r = 0; r < kP; r++) {
+            if (r & b) continue;
+            const uint32_t t = ((a[r] >> (b * kBits)) ^ a[r + b]) & mask;
+            a[r + b] ^= t;
+            a[r] ^= t << (b * kBits);
+        }
+    }
+}
+
+// kTileWords: input word columns per tile (a multiple of 4, at most 64);
+// kTileCols: output word columns per tile (input rows / kP).
+template <int kP, int kTileWords, int kTileCols>
+__global__ __launch_bounds__(kTileWords / 4 * kTileCols) void repack_tile_kernel(TileArgs a) {
+    constexpr int kQuads = kTileWords / 4;   // 16-byte word quads per tile row of the input
+    constexpr int kT = kQuads * kTileCols;   // threads
+    constexpr int kTileRows = kTileWords * kP;  // output rows (p values) per tile
+    constexpr int kRot = 64 / kQuads >= 4 ? 64 / kQuads : 4;
+    __shared__ uint32_t lds[kTileRows * kTileCols];
+    const uint32_t pq = threadIdx.x % kQuads, lw = threadIdx.x / kQuads;
+    const uint32_t pw0 = blockIdx.x * kTileWords, lw0 = blockIdx.y * kTileCols;
+    uint64_t in_base = 0, out_base = 0;
+    {
+        uint32_t rem = blockIdx.z;
+        for (int d = static_cast<int>(a.num_batch_dims) - 1; d >= 0; d--) {
+            const uint32_t c = rem % a.batch_shape[d];
+            rem /= a.batch_shape[d];
+            in_base += c * a.batch_in[d];
+            out_base += c * a.batch_out[d];
+        }
+    }
+    const uint32_t pw = pw0 + 4 * pq;
+    if (pw < a.wp && lw0 + lw < a.wl) {
+        u32x4 raw[kP];
+        const uint32_t* src = a.in + in_base + static_cast<uint64_t>(lw0 + lw) * kP * a.in_l_stride + pw;
+#pragma unroll
+        for (int i = 0; i < kP; i++) raw[i] = stream_load(reinterpret_cast<const u32x4*>(src + i * a.in_l_stride));
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            uint32_t blk[kP];
+#pragma unroll
+            for (int i = 0; i < kP; i++) blk[i] = raw[i][q];
+            transpose_fields<kP>(blk);
+            // all rows start at the same bank; rotating the columns by a multiple of pq
+            // spreads the lanes of a wave evenly over the banks
+            const uint32_t col = (lw + pq * kRot) % kTileCols;
+#pragma unroll
+            for (int s = 0; s < kP; s++) lds[((4 * pq + q) * kP + s) * kTileCols + col] = blk[s];
+        }
+    }
+    __syncthreads();
+    constexpr int kRowsPerPass = kT / (kTileCols / 4);
+#pragma unroll
+    for (int r = 0; r < kTileRows / kRowsPerPass; r++) {
+        const uint32_t row = r * kRowsPerPass + threadIdx.x / (kTileCols / 4), c4 = (threadIdx.x % (kTileCols / 4)) * 4;
+        const uint64_t p = static_cast<uint64_t>(pw0) * kP + row;
+        if (p < static_cast<uint64_t>(a.wp) * kP && lw0 + c4 < a.wl) {
+            const uint32_t col = (c4 + (row / (4 * kP)) * kRot) % kTileCols;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(&lds[row * kTileCols + col]);
+            stream_store(v, reinterpret_cast<u32x4*>(a.out + out_base + p * a.out_p_stride + lw0 + c4));
+        }
+    }
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Fills `t` and returns true when the tiled kernel can take the launch.
+bool plan_tiles(const RepackArgs& a, TileArgs* t, dim3* grid, uint32_t tile_words, uint32_t tile_cols) {
+    const uint32_t last = a.rank - 1, pd = a.packed_dim;
+    if (a.elem_bytes != 4 || (a.packing != 4 && a.packing != 8 && a.packing != 16)) return false;
+    if (a.rank < 2 || pd == last || a.strides[pd] != 1) return false;
+    if (!aligned16(a.input) || !aligned16(a.output)) return false;
+    std::memset(t, 0, sizeof(*t));
+    t->in = static_cast<const uint32_t*>(a.input);
+    t->out = static_cast<uint32_t*>(a.output);
+    t->wp = a.shape[pd] / a.packing;
+    t->wl = a.shape[last] / a.packing;
+    if (t->wp % 4 || t->wl % 4) return false;
+    t->in_l_stride = a.strides[last];
+    if (t->in_l_stride % 4) return false;
+    // contiguous strides of the output [.., shape[last] / packing]
+    uint64_t ostride[CQ_MAX_RANK], acc = 1;
+    for (int d = static_cast<int>(last); d >= 0; d--) {
+        ostride[d] = acc;
+        acc *= static_cast<uint32_t>(d) == last ? t->wl : a.shape[d];
+    }
+    t->out_p_stride = ostride[pd];
+    uint64_t batches = 1;
+    for (uint32_t d = 0; d < a.rank; d++) {
+        if (d == pd || d == last) continue;
+        if (a.strides[d] % 4) return false;
+        t->batch_shape[t->num_batch_dims] = a.shape[d];
+        t->batch_in[t->num_batch_dims] = a.strides[d];
+        t->batch_out[t->num_batch_dims] = ostride[d];
+        t->num_batch_dims++;
+        batches *= a.shape[d];
+    }
+    const uint64_t tiles_p = (t->wp + tile_words - 1) / tile_words;
+    const uint64_t tiles_l = (t->wl + tile_cols - 1) / tile_cols;
+    if (batches > 65535 || tiles_l > 65535 || tiles_p > 0x7fffffffull) return false;
+    *grid = dim3(static_cast<uint32_t>(tiles_p), static_cast<uint32_t>(tiles_l), static_cast<uint32_t>(batches));
+    return true;
+}
+
 }  // namespace
 
 hipError_t launch_repack(hipStream_t s, const RepackArgs& a) {
     if (a.num_out == 0) return hipSuccess;
+    TileArgs t;
+    dim3 tile_grid;
+    // tile = 32 output word columns x (64 | 32 | 32) input word columns for P = 4 | 8 | 16:
+    // both sides move whole 128-byte lines (64-byte segments measured at two thirds of this)
+    const uint32_t tile_words = a.packing == 4 ? 64 : 32;
+    if (plan_tiles(a, &t, &tile_grid, tile_words, 32)) {
+        switch (a.packing) {
+            case 4: hipLaunchKernelGGL((repack_tile_kernel<4, 64, 32>), tile_grid, dim3(512), 0, s, t); break;
+            case 8: hipLaunchKernelGGL((repack_tile_kernel<8, 32, 32>), tile_grid, dim3(256), 0, s, t); break;
+            default: hipLaunchKernelGGL((repack_tile_kernel<16, 32, 32>), tile_grid, dim3(256), 0, s, t); break;
+        }
+        return hipGetLastError();
+    }
     const dim3 grid(static_cast<uint32_t>((a.num_out + kThreads - 1) / kThreads));
     if (a.elem_bytes == 4)
         hipLaunchKernelGGL((repack_generic_kernel<uint32_t>), grid, dim3(kThreads), 0, s, a);

@@ -253,4 +253,21 @@ inline void max_abs(const ComputeClient& client, const TensorHandleRef& input, c
 }
 }  // namespace reduce
 
+namespace contiguous {
+// cubecl_std::tensor::into_contiguous_packed_ref as cubek-matmul uses it on quantized operands
+// (crates/cubek-matmul/src/base.rs:505-529): `shape` is the logical shape, `packing` the values per
+// stored element; `output` is contiguous with the last dimension of `shape` divided by `packing`.
+inline void into_contiguous_packed_ref(const ComputeClient& client, const TensorHandleRef& input,
+                                       const TensorHandleRef& output, const std::vector<uint64_t>& shape,
+                                       uint32_t packing) {
+    cq_tensor i = input.as_c(), o = output.as_c();
+    const cq_status st = cq_into_contiguous_packed(client.stream, &i, &o, shape.data(),
+                                                   static_cast<uint32_t>(shape.size()), packing);
+    if (st == CQ_OK) return;
+    if (st == CQ_ERR_HIP)
+        throw LaunchError(std::string(cq_strerror(st)) + " (hipError_t " + std::to_string(cq_last_hip_error()) + ")");
+    throw std::invalid_argument(cq_strerror(st));
+}
+}  // namespace contiguous
+
 }  // namespace cubek_quant

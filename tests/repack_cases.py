@@ -3,7 +3,7 @@ that builds the strided, packed input from a logical array (the inverse directio
 import numpy as np
 
 # (name, stored dtype, packing, logical shape, packed_dim, memory order of the input's dims
-#  from slowest to fastest; padding is added to the slowest one)
+#  from slowest to fastest)
 CASES = [
     ("u32x4_rows_pitched", np.uint32, 4, (6, 32), 1, (0, 1)),
     ("u32x8_transposed", np.uint32, 8, (16, 24), 0, (1, 0)),
@@ -27,9 +27,9 @@ def pack_last(logical: np.ndarray, dtype, packing: int) -> np.ndarray:
     return out.astype(dtype)
 
 
-def scatter_packed(logical: np.ndarray, dtype, packing: int, packed_dim: int, order, rng):
+def scatter_packed(logical: np.ndarray, dtype, packing: int, packed_dim: int, order, rng, pad: int = 3):
     """Pack `logical` along packed_dim and lay the result out in memory with the dims
-    ordered `order` (slowest first, the slowest padded).  Returns (buffer, strides in elements)."""
+    ordered `order` (slowest first); the rows of the fastest dim get `pad` extra elements.  Returns (buffer, strides in elements)."""
     moved = np.moveaxis(logical, packed_dim, -1)
     packed = np.moveaxis(pack_last(moved, dtype, packing), -1, packed_dim)  # shape with packed_dim / packing
     in_shape = packed.shape
@@ -37,7 +37,7 @@ def scatter_packed(logical: np.ndarray, dtype, packing: int, packed_dim: int, or
     acc = 1
     for i, d in enumerate(reversed(order)):
         strides[d] = acc
-        acc *= in_shape[d] + (3 if i == len(order) - 2 else 0)  # pad the pitch of the second fastest dim
+        acc *= in_shape[d] + (pad if i == 0 else 0)  # pad the pitch of the fastest dim
     reach = 1 + sum((n - 1) * st for n, st in zip(in_shape, strides))
     info = np.iinfo(dtype)
     buf = rng.integers(0, int(info.max) + 1, size=reach, dtype=np.uint64).astype(dtype)  # garbage in the gaps

@@ -10,7 +10,11 @@ pytestmark = pytest.mark.gpu
 
 BIG = [
     ("u32x8_transposed_big", np.uint32, 8, (1024, 768), 0, (1, 0)),
-    ("u32x4_transposed_ragged_tiles", np.uint32, 4, (520, 1000), 0, (1, 0)),
+    ("u32x4_transposed_ragged_tiles", np.uint32, 4, (528, 1008), 0, (1, 0)),
+    ("u32x8_transposed_ragged_tiles", np.uint32, 8, (2080, 2336), 0, (1, 0)),
+    ("u32x16_transposed_ragged_tiles", np.uint32, 16, (320, 1088), 0, (1, 0)),
+    ("u32x8_rank4_batched_transposed", np.uint32, 8, (2, 3, 64, 96), 2, (1, 0, 3, 2)),
+    ("u32x8_batch_between", np.uint32, 8, (64, 5, 128), 0, (1, 2, 0)),
     ("u32x16_transposed_big", np.uint32, 16, (512, 2048), 0, (1, 0)),
     ("u32x8_batched_transposed_big", np.uint32, 8, (3, 256, 640), 1, (0, 2, 1)),
     ("u32x8_rows_pitched_big", np.uint32, 8, (300, 4096), 1, (0, 1)),
@@ -38,13 +42,16 @@ def run(gpu, buf, dtype, packing, shape, in_strides, packed_dim):
     return gpu.to_host(d_out).view(dtype)
 
 
+@pytest.mark.parametrize("pad", [0, 3, 4], ids=lambda p: f"pad{p}")
 @pytest.mark.parametrize("case", CASES + BIG, ids=[c[0] for c in CASES + BIG])
-def test_into_contiguous_packed(gpu, oracle, case):
+def test_into_contiguous_packed(gpu, oracle, case, pad):
+    # pad 0 / 4 keep the rows 16-byte aligned (tiled transposition where it applies),
+    # pad 3 does not (per-element kernel)
     name, dtype, packing, shape, packed_dim, order = case
     rng = np.random.default_rng(len(name) * 5 + packing)
     bits = 8 * np.dtype(dtype).itemsize // packing
     logical = rng.integers(0, 1 << bits, size=shape, dtype=np.uint64)
-    buf, in_strides = scatter_packed(logical, dtype, packing, packed_dim, order, rng)
+    buf, in_strides = scatter_packed(logical, dtype, packing, packed_dim, order, rng, pad)
     want = oracle.into_contiguous_packed(buf, packing, shape, in_strides, packed_dim)
     assert np.array_equal(want, pack_last(logical, dtype, packing))
     got = run(gpu, buf, dtype, packing, shape, in_strides, packed_dim)
