@@ -184,10 +184,33 @@ bool plan_tiles(const RepackArgs& a, TileArgs* t, dim3* grid, uint32_t tile_word
     return true;
 }
 
+// Bytes holding two 4-bit values, low nibble first, are bit for bit u32 words holding
+// eight (little endian): when everything is a multiple of a word, re-express the launch
+// in words so that the tiled kernel can take it.
+bool bytes_as_words(const RepackArgs& a, RepackArgs* w) {
+    const uint32_t last = a.rank - 1, pd = a.packed_dim;
+    if (a.elem_bytes != 1 || a.packing != 2 || a.rank < 2 || pd == last || a.strides[pd] != 1) return false;
+    if (a.shape[pd] % 8 || a.shape[last] % 8) return false;
+    *w = a;
+    w->elem_bytes = 4;
+    w->packing = 8;
+    w->bits = 4;
+    for (uint32_t d = 0; d < a.rank; d++) {
+        if (d == pd) continue;
+        if (a.strides[d] % 4) return false;
+        w->strides[d] = a.strides[d] / 4;
+    }
+    w->num_out = a.num_out / 4;
+    return true;
+}
+
 }  // namespace
 
-hipError_t launch_repack(hipStream_t s, const RepackArgs& a) {
-    if (a.num_out == 0) return hipSuccess;
+hipError_t launch_repack(hipStream_t s, const RepackArgs& bytes_or_words) {
+    if (bytes_or_words.num_out == 0) return hipSuccess;
+    RepackArgs as_words;
+    const RepackArgs& a = bytes_as_words(bytes_or_words, &as_words) ? as_words : bytes_or_words;
+    const RepackArgs& g = bytes_or_words;  // the per-element kernel takes the launch as it came
     TileArgs t;
     dim3 tile_grid;
     // tile = 32 output word columns x (64 | 32 | 32) input word columns for P = 4 | 8 | 16:
@@ -201,11 +224,11 @@ hipError_t launch_repack(hipStream_t s, const RepackArgs& a) {
         }
         return hipGetLastError();
     }
-    const dim3 grid(static_cast<uint32_t>((a.num_out + kThreads - 1) / kThreads));
-    if (a.elem_bytes == 4)
-        hipLaunchKernelGGL((repack_generic_kernel<uint32_t>), grid, dim3(kThreads), 0, s, a);
+    const dim3 grid(static_cast<uint32_t>((g.num_out + kThreads - 1) / kThreads));
+    if (g.elem_bytes == 4)
+        hipLaunchKernelGGL((repack_generic_kernel<uint32_t>), grid, dim3(kThreads), 0, s, g);
     else
-        hipLaunchKernelGGL((repack_generic_kernel<uint8_t>), grid, dim3(kThreads), 0, s, a);
+        hipLaunchKernelGGL((repack_generic_kernel<uint8_t>), grid, dim3(kThreads), 0, s, g);
     return hipGetLastError();
 }
 

@@ -19,6 +19,9 @@ BIG = [
     ("u32x8_batched_transposed_big", np.uint32, 8, (3, 256, 640), 1, (0, 2, 1)),
     ("u32x8_rows_pitched_big", np.uint32, 8, (300, 4096), 1, (0, 1)),
     ("u8x2_transposed_big", np.uint8, 2, (512, 384), 0, (1, 0)),
+    ("u8x2_transposed_ragged_tiles", np.uint8, 2, (2080, 1312), 0, (1, 0)),
+    ("u8x2_batched_transposed_big", np.uint8, 2, (3, 256, 640), 1, (0, 2, 1)),
+    ("u8x2_transposed_not_word_multiple", np.uint8, 2, (516, 388), 0, (1, 0)),
 ]
 
 
