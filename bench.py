@@ -211,6 +211,50 @@ def cpu_baseline(torch, w, path, budget_s=12.0):
     }
 
 
+def adjacent_kernels(torch):
+    """The steps either side of the path on the headline tensor: abs-max along an axis
+    (cq_reduce_max_abs) in front of it, re-packing of a transposed quantized tensor
+    (cq_into_contiguous_packed) behind it.  Reported only; `value` does not include them."""
+    from cubek_amd import ComputeClient, ElemType, TensorHandleRef
+    from cubek_amd import contiguous as cq_contiguous
+    from cubek_amd import reduce as cq_reduce
+
+    client = ComputeClient.current()
+    h = TensorHandleRef.from_torch
+    rows, cols = WORKLOADS["cfg5"]["shape"]
+    sets = 4  # 4 x 470 MB: each launch reads a tensor that has left the Infinity Cache
+    xs = [torch.randn((rows, cols), device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
+    out = []
+    for axis in (1, 0):
+        o = torch.zeros((rows, 1) if axis == 1 else (1, cols), device="cuda", dtype=torch.bfloat16)
+        nbytes = cq_reduce.workspace_bytes(h(xs[0]), axis, ElemType.BF16)
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+        hs, ho = [h(x) for x in xs], h(o)
+        fn = lambda i: cq_reduce.max_abs(client, hs[i % sets], ho, axis, ElemType.BF16, ws.data_ptr() if nbytes else 0,
+                                         nbytes)
+        ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
+        b = rows * cols * 2
+        out.append({"kernel": f"reduce_max_abs axis {axis} of bf16 [{rows}, {cols}]", "algorithmic_bytes": b,
+                    "workspace_bytes": nbytes, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                    "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+    del xs
+    torch.cuda.empty_cache()
+    # 4-bit codes of a [rows, cols] weight, 8 per u32 word along cols, viewed transposed as [cols, rows]
+    packing = 8
+    srcs = [torch.randint(-2**31, 2**31 - 1, (rows, cols // packing), dtype=torch.int32, device="cuda")
+            for _ in range(8)]
+    dst = torch.zeros((cols, rows // packing), dtype=torch.int32, device="cuda")
+    hs = [TensorHandleRef(h(t).handle, (cols // packing, rows), (1, cols // packing), 4) for t in srcs]
+    hd = h(dst)
+    fn = lambda i: cq_contiguous.into_contiguous_packed_ref(client, hs[i % len(hs)], hd, (cols, rows), packing)
+    ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
+    b = 2 * rows * cols // packing * 4
+    out.append({"kernel": f"into_contiguous_packed of transposed 4-bit [{cols}, {rows}] (u32 x 8)",
+                "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -313,6 +357,7 @@ def main():
             del ps, p, xi
             torch.cuda.empty_cache()
         result["per_config"] = table
+        result["adjacent_kernels"] = adjacent_kernels(torch)
 
     print(json.dumps(result))
 
