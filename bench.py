@@ -263,6 +263,8 @@ def main():
     ap.add_argument("--workload", default="cfg5", choices=sorted(WORKLOADS))
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-config table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--adjacent-only", action="store_true",
+                    help="run only the abs-max / re-pack kernels on the headline tensor (for profiling)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run 3 plain device copies of the input (known bytes) to calibrate rocprof counters")
     args = ap.parse_args()
@@ -277,6 +279,10 @@ def main():
     _ffi.lib()  # fail loudly if the HIP library is not built
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+
+    if args.adjacent_only:
+        print(json.dumps({"adjacent_kernels": adjacent_kernels(torch)}))
+        return
 
     w = WORKLOADS[args.workload]
     x = make_input(torch, w)
