@@ -279,8 +279,16 @@ __device__ __forceinline__ float scale_from_absmax_tame(float amax, const QuantP
 //   is within 2^-21 relative of a half-integer; such lanes redo the chunk with
 //   IEEE division.  Clamping to [lo-1/4, hi+1/4] first removes the ties that
 //   clamp anyway and bounds the window by a per-range constant.
-// f16 : IEEE division (the f16 boundaries are too close for the shortcut).
-// Negation commutes with every step (multiply, RNE rounding to bf16, rint).
+// f16 : the f16 boundaries are too close for x * rcp(d) alone (a quotient of two
+//   f16 numbers can sit 2^-23 relative from a boundary), so one residual step
+//   follows: t = x*r, e = x - t*d (exact in one FMA up to its rounding), q = t + e*r.
+//   q is x/d with a relative error near 2^-44 before its final rounding, and a
+//   quotient of two 11-bit significands is at least 2^-36 relative away from
+//   every f32 rounding boundary, so q is bit for bit the IEEE f32 quotient.
+//   t is clamped to [lo-1, hi+1] first: that leaves t alone wherever the code is
+//   not decided by the clamp, and turns an infinite t (infinite x) into a finite
+//   one so that the residual is +-inf (clamped like the IEEE quotient), not NaN.
+// Negation commutes with every step (multiply, RNE rounding, rint).
 template <class F, int kN>
 __device__ __forceinline__ void quantize_values_neg(const float* x, float d, bool d_tame, float lo,
                                                     float hi, float* qn) {
@@ -295,6 +303,19 @@ __device__ __forceinline__ void quantize_values_neg(const float* x, float d, boo
                 const uint32_t p = BF16::pack2(a, b);
                 qn[i] = __builtin_rintf(bits_f32(p << 16));
                 qn[i + 1] = __builtin_rintf(bits_f32(p & 0xffff0000u));
+            }
+            return;
+        }
+    } else if constexpr (F::kDtype == CQ_F16) {
+        if (d_tame) {
+            const float nr = -__builtin_amdgcn_rcpf(d);
+            const float nhi = -hi, nlo = -lo, nhi_t = -(hi + 1.0f), nlo_t = -(lo - 1.0f);
+#pragma unroll
+            for (int i = 0; i < kN; i++) {
+                const float tn = neg_clamp_of_neg(x[i] * nr, nhi_t, nlo_t);  // -t
+                const float e = __builtin_fmaf(tn, d, x[i]);                 // x - t*d
+                const float qn1 = __builtin_fmaf(e, nr, tn);                 // -(t + e*r)
+                qn[i] = __builtin_rintf(F16::round(neg_clamp_of_neg(qn1, nhi, nlo)));
             }
             return;
         }

@@ -446,3 +446,30 @@ def test_scale_division_all_significands(gpu):
                     (value, exp_field, k)
                 assert np.array_equal(out_scale.cpu().numpy().reshape(-1).view(np.uint32), ref.view(np.uint32)), \
                     (value, exp_field, k)
+
+
+@pytest.mark.parametrize("value", [QuantValue.E5M2, QuantValue.Q2S], ids=lambda v: v.name)
+def test_f16_every_input_every_divisor(gpu, oracle, value):
+    """The f16 kernels replace the division by a reciprocal and one residual step.  All
+    65536 x 65536 (element, divisor) bit patterns, NaN, infinities, zeros and subnormals
+    included, against the oracle's IEEE division; a wide and a narrow clamp range."""
+    import torch
+    from cubek_amd import ComputeClient
+    from cubek_amd import quantize as qz
+
+    client = ComputeClient.current()
+    rows = 2048
+    x = np.ascontiguousarray(np.broadcast_to(np.arange(65536, dtype=np.uint16), (rows, 65536)))
+    dx = gpu.to_dev(x)
+    scheme = QuantScheme.default().with_value(value).with_level(QuantLevel.block([128]))
+    pshape = scheme.packed_shape((rows, 65536))
+    for d0 in range(0, 65536, rows):
+        d = np.arange(d0, d0 + rows, dtype=np.uint16)
+        scale = np.ascontiguousarray(np.broadcast_to(d[:, None], (rows, 512)))
+        dout = torch.zeros(pshape, dtype=torch.int32, device="cuda")
+        dos = torch.zeros((rows, 512), dtype=torch.float32, device="cuda")
+        qz.launch_ref(client, gpu.handle(dx), gpu.handle(dout), gpu.handle(gpu.to_dev(scale)), gpu.handle(dos),
+                      scheme, ElemType.F16)
+        torch.cuda.synchronize()
+        want, _ = oracle.quantize(x, ElemType.F16, (rows, 65536), scale, scheme, threads=16)
+        assert np.array_equal(gpu.to_host(dout).reshape(-1), want.reshape(-1)), (value.name, d0)
