@@ -25,11 +25,14 @@ int group_of(int dtype, uint32_t block) {
 
 // Launch shapes from a sweep on MI355X (batches of back-to-back launches,
 // 117 MB - 470 MB tensors): quantize is best with four 16-byte loads in flight
-// per lane; dequantize, which is store-dominated, with 16 output elements per
-// lane (two 16-byte stores for 16-bit outputs, four for f32 outputs).
+// per lane; dequantize, which is store-dominated, with two 16-byte stores per lane
+// for 16-bit outputs.  For f32 outputs the best depth follows the share of reads:
+// four stores per lane where the codes and scales are under ~15 % of the bytes
+// written (measured 87-91 % of HBM peak against 78-87 % with two), two stores
+// where they are more (8-bit codes, 4-bit codes with blocks of 32: 81-83 % against 73-75 %).
 constexpr int kUnrollQ = 4;
-template <class F>
-constexpr int kUnrollD = F::kBytes == 4 ? 4 : 2;
+template <class F, int kBits, int kGroup>
+constexpr int kUnrollD = F::kBytes != 4 ? 2 : ((kBits == 8 || (kBits == 4 && kGroup > 0 && kGroup <= 8)) ? 2 : 4);
 
 QuantParams quant_params(const Range& r) {
     QuantParams p;
@@ -117,12 +120,12 @@ hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
     auto in = static_cast<const uint32_t*>(a.input);
     auto out = static_cast<u32x4*>(a.output);
     const bool p32 = a.param_dtype == CQ_F32;
-    return launch_tiles(a.num_chunks, kUnrollD<F>, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
+    return launch_tiles(a.num_chunks, kUnrollD<F, kBits, kGroup>, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
         auto kernel =
-            checked ? (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F>, kThreads, true, kEnc>
-                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F>, kThreads, true, kEnc>)
-                    : (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F>, kThreads, false, kEnc>
-                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F>, kThreads, false, kEnc>);
+            checked ? (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F, kBits, kGroup>, kThreads, true, kEnc>
+                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F, kBits, kGroup>, kThreads, true, kEnc>)
+                    : (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F, kBits, kGroup>, kThreads, false, kEnc>
+                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F, kBits, kGroup>, kThreads, false, kEnc>);
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, begin, end);
     });
 }
