@@ -196,6 +196,61 @@ int flat_encoding(const cq_scheme* s) {
     }
 }
 
+// Row kernels: last dimension contiguous on both sides and everything a multiple of a
+// unit (see cq_kernels_rows.hip).  `values` may be NULL when only the float tensor
+// takes part (scale production).  Fills `r` except the data pointers and dtypes.
+bool rows_args(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
+               cq::RowArgs* r) {
+    const uint32_t last = p.rank - 1;
+    const uint32_t per_chunk = 16u / dtype_size(dtype);
+    const uint32_t unit = values ? cq::rows_unit_values(dtype, static_cast<int>(p.bits)) : per_chunk;
+    const uint64_t cols = p.shape[last];
+    if (cols == 0 || cols % unit || cols > (1ull << 26)) return false;
+    if (!p.tensor_level && p.layout.block[last] % unit) return false;
+    if (floats->strides[last] != 1 || !aligned(floats->ptr, 16)) return false;
+    const bool native = s->store == CQ_STORE_NATIVE;
+    if (values && (values->strides[last] != 1 || !aligned(values->ptr, 4))) return false;
+    std::memset(r, 0, sizeof(*r));
+    r->rank = p.rank;
+    r->tensor_level = p.tensor_level ? 1u : 0u;
+    r->rows = 1;
+    for (uint32_t d = 0; d < p.rank; d++) {
+        r->shape[d] = static_cast<uint32_t>(p.shape[d]);
+        r->block[d] = p.tensor_level ? 1u : p.layout.block[d];
+        r->sa[d] = p.layout.stride_a[d];
+        r->sb[d] = p.layout.stride_b[d];
+        if (d == last) continue;
+        r->rows *= p.shape[d];
+        if (p.shape[d] == 1) continue;  // its stride never contributes
+        if (floats->strides[d] % per_chunk) return false;
+        r->fstride[d] = floats->strides[d];
+        if (values) {
+            if (native && values->strides[d] % 4) return false;
+            r->vstride[d] = native ? values->strides[d] / 4 : values->strides[d];
+        }
+    }
+    if (r->rows >= (1ull << 31)) return false;
+    r->fstride[last] = 1;
+    r->vstride[last] = 1;
+    const uint32_t bc = r->block[last];
+    r->bc_shift = -1;
+    if ((bc & (bc - 1)) == 0)
+        for (int k = 0; k < 9; k++)
+            if ((1u << k) == bc) r->bc_shift = k;
+    r->param_dtype = param_to_dtype(s->param);
+    r->encoding = flat_encoding(s);
+    r->range = p.range;
+    return true;
+}
+
+// Block abs-max by the row kernels: blocks over the last two dimensions only.
+bool scales_rows_ok(const Plan& p) {
+    if (p.tensor_level) return false;
+    for (uint32_t d = 0; d + 2 < p.rank; d++)
+        if (p.layout.block[d] != 1) return false;
+    return true;
+}
+
 cq::GenericArgs generic_args(const Plan& p, const cq_scheme* s) {
     cq::GenericArgs g;
     std::memset(&g, 0, sizeof(g));
@@ -293,6 +348,15 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         if (st != CQ_OK) return st;
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
+    cq::RowArgs r;
+    if (flat_words == 0 && rows_args(p, scheme, input_dtype, input, output, &r)) {
+        r.input = input->ptr;
+        r.output = output->ptr;
+        r.scale_in = scale->ptr;
+        r.scale_in_dtype = input_dtype;
+        r.scale_out = out_scale->ptr;
+        return hip_status(cq::launch_quantize_rows(stream, input_dtype, static_cast<int>(p.bits), r));
+    }
     if (flat_words < p.n / p.nq) {
         cq::GenericArgs g = generic_args(p, scheme);
         g.input = input->ptr;
@@ -335,6 +399,13 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         if (st != CQ_OK) return st;
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
+    cq::RowArgs r;
+    if (flat_words == 0 && rows_args(p, scheme, output_dtype, output, values, &r)) {
+        r.input = values->ptr;
+        r.output = output->ptr;
+        r.scale_in = params->ptr;
+        return hip_status(cq::launch_dequantize_rows(stream, output_dtype, static_cast<int>(p.bits), r));
+    }
     if (flat_words < p.n / p.nq) {
         cq::GenericArgs g = generic_args(p, scheme);
         g.input = values->ptr;
@@ -359,7 +430,12 @@ static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_sche
         if (!aligned(workspace, 4)) return CQ_ERR_INVALID_ARGUMENT;
         uint32_t num_partials = 0;
         cq_status st;
-        if (p.vs.on) {
+        cq::RowArgs r;
+        if (p.vs.on && rows_args(p, scheme, input_dtype, input, nullptr, &r)) {
+            r.input = input->ptr;
+            st = hip_status(cq::launch_absmax_partials_rows(stream, input_dtype, r, static_cast<float*>(workspace),
+                                                            &num_partials));
+        } else if (p.vs.on) {
             cq::GenericArgs g = generic_args(p, scheme);
             g.input = input->ptr;
             st = hip_status(cq::launch_absmax_partials_strided(stream, input_dtype, g, p.n,
@@ -372,6 +448,12 @@ static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_sche
         return hip_status(cq::launch_tensor_scale(stream, input_dtype, out_dtype,
                                                   static_cast<const float*>(workspace), num_partials,
                                                   p.range, scales->ptr));
+    }
+    cq::RowArgs r;
+    if (scales_rows_ok(p) && rows_args(p, scheme, input_dtype, input, nullptr, &r)) {
+        r.input = input->ptr;
+        r.scale_out = scales->ptr;
+        return hip_status(cq::launch_scales_rows(stream, input_dtype, out_dtype, r));
     }
     cq::GenericArgs g = generic_args(p, scheme);
     g.input = input->ptr;
@@ -474,6 +556,15 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         // (the divisor F(FS(scale)) is the same either way)
         st = produce_scales(stream, p, scheme, input, input_dtype, out_scale, pd, workspace, workspace_bytes);
         if (st != CQ_OK) return st;
+    }
+    cq::RowArgs r;
+    if (flat_words == 0 && rows_args(p, scheme, input_dtype, input, output, &r)) {
+        r.input = input->ptr;
+        r.output = output->ptr;
+        r.scale_in = out_scale->ptr;
+        r.scale_in_dtype = pd;
+        r.scale_out = nullptr;
+        return hip_status(cq::launch_quantize_rows(stream, input_dtype, static_cast<int>(p.bits), r));
     }
     if (flat_words < p.n / p.nq) {
         cq::GenericArgs g = generic_args(p, scheme);

@@ -111,6 +111,38 @@ hipError_t launch_reduce_max_abs(hipStream_t s, int dtype, const ReduceArgs& a);
 uint64_t reduce_workspace_bytes(uint64_t outer, uint64_t len, uint64_t inner, int dtype);
 
 
+// Row kernels: any layout whose last dimension is contiguous in both value tensors
+// (N-D blocks, odd block sizes, strided scales, pitched / sliced / permuted rows).
+struct RowArgs {
+    const void* input;       // floats (quantize, scales) / stored words (dequantize)
+    void* output;
+    const void* scale_in;    // quantize: typed scale_in_dtype; dequantize: typed param_dtype
+    void* scale_out;         // quantize: out_scale or NULL; scales: destination
+    int scale_in_dtype, param_dtype;
+    int encoding;            // cq::Encoding of the stored values
+    Range range;
+    uint32_t rank;
+    uint32_t tensor_level;   // 1: one scale for the whole tensor
+    uint32_t shape[CQ_MAX_RANK];    // unpacked shape
+    uint32_t block[CQ_MAX_RANK];    // block extents left-padded with 1 (block level only)
+    uint64_t fstride[CQ_MAX_RANK];  // float tensor, elements; leading strides are multiples of a 16-byte chunk
+    uint64_t vstride[CQ_MAX_RANK];  // stored tensor, in 32-bit words
+    uint64_t sa[CQ_MAX_RANK], sb[CQ_MAX_RANK];  // strides of scale_in / scale_out
+    uint64_t rows;           // product of the leading dimensions (< 2^31)
+    int32_t bc_shift;        // log2(block[last]) if a power of two, else -1
+    uint32_t units_per_row, tj_log2;  // filled by the launchers
+};
+// values per unit of the row kernels: the last dimension and the last block extent must be multiples of it
+uint32_t rows_unit_values(int dtype, int bits);
+hipError_t launch_quantize_rows(hipStream_t s, int dtype, int bits, const RowArgs& a);
+hipError_t launch_dequantize_rows(hipStream_t s, int dtype, int bits, const RowArgs& a);
+// block abs-max -> out_dtype(dtype(2*absmax/(hi-lo))) through `sb` into scale_out; blocks may
+// extend over the last two dimensions only, the last extent is a multiple of a chunk
+hipError_t launch_scales_rows(hipStream_t s, int dtype, int out_dtype, const RowArgs& a);
+// per-tensor abs-max partials (same contract as launch_absmax_partials)
+hipError_t launch_absmax_partials_rows(hipStream_t s, int dtype, const RowArgs& a, float* partials,
+                                       uint32_t* num_partials);
+
 // Re-packing of a strided quantized tensor (cq_into_contiguous_packed).
 struct RepackArgs {
     const void* input;

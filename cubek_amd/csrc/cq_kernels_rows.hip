@@ -1,0 +1,378 @@
+// Row kernels: quantize / dequantize / block abs-max for every layout whose last
+// dimension is contiguous but which the flat streaming kernels cannot take:
+// N-D blocks (e.g. 128 x 128), block sizes that are not a power-of-two number of
+// lanes (e.g. 24), strided scale tensors, pitched or sliced rows, permuted leading
+// dimensions.  Same arithmetic as the flat kernels (cq_device.hpp), same addressing
+// rules as the reference's layouts (crates/cubek-quant/src/layout/scales.rs:144-194).
+//
+// A workgroup covers TR rows x TJ units (TR * TJ = 256, TJ a power of two chosen on
+// the host from the row length).  A unit is the smallest run of elements that is
+// whole on both sides: max(values per stored word, values per 16-byte chunk).  Each
+// thread decomposes its row index once (strides and block coordinates of the
+// leading dimensions) and then walks kUnits units of that row; loads and stores are
+// 16 bytes of floats and whole 32-bit words.
+#include "cq_device.hpp"
+#include "cq_internal.hpp"
+
+namespace cq {
+namespace {
+
+constexpr int kThreads = 256;
+
+template <class F, int kBits>
+struct Unit {
+    static constexpr int kN = F::kPerChunk;           // values per 16-byte chunk
+    static constexpr int kNq = 32 / kBits;            // values per stored word
+    static constexpr int kV = kNq > kN ? kNq : kN;    // values per unit
+    static constexpr int kChunks = kV / kN;
+    static constexpr int kWords = kV / kNq;
+    static constexpr int kUnits = kChunks >= 4 ? 2 : 4;  // units per thread
+};
+
+// What a thread knows about its row.
+struct RowPos {
+    uint64_t f, v, sa, sb;  // offsets: floats (elements), stored (words), scale_in, scale_out
+    bool start;             // every leading coordinate sits on a block start
+    bool live;
+};
+
+__device__ __forceinline__ RowPos row_pos(const RowArgs& a, uint32_t row) {
+    RowPos r{0, 0, 0, 0, true, row < a.rows};
+    uint32_t rem = r.live ? row : 0;
+    for (int d = static_cast<int>(a.rank) - 2; d >= 0; d--) {
+        const uint32_t c = rem % a.shape[d];
+        rem /= a.shape[d];
+        r.f += static_cast<uint64_t>(c) * a.fstride[d];
+        r.v += static_cast<uint64_t>(c) * a.vstride[d];
+        if (a.tensor_level) {
+            r.start = r.start && c == 0;
+        } else {
+            const uint32_t cb = c / a.block[d];
+            r.sa += static_cast<uint64_t>(cb) * a.sa[d];
+            r.sb += static_cast<uint64_t>(cb) * a.sb[d];
+            r.start = r.start && (c % a.block[d]) == 0;
+        }
+    }
+    return r;
+}
+
+// Scale offsets and block-start flag of the unit that begins at column `e`.
+struct ScaleAt {
+    uint64_t a, b;
+    bool start;
+};
+__device__ __forceinline__ ScaleAt scale_at(const RowArgs& a, const RowPos& r, uint32_t e) {
+    if (a.tensor_level) return ScaleAt{0, 0, r.start && e == 0};
+    const int last = static_cast<int>(a.rank) - 1;
+    const uint32_t bc = a.block[last];
+    const uint32_t cb = a.bc_shift >= 0 ? e >> a.bc_shift : e / bc;
+    return ScaleAt{r.sa + static_cast<uint64_t>(cb) * a.sa[last], r.sb + static_cast<uint64_t>(cb) * a.sb[last],
+                   r.start && e == cb * bc};
+}
+
+template <class F, int kBits, bool kWide, int kEnc>
+__global__ __launch_bounds__(kThreads) void quantize_rows_kernel(RowArgs a) {
+    using U = Unit<F, kBits>;
+    constexpr int kN = U::kN;
+    const uint32_t tj = 1u << a.tj_log2;
+    const uint32_t row = blockIdx.x * (kThreads >> a.tj_log2) + (threadIdx.x >> a.tj_log2);
+    const uint32_t jl = threadIdx.x & (tj - 1);
+    const RowPos r = row_pos(a, row);
+    const u32x4* in = static_cast<const u32x4*>(a.input);
+    uint32_t* out = static_cast<uint32_t*>(a.output);
+
+    u32x4 raw[U::kUnits][U::kChunks];
+    float s_f[U::kUnits];
+    ScaleAt sp[U::kUnits];
+#pragma unroll
+    for (int u = 0; u < U::kUnits; u++) {
+        uint32_t j = (blockIdx.y * U::kUnits + u) * tj + jl;
+        j = j < a.units_per_row ? j : a.units_per_row - 1;  // clamp instead of branching around loads
+        const uint32_t e = j * U::kV;
+        sp[u] = scale_at(a, r, e);
+        s_f[u] = load_dtype(a.scale_in_dtype, a.scale_in, sp[u].a);
+#pragma unroll
+        for (int i = 0; i < U::kChunks; i++) raw[u][i] = stream_load(in + (r.f + e) / kN + i);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < U::kUnits; u++) {
+        const uint32_t j = (blockIdx.y * U::kUnits + u) * tj + jl;
+        const bool live = r.live && j < a.units_per_row;
+        // write_scale (src/quantize.rs:83-98): FS(scale), stored by the block's first element
+        const float s_fs = round_to_dtype(a.param_dtype, s_f[u]);
+        if (a.scale_out != nullptr && live && sp[u].start) store_dtype(a.param_dtype, a.scale_out, sp[u].b, s_fs);
+        const float d = F::round(s_fs);
+        const bool tame = divisor_is_tame(d);
+        uint32_t w[2] = {0, 0};
+#pragma unroll
+        for (int i = 0; i < U::kChunks; i++) {
+            float v[kN], qn[kN];
+            F::unpack(raw[u][i], v);
+            quantize_values_neg<F, kN>(v, d, tame, a.range.lo, a.range.hi, qn);
+            uint32_t cw[2] = {0, 0};
+            if constexpr (kEnc == kEncInt)
+                pack_chunk_neg<kBits, kN, kWide>(qn, cw);
+            else
+                encode_chunk_neg<kEnc, kN>(qn, cw);
+            if constexpr (U::kChunks == 1) {
+                w[0] = cw[0];
+                w[1] = cw[1];
+            } else {
+                w[0] |= cw[0] << (i * kN * kBits);  // sub-word chunks, upper bits are zero
+            }
+        }
+        if (live) {
+            uint32_t* dst = out + r.v + static_cast<uint64_t>(j) * U::kWords;
+            stream_store(w[0], dst);
+            if constexpr (U::kWords == 2) stream_store(w[1], dst + 1);
+        }
+    }
+}
+
+template <class F, int kBits, int kEnc>
+__global__ __launch_bounds__(kThreads) void dequantize_rows_kernel(RowArgs a) {
+    using U = Unit<F, kBits>;
+    constexpr int kN = U::kN;
+    const uint32_t tj = 1u << a.tj_log2;
+    const uint32_t row = blockIdx.x * (kThreads >> a.tj_log2) + (threadIdx.x >> a.tj_log2);
+    const uint32_t jl = threadIdx.x & (tj - 1);
+    const RowPos r = row_pos(a, row);
+    const uint32_t* in = static_cast<const uint32_t*>(a.input);
+    u32x4* out = static_cast<u32x4*>(a.output);
+
+    uint32_t w[U::kUnits][U::kWords];
+    float sc[U::kUnits];
+#pragma unroll
+    for (int u = 0; u < U::kUnits; u++) {
+        uint32_t j = (blockIdx.y * U::kUnits + u) * tj + jl;
+        j = j < a.units_per_row ? j : a.units_per_row - 1;
+        const ScaleAt sp = scale_at(a, r, j * U::kV);
+        sc[u] = F::round(load_dtype(a.param_dtype, a.scale_in, sp.a));  // Line::cast_from(scale)
+#pragma unroll
+        for (int k = 0; k < U::kWords; k++) w[u][k] = stream_load(in + r.v + static_cast<uint64_t>(j) * U::kWords + k);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < U::kUnits; u++) {
+        const uint32_t j = (blockIdx.y * U::kUnits + u) * tj + jl;
+        float y[U::kV];
+#pragma unroll
+        for (int k = 0; k < U::kWords; k++) decode_fields<kEnc, kBits, U::kNq>(w[u][k], y + k * U::kNq);
+#pragma unroll
+        for (int i = 0; i < U::kV; i++) y[i] = sc[u] * y[i];
+        if (r.live && j < a.units_per_row) {
+#pragma unroll
+            for (int i = 0; i < U::kChunks; i++)
+                stream_store(F::pack(y + i * kN), out + (r.f + static_cast<uint64_t>(j) * U::kV) / kN + i);  // pack rounds to F
+        }
+    }
+}
+
+// Abs-max of every block [BR rows x BC columns] (blocks extend over the last two
+// dimensions only) -> scale typed `out_dtype` through the strides `sb`.
+// Thread = (block row, 16-byte chunk column); it walks the BR rows of its block
+// row, then the chunk columns of one block meet in LDS.
+template <class F>
+__global__ __launch_bounds__(kThreads) void scales_rows_kernel(RowArgs a, int out_dtype, uint32_t block_rows,
+                                                               uint32_t chunks_per_block, uint32_t tj_eff) {
+    constexpr int kN = F::kPerChunk;
+    constexpr int kUnroll = 4;
+    __shared__ float lds[kThreads];
+    const int last = static_cast<int>(a.rank) - 1;
+    const uint32_t tj = 1u << a.tj_log2;
+    const uint32_t rbi = blockIdx.x * (kThreads >> a.tj_log2) + (threadIdx.x >> a.tj_log2);
+    const uint32_t jl = threadIdx.x & (tj - 1);
+    const uint32_t jc = blockIdx.y * tj_eff + jl;
+    const uint32_t chunks_per_row = a.shape[last] / kN;
+    const uint32_t br = a.rank >= 2 ? a.block[last - 1] : 1u;
+    const bool live = rbi < block_rows && jl < tj_eff && jc < chunks_per_row;
+    // the block row's first row, as a flattened row index
+    const RowPos r = row_pos(a, live ? rbi * br : 0);
+    float amax = 0.0f;
+    if (live) {
+        const u32x4* p = static_cast<const u32x4*>(a.input) + r.f / kN + jc;
+        const uint64_t pitch = a.rank >= 2 ? a.fstride[last - 1] / kN : 0;
+        for (uint32_t r0 = 0; r0 < br; r0 += kUnroll) {
+            u32x4 raw[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) raw[u] = stream_load(p + (r0 + u < br ? r0 + u : br - 1) * pitch);
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                float v[kN];
+                F::unpack(raw[u], v);
+#pragma unroll
+                for (int i = 0; i < kN; i++) amax = fmaxf(amax, fabsf(v[i]));  // NaN elements drop out
+            }
+        }
+    }
+    lds[threadIdx.x] = amax;
+    __syncthreads();
+    if (live && jc % chunks_per_block == 0) {
+        for (uint32_t k = 1; k < chunks_per_block; k++) amax = fmaxf(amax, lds[threadIdx.x + k]);
+        const float s = F::round(scale_from_absmax(amax, a.range.hi - a.range.lo));
+        store_dtype(out_dtype, a.scale_out, r.sb + static_cast<uint64_t>(jc / chunks_per_block) * a.sb[last],
+                    round_to_dtype(out_dtype, s));
+    }
+}
+
+// Per-tensor abs-max, pass 1, over strided rows: gridDim.x <= kMaxPartials workgroups
+// stride over the (row tile, chunk tile) pairs; one f32 partial per workgroup.
+template <class F>
+__global__ __launch_bounds__(kThreads) void absmax_rows_kernel(RowArgs a, float* __restrict__ partials,
+                                                               uint32_t row_tiles, uint32_t col_tiles) {
+    constexpr int kN = F::kPerChunk;
+    __shared__ float lds[kThreads / kWave];
+    const int last = static_cast<int>(a.rank) - 1;
+    const uint32_t tj = 1u << a.tj_log2;
+    const uint32_t chunks_per_row = a.shape[last] / kN;
+    const u32x4* in = static_cast<const u32x4*>(a.input);
+    float amax = 0.0f;
+    for (uint64_t t = blockIdx.x; t < static_cast<uint64_t>(row_tiles) * col_tiles; t += gridDim.x) {
+        const uint32_t rt = static_cast<uint32_t>(t / col_tiles), ct = static_cast<uint32_t>(t % col_tiles);
+        const uint32_t row = rt * (kThreads >> a.tj_log2) + (threadIdx.x >> a.tj_log2);
+        const uint32_t jc = ct * tj + (threadIdx.x & (tj - 1));
+        const RowPos r = row_pos(a, row);
+        if (r.live && jc < chunks_per_row) {
+            float v[kN];
+            F::unpack(stream_load(in + r.f / kN + jc), v);
+#pragma unroll
+            for (int i = 0; i < kN; i++) amax = fmaxf(amax, fabsf(v[i]));
+        }
+    }
+    amax = group_max<kWave>(amax);
+    if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kThreads / kWave; w++) amax = fmaxf(amax, lds[w]);
+        partials[blockIdx.x] = amax;
+    }
+}
+
+// lanes along the row: the smallest power of two that covers `units`, at most 256
+uint32_t lanes_log2(uint64_t units) {
+    uint32_t l = 0;
+    while (l < 8 && (1ull << l) < units) l++;
+    return l;
+}
+
+#define CQ_SWITCH_DTYPE(D, ...)                              \
+    switch (D) {                                             \
+        case CQ_F32: { using kF = F32; __VA_ARGS__; }        \
+        case CQ_BF16: { using kF = BF16; __VA_ARGS__; }      \
+        case CQ_F16: { using kF = F16; __VA_ARGS__; }        \
+        default: return hipErrorInvalidValue;                \
+    }
+
+template <class F, int kBits>
+dim3 unit_grid(RowArgs* a) {
+    using U = Unit<F, kBits>;
+    a->units_per_row = a->shape[a->rank - 1] / U::kV;
+    a->tj_log2 = lanes_log2((a->units_per_row + U::kUnits - 1) / U::kUnits);
+    const uint32_t tr = kThreads >> a->tj_log2;
+    const uint32_t per_group = U::kUnits << a->tj_log2;
+    return dim3(static_cast<uint32_t>((a->rows + tr - 1) / tr), (a->units_per_row + per_group - 1) / per_group);
+}
+
+template <class F>
+hipError_t quantize_rows(hipStream_t s, int bits, RowArgs a) {
+    const bool wide = a.range.hi > 127.0f || a.range.lo < -128.0f;
+#define CQ_LAUNCH(B, W, E)                                                                                    \
+    {                                                                                                         \
+        const dim3 grid = unit_grid<F, B>(&a);                                                                \
+        hipLaunchKernelGGL((quantize_rows_kernel<F, B, W, E>), grid, dim3(kThreads), 0, s, a);                \
+        return hipGetLastError();                                                                             \
+    }
+    switch (a.encoding) {
+        case kEncInt:
+            if (bits == 2) CQ_LAUNCH(2, false, kEncInt)
+            if (bits == 4) CQ_LAUNCH(4, false, kEncInt)
+            if (bits == 8 && wide) CQ_LAUNCH(8, true, kEncInt)
+            if (bits == 8) CQ_LAUNCH(8, false, kEncInt)
+            break;
+        case kEncE4M3: if (bits == 8) CQ_LAUNCH(8, false, kEncE4M3) break;
+        case kEncE5M2: if (bits == 8) CQ_LAUNCH(8, false, kEncE5M2) break;
+        case kEncE2M1: if (bits == 4) CQ_LAUNCH(4, false, kEncE2M1) break;
+    }
+#undef CQ_LAUNCH
+    return hipErrorInvalidValue;
+}
+
+template <class F>
+hipError_t dequantize_rows(hipStream_t s, int bits, RowArgs a) {
+#define CQ_LAUNCH(B, E)                                                                                       \
+    {                                                                                                         \
+        const dim3 grid = unit_grid<F, B>(&a);                                                                \
+        hipLaunchKernelGGL((dequantize_rows_kernel<F, B, E>), grid, dim3(kThreads), 0, s, a);                 \
+        return hipGetLastError();                                                                             \
+    }
+    switch (a.encoding) {
+        case kEncInt:
+            if (bits == 2) CQ_LAUNCH(2, kEncInt)
+            if (bits == 4) CQ_LAUNCH(4, kEncInt)
+            if (bits == 8) CQ_LAUNCH(8, kEncInt)
+            break;
+        case kEncE4M3: if (bits == 8) CQ_LAUNCH(8, kEncE4M3) break;
+        case kEncE5M2: if (bits == 8) CQ_LAUNCH(8, kEncE5M2) break;
+        case kEncE2M1: if (bits == 4) CQ_LAUNCH(4, kEncE2M1) break;
+    }
+#undef CQ_LAUNCH
+    return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+uint32_t rows_unit_values(int dtype, int bits) {
+    const uint32_t per_chunk = dtype == CQ_F32 ? 4 : 8, per_word = 32u / static_cast<uint32_t>(bits);
+    return per_chunk > per_word ? per_chunk : per_word;
+}
+
+hipError_t launch_quantize_rows(hipStream_t s, int dtype, int bits, const RowArgs& a) {
+    if (a.rows == 0 || a.shape[a.rank - 1] == 0) return hipSuccess;
+    CQ_SWITCH_DTYPE(dtype, return quantize_rows<kF>(s, bits, a))
+}
+
+hipError_t launch_dequantize_rows(hipStream_t s, int dtype, int bits, const RowArgs& a) {
+    if (a.rows == 0 || a.shape[a.rank - 1] == 0) return hipSuccess;
+    CQ_SWITCH_DTYPE(dtype, return dequantize_rows<kF>(s, bits, a))
+}
+
+hipError_t launch_scales_rows(hipStream_t s, int dtype, int out_dtype, const RowArgs& args) {
+    RowArgs a = args;
+    const uint32_t last = a.rank - 1;
+    const uint32_t per_chunk = dtype == CQ_F32 ? 4 : 8;
+    const uint32_t br = a.rank >= 2 ? a.block[last - 1] : 1u;
+    const uint32_t chunks_per_row = a.shape[last] / per_chunk;
+    const uint32_t chunks_per_block = a.block[last] / per_chunk;
+    const uint64_t block_rows = a.rows / br;
+    if (block_rows == 0 || chunks_per_row == 0) return hipSuccess;
+    // lanes along the row: whole blocks only, so that a block never straddles two workgroups
+    a.tj_log2 = lanes_log2(chunks_per_row);
+    while ((1u << a.tj_log2) < chunks_per_block) a.tj_log2++;
+    if (a.tj_log2 > 8) return hipErrorInvalidValue;  // a block wider than a workgroup: not for this kernel
+    const uint32_t tj_eff = ((1u << a.tj_log2) / chunks_per_block) * chunks_per_block;
+    const uint32_t tr = kThreads >> a.tj_log2;
+    const dim3 grid(static_cast<uint32_t>((block_rows + tr - 1) / tr), (chunks_per_row + tj_eff - 1) / tj_eff);
+    CQ_SWITCH_DTYPE(dtype, hipLaunchKernelGGL((scales_rows_kernel<kF>), grid, dim3(kThreads), 0, s, a, out_dtype,
+                                              static_cast<uint32_t>(block_rows), chunks_per_block, tj_eff);
+                    return hipGetLastError())
+}
+
+hipError_t launch_absmax_partials_rows(hipStream_t s, int dtype, const RowArgs& args, float* partials,
+                                       uint32_t* num_partials) {
+    RowArgs a = args;
+    const uint32_t per_chunk = dtype == CQ_F32 ? 4 : 8;
+    const uint32_t chunks_per_row = a.shape[a.rank - 1] / per_chunk;
+    a.tj_log2 = lanes_log2(chunks_per_row);
+    const uint32_t tr = kThreads >> a.tj_log2;
+    const uint32_t row_tiles = static_cast<uint32_t>((a.rows + tr - 1) / tr);
+    const uint32_t col_tiles = (chunks_per_row + (1u << a.tj_log2) - 1) >> a.tj_log2;
+    const uint64_t tiles = static_cast<uint64_t>(row_tiles) * col_tiles;
+    const uint32_t grid = static_cast<uint32_t>(tiles < 1 ? 1 : (tiles > kMaxPartials ? kMaxPartials : tiles));
+    *num_partials = grid;
+    CQ_SWITCH_DTYPE(dtype, hipLaunchKernelGGL((absmax_rows_kernel<kF>), dim3(grid), dim3(kThreads), 0, s, a, partials,
+                                              row_tiles, col_tiles);
+                    return hipGetLastError())
+}
+
+}  // namespace cq

@@ -71,11 +71,11 @@ def test_native_store_and_scheme_checks():
     e4m3 = QuantScheme.default().with_value(QuantValue.E4M3).with_store(QuantStore.Native)
     assert status(lambda: qz.launch_ref(CLIENT, x, t((8, 64), 4), sc, sc, e4m3, ElemType.F32)) \
         == _ffi.ERR_SHAPE_MISMATCH                                                 # native store is bytes
-    raw = QuantScheme.default().to_c()
+    raw = type(QuantScheme.default().to_c()).from_buffer_copy(QuantScheme.default().to_c())  # to_c() is cached
     raw.reserved = 1
     assert _ffi.lib().cq_quantize(None, x.as_c(), x.as_c(), sc.as_c(), sc.as_c(), ctypes.byref(raw), 0) \
         == _ffi.ERR_INVALID_ARGUMENT
-    raw = QuantScheme.default().to_c()
+    raw = type(raw).from_buffer_copy(QuantScheme.default().to_c())
     raw.value = 42
     assert _ffi.lib().cq_dequantize(None, x.as_c(), x.as_c(), sc.as_c(), ctypes.byref(raw), 0) \
         == _ffi.ERR_INVALID_ARGUMENT
