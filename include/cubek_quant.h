@@ -127,8 +127,8 @@ cq_status cq_value_range(uint8_t value, float* range_min, float* range_max);
 /* ---- the path ---- */
 
 /* Replaces cubek_quant::quantize::launch_ref (src/quantize.rs:174-221).
- *   input      : float tensor of dtype `input_dtype`, any strides (contiguous row-major
- *                tensors take the streaming kernels, anything else a per-element path)
+ *   input      : float tensor of dtype `input_dtype`, any strides (fastest when
+ *                contiguous row-major; a contiguous last dimension is the next best)
  *   output     : U32 store -> u32 tensor, shape = input shape with the last
  *                dimension divided by num_quants (tests/suite/symmetric.rs:68-69);
  *                NATIVE store -> 1-byte tensor (E2M1: last dimension / 2);
