@@ -524,6 +524,17 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
     }
 
+    // blocks over the last two dimensions (or 1-D blocks on layouts the flat kernel refuses): one
+    // launch that owns whole blocks
+    cq::RowArgs rb;
+    if (!p.tensor_level && scales_rows_ok(p) && rows_args(p, scheme, input_dtype, input, output, &rb) &&
+        cq::blocks_dynamic_supported(input_dtype, rb)) {
+        rb.input = input->ptr;
+        rb.output = output->ptr;
+        rb.scale_out = out_scale->ptr;
+        return hip_status(cq::launch_quantize_blocks_dynamic(stream, input_dtype, static_cast<int>(p.bits), rb));
+    }
+
     uint64_t flat_words = 0;
     const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
     const uint64_t flat_chunks = flat ? (p.n / chunk_elems) * chunk_elems / per_chunk : 0;

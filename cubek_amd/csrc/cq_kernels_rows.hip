@@ -216,6 +216,118 @@ __global__ __launch_bounds__(kThreads) void scales_rows_kernel(RowArgs a, int ou
     }
 }
 
+// Fused dynamic quantize for blocks of BR rows x BC columns (BC a power-of-two number
+// of chunks): abs-max, scale, out_scale and codes in one launch that reads the input
+// once.  A workgroup owns whole blocks: TJ chunk columns x (256 / TJ) row phases; PH
+// phases share a block row and each keeps every PH-th row of it in registers (at most
+// kRows 16-byte chunks), so small BR puts several block rows into one workgroup.  The
+// abs-max meets across the chunk columns of a block by DPP and across the phases in LDS.
+template <int kLog2>
+__device__ __forceinline__ float group_max_log2(float v, uint32_t log2) {
+    if constexpr (kLog2 > 5) {
+        return v;
+    } else {
+        if (log2 == kLog2) return group_max<(1 << kLog2)>(v);
+        return group_max_log2<kLog2 + 1>(v, log2);
+    }
+}
+
+template <class F, int kBits, bool kWide, int kEnc, int kRows, int kCols>
+__global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, uint32_t cpb_log2, uint32_t ph_per_block,
+                                                                   uint32_t block_rows_per_group,
+                                                                   uint32_t num_block_rows, QuantParams qp) {
+    constexpr int kN = F::kPerChunk;
+    constexpr int kChunkBits = kN * kBits;
+    __shared__ float lds[kCols][kThreads];
+    const int last = static_cast<int>(a.rank) - 1;
+    const uint32_t tj = 1u << a.tj_log2;
+    const uint32_t ph = threadIdx.x >> a.tj_log2, jl = threadIdx.x & (tj - 1);
+    const uint32_t bsub = ph / ph_per_block, pin = ph % ph_per_block;
+    const uint32_t rbi = blockIdx.x * block_rows_per_group + bsub;
+    const uint32_t chunks_per_row = a.shape[last] / kN;
+    const uint32_t br = a.rank >= 2 ? a.block[last - 1] : 1u;
+    const bool row_group_live = bsub < block_rows_per_group && rbi < num_block_rows;
+    const RowPos r = row_pos(a, row_group_live ? rbi * br : 0);
+    const uint64_t pitch_f = a.rank >= 2 ? a.fstride[last - 1] / kN : 0;
+    const uint64_t pitch_v = a.rank >= 2 ? a.vstride[last - 1] : 0;
+    const u32x4* src = static_cast<const u32x4*>(a.input) + r.f / kN;
+
+    // kCols tiles of TJ chunk columns side by side; blocks never straddle a tile
+    uint32_t jc[kCols];
+    bool live[kCols];
+    u32x4 raw[kCols][kRows];
+#pragma unroll
+    for (int c = 0; c < kCols; c++) {
+        jc[c] = (blockIdx.y * kCols + c) * tj + jl;
+        live[c] = row_group_live && jc[c] < chunks_per_row;
+#pragma unroll
+        for (int k = 0; k < kRows; k++) {
+            const uint32_t rr = pin + k * ph_per_block;
+            raw[c][k] = u32x4{0, 0, 0, 0};
+            if (live[c] && rr < br) raw[c][k] = stream_load(src + rr * pitch_f + jc[c]);
+        }
+    }
+    float amax[kCols];
+#pragma unroll
+    for (int c = 0; c < kCols; c++) {
+        amax[c] = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kRows; k++) {
+            float v[kN];
+            F::unpack(raw[c][k], v);
+#pragma unroll
+            for (int i = 0; i < kN; i++) amax[c] = fmaxf(amax[c], fabsf(v[i]));  // NaN elements drop out
+        }
+        amax[c] = group_max_log2<0>(amax[c], cpb_log2);  // over the chunk columns of the block
+        lds[c][threadIdx.x] = amax[c];
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int c = 0; c < kCols; c++) {
+        if (bsub < block_rows_per_group)  // phases beyond the last whole block row hold nothing
+            for (uint32_t p = 0; p < ph_per_block; p++)
+                amax[c] = fmaxf(amax[c], lds[c][((bsub * ph_per_block + p) << a.tj_log2) + jl]);
+        const float s32 =
+            absmax_is_tame(amax[c]) ? scale_from_absmax_tame(amax[c], qp) : scale_from_absmax(amax[c], qp.width);
+        const float s_fs = round_to_dtype(a.param_dtype, F::round(s32));
+        if (live[c] && pin == 0 && (jc[c] & ((1u << cpb_log2) - 1)) == 0)
+            store_dtype(a.param_dtype, a.scale_out, r.sb + static_cast<uint64_t>(jc[c] >> cpb_log2) * a.sb[last], s_fs);
+        const float d = F::round(s_fs);
+        const bool tame = divisor_is_tame(d);
+        if (!live[c]) continue;  // the same for every lane of a word
+        uint32_t* out = static_cast<uint32_t*>(a.output) + r.v;
+#pragma unroll
+        for (int k = 0; k < kRows; k++) {
+            const uint32_t rr = pin + k * ph_per_block;
+            const bool row_live = rr < br;  // the same for every lane of a word
+            float v[kN], qn[kN];
+            F::unpack(raw[c][k], v);
+            quantize_values_neg<F, kN>(v, d, tame, qp.lo, qp.hi, qn);
+            uint32_t w[2] = {0, 0};
+            if constexpr (kEnc == kEncInt)
+                pack_chunk_neg<kBits, kN, kWide>(qn, w);
+            else
+                encode_chunk_neg<kEnc, kN>(qn, w);
+            uint32_t* dst = out + rr * pitch_v;
+            if constexpr (kChunkBits == 64) {
+                if (row_live) {
+                    stream_store(w[0], dst + 2 * static_cast<uint64_t>(jc[c]));
+                    stream_store(w[1], dst + 2 * static_cast<uint64_t>(jc[c]) + 1);
+                }
+            } else if constexpr (kChunkBits == 32) {
+                if (row_live) stream_store(w[0], dst + jc[c]);
+            } else {
+                // neighbouring lanes (same row) hold the other parts of the word
+                constexpr int kLanesPerWord = 32 / kChunkBits;
+                const uint32_t sub = jc[c] & (kLanesPerWord - 1);
+                const uint32_t word = group_or<kLanesPerWord>(w[0] << (sub * kChunkBits));
+                if (row_live && sub == 0) stream_store(word, dst + jc[c] / kLanesPerWord);
+            }
+        }
+    }
+}
+
 // Per-tensor abs-max, pass 1, over strided rows: gridDim.x <= kMaxPartials workgroups
 // stride over the (row tile, chunk tile) pairs; one f32 partial per workgroup.
 template <class F>
@@ -227,15 +339,25 @@ __global__ __launch_bounds__(kThreads) void absmax_rows_kernel(RowArgs a, float*
     const uint32_t tj = 1u << a.tj_log2;
     const uint32_t chunks_per_row = a.shape[last] / kN;
     const u32x4* in = static_cast<const u32x4*>(a.input);
+    constexpr int kUnroll = 4;  // tiles in flight per thread
+    const uint64_t tiles = static_cast<uint64_t>(row_tiles) * col_tiles;
     float amax = 0.0f;
-    for (uint64_t t = blockIdx.x; t < static_cast<uint64_t>(row_tiles) * col_tiles; t += gridDim.x) {
-        const uint32_t rt = static_cast<uint32_t>(t / col_tiles), ct = static_cast<uint32_t>(t % col_tiles);
-        const uint32_t row = rt * (kThreads >> a.tj_log2) + (threadIdx.x >> a.tj_log2);
-        const uint32_t jc = ct * tj + (threadIdx.x & (tj - 1));
-        const RowPos r = row_pos(a, row);
-        if (r.live && jc < chunks_per_row) {
+    for (uint64_t t0 = blockIdx.x; t0 < tiles; t0 += static_cast<uint64_t>(gridDim.x) * kUnroll) {
+        u32x4 raw[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const uint64_t t = t0 + static_cast<uint64_t>(u) * gridDim.x;
+            const uint32_t rt = static_cast<uint32_t>(t / col_tiles), ct = static_cast<uint32_t>(t % col_tiles);
+            const uint32_t row = rt * (kThreads >> a.tj_log2) + (threadIdx.x >> a.tj_log2);
+            const uint32_t jc = ct * tj + (threadIdx.x & (tj - 1));
+            const RowPos r = row_pos(a, row);
+            raw[u] = u32x4{0, 0, 0, 0};
+            if (t < tiles && r.live && jc < chunks_per_row) raw[u] = stream_load(in + r.f / kN + jc);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
             float v[kN];
-            F::unpack(stream_load(in + r.f / kN + jc), v);
+            F::unpack(raw[u], v);
 #pragma unroll
             for (int i = 0; i < kN; i++) amax = fmaxf(amax, fabsf(v[i]));
         }
@@ -320,7 +442,108 @@ hipError_t dequantize_rows(hipStream_t s, int bits, RowArgs a) {
     return hipErrorInvalidValue;
 }
 
+constexpr uint32_t kMaxRowsPerThread = 16;
+constexpr uint32_t kPreferredRowsPerThread = 8;  // more, smaller workgroups overlap their load and compute phases better
+
+// Geometry of quantize_blocks_kernel for one launch; false when a block row does not fit
+// the registers of one workgroup.
+struct BlocksGeom {
+    uint32_t cpb_log2, tj_log2, ph_per_block, per_group, rows_per_thread;
+};
+bool blocks_geom(uint32_t per_chunk, const RowArgs& a, BlocksGeom* g) {
+    const uint32_t last = a.rank - 1;
+    const uint32_t br = a.rank >= 2 ? a.block[last - 1] : 1u;
+    const uint32_t chunks_per_row = a.shape[last] / per_chunk, cpb = a.block[last] / per_chunk;
+    g->cpb_log2 = 0;
+    while ((1u << g->cpb_log2) < cpb) g->cpb_log2++;
+    const uint32_t min_log2 = g->cpb_log2 > 2 ? g->cpb_log2 : 2;  // at least one block and one word
+    // as many lanes along the row as the rows allow, while a block row still fits the registers
+    uint32_t tj_log2 = lanes_log2(chunks_per_row);
+    if (tj_log2 < min_log2) tj_log2 = min_log2;
+    while (tj_log2 > min_log2 && br > kPreferredRowsPerThread * (kThreads >> tj_log2)) tj_log2--;
+    const uint32_t phases = kThreads >> tj_log2;
+    g->tj_log2 = tj_log2;
+    g->ph_per_block = br >= phases ? phases : br;
+    g->per_group = br >= phases ? 1u : phases / br;
+    g->rows_per_thread = (br + g->ph_per_block - 1) / g->ph_per_block;
+    return g->rows_per_thread <= kMaxRowsPerThread;
+}
+
+// kRows x kCols chunks per thread: tall blocks keep their rows, flat ones take several
+// column tiles so that a thread still has 4-16 loads in flight.
+inline uint32_t blocks_cols_per_thread(uint32_t rows_per_thread) {
+    return rows_per_thread <= 2 ? 4u : (rows_per_thread <= 4 ? 2u : 1u);
+}
+
+template <class F, int kBits, bool kWide, int kEnc>
+hipError_t quantize_blocks_rows(hipStream_t s, RowArgs a, const BlocksGeom& g, dim3 grid, uint32_t num_block_rows,
+                                const QuantParams& qp) {
+#define CQ_ROWS(R, C)                                                                                           \
+    hipLaunchKernelGGL((quantize_blocks_kernel<F, kBits, kWide, kEnc, R, C>), grid, dim3(kThreads), 0, s, a,    \
+                       g.cpb_log2, g.ph_per_block, g.per_group, num_block_rows, qp)
+    if (g.rows_per_thread <= 1)
+        CQ_ROWS(1, 4);
+    else if (g.rows_per_thread <= 2)
+        CQ_ROWS(2, 4);
+    else if (g.rows_per_thread <= 4)
+        CQ_ROWS(4, 2);
+    else if (g.rows_per_thread <= 8)
+        CQ_ROWS(8, 1);
+    else
+        CQ_ROWS(16, 1);
+#undef CQ_ROWS
+    return hipGetLastError();
+}
+
+template <class F>
+hipError_t quantize_blocks(hipStream_t s, int bits, RowArgs a) {
+    constexpr uint32_t kN = F::kPerChunk;
+    BlocksGeom g;
+    if (!blocks_geom(kN, a, &g)) return hipErrorInvalidValue;
+    const uint32_t last = a.rank - 1;
+    const uint32_t br = a.rank >= 2 ? a.block[last - 1] : 1u;
+    const uint32_t chunks_per_row = a.shape[last] / kN;
+    a.tj_log2 = g.tj_log2;
+    const uint64_t num_block_rows = a.rows / br;
+    const uint32_t per_group_cols = blocks_cols_per_thread(g.rows_per_thread) << g.tj_log2;
+    const dim3 grid(static_cast<uint32_t>((num_block_rows + g.per_group - 1) / g.per_group),
+                    (chunks_per_row + per_group_cols - 1) / per_group_cols);
+    QuantParams qp;
+    qp.lo = a.range.lo;
+    qp.hi = a.range.hi;
+    qp.width = a.range.hi - a.range.lo;
+    qp.rwidth = 1.0f / qp.width;  // IEEE division on the host: correctly rounded
+    const bool wide = a.range.hi > 127.0f || a.range.lo < -128.0f;
+    const uint32_t nbr = static_cast<uint32_t>(num_block_rows);
+    switch (a.encoding) {
+        case kEncInt:
+            if (bits == 2) return quantize_blocks_rows<F, 2, false, kEncInt>(s, a, g, grid, nbr, qp);
+            if (bits == 4) return quantize_blocks_rows<F, 4, false, kEncInt>(s, a, g, grid, nbr, qp);
+            if (bits == 8 && wide) return quantize_blocks_rows<F, 8, true, kEncInt>(s, a, g, grid, nbr, qp);
+            if (bits == 8) return quantize_blocks_rows<F, 8, false, kEncInt>(s, a, g, grid, nbr, qp);
+            break;
+        case kEncE4M3: if (bits == 8) return quantize_blocks_rows<F, 8, false, kEncE4M3>(s, a, g, grid, nbr, qp); break;
+        case kEncE5M2: if (bits == 8) return quantize_blocks_rows<F, 8, false, kEncE5M2>(s, a, g, grid, nbr, qp); break;
+        case kEncE2M1: if (bits == 4) return quantize_blocks_rows<F, 4, false, kEncE2M1>(s, a, g, grid, nbr, qp); break;
+    }
+    return hipErrorInvalidValue;
+}
+
 }  // namespace
+
+bool blocks_dynamic_supported(int dtype, const RowArgs& a) {
+    const uint32_t per_chunk = dtype == CQ_F32 ? 4 : 8;
+    if (a.tensor_level) return false;
+    const uint32_t bc = a.block[a.rank - 1];
+    if (bc % per_chunk) return false;
+    const uint32_t cpb = bc / per_chunk;
+    BlocksGeom g;
+    return (cpb & (cpb - 1)) == 0 && a.rows != 0 && a.shape[a.rank - 1] != 0 && blocks_geom(per_chunk, a, &g);
+}
+
+hipError_t launch_quantize_blocks_dynamic(hipStream_t s, int dtype, int bits, const RowArgs& a) {
+    CQ_SWITCH_DTYPE(dtype, return quantize_blocks<kF>(s, bits, a))
+}
 
 uint32_t rows_unit_values(int dtype, int bits) {
     const uint32_t per_chunk = dtype == CQ_F32 ? 4 : 8, per_word = 32u / static_cast<uint32_t>(bits);
