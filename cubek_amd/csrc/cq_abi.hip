@@ -126,9 +126,10 @@ cq_status make_plan(const cq_scheme* s, const cq_tensor* floats, int dtype, cons
         p->shape[d] = floats->shape[d];
         uint64_t want = d + 1 == p->rank ? values->shape[d] * p->nq : values->shape[d];
         if (floats->shape[d] != want) return CQ_ERR_SHAPE_MISMATCH;
-        if (floats->shape[d] == 0 || floats->shape[d] > 0xffffffffull) return CQ_ERR_TOO_LARGE;
+        if (floats->shape[d] > 0xffffffffull) return CQ_ERR_TOO_LARGE;
     }
     p->n = numel(floats);
+    if (p->n == 0) return CQ_OK;  // an empty tensor: the callers launch nothing
     std::memset(&p->vs, 0, sizeof(p->vs));
     p->vs.on = !is_contiguous(floats) || !is_contiguous(values);
     p->vs.rank = p->rank;
@@ -325,6 +326,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     st = make_plan(scheme, input, input_dtype, output, scale, dtype_size(input_dtype), out_scale,
                    dtype_size(pd), &p);
     if (st != CQ_OK) return st;
+    if (p.n == 0) return CQ_OK;
     if (!out_scale) return CQ_ERR_INVALID_ARGUMENT;
 
     const bool native = scheme->store == CQ_STORE_NATIVE;
@@ -380,6 +382,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
     int pd = param_to_dtype(scheme->param);
     st = make_plan(scheme, output, output_dtype, values, params, dtype_size(pd), nullptr, 0, &p);
     if (st != CQ_OK) return st;
+    if (p.n == 0) return CQ_OK;
 
     const bool native = scheme->store == CQ_STORE_NATIVE;
     const uint64_t per_chunk = 16 / dtype_size(output_dtype);
@@ -481,6 +484,7 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
     Plan p;
     st = make_plan(scheme, input, input_dtype, &values, scales, dtype_size(input_dtype), nullptr, 0, &p);
     if (st != CQ_OK) return st;
+    if (p.n == 0) return CQ_OK;
 
     if (!p.vs.on && !p.tensor_level && p.last_dim_blocks && is_contiguous(scales) && aligned(input->ptr, 16) &&
         cq::flat_block_supported(input_dtype, p.block_last)) {
@@ -505,6 +509,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
     int pd = param_to_dtype(scheme->param);
     st = make_plan(scheme, input, input_dtype, output, out_scale, dtype_size(pd), nullptr, 0, &p);
     if (st != CQ_OK) return st;
+    if (p.n == 0) return CQ_OK;
 
     const uint64_t per_chunk = 16 / dtype_size(input_dtype);
     const bool native = scheme->store == CQ_STORE_NATIVE;

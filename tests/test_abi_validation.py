@@ -114,3 +114,15 @@ def test_into_contiguous_packed_checks():
     assert status(lambda: run(shape=(16, 4, 8))) == _ffi.ERR_SHAPE_MISMATCH     # rank
     # transposed source: logical [32, 16] packed along dim 0 (stride 1): source shape must be [4, 16]
     assert status(lambda: run(src=t((32, 2), 4, (1, 4)), dst=t((32, 2), 4), shape=(32, 16))) == _ffi.ERR_SHAPE_MISMATCH
+
+
+def test_empty_tensors_are_a_no_op():
+    """Zero elements: nothing to launch, success (shapes still have to agree)."""
+    x, out, sc = t((0, 64), 4), t((0, 16), 4), t((0, 2), 4)
+    qz.launch_ref(CLIENT, x, out, sc, sc, Q8_B32, ElemType.F32)
+    dq.launch_ref(CLIENT, out, x, sc, Q8_B32, ElemType.F32)
+    qz.launch_dynamic(CLIENT, x, out, sc, Q8_B32, ElemType.F32)
+    qz.compute_scales(CLIENT, x, sc, Q8_B32, ElemType.F32)
+    assert status(lambda: qz.launch_ref(CLIENT, x, t((0, 15), 4), sc, sc, Q8_B32, ElemType.F32)) == _ffi.ERR_SHAPE_MISMATCH
+    cq_reduce.max_abs(CLIENT, t((0, 8), 4), t((0, 1), 4), 1, ElemType.F32)   # no outputs
+    cq_contiguous.into_contiguous_packed_ref(CLIENT, t((0, 4), 4), t((0, 4), 4), (0, 32), 8)
