@@ -133,3 +133,35 @@ def test_reduce_reference_matrix(gpu, oracle, elem):
         want = oracle.reduce_max_abs(x, elem, shape, axis, in_strides=strides).reshape(-1)
         got, n_out = run(torch, gpu, x, elem, shape, axis, in_strides=strides)
         assert np.array_equal(got[:n_out].view(np.uint8), want.view(np.uint8)), (shape, strides, axis)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_reduce_random_shapes_axes_and_layouts(gpu, oracle, seed):
+    """Seeded random rank / shape / axis / strides / float type, with and without workspace."""
+    import torch
+
+    rng = np.random.default_rng(1000 + seed)
+    for _ in range(12):
+        rank = int(rng.integers(1, 5))
+        shape = [int(rng.choice([1, 2, 3, 5, 8, 16, 24, 33, 64, 100, 256, 1000, 4096])) for _ in range(rank)]
+        while int(np.prod(shape)) > (1 << 20):
+            shape[int(np.argmax(shape))] //= 2
+        shape = tuple(shape)
+        axis = int(rng.integers(rank))
+        elem = ELEMS[int(rng.integers(3))]
+        order = list(range(rank))
+        kind = int(rng.integers(3))
+        if kind == 2:
+            rng.shuffle(order)
+        strides, acc = [0] * rank, 1
+        for i, d in enumerate(reversed(order)):
+            strides[d] = acc
+            acc *= shape[d] + (4 if kind == 1 and i == 0 else 0)
+        reach = 1 + sum((n - 1) * st for n, st in zip(shape, strides))
+        x32 = rng.normal(0, 1, reach).astype(np.float32)
+        x32[rng.random(reach) < 0.01] = np.nan
+        x = oracle.to_bits(x32, elem)
+        want = oracle.reduce_max_abs(x, elem, shape, axis, in_strides=strides).reshape(-1)
+        for use_ws in (True, False):
+            got, n_out = run(torch, gpu, x, elem, shape, axis, use_workspace=use_ws, in_strides=strides)
+            assert np.array_equal(got[:n_out].view(np.uint8), want.view(np.uint8)), (shape, strides, axis, elem.name, use_ws)

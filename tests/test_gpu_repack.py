@@ -98,3 +98,35 @@ def test_into_contiguous_packed_errors(gpu):
         == _ffi.ERR_INVALID_ARGUMENT
     assert status(lambda: cq_contiguous.into_contiguous_packed_ref(client, h(src), h(dst, (16, 4), (8, 1)), (16, 32), 8)) \
         == _ffi.ERR_NON_CONTIGUOUS
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_into_contiguous_packed_random(gpu, oracle, seed):
+    """Seeded random rank / shape / packed dimension / memory order / padding."""
+    rng = np.random.default_rng(500 + seed)
+    for _ in range(10):
+        dtype, packing = [(np.uint32, 4), (np.uint32, 8), (np.uint32, 16), (np.uint8, 2)][int(rng.integers(4))]
+        rank = int(rng.integers(1, 5))
+        shape = [int(rng.choice([1, 2, 3, 5, 8, 12])) for _ in range(rank)]
+        packed_dim = int(rng.integers(rank))
+        mult = packing * (4 if rng.random() < 0.5 else 1)  # word-quad multiples reach the tiled kernel
+        shape[packed_dim] = mult * int(rng.integers(1, 12))
+        shape[-1] = (mult if packed_dim != rank - 1 else shape[-1]) * (int(rng.integers(1, 12)) if packed_dim != rank - 1 else 1)
+        shape = tuple(shape)
+        # memory order: the packed dimension is the fastest one (stride 1)
+        lead = [d for d in range(rank) if d != packed_dim]
+        rng.shuffle(lead)
+        order = tuple(lead + [packed_dim])
+        pad = int(rng.choice([0, 3, 4]))
+        bits = 8 * np.dtype(dtype).itemsize // packing
+        logical = rng.integers(0, 1 << bits, size=shape, dtype=np.uint64)
+        buf, in_strides = scatter_packed(logical, dtype, packing, packed_dim, order, rng, pad)
+        # the library finds the packed dimension itself: the rightmost one with stride 1
+        in_shape = tuple(s // packing if d == packed_dim else s for d, s in enumerate(shape))
+        rightmost = max(d for d in range(rank) if in_strides[d] == 1)
+        if rightmost != packed_dim:
+            continue  # another dimension of extent 1 also has stride 1: ambiguous by construction
+        want = oracle.into_contiguous_packed(buf, packing, shape, in_strides, packed_dim)
+        assert np.array_equal(want, pack_last(logical, dtype, packing))
+        got = run(gpu, buf, dtype, packing, shape, in_strides, packed_dim)
+        assert np.array_equal(got, want), (dtype.__name__, packing, shape, packed_dim, order, pad)
