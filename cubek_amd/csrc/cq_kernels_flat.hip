@@ -216,7 +216,8 @@ hipError_t launch_absmax_partials(hipStream_t s, int dtype, const void* input, u
     const uint64_t chunks = num_elems / per_chunk;
     const uint64_t per_group = static_cast<uint64_t>(kReduceThreads) * kReduceUnroll;
     const uint64_t want = (chunks + per_group - 1) / per_group;
-    const uint32_t grid = static_cast<uint32_t>(want < 1 ? 1 : (want > kMaxPartials ? kMaxPartials : want));
+    uint32_t grid = static_cast<uint32_t>(want < 1 ? 1 : (want > kMaxPartials ? kMaxPartials : want));
+    if (grid > 8) grid = (grid + 7) & ~7u;  // a multiple of the 8 XCDs: block b of the tensor is read on XCD b % 8
     const bool is_aligned = (reinterpret_cast<uintptr_t>(input) & 15u) == 0;
     *num_partials = grid;
     CQ_SWITCH_DTYPE(dtype,

@@ -46,8 +46,16 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
     constexpr int kChunkBits = kN * kBits;  // 64, 32, 16 or 8
     const int param_dtype = kParamF32 ? static_cast<int>(CQ_F32) : param_dtype_rt;
     const auto load_scale = [&](uint64_t i) { return F::load(scale_in, i); };
-    const uint64_t first =
-        chunk_begin + static_cast<uint64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+    // Pass 2 of the per-tensor reduction walks the tiles last to first: pass 1 has just read the
+    // tensor first to last, so what it read last is what the L2 caches still hold.  Groups of
+    // eight consecutive tiles keep their places, because workgroup i runs on XCD i % 8 and tile
+    // i was read there in pass 1 (each XCD has its own L2).
+    uint32_t tile = blockIdx.x;
+    if constexpr (kScaleSrc == kScalePartials) {
+        const uint32_t whole = gridDim.x & ~7u;
+        if (tile < whole) tile = (whole - 8 - (tile & ~7u)) + (tile & 7u);
+    }
+    const uint64_t first = chunk_begin + static_cast<uint64_t>(tile) * (kThreads * kUnroll) + threadIdx.x;
 
     // All kUnroll loads are issued back to back.  Checked launches let
     // out-of-range lanes re-read the last chunk instead of branching.
