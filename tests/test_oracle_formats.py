@@ -95,3 +95,27 @@ def test_minifloats_match_table_search(oracle):
     assert [L.cqo_e2m1_to_f32(c) for c in range(8)] == [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
     assert L.cqo_e4m3_to_f32(0x7E) == 448.0 and L.cqo_e4m3_to_f32(0x01) == 2.0 ** -9
     assert L.cqo_e5m2_to_f32(0x7B) == 57344.0 and L.cqo_e5m2_to_f32(0x01) == 2.0 ** -16
+
+
+def test_fp8_matches_torch_float8(oracle):
+    """e4m3 / e5m2 against torch's CPU float8 conversions (a library routine): every byte
+    decodes to the same value, and in-range floats encode to the same byte."""
+    import torch
+
+    L = oracle.lib()
+    rng = np.random.default_rng(8)
+    for name, tdt, top in (("e4m3", torch.float8_e4m3fn, 448.0), ("e5m2", torch.float8_e5m2, 57344.0)):
+        enc = getattr(L, f"cqo_f32_to_{name}")
+        dec = getattr(L, f"cqo_{name}_to_f32")
+        decoded = torch.arange(256, dtype=torch.uint8).view(tdt).to(torch.float32).numpy()
+        for code in range(256):
+            ours = dec(code)
+            if np.isfinite(decoded[code]):
+                assert ours == decoded[code], (name, code)
+        xs = np.concatenate([rng.uniform(-top, top, 20000), rng.normal(0, 1, 20000), rng.normal(0, 2.0 ** -8, 5000),
+                             np.arange(-448, 449, dtype=np.float64)]).astype(np.float32)
+        xs = xs[np.abs(xs) <= top]
+        want = torch.from_numpy(xs).to(tdt).view(torch.uint8).numpy()
+        got = np.array([enc(ctypes.c_float(float(v))) for v in xs], dtype=np.uint8)
+        # -0.0 and +0.0: both sides keep the sign of a float cast
+        assert np.array_equal(got, want), (name, xs[got != want][:5], got[got != want][:5], want[got != want][:5])
