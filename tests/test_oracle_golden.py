@@ -204,3 +204,32 @@ def test_param_dtype_rounds_the_divisor(oracle):
     assert d != sc[0]
     want = np.clip(np.rint(x / d), -127, 127).astype(np.int8).reshape(-1)
     assert np.array_equal(w.reshape(-1).view(np.int8), want)
+
+
+def test_native_fp8_store_matches_torch_composition(oracle):
+    """cqo_quantize_native / cqo_dequantize_native for e4m3 and e5m2 against the same
+    computation spelled with torch CPU routines: IEEE divide, round half to even, clamp,
+    cast to float8; and float8 -> f32 times scale.  (That the reference's native arm means
+    exactly this composition is a decision; that the oracle computes it is what this pins.)"""
+    import torch
+    from cubek_amd import ElemType, QuantLevel, QuantScheme, QuantStore, QuantValue
+
+    rng = np.random.default_rng(21)
+    for value, tdt, top in ((QuantValue.E4M3, torch.float8_e4m3fn, 448.0), (QuantValue.E5M2, torch.float8_e5m2, 57344.0)):
+        for block in (None, 16):
+            shape = (24, 64)
+            level = QuantLevel.Tensor if block is None else QuantLevel.block([block])
+            scheme = QuantScheme.default().with_value(value).with_store(QuantStore.Native).with_level(level)
+            x = rng.normal(0, 3, shape).astype(np.float32)
+            s = oracle.compute_scales(x, ElemType.F32, shape, scheme)
+            codes, out_scale = oracle.quantize(x, ElemType.F32, shape, s, scheme)
+            if block is None:
+                s_full = np.full(shape, s.reshape(-1)[0], dtype=np.float32)
+            else:
+                s_full = np.repeat(s.reshape(shape[0], -1), block, axis=1)
+            q = torch.clamp(torch.round(torch.from_numpy(x) / torch.from_numpy(s_full)), -top, top)
+            want = q.to(tdt).view(torch.uint8).numpy()
+            assert np.array_equal(codes.reshape(shape), want), value.name
+            y = oracle.dequantize(codes, shape, out_scale, ElemType.F32, scheme)
+            y_want = (torch.from_numpy(want).view(tdt).to(torch.float32) * torch.from_numpy(s_full)).numpy()
+            assert np.array_equal(y.reshape(shape), y_want), value.name
