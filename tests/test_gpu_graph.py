@@ -13,13 +13,15 @@ from cubek_amd import quantize as qz
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("level", ["block32", "tensor"])
+@pytest.mark.parametrize("level", ["block32", "tensor", "block64x64"])
 def test_graph_replays_match_eager(level):
     import torch
 
     scheme = QuantScheme.default().with_value(QuantValue.Q4S)
     if level == "block32":
         scheme = scheme.with_level(QuantLevel.block([32]))
+    elif level == "block64x64":  # the pipelined block kernel (looks up its occupancy on first use)
+        scheme = scheme.with_level(QuantLevel.block([64, 64]))
     shape = (512, 1024)
     h = TensorHandleRef.from_torch
     gen = torch.Generator(device="cuda").manual_seed(7)
