@@ -4,7 +4,7 @@
 // They are the counterparts of the public #[cube] functions of the reference
 // crate, which other kernels (its matmul) inline to dequantize while loading:
 //   dequantize_symmetric                  crates/cubek-quant/src/dequantize.rs:20-25
-//   dequantize_symmetric_packed_value(s)  src/dequantize.rs:27-79
+//   dequantize_symmetric_packed_value(s), dequantize_symmetric_packed_value_at   src/dequantize.rs:27-79
 //   unpack_q                              src/dequantize.rs:81-118
 //   ScalesLayout::{to_source_pos, is_block_start}   src/layout/scales.rs:15-195
 // Results are bit-identical to cq_dequantize for the same inputs.
@@ -91,14 +91,23 @@ __device__ __forceinline__ void dequantize_symmetric_packed_value(uint32_t word,
     for (int i = 0; i < 32 / kBits; i++) out[i] = round_to<kF>(s * q[i]);
 }
 
-// dequantize_symmetric_packed_values: word `position` of a packed tensor, its scale
-// looked up through the layout (`scales` holds f32 parameters).
+// dequantize_symmetric_packed_value_at: a word the caller already holds (`position` is its
+// index in the packed tensor), its scale looked up through the layout (`scales` holds f32
+// parameters): the scale of the word's first element, as the reference indexes its scales view.
+template <Float kF, int kBits>
+__device__ __forceinline__ void dequantize_symmetric_packed_value_at(uint64_t position, uint32_t word,
+                                                                     const float* scales, const ScalesLayout& layout,
+                                                                     float* out) {
+    const uint64_t elem = position * (32 / kBits);
+    dequantize_symmetric_packed_value<kF, kBits>(word, scales[layout.to_source_pos(elem)], out);
+}
+
+// dequantize_symmetric_packed_values: word `position` of a packed tensor.
 template <Float kF, int kBits>
 __device__ __forceinline__ void dequantize_symmetric_packed_values(uint64_t position, const uint32_t* values,
                                                                    const float* scales, const ScalesLayout& layout,
                                                                    float* out) {
-    const uint64_t elem = position * (32 / kBits);
-    dequantize_symmetric_packed_value<kF, kBits>(values[position], scales[layout.to_source_pos(elem)], out);
+    dequantize_symmetric_packed_value_at<kF, kBits>(position, values[position], scales, layout, out);
 }
 
 }  // namespace device
