@@ -6,7 +6,7 @@
 //   dequantize_symmetric                  crates/cubek-quant/src/dequantize.rs:20-25
 //   dequantize_symmetric_packed_value(s), dequantize_symmetric_packed_value_at   src/dequantize.rs:27-79
 //   unpack_q                              src/dequantize.rs:81-118
-//   ScalesLayout::{to_source_pos, is_block_start}   src/layout/scales.rs:15-195
+//   ScalesLayout::{to_source_pos, is_block_start}, scales_layout   src/layout/scales.rs:15-247
 // Results are bit-identical to cq_dequantize for the same inputs.
 #pragma once
 
@@ -50,6 +50,26 @@ struct ScalesLayout {
         return start;
     }
 };
+
+// scales_layout (src/layout/scales.rs:220-247), host side: the layout of the scales that belong
+// to a quantized tensor.
+//   values_shape   : shape of the QUANTIZED tensor (its last dimension counts stored elements)
+//   num_quants     : values per stored element (the last dimension is multiplied by it)
+//   scales_strides : strides of the scales tensor, in elements
+//   block          : block size per trailing dimension, block_rank entries (0: one scale per tensor);
+//                    left-padded with 1 up to the tensor rank, as BlockSize::to_dim_vec does
+inline ScalesLayout scales_layout(const uint64_t* values_shape, uint32_t rank, uint32_t num_quants,
+                                  const uint64_t* scales_strides, const uint8_t* block, uint32_t block_rank) {
+    ScalesLayout l;
+    if (block_rank == 0) return l;  // per tensor
+    l.rank = rank;
+    for (uint32_t d = 0; d < rank; d++) {
+        l.shape[d] = static_cast<uint32_t>(d + 1 == rank ? values_shape[d] * num_quants : values_shape[d]);
+        l.block[d] = d + block_rank < rank ? 1u : block[d + block_rank - rank];
+        l.strides[d] = scales_strides[d];
+    }
+    return l;
+}
 
 // Round an f32 value to `kF` (round-to-nearest-even), widened back to f32.
 template <Float kF>

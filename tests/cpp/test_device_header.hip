@@ -131,13 +131,10 @@ static void run_case(const char* name, QuantValue value, std::vector<uint64_t> s
     quantize::launch_dynamic(client, t_in, t_words, t_scales, scheme, elem);
     dequantize::launch_ref(client, t_words, t_ref, t_scales, scheme, elem);
 
-    dev::ScalesLayout layout;
-    layout.rank = static_cast<uint32_t>(shape.size());
-    for (size_t d = 0; d < shape.size(); d++) {
-        layout.shape[d] = static_cast<uint32_t>(shape[d]);
-        layout.block[d] = blk[d];
-        layout.strides[d] = t_scales.strides[d];
-    }
+    // as the reference's scales_layout(client, values, scales, 1, scheme): from the quantized tensor's shape
+    const dev::ScalesLayout layout =
+        dev::scales_layout(pshape.data(), static_cast<uint32_t>(pshape.size()), static_cast<uint32_t>(nq),
+                           t_scales.strides.data(), block.data(), static_cast<uint32_t>(block.size()));
     const uint64_t num_words = n / nq;
     hipLaunchKernelGGL((dequant_on_read<kF, kBits>), dim3(static_cast<uint32_t>((num_words + 255) / 256)), dim3(256), 0, 0,
                        d_words, d_scales, layout, num_words, d_got);
