@@ -40,17 +40,21 @@ __device__ __forceinline__ RowPos row_pos(const RowArgs& a, uint32_t row) {
     RowPos r{0, 0, 0, 0, true, row < a.rows};
     uint32_t rem = r.live ? row : 0;
     for (int d = static_cast<int>(a.rank) - 2; d >= 0; d--) {
-        const uint32_t c = rem % a.shape[d];
-        rem /= a.shape[d];
+        // the outermost coordinate is what is left; integer division is a long instruction sequence
+        const uint32_t c = d == 0 ? rem : rem % a.shape[d];
+        if (d != 0) rem /= a.shape[d];
         r.f += static_cast<uint64_t>(c) * a.fstride[d];
         r.v += static_cast<uint64_t>(c) * a.vstride[d];
         if (a.tensor_level) {
             r.start = r.start && c == 0;
+        } else if (a.block[d] == 1) {
+            r.sa += static_cast<uint64_t>(c) * a.sa[d];
+            r.sb += static_cast<uint64_t>(c) * a.sb[d];
         } else {
             const uint32_t cb = c / a.block[d];
             r.sa += static_cast<uint64_t>(cb) * a.sa[d];
             r.sb += static_cast<uint64_t>(cb) * a.sb[d];
-            r.start = r.start && (c % a.block[d]) == 0;
+            r.start = r.start && c == cb * a.block[d];
         }
     }
     return r;
