@@ -237,7 +237,28 @@ def adjacent_kernels(torch):
         out.append({"kernel": f"reduce_max_abs axis {axis} of bf16 [{rows}, {cols}]", "algorithmic_bytes": b,
                     "workspace_bytes": nbytes, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
-    del xs
+    # weight-style 128 x 128 blocks, fp8 e4m3 bytes: the fused block kernel (one launch, one read)
+    from cubek_amd import QuantLevel, QuantScheme, QuantStore, QuantValue
+    from cubek_amd import dequantize as cq_dequantize
+    from cubek_amd import quantize as cq_quantize
+
+    scheme = (QuantScheme.default().with_value(QuantValue.E4M3).with_store(QuantStore.Native)
+              .with_level(QuantLevel.block([128, 128])))
+    codes = [torch.empty((rows, cols), dtype=torch.uint8, device="cuda") for _ in range(sets)]
+    scales = [torch.empty((rows // 128, cols // 128), dtype=torch.float32, device="cuda") for _ in range(sets)]
+    ys = [torch.empty((rows, cols), dtype=torch.bfloat16, device="cuda") for _ in range(2)]
+    hx, hc, hs, hy = [h(x) for x in xs], [h(c) for c in codes], [h(s) for s in scales], [h(y) for y in ys]
+    b = rows * cols * 3 + scales[0].numel() * 4
+    for label, fn in (
+            ("quantize_dynamic", lambda i: cq_quantize.launch_dynamic(client, hx[i % sets], hc[i % sets], hs[i % sets],
+                                                                       scheme, ElemType.BF16)),
+            ("dequantize", lambda i: cq_dequantize.launch_ref(client, hc[i % sets], hy[i % 2], hs[i % sets], scheme,
+                                                              ElemType.BF16))):
+        ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
+        out.append({"kernel": f"{label}, 128 x 128 blocks, e4m3 native store, bf16 [{rows}, {cols}]",
+                    "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                    "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+    del xs, codes, scales, ys, hx, hc, hs, hy
     torch.cuda.empty_cache()
     # 4-bit codes of a [rows, cols] weight, 8 per u32 word along cols, viewed transposed as [cols, rows]
     packing = 8
