@@ -533,7 +533,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
     // launch that owns whole blocks
     cq::RowArgs rb;
     if (!p.tensor_level && scales_rows_ok(p) && rows_args(p, scheme, input_dtype, input, output, &rb) &&
-        cq::blocks_dynamic_supported(input_dtype, rb)) {
+        cq::blocks_dynamic_supported(input_dtype, static_cast<int>(p.bits), rb)) {
         rb.input = input->ptr;
         rb.output = output->ptr;
         rb.scale_out = out_scale->ptr;

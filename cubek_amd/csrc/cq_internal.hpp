@@ -140,8 +140,8 @@ hipError_t launch_dequantize_rows(hipStream_t s, int dtype, int bits, const RowA
 // extend over the last two dimensions only, the last extent is a multiple of a chunk
 hipError_t launch_scales_rows(hipStream_t s, int dtype, int out_dtype, const RowArgs& a);
 // fused abs-max + scale + quantize for blocks over the last two dimensions whose last extent is a
-// power-of-two number of 16-byte chunks; writes scale_out (typed param_dtype), reads no scale_in
-bool blocks_dynamic_supported(int dtype, const RowArgs& a);
+// whole number of 16-byte chunks; writes scale_out (typed param_dtype), reads no scale_in
+bool blocks_dynamic_supported(int dtype, int bits, const RowArgs& a);
 hipError_t launch_quantize_blocks_dynamic(hipStream_t s, int dtype, int bits, const RowArgs& a);
 // per-tensor abs-max partials (same contract as launch_absmax_partials)
 hipError_t launch_absmax_partials_rows(hipStream_t s, int dtype, const RowArgs& a, float* partials,

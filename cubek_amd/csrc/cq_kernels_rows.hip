@@ -220,13 +220,14 @@ __global__ __launch_bounds__(kThreads) void scales_rows_kernel(RowArgs a, int ou
     }
 }
 
-// Fused dynamic quantize for blocks of BR rows x BC columns (BC a power-of-two number
-// of chunks): abs-max, scale, out_scale and codes in one launch that reads the input
+// Fused dynamic quantize for blocks of BR rows x BC columns (BC a whole number of
+// chunks): abs-max, scale, out_scale and codes in one launch that reads the input
 // once.  A tile is what one workgroup holds at a time: TJ chunk columns (x kCols tiles
 // side by side) x (256 / TJ) row phases; PH phases share a block row and each keeps
 // every PH-th row of it in registers (at most kRows 16-byte chunks), so small BR puts
 // several block rows into one tile.  The abs-max meets across the chunk columns of a
-// block by DPP and across the phases in LDS.
+// block by DPP (power-of-two widths; other widths use only the lanes that hold whole
+// blocks and meet in LDS) and across the phases in LDS.
 // kPipeline (tall tiles): as many workgroups as the GPU holds at once walk the tiles
 // with a stride of gridDim.x and load tile i+1 before they work on tile i, so every
 // wave has loads in flight while it computes, whatever the other workgroups of its CU
@@ -244,7 +245,9 @@ __device__ __forceinline__ float group_max_log2(float v, uint32_t log2) {
 }
 
 struct BlocksGeom {
-    uint32_t cpb_log2, tj_log2, ph_per_block, per_group, rows_per_thread;
+    uint32_t cpb, cpb_log2;  // chunks per block along the row; its log2, or 32 when not a power of two
+    uint32_t tj_log2, tj_eff;  // lanes along the row, and how many of them hold whole blocks
+    uint32_t ph_per_block, per_group, rows_per_thread;
     uint32_t num_block_rows, col_groups, tiles;
 };
 
@@ -277,19 +280,20 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
         p.f = r.f / kN;
         p.v = r.v;
         p.sb = r.sb;
-        p.jc0 = cg * (kCols << g.tj_log2) + jl;
+        p.jc0 = cg * (kCols * g.tj_eff) + jl;
         return p;
     };
     auto load = [&](const Pos& p, u32x4 (&raw)[kCols][kRows]) {
         const u32x4* src = static_cast<const u32x4*>(a.input) + p.f;
 #pragma unroll
         for (int c = 0; c < kCols; c++) {
-            const uint32_t jc = p.jc0 + c * tj;
+            const uint32_t jc = p.jc0 + c * g.tj_eff;
 #pragma unroll
             for (int k = 0; k < kRows; k++) {
                 const uint32_t rr = pin + k * g.ph_per_block;
                 raw[c][k] = u32x4{0, 0, 0, 0};
-                if (p.rows_live && jc < chunks_per_row && rr < br) raw[c][k] = stream_load(src + rr * pitch_f + jc);
+                if (p.rows_live && jl < g.tj_eff && jc < chunks_per_row && rr < br)
+                    raw[c][k] = stream_load(src + rr * pitch_f + jc);
             }
         }
     };
@@ -323,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
 #pragma unroll
                 for (int i = 0; i < kN; i++) amax[c] = fmaxf(amax[c], fabsf(v[i]));  // NaN elements drop out
             }
-            amax[c] = group_max_log2<0>(amax[c], g.cpb_log2);  // over the chunk columns of the block
+            amax[c] = group_max_log2<0>(amax[c], g.cpb_log2);  // over the chunk columns of a power-of-two block
             lds[buf][c][threadIdx.x] = amax[c];
         }
         // LDS writes done, then the barrier; no wait for the global loads in flight.  The two LDS
@@ -332,16 +336,23 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
 
 #pragma unroll
         for (int c = 0; c < kCols; c++) {
-            const uint32_t jc = pos.jc0 + c * tj;
-            const bool live = pos.rows_live && jc < chunks_per_row;  // the same for every lane of a word
+            const uint32_t jc = pos.jc0 + c * g.tj_eff;
+            const bool live = pos.rows_live && jl < g.tj_eff && jc < chunks_per_row;  // the same for every lane of a word
+            const bool pow2 = g.cpb_log2 < 32;
+            // first lane and number of LDS entries of this block in a phase: after the DPP step every
+            // lane of a power-of-two block holds its maximum; other widths meet here, entry by entry
+            const uint32_t lane0 = pow2 ? jl : (jl < g.tj_eff ? jl / g.cpb * g.cpb : 0);
+            const uint32_t entries = pow2 ? 1u : g.cpb;
             if (bsub < g.per_group)  // phases beyond the last whole block row hold nothing
                 for (uint32_t p = 0; p < g.ph_per_block; p++)
-                    amax[c] = fmaxf(amax[c], lds[buf][c][((bsub * g.ph_per_block + p) << g.tj_log2) + jl]);
+                    for (uint32_t k = 0; k < entries; k++)
+                        amax[c] = fmaxf(amax[c], lds[buf][c][((bsub * g.ph_per_block + p) << g.tj_log2) + lane0 + k]);
             const float s32 =
                 absmax_is_tame(amax[c]) ? scale_from_absmax_tame(amax[c], qp) : scale_from_absmax(amax[c], qp.width);
             const float s_fs = round_to_dtype(a.param_dtype, F::round(s32));
-            if (live && pin == 0 && (jc & ((1u << g.cpb_log2) - 1)) == 0)
-                store_dtype(a.param_dtype, a.scale_out, pos.sb + static_cast<uint64_t>(jc >> g.cpb_log2) * a.sb[last], s_fs);
+            const uint32_t block_col = pow2 ? jc >> g.cpb_log2 : jc / g.cpb;
+            if (live && pin == 0 && jc == block_col * g.cpb)
+                store_dtype(a.param_dtype, a.scale_out, pos.sb + static_cast<uint64_t>(block_col) * a.sb[last], s_fs);
             const float d = F::round(s_fs);
             const bool tame = divisor_is_tame(d);
             if (!live) continue;
@@ -510,25 +521,34 @@ inline uint32_t blocks_cols_per_thread(uint32_t rows_per_thread) {
 
 // Geometry of quantize_blocks_kernel for one launch; false when a block row does not fit
 // the registers of one workgroup or there are too many tiles for 32-bit indices.
-bool blocks_geom(uint32_t per_chunk, const RowArgs& a, BlocksGeom* g) {
+bool blocks_geom(uint32_t per_chunk, uint32_t bits, const RowArgs& a, BlocksGeom* g) {
     const uint32_t last = a.rank - 1;
     const uint32_t br = a.rank >= 2 ? a.block[last - 1] : 1u;
     const uint32_t chunks_per_row = a.shape[last] / per_chunk, cpb = a.block[last] / per_chunk;
-    g->cpb_log2 = 0;
-    while ((1u << g->cpb_log2) < cpb) g->cpb_log2++;
-    const uint32_t min_log2 = g->cpb_log2 > 2 ? g->cpb_log2 : 2;  // at least one block and one word
+    g->cpb = cpb;
+    uint32_t cover_log2 = 0;  // lanes that cover one block
+    while ((1u << cover_log2) < cpb) cover_log2++;
+    g->cpb_log2 = (1u << cover_log2) == cpb ? cover_log2 : 32u;
+    const uint32_t min_log2 = cover_log2 > 2 ? cover_log2 : 2;  // at least one block and one word
     // as many lanes along the row as the rows allow, while a block row still fits the registers
     uint32_t tj_log2 = lanes_log2(chunks_per_row);
     if (tj_log2 < min_log2) tj_log2 = min_log2;
     while (tj_log2 > min_log2 && br > kPreferredRowsPerThread * (kThreads >> tj_log2)) tj_log2--;
     const uint32_t phases = kThreads >> tj_log2;
     g->tj_log2 = tj_log2;
+    // whole blocks and whole stored words only (lanes that share a word exchange their parts by lane number)
+    const uint32_t chunk_bits = per_chunk * bits;
+    const uint32_t word_lanes = chunk_bits >= 32 ? 1u : 32u / chunk_bits;
+    uint32_t step = cpb;
+    while (step % word_lanes) step += cpb;
+    g->tj_eff = ((1u << tj_log2) / step) * step;
+    if (g->tj_eff == 0) return false;
     g->ph_per_block = br >= phases ? phases : br;
     g->per_group = br >= phases ? 1u : phases / br;
     g->rows_per_thread = (br + g->ph_per_block - 1) / g->ph_per_block;
     if (g->rows_per_thread > kMaxRowsPerThread) return false;
     const uint64_t num_block_rows = a.rows / br;
-    const uint32_t per_group_cols = blocks_cols_per_thread(g->rows_per_thread) << tj_log2;
+    const uint32_t per_group_cols = blocks_cols_per_thread(g->rows_per_thread) * g->tj_eff;
     const uint64_t row_groups = (num_block_rows + g->per_group - 1) / g->per_group;
     g->num_block_rows = static_cast<uint32_t>(num_block_rows);
     g->col_groups = (chunks_per_row + per_group_cols - 1) / per_group_cols;
@@ -572,7 +592,7 @@ hipError_t quantize_blocks_rows(hipStream_t s, const RowArgs& a, const BlocksGeo
 template <class F>
 hipError_t quantize_blocks(hipStream_t s, int bits, const RowArgs& a) {
     BlocksGeom g;
-    if (!blocks_geom(F::kPerChunk, a, &g)) return hipErrorInvalidValue;
+    if (!blocks_geom(F::kPerChunk, static_cast<uint32_t>(bits), a, &g)) return hipErrorInvalidValue;
     if (g.tiles == 0) return hipSuccess;
     QuantParams qp;
     qp.lo = a.range.lo;
@@ -596,14 +616,13 @@ hipError_t quantize_blocks(hipStream_t s, int bits, const RowArgs& a) {
 
 }  // namespace
 
-bool blocks_dynamic_supported(int dtype, const RowArgs& a) {
+bool blocks_dynamic_supported(int dtype, int bits, const RowArgs& a) {
     const uint32_t per_chunk = dtype == CQ_F32 ? 4 : 8;
     if (a.tensor_level) return false;
     const uint32_t bc = a.block[a.rank - 1];
     if (bc % per_chunk) return false;
-    const uint32_t cpb = bc / per_chunk;
     BlocksGeom g;
-    return (cpb & (cpb - 1)) == 0 && a.rows != 0 && a.shape[a.rank - 1] != 0 && blocks_geom(per_chunk, a, &g);
+    return a.rows != 0 && a.shape[a.rank - 1] != 0 && blocks_geom(per_chunk, static_cast<uint32_t>(bits), a, &g);
 }
 
 hipError_t launch_quantize_blocks_dynamic(hipStream_t s, int dtype, int bits, const RowArgs& a) {
