@@ -11,6 +11,11 @@
 // thread decomposes its row index once (strides and block coordinates of the
 // leading dimensions) and then walks kUnits units of that row; loads and stores are
 // 16 bytes of floats and whole 32-bit words.
+//
+//   quantize_rows_kernel / dequantize_rows_kernel   scales given / stored
+//   scales_rows_kernel        abs-max of BR x BC blocks -> scales
+//   quantize_blocks_kernel    abs-max + scale + quantize of BR x BC blocks in one launch
+//   absmax_rows_kernel        per-tensor abs-max partials over strided rows
 #include "cq_device.hpp"
 #include "cq_internal.hpp"
 
