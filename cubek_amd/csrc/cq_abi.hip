@@ -244,6 +244,77 @@ bool rows_args(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* fl
     return true;
 }
 
+// Transposed float tensor (stride 1 on the second to last dimension), stored tensor with a
+// contiguous last dimension, blocks along the last dimension only (see cq_kernels_transposed.hip).
+// Fills `t` except the data pointers and scale_in_dtype.
+bool transposed_args(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
+                     cq::TransposedArgs* t) {
+    if (p.rank < 2) return false;
+    const uint32_t last = p.rank - 1, rdim = p.rank - 2;
+    if (floats->strides[rdim] != 1 || p.shape[rdim] < 2) return false;
+    if (values->strides[last] != 1 || !aligned(values->ptr, 4)) return false;
+    const bool native = s->store == CQ_STORE_NATIVE;
+    const uint32_t unit = cq::rows_unit_values(dtype, static_cast<int>(p.bits));
+    const uint64_t cols = p.shape[last];
+    std::memset(t, 0, sizeof(*t));
+    if (p.tensor_level) {
+        t->segment = cols % 32 == 0 ? 32u : unit;
+    } else {
+        for (uint32_t d = 0; d < last; d++)
+            if (p.layout.block[d] != 1) return false;
+        t->segment = p.layout.block[last];
+    }
+    if (t->segment % unit || cols % t->segment || cols == 0) return false;
+    if (native && values->strides[rdim] % 4) return false;
+    t->tensor_level = p.tensor_level ? 1u : 0u;
+    t->rows = static_cast<uint32_t>(p.shape[rdim]);
+    t->segments = static_cast<uint32_t>(cols / t->segment);
+    t->pitch_f = floats->strides[last];
+    t->vrow = native ? values->strides[rdim] / 4 : values->strides[rdim];
+    t->sa_row = p.layout.stride_a[rdim];
+    t->sa_col = p.layout.stride_a[last];
+    t->sb_row = p.layout.stride_b[rdim];
+    t->sb_col = p.layout.stride_b[last];
+    uint64_t batches = 1;
+    for (uint32_t d = 0; d < rdim; d++) {
+        if (p.shape[d] == 1) continue;
+        if (native && values->strides[d] % 4) return false;
+        const uint32_t k = t->num_batch_dims++;
+        t->batch_shape[k] = static_cast<uint32_t>(p.shape[d]);
+        t->batch_f[k] = floats->strides[d];
+        t->batch_v[k] = native ? values->strides[d] / 4 : values->strides[d];
+        t->batch_sa[k] = p.layout.stride_a[d];
+        t->batch_sb[k] = p.layout.stride_b[d];
+        batches *= p.shape[d];
+    }
+    if (batches > 65535 || (t->segments + 3) / 4 > 65535) return false;
+    t->batches = static_cast<uint32_t>(batches);
+    t->param_dtype = param_to_dtype(s->param);
+    t->encoding = flat_encoding(s);
+    t->range = p.range;
+    return true;
+}
+
+// A tensor whose elements fill a buffer without gaps or overlap (a permutation of a contiguous
+// layout): order-free reductions may read the buffer front to back.
+bool is_dense_permutation(const cq_tensor* t) {
+    uint32_t order[CQ_MAX_RANK], n = 0;
+    for (uint32_t d = 0; d < t->rank; d++)
+        if (t->shape[d] != 1) order[n++] = d;
+    for (uint32_t i = 1; i < n; i++)  // insertion sort by stride
+        for (uint32_t j = i; j > 0 && t->strides[order[j]] < t->strides[order[j - 1]]; j--) {
+            const uint32_t tmp = order[j];
+            order[j] = order[j - 1];
+            order[j - 1] = tmp;
+        }
+    uint64_t expect = 1;
+    for (uint32_t i = 0; i < n; i++) {
+        if (t->strides[order[i]] != expect) return false;
+        expect *= t->shape[order[i]];
+    }
+    return true;
+}
+
 // Block abs-max by the row kernels: blocks over the last two dimensions only.
 bool scales_rows_ok(const Plan& p) {
     if (p.tensor_level) return false;
@@ -359,6 +430,15 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         r.scale_out = out_scale->ptr;
         return hip_status(cq::launch_quantize_rows(stream, input_dtype, static_cast<int>(p.bits), r));
     }
+    cq::TransposedArgs tr;
+    if (flat_words == 0 && transposed_args(p, scheme, input_dtype, input, output, &tr)) {
+        tr.input = input->ptr;
+        tr.output = output->ptr;
+        tr.scale_in = scale->ptr;
+        tr.scale_in_dtype = input_dtype;
+        tr.scale_out = out_scale->ptr;
+        return hip_status(cq::launch_quantize_transposed(stream, input_dtype, static_cast<int>(p.bits), false, tr));
+    }
     if (flat_words < p.n / p.nq) {
         cq::GenericArgs g = generic_args(p, scheme);
         g.input = input->ptr;
@@ -409,6 +489,13 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         r.scale_in = params->ptr;
         return hip_status(cq::launch_dequantize_rows(stream, output_dtype, static_cast<int>(p.bits), r));
     }
+    cq::TransposedArgs tr;
+    if (flat_words == 0 && transposed_args(p, scheme, output_dtype, output, values, &tr)) {
+        tr.input = values->ptr;
+        tr.output = output->ptr;
+        tr.scale_in = params->ptr;
+        return hip_status(cq::launch_dequantize_transposed(stream, output_dtype, static_cast<int>(p.bits), tr));
+    }
     if (flat_words < p.n / p.nq) {
         cq::GenericArgs g = generic_args(p, scheme);
         g.input = values->ptr;
@@ -434,7 +521,11 @@ static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_sche
         uint32_t num_partials = 0;
         cq_status st;
         cq::RowArgs r;
-        if (p.vs.on && rows_args(p, scheme, input_dtype, input, nullptr, &r)) {
+        if (p.vs.on && is_dense_permutation(input)) {
+            // the order does not matter for a maximum: read the buffer front to back
+            st = hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n,
+                                                       static_cast<float*>(workspace), &num_partials));
+        } else if (p.vs.on && rows_args(p, scheme, input_dtype, input, nullptr, &r)) {
             r.input = input->ptr;
             st = hip_status(cq::launch_absmax_partials_rows(stream, input_dtype, r, static_cast<float*>(workspace),
                                                             &num_partials));
@@ -540,6 +631,15 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         return hip_status(cq::launch_quantize_blocks_dynamic(stream, input_dtype, static_cast<int>(p.bits), rb));
     }
 
+    cq::TransposedArgs tr;
+    const bool transposed = !flat && transposed_args(p, scheme, input_dtype, input, output, &tr);
+    if (transposed && !p.tensor_level) {  // each thread owns whole blocks: one launch
+        tr.input = input->ptr;
+        tr.output = output->ptr;
+        tr.scale_out = out_scale->ptr;
+        return hip_status(cq::launch_quantize_transposed(stream, input_dtype, static_cast<int>(p.bits), true, tr));
+    }
+
     uint64_t flat_words = 0;
     const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
     const uint64_t flat_chunks = flat ? (p.n / chunk_elems) * chunk_elems / per_chunk : 0;
@@ -581,6 +681,14 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         r.scale_in_dtype = pd;
         r.scale_out = nullptr;
         return hip_status(cq::launch_quantize_rows(stream, input_dtype, static_cast<int>(p.bits), r));
+    }
+    if (flat_words == 0 && transposed) {
+        tr.input = input->ptr;
+        tr.output = output->ptr;
+        tr.scale_in = out_scale->ptr;
+        tr.scale_in_dtype = pd;
+        tr.scale_out = nullptr;
+        return hip_status(cq::launch_quantize_transposed(stream, input_dtype, static_cast<int>(p.bits), false, tr));
     }
     if (flat_words < p.n / p.nq) {
         cq::GenericArgs g = generic_args(p, scheme);

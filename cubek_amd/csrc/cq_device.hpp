@@ -120,14 +120,19 @@ struct F16 {
     static constexpr int kDtype = CQ_F16;
     static constexpr int kBytes = 2;
     static constexpr int kPerChunk = 8;
-    __device__ static __forceinline__ float round(float v) {
-        return static_cast<float>(static_cast<_Float16>(v));  // v_cvt_f16_f32 (RNE), widen back
+    // f32 -> f16 (RNE).  `v` is first pinned as an f32 value of its own: when it is a product, the
+    // compiler otherwise fuses the multiply and the conversion into v_fma_mixlo_f16 with a +0
+    // addend, and (-0) + (+0) = +0 loses the sign of a negative zero.
+    __device__ static __forceinline__ _Float16 narrow(float v) {
+        asm("" : "+v"(v));
+        return static_cast<_Float16>(v);
     }
+    __device__ static __forceinline__ float round(float v) { return static_cast<float>(narrow(v)); }
     __device__ static __forceinline__ float load(const void* p, uint64_t i) {
         return static_cast<float>(static_cast<const _Float16*>(p)[i]);
     }
     __device__ static __forceinline__ void store(void* p, uint64_t i, float v) {
-        static_cast<_Float16*>(p)[i] = static_cast<_Float16>(v);
+        static_cast<_Float16*>(p)[i] = narrow(v);
     }
     __device__ static __forceinline__ void unpack(u32x4 raw, float* v) {
 #pragma unroll
@@ -142,7 +147,7 @@ struct F16 {
         u32x4 r;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            f16x2 h = {static_cast<_Float16>(v[2 * j]), static_cast<_Float16>(v[2 * j + 1])};
+            f16x2 h = {narrow(v[2 * j]), narrow(v[2 * j + 1])};
             r[j] = __builtin_bit_cast(uint32_t, h);
         }
         return r;

@@ -147,6 +147,31 @@ hipError_t launch_quantize_blocks_dynamic(hipStream_t s, int dtype, int bits, co
 hipError_t launch_absmax_partials_rows(hipStream_t s, int dtype, const RowArgs& a, float* partials,
                                        uint32_t* num_partials);
 
+// Transposed float tensors: the memory-fastest dimension is the second to last logical one.
+// Blocks run along the last dimension only (or one scale per tensor).
+struct TransposedArgs {
+    const void* input;       // floats (quantize) / stored words (dequantize)
+    void* output;
+    const void* scale_in;    // quantize with given scales: typed scale_in_dtype; dequantize: typed param_dtype
+    void* scale_out;         // quantize: out_scale or NULL
+    int scale_in_dtype, param_dtype;
+    int encoding;            // cq::Encoding
+    Range range;
+    uint32_t tensor_level;
+    uint32_t rows;           // extent of the second to last dimension (float stride 1)
+    uint32_t segment;        // columns one thread handles: the block size, or 32 per tensor
+    uint32_t segments;       // last dimension / segment
+    uint32_t batches;        // product of the leading dimensions (<= 65535)
+    uint64_t pitch_f;        // float stride of the last dimension
+    uint64_t vrow;           // stored stride of the second to last dimension, in 32-bit words
+    uint64_t sa_row, sa_col, sb_row, sb_col;  // scale strides along the two dimensions
+    uint32_t num_batch_dims;
+    uint32_t batch_shape[CQ_MAX_RANK];
+    uint64_t batch_f[CQ_MAX_RANK], batch_v[CQ_MAX_RANK], batch_sa[CQ_MAX_RANK], batch_sb[CQ_MAX_RANK];
+};
+hipError_t launch_quantize_transposed(hipStream_t s, int dtype, int bits, bool dynamic, const TransposedArgs& a);
+hipError_t launch_dequantize_transposed(hipStream_t s, int dtype, int bits, const TransposedArgs& a);
+
 // Re-packing of a strided quantized tensor (cq_into_contiguous_packed).
 struct RepackArgs {
     const void* input;

@@ -77,6 +77,9 @@ __device__ __forceinline__ float round_to(float v) {
     if constexpr (kF == Float::F32) {
         return v;
     } else if constexpr (kF == Float::F16) {
+        // pin `v` first: fused with a preceding multiply (v_fma_mixlo_f16, +0 addend) the conversion
+        // would turn a negative zero product into +0
+        asm("" : "+v"(v));
         return static_cast<float>(static_cast<_Float16>(v));
     } else {
         return static_cast<float>(static_cast<__bf16>(v));

@@ -468,8 +468,45 @@ def test_f16_every_input_every_divisor(gpu, oracle, value):
         scale = np.ascontiguousarray(np.broadcast_to(d[:, None], (rows, 512)))
         dout = torch.zeros(pshape, dtype=torch.int32, device="cuda")
         dos = torch.zeros((rows, 512), dtype=torch.float32, device="cuda")
-        qz.launch_ref(client, gpu.handle(dx), gpu.handle(dout), gpu.handle(gpu.to_dev(scale)), gpu.handle(dos),
+        dscale = gpu.to_dev(scale)  # the handle only borrows it
+        qz.launch_ref(client, gpu.handle(dx), gpu.handle(dout), gpu.handle(dscale), gpu.handle(dos),
                       scheme, ElemType.F16)
         torch.cuda.synchronize()
         want, _ = oracle.quantize(x, ElemType.F16, (rows, 65536), scale, scheme, threads=16)
         assert np.array_equal(gpu.to_host(dout).reshape(-1), want.reshape(-1)), (value.name, d0)
+
+
+@pytest.mark.parametrize("elem", ELEMS, ids=lambda e: e.name)
+def test_negative_zero_survives_every_dequantize_path(gpu, oracle, elem):
+    """-0 codes (fp8 / fp4 sign bit with zero magnitude) and zero codes under a negative scale
+    dequantize to -0, whichever kernel takes the layout: contiguous, pitched rows, transposed,
+    transposed with an odd pitch (per-element)."""
+    import torch
+    from cubek_amd import ComputeClient
+    from cubek_amd import dequantize as dq
+
+    client = ComputeClient.current()
+    rows, cols = 64, 64
+    cases = [(QuantValue.E4M3, QuantStore.Native, np.uint8, 0x80, 0.5), (QuantValue.E5M2, QuantStore.Native, np.uint8, 0x80, 0.5),
+             (QuantValue.E2M1, QuantStore.Native, np.uint8, 0x88, 0.5), (QuantValue.Q8S, QuantStore.U32, np.uint32, 0, -0.5),
+             (QuantValue.Q4S, QuantStore.U32, np.uint32, 0, -0.5)]
+    for value, store, sdt, code, scale in cases:
+        scheme = QuantScheme.default().with_value(value).with_store(store)
+        pshape = scheme.packed_shape((rows, cols))
+        codes = np.full(pshape, code, dtype=sdt)
+        params = np.array([scale], dtype=np.float32)
+        want = oracle.dequantize(codes, (rows, cols), params, elem, scheme).reshape(rows, cols)
+        assert np.signbit(oracle.from_bits(want, elem)).all()
+        for name, fstr in (("contiguous", (cols, 1)), ("pitched", (cols + 8, 1)), ("transposed", (1, rows)),
+                           ("transposed_odd_pitch", (1, rows + 1))):
+            n = 1 + (rows - 1) * fstr[0] + (cols - 1) * fstr[1]
+            d_y = torch.full((n,), 7.0, dtype={ElemType.F32: torch.float32, ElemType.BF16: torch.bfloat16,
+                                               ElemType.F16: torch.float16}[elem], device="cuda")
+            d_codes, d_params = gpu.to_dev(codes), gpu.to_dev(params)  # the handles only borrow: keep them alive
+            dq.launch_ref(client, gpu.handle(d_codes), gpu.handle(d_y, (rows, cols), fstr), gpu.handle(d_params),
+                          scheme, elem)
+            torch.cuda.synchronize()
+            raw = d_y.view(torch.int32 if elem == ElemType.F32 else torch.int16)
+            got = torch.as_strided(raw, (rows, cols), fstr).cpu().numpy()
+            bits = np.uint32 if elem == ElemType.F32 else np.uint16
+            assert np.array_equal(got.view(bits), np.ascontiguousarray(want).view(bits)), (value.name, elem.name, name)

@@ -58,6 +58,20 @@ def layouts(shape, per):
            ("transposed_stored", contiguous(shape), permuted(pshape)),
            ("both", permuted(shape), permuted(pshape))]
     if rank >= 2:
+        # last two dimensions swapped in memory (rows of the buffer = logical columns), padded pitch,
+        # leading dimensions outermost: the transposed-float kernels
+        def swapped(sh, pad):
+            st = [0] * len(sh)
+            st[-2] = 1
+            st[-1] = sh[-2] + pad
+            acc = st[-1] * sh[-1]
+            for d in range(len(sh) - 3, -1, -1):
+                st[d] = acc
+                acc *= sh[d]
+            return tuple(st)
+
+        out.append(("last_two_swapped", swapped(shape, 0), contiguous(pshape)))
+        out.append(("last_two_swapped_pitched", swapped(shape, 6), contiguous(pshape, 3)))
         out.append(("every_other_row", tuple(s * (2 if d == 0 else 1) for d, s in enumerate(contiguous(shape))),
                     tuple(s * (2 if d == 0 else 1) for d, s in enumerate(contiguous(pshape)))))
     return pshape, out
@@ -86,7 +100,7 @@ def test_strided_value_tensors(gpu, oracle, elem, name, scheme):
     per = scheme.num_quants()
     stored_np = np.uint32 if scheme.store == QuantStore.U32 else np.uint8
     pe = gpu.param_elem(scheme)
-    for shape in ((6, 64), (2, 4, 96)):
+    for shape in ((6, 64), (2, 4, 96), (3, 70, 128)):
         pshape, cases = layouts(shape, per)
         sshape = scheme.scales_shape(shape)
         for case, fstr, vstr in cases:
