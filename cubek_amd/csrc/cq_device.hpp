@@ -127,7 +127,9 @@ struct F16 {
         asm("" : "+v"(v));
         return static_cast<_Float16>(v);
     }
-    __device__ static __forceinline__ float round(float v) { return static_cast<float>(narrow(v)); }
+    // not pinned: no caller rounds a product that can be a negative zero (scales are positive,
+    // quotients come out of inline assembly), and the hot dequantize kernels round a scale per chunk
+    __device__ static __forceinline__ float round(float v) { return static_cast<float>(static_cast<_Float16>(v)); }
     __device__ static __forceinline__ float load(const void* p, uint64_t i) {
         return static_cast<float>(static_cast<const _Float16*>(p)[i]);
     }
@@ -147,7 +149,10 @@ struct F16 {
         u32x4 r;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            f16x2 h = {narrow(v[2 * j]), narrow(v[2 * j + 1])};
+            // plain casts: pairs become v_cvt_pk_f16_f32, which keeps the sign of zero, and pinning the
+            // inputs as narrow() does costs the 4-bit dequantize kernels 8 % (the negative-zero test
+            // watches this path too)
+            f16x2 h = {static_cast<_Float16>(v[2 * j]), static_cast<_Float16>(v[2 * j + 1])};
             r[j] = __builtin_bit_cast(uint32_t, h);
         }
         return r;
