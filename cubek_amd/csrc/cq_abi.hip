@@ -246,14 +246,15 @@ bool rows_args(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* fl
 
 // Transposed float tensor (stride 1 on the second to last dimension), stored tensor with a
 // contiguous last dimension, blocks along the last dimension only (see cq_kernels_transposed.hip).
-// Fills `t` except the data pointers and scale_in_dtype.
+// Fills `t` except the data pointers and scale_in_dtype; `values` may be NULL for a launch that only
+// reads the floats (scale production).
 bool transposed_args(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
                      cq::TransposedArgs* t) {
     if (p.rank < 2) return false;
     const uint32_t last = p.rank - 1, rdim = p.rank - 2;
     if (floats->strides[rdim] != 1 || p.shape[rdim] < 2) return false;
-    if (values->strides[last] != 1 || !aligned(values->ptr, 4)) return false;
-    const bool native = s->store == CQ_STORE_NATIVE;
+    if (values && (values->strides[last] != 1 || !aligned(values->ptr, 4))) return false;
+    const bool native = values && s->store == CQ_STORE_NATIVE;
     const uint32_t unit = cq::rows_unit_values(dtype, static_cast<int>(p.bits));
     const uint64_t cols = p.shape[last];
     std::memset(t, 0, sizeof(*t));
@@ -270,7 +271,7 @@ bool transposed_args(const Plan& p, const cq_scheme* s, int dtype, const cq_tens
     t->rows = static_cast<uint32_t>(p.shape[rdim]);
     t->segments = static_cast<uint32_t>(cols / t->segment);
     t->pitch_f = floats->strides[last];
-    t->vrow = native ? values->strides[rdim] / 4 : values->strides[rdim];
+    if (values) t->vrow = native ? values->strides[rdim] / 4 : values->strides[rdim];
     t->sa_row = p.layout.stride_a[rdim];
     t->sa_col = p.layout.stride_a[last];
     t->sb_row = p.layout.stride_b[rdim];
@@ -282,7 +283,7 @@ bool transposed_args(const Plan& p, const cq_scheme* s, int dtype, const cq_tens
         const uint32_t k = t->num_batch_dims++;
         t->batch_shape[k] = static_cast<uint32_t>(p.shape[d]);
         t->batch_f[k] = floats->strides[d];
-        t->batch_v[k] = native ? values->strides[d] / 4 : values->strides[d];
+        if (values) t->batch_v[k] = native ? values->strides[d] / 4 : values->strides[d];
         t->batch_sa[k] = p.layout.stride_a[d];
         t->batch_sb[k] = p.layout.stride_b[d];
         batches *= p.shape[d];
@@ -548,6 +549,12 @@ static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_sche
         r.input = input->ptr;
         r.scale_out = scales->ptr;
         return hip_status(cq::launch_scales_rows(stream, input_dtype, out_dtype, r));
+    }
+    cq::TransposedArgs tr;
+    if (transposed_args(p, scheme, input_dtype, input, nullptr, &tr)) {
+        tr.input = input->ptr;
+        tr.scale_out = scales->ptr;
+        return hip_status(cq::launch_scales_transposed(stream, input_dtype, out_dtype, tr));
     }
     cq::GenericArgs g = generic_args(p, scheme);
     g.input = input->ptr;

@@ -171,6 +171,8 @@ struct TransposedArgs {
 };
 hipError_t launch_quantize_transposed(hipStream_t s, int dtype, int bits, bool dynamic, const TransposedArgs& a);
 hipError_t launch_dequantize_transposed(hipStream_t s, int dtype, int bits, const TransposedArgs& a);
+// block abs-max -> out_dtype(dtype(2*absmax/(hi-lo))) through sb_row / sb_col into scale_out (block level only)
+hipError_t launch_scales_transposed(hipStream_t s, int dtype, int out_dtype, const TransposedArgs& a);
 
 // Re-packing of a strided quantized tensor (cq_into_contiguous_packed).
 struct RepackArgs {

@@ -177,6 +177,31 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_kernel(Transpose
     }
 }
 
+// Block abs-max -> scale typed `out_dtype` (what cq_compute_scales produces), same mapping.
+template <class F>
+__global__ __launch_bounds__(kThreads) void scales_transposed_kernel(TransposedArgs a, int out_dtype, QuantParams qp) {
+    const uint32_t r = blockIdx.x * kWave + (threadIdx.x & (kWave - 1));
+    const uint32_t seg = blockIdx.y * kSegmentsPerGroup + threadIdx.x / kWave;
+    if (r >= a.rows || seg >= a.segments) return;
+    const BatchPos b = batch_pos(a, blockIdx.z);
+    const uint64_t f0 = b.f + r + static_cast<uint64_t>(seg) * a.segment * a.pitch_f;
+    constexpr uint32_t kPiece = 32;
+    float amax = 0.0f;
+    for (uint32_t c = 0; c < a.segment; c += kPiece) {
+        float v[kPiece];
+#pragma unroll
+        for (uint32_t i = 0; i < kPiece; i++) {
+            v[i] = 0.0f;
+            if (c + i < a.segment) v[i] = F::load(a.input, f0 + static_cast<uint64_t>(c + i) * a.pitch_f);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < kPiece; i++) amax = fmaxf(amax, fabsf(v[i]));  // NaN elements drop out
+    }
+    const float s32 = absmax_is_tame(amax) ? scale_from_absmax_tame(amax, qp) : scale_from_absmax(amax, qp.width);
+    store_dtype(out_dtype, a.scale_out, b.sb + static_cast<uint64_t>(r) * a.sb_row + static_cast<uint64_t>(seg) * a.sb_col,
+                round_to_dtype(out_dtype, F::round(s32)));
+}
+
 template <class F, int kBits, int kEnc>
 __global__ __launch_bounds__(kThreads) void dequantize_transposed_kernel(TransposedArgs a) {
     using U = Unit<F, kBits>;
@@ -277,6 +302,18 @@ hipError_t launch_quantize_transposed(hipStream_t s, int dtype, int bits, bool d
         CQ_SWITCH_DTYPE(dtype, return (quantize_transposed<kF, 0>(s, bits, a)))
     }
     CQ_SWITCH_DTYPE(dtype, return (quantize_transposed<kF, 1>(s, bits, a)))
+}
+
+hipError_t launch_scales_transposed(hipStream_t s, int dtype, int out_dtype, const TransposedArgs& a) {
+    if (a.rows == 0 || a.segments == 0 || a.batches == 0) return hipSuccess;
+    QuantParams qp;
+    qp.lo = a.range.lo;
+    qp.hi = a.range.hi;
+    qp.width = a.range.hi - a.range.lo;
+    qp.rwidth = 1.0f / qp.width;  // IEEE division on the host: correctly rounded
+    CQ_SWITCH_DTYPE(dtype, hipLaunchKernelGGL((scales_transposed_kernel<kF>), grid_of(a), dim3(kThreads), 0, s, a,
+                                              out_dtype, qp);
+                    return hipGetLastError())
 }
 
 hipError_t launch_dequantize_transposed(hipStream_t s, int dtype, int bits, const TransposedArgs& a) {
