@@ -128,7 +128,13 @@ cq_status make_plan(const cq_scheme* s, const cq_tensor* floats, int dtype, cons
         if (floats->shape[d] != want) return CQ_ERR_SHAPE_MISMATCH;
         if (floats->shape[d] > 0xffffffffull) return CQ_ERR_TOO_LARGE;
     }
-    p->n = numel(floats);
+    p->n = 1;
+    for (uint32_t d = 0; d < p->rank; d++)
+        if (p->shape[d] == 0) p->n = 0;
+    for (uint32_t d = 0; d < p->rank && p->n != 0; d++) {
+        if (p->n > (1ull << 48) / p->shape[d]) return CQ_ERR_TOO_LARGE;  // far beyond any HBM; keeps products in 64 bits
+        p->n *= p->shape[d];
+    }
     if (p->n == 0) return CQ_OK;  // an empty tensor: the callers launch nothing
     std::memset(&p->vs, 0, sizeof(p->vs));
     p->vs.on = !is_contiguous(floats) || !is_contiguous(values);
@@ -398,8 +404,8 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     st = make_plan(scheme, input, input_dtype, output, scale, dtype_size(input_dtype), out_scale,
                    dtype_size(pd), &p);
     if (st != CQ_OK) return st;
-    if (p.n == 0) return CQ_OK;
     if (!out_scale) return CQ_ERR_INVALID_ARGUMENT;
+    if (p.n == 0) return CQ_OK;
 
     const bool native = scheme->store == CQ_STORE_NATIVE;
     const uint64_t per_chunk = 16 / dtype_size(input_dtype);

@@ -116,6 +116,14 @@ def test_into_contiguous_packed_checks():
     assert status(lambda: run(src=t((32, 2), 4, (1, 4)), dst=t((32, 2), 4), shape=(32, 16))) == _ffi.ERR_SHAPE_MISMATCH
 
 
+def test_element_counts_beyond_64_bit_products_are_refused():
+    scheme = QuantScheme.default().with_value(QuantValue.Q8S)
+    big = 1 << 31
+    x, out, one = t((big, big, 4), 4), t((big, big, 1), 4), t((1,), 4)
+    assert status(lambda: qz.launch_ref(CLIENT, x, out, one, one, scheme, ElemType.F32)) == _ffi.ERR_TOO_LARGE
+    assert status(lambda: dq.launch_ref(CLIENT, out, x, one, scheme, ElemType.F32)) == _ffi.ERR_TOO_LARGE
+
+
 def test_empty_tensors_are_a_no_op():
     """Zero elements: nothing to launch, success (shapes still have to agree)."""
     x, out, sc = t((0, 64), 4), t((0, 16), 4), t((0, 2), 4)

@@ -165,3 +165,18 @@ def test_reduce_random_shapes_axes_and_layouts(gpu, oracle, seed):
         for use_ws in (True, False):
             got, n_out = run(torch, gpu, x, elem, shape, axis, use_workspace=use_ws, in_strides=strides)
             assert np.array_equal(got[:n_out].view(np.uint8), want.view(np.uint8)), (shape, strides, axis, elem.name, use_ws)
+
+
+def test_reduce_over_an_empty_axis_writes_the_identity(gpu):
+    """No elements along the axis: every output is the identity of max-abs, 0."""
+    import torch
+
+    for elem in ELEMS:
+        dt = gpu.storage_dtype(elem)
+        din = torch.zeros(16, dtype=dt, device="cuda")
+        dout = torch.ones(32, dtype=dt, device="cuda")   # 1.0f / the bits 0x0001: anything but zero
+        hin = gpu.handle(din, (4, 0, 8), (8, 8, 1))
+        hout = gpu.handle(dout, (4, 1, 8), (8, 8, 1))
+        cq_reduce.max_abs(ComputeClient.current(), hin, hout, 1, elem, 0, 0)
+        torch.cuda.synchronize()
+        assert not dout.view(torch.uint8).any().item(), elem
