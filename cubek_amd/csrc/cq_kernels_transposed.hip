@@ -6,9 +6,15 @@
 // A wave holds 64 consecutive r of one block (or, per tensor, one 32-column segment): lane
 // l walks the block's columns for its own r, so every load or store of floats is one
 // contiguous run across the wave, and the abs-max of a block never leaves the thread.
-// A fused dynamic launch reads the block twice (abs-max, then quantize); the second read
-// finds the lines in cache.  Stored words are written / read per thread (a few words per
-// row and block, rows far apart): that side moves 1/4 - 1/16 of the bytes.
+// Column addresses are wave-uniform (scalar registers) plus a 32-bit lane offset.  Blocks of
+// up to 32 columns stay in registers between the abs-max and the quantize pass; blocks of 64
+// or 128 columns are shared by 2 or 4 lanes (quantize_transposed_quads_kernel); longer ones
+// are read twice, the second time from cache.  Stored words are written / read per thread (a
+// few words per row and block, rows far apart): that side moves 1/4 - 1/16 of the bytes.
+//
+// Kernels: quantize_transposed_kernel (given scales or fused abs-max), its variant
+// quantize_transposed_quads_kernel, scales_transposed_kernel (abs-max -> scale only),
+// dequantize_transposed_kernel.
 #include "cq_device.hpp"
 #include "cq_internal.hpp"
 
@@ -44,6 +50,46 @@ __device__ __forceinline__ BatchPos batch_pos(const TransposedArgs& a, uint32_t 
         p.sb += static_cast<uint64_t>(c) * a.batch_sb[d];
     }
     return p;
+}
+
+// A wave's place: 64 consecutive r (one per lane) of segment `seg`.  seg is the same for the whole
+// wave, and said so to the compiler, so that everything derived from it stays in scalar registers
+// and a float access is "scalar base + 32-bit lane offset" with no address arithmetic per lane.
+struct Lane {
+    uint32_t r, seg;
+    uint32_t byte;  // lane's offset from the wave's first r, in bytes
+    bool live;
+};
+template <class F>
+__device__ __forceinline__ Lane lane_of(const TransposedArgs& a) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    Lane t;
+    t.r = blockIdx.x * kWave + lane;
+    t.seg = __builtin_amdgcn_readfirstlane(blockIdx.y * kSegmentsPerGroup + threadIdx.x / kWave);
+    t.byte = lane * F::kBytes;
+    t.live = t.r < a.rows && t.seg < a.segments;
+    return t;
+}
+// A wave-uniform address handed over as a scalar value of its own (64-bit products come out of
+// the vector unit, and the compiler otherwise folds the lane offset into the base first and
+// computes every column's address per lane).  Rebuilt as a pointer into global memory, which it
+// is: a bare integer would become a flat pointer.
+__device__ __forceinline__ const char* scalar_address(const char* ptr) {
+    const uint64_t p = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(p));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(p >> 32));
+    typedef const char __attribute__((address_space(1))) * GlobalPtr;
+    return (const char*)(GlobalPtr)(static_cast<uint64_t>(hi) << 32 | lo);
+}
+// address of (first r of the wave, column c0) / of column c0 + c in the same rows
+template <class F>
+__device__ __forceinline__ const char* wave_base(const void* base, const TransposedArgs& a, uint64_t batch, uint32_t c0) {
+    return scalar_address(static_cast<const char*>(base) +
+                          (batch + static_cast<uint64_t>(blockIdx.x) * kWave + static_cast<uint64_t>(c0) * a.pitch_f) * F::kBytes);
+}
+template <class F>
+__device__ __forceinline__ const char* column(const char* base, const TransposedArgs& a, uint32_t c) {
+    return scalar_address(base + static_cast<uint64_t>(c) * a.pitch_f * F::kBytes);
 }
 
 // kCount consecutive words of one thread, as one 16- or 8-byte access when the address allows:
@@ -93,27 +139,70 @@ __device__ __forceinline__ void load_words(const uint32_t* src, uint32_t* w, uin
     for (int k = 0; k < kCount; k++) w[k] = static_cast<uint32_t>(k) < valid ? src[k] : 0u;
 }
 
+// 32 values of one row -> codes -> the piece's stored words
+template <class F, int kBits, bool kWide, int kEnc>
+__device__ __forceinline__ void quantize_piece_words(const float* v, float d, bool tame, const QuantParams& qp, uint32_t* pw) {
+    using U = Unit<F, kBits>;
+    constexpr int kN = U::kN;
+    constexpr uint32_t kPiece = 32;
+#pragma unroll
+    for (uint32_t u = 0; u < kPiece / U::kV; u++) {
+        uint32_t w[2] = {0, 0};
+#pragma unroll
+        for (int i = 0; i < U::kChunks; i++) {
+            float qn[kN];
+            quantize_values_neg<F, kN>(v + u * U::kV + i * kN, d, tame, qp.lo, qp.hi, qn);
+            uint32_t cw[2] = {0, 0};
+            if constexpr (kEnc == kEncInt)
+                pack_chunk_neg<kBits, kN, kWide>(qn, cw);
+            else
+                encode_chunk_neg<kEnc, kN>(qn, cw);
+            if constexpr (U::kChunks == 1) {
+                w[0] = cw[0];
+                w[1] = cw[1];
+            } else {
+                w[0] |= cw[0] << (i * kN * kBits);  // sub-word chunks, upper bits are zero
+            }
+        }
+        pw[u * U::kWords] = w[0];
+        if constexpr (U::kWords == 2) pw[u * U::kWords + 1] = w[1];
+    }
+}
+// ... and `valid` of them stored at `out`
+template <class F, int kBits, bool kWide, int kEnc>
+__device__ __forceinline__ void quantize_piece(const float* v, float d, bool tame, const QuantParams& qp, uint32_t* out,
+                                               uint32_t valid) {
+    constexpr int kPieceWords = 32 / Unit<F, kBits>::kNq;
+    uint32_t pw[kPieceWords];
+    quantize_piece_words<F, kBits, kWide, kEnc>(v, d, tame, qp, pw);
+    store_words<kPieceWords>(out, pw, valid);
+}
+
 // kScale: 0 dynamic (abs-max of the block), 1 given (scale_in typed scale_in_dtype)
 template <class F, int kBits, bool kWide, int kEnc, int kScale>
 __global__ __launch_bounds__(kThreads) void quantize_transposed_kernel(TransposedArgs a, QuantParams qp) {
     using U = Unit<F, kBits>;
-    constexpr int kN = U::kN;
-    const uint32_t r = blockIdx.x * kWave + (threadIdx.x & (kWave - 1));
-    const uint32_t seg = blockIdx.y * kSegmentsPerGroup + threadIdx.x / kWave;
-    if (r >= a.rows || seg >= a.segments) return;  // nothing below needs the whole wave
+    const Lane t = lane_of<F>(a);
+    if (!t.live) return;  // nothing below needs the whole wave
+    const uint32_t r = t.r, seg = t.seg;
     const BatchPos b = batch_pos(a, blockIdx.z);
     const uint32_t c0 = seg * a.segment;
-    const uint64_t f0 = b.f + r + static_cast<uint64_t>(c0) * a.pitch_f;
+    const char* in0 = wave_base<F>(a.input, a, b.f, c0);
 
     // a piece = up to 32 columns of the segment held in registers (32 loads in flight per lane)
     constexpr uint32_t kPiece = 32;
     static_assert(kPiece % U::kV == 0, "pieces hold whole units");
     float v[kPiece];
     const auto load_piece = [&](uint32_t c) {
+        if (c + kPiece <= a.segment) {
 #pragma unroll
-        for (uint32_t i = 0; i < kPiece; i++) {
-            v[i] = 0.0f;
-            if (c + i < a.segment) v[i] = F::load(a.input, f0 + static_cast<uint64_t>(c + i) * a.pitch_f);
+            for (uint32_t i = 0; i < kPiece; i++) v[i] = F::load(column<F>(in0, a, c + i) + t.byte, 0);
+        } else {
+#pragma unroll
+            for (uint32_t i = 0; i < kPiece; i++) {
+                v[i] = 0.0f;
+                if (c + i < a.segment) v[i] = F::load(column<F>(in0, a, c + i) + t.byte, 0);
+            }
         }
     };
     const bool single_piece = a.segment <= kPiece;  // then the abs-max pass and the quantize pass share the registers
@@ -148,51 +237,151 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_kernel(Transpose
     uint32_t* out = static_cast<uint32_t*>(a.output) + b.v + static_cast<uint64_t>(r) * a.vrow + c0 / U::kNq;
     for (uint32_t c = 0; c < a.segment; c += kPiece) {
         if (kScale != 0 || !single_piece) load_piece(c);  // a second read finds the lines in cache
-        constexpr int kPieceWords = kPiece / U::kNq;
-        uint32_t pw[kPieceWords];
-#pragma unroll
-        for (uint32_t u = 0; u < kPiece / U::kV; u++) {
-            uint32_t w[2] = {0, 0};
-#pragma unroll
-            for (int i = 0; i < U::kChunks; i++) {
-                float qn[kN];
-                quantize_values_neg<F, kN>(v + u * U::kV + i * kN, d, tame, qp.lo, qp.hi, qn);
-                uint32_t cw[2] = {0, 0};
-                if constexpr (kEnc == kEncInt)
-                    pack_chunk_neg<kBits, kN, kWide>(qn, cw);
-                else
-                    encode_chunk_neg<kEnc, kN>(qn, cw);
-                if constexpr (U::kChunks == 1) {
-                    w[0] = cw[0];
-                    w[1] = cw[1];
-                } else {
-                    w[0] |= cw[0] << (i * kN * kBits);  // sub-word chunks, upper bits are zero
-                }
-            }
-            pw[u * U::kWords] = w[0];
-            if constexpr (U::kWords == 2) pw[u * U::kWords + 1] = w[1];
-        }
         const uint32_t left = a.segment - c;
-        store_words<kPieceWords>(out + c / U::kNq, pw, left >= kPiece ? kPieceWords : left / U::kNq);
+        quantize_piece<F, kBits, kWide, kEnc>(v, d, tame, qp, out + c / U::kNq, left >= kPiece ? kPiece / U::kNq : left / U::kNq);
+    }
+}
+
+// Blocks of 64 or 128 columns: the lane-per-row kernel above would read them twice (abs-max, then
+// quantize, 32 columns at a time).  Here 2 or 4 neighbouring lanes share a block, 32 columns
+// each, and combine their maxima through DPP, so a block is read once and stays in registers.
+// To keep the float runs long with fewer lanes along r, a lane holds kR = 2 (f32) or 4 (16-bit
+// types) consecutive r through one 8-byte load: a wave covers 16 * kR rows by 128 columns, a
+// load instruction fetches four runs of 128 bytes, and the words of a row leave as one
+// contiguous run per quad of lanes.  Needs 8-byte aligned runs (base address, pitch, batch
+// strides), a row count that is a multiple of kR and 128 columns within 2 GiB of each other.
+template <class F>
+constexpr int kRowsPerLane = 8 / F::kBytes;
+constexpr int kQuad = 4;
+
+// element j of the kR a lane loaded together
+template <class F>
+__device__ __forceinline__ float lane_row(u32x2 raw, int j) {
+    if constexpr (F::kBytes == 4) {
+        return bits_f32(raw[j]);
+    } else {
+        const uint32_t w = raw[j >> 1];
+        if constexpr (F::kDtype == CQ_BF16) {
+            return bits_f32((j & 1) ? (w & 0xffff0000u) : (w << 16));
+        } else {
+            const f16x2 h = __builtin_bit_cast(f16x2, w);
+            return static_cast<float>(h[j & 1]);
+        }
+    }
+}
+
+// Eight words per lane (32 columns of 8-bit codes), four lanes side by side = 128 contiguous
+// bytes: written as two instructions of 64 contiguous bytes per quad instead of two of 4 x 16
+// scattered ones.  Piece q (16 bytes) of the run sits in lane q / 2, words 4 * (q % 2)...; in
+// instruction k lane s writes piece 4 k + s.  `run` is the quad's first word; all four lanes
+// of the quad are here.
+__device__ __forceinline__ void store_quad_run(uint32_t* run, const uint32_t* pw, uint32_t s) {
+    constexpr int kFrom01 = 0x50, kFrom23 = 0xfa;  // quad_perm [0,0,1,1] and [2,2,3,3]
+    const bool upper = (s & 1u) != 0;
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        u32x4 piece;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const uint32_t lo = k == 0 ? dpp<kFrom01>(pw[w]) : dpp<kFrom23>(pw[w]);
+            const uint32_t hi = k == 0 ? dpp<kFrom01>(pw[4 + w]) : dpp<kFrom23>(pw[4 + w]);
+            piece[w] = upper ? hi : lo;
+        }
+        *reinterpret_cast<u32x4*>(run + (4 * k + s) * 4) = piece;
+    }
+}
+
+template <class F, int kBits, bool kWide, int kEnc, int kScale>
+__global__ __launch_bounds__(kThreads) void quantize_transposed_quads_kernel(TransposedArgs a, QuantParams qp) {
+    using U = Unit<F, kBits>;
+    constexpr int kR = kRowsPerLane<F>;
+    constexpr uint32_t kPart = 32;                 // columns per lane
+    constexpr uint32_t kLaneRows = kWave / kQuad;  // lanes along r
+    constexpr uint32_t kPartWords = kPart / U::kNq;
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t s = lane & (kQuad - 1);
+    const uint32_t r0 = (blockIdx.x * kLaneRows + lane / kQuad) * kR;
+    // parts of 32 columns: the quad's first, the lane's own; a block is 2 or 4 parts, so the lanes of a block sit in one quad
+    const uint32_t part0 = __builtin_amdgcn_readfirstlane((blockIdx.y * kSegmentsPerGroup + threadIdx.x / kWave) * kQuad);
+    const uint32_t parts_per_block = a.segment / kPart;
+    const uint32_t parts = a.segments * parts_per_block;
+    if (r0 >= a.rows || part0 + s >= parts) return;  // rows is a multiple of kR: a lane's rows all exist
+    const bool whole_quad = part0 + kQuad <= parts;  // else blocks of two parts, and only the first is here
+    const uint32_t seg = (part0 + s) / parts_per_block;
+    const bool first_part = (s & (parts_per_block - 1)) == 0;
+    const BatchPos b = batch_pos(a, blockIdx.z);
+    const char* in0 = scalar_address(static_cast<const char*>(a.input) +
+                                     (b.f + static_cast<uint64_t>(blockIdx.x) * kLaneRows * kR +
+                                      static_cast<uint64_t>(part0) * kPart * a.pitch_f) * F::kBytes);
+    // the lane's own corner: its part's first column, its first r (below 2 GiB, the launcher checks)
+    const uint32_t corner = s * kPart * static_cast<uint32_t>(a.pitch_f) * F::kBytes + (lane / kQuad) * 8;
+
+    u32x2 raw[kPart];
+#pragma unroll
+    for (uint32_t i = 0; i < kPart; i++) raw[i] = *reinterpret_cast<const u32x2*>(column<F>(in0, a, i) + corner);
+
+    float d[kR];
+#pragma unroll
+    for (int j = 0; j < kR; j++) {
+        float s_f;
+        if constexpr (kScale == 0) {
+            float amax = 0.0f;
+#pragma unroll
+            for (uint32_t i = 0; i < kPart; i++) amax = fmaxf(amax, fabsf(lane_row<F>(raw[i], j)));  // NaN elements drop out
+            uint32_t bits = f32_bits(amax);  // non-negative floats order like their bits
+            bits = max(bits, dpp<kDppXor1>(bits));
+            if (parts_per_block == kQuad) bits = max(bits, dpp<kDppXor2>(bits));
+            amax = bits_f32(bits);
+            const float s32 = absmax_is_tame(amax) ? scale_from_absmax_tame(amax, qp) : scale_from_absmax(amax, qp.width);
+            s_f = F::round(s32);
+        } else {
+            s_f = load_dtype(a.scale_in_dtype, a.scale_in,
+                             b.sa + static_cast<uint64_t>(r0 + j) * a.sa_row + static_cast<uint64_t>(seg) * a.sa_col);
+        }
+        const float s_fs = round_to_dtype(a.param_dtype, s_f);  // write_scale (src/quantize.rs:83-98)
+        if (a.scale_out != nullptr && first_part)
+            store_dtype(a.param_dtype, a.scale_out,
+                        b.sb + static_cast<uint64_t>(r0 + j) * a.sb_row + static_cast<uint64_t>(seg) * a.sb_col, s_fs);
+        d[j] = F::round(s_fs);
+    }
+
+    uint32_t* run = static_cast<uint32_t*>(a.output) + b.v + static_cast<uint64_t>(r0) * a.vrow + part0 * kPartWords;
+#pragma unroll
+    for (int j = 0; j < kR; j++) {
+        float v[kPart];
+#pragma unroll
+        for (uint32_t i = 0; i < kPart; i++) v[i] = lane_row<F>(raw[i], j);
+        uint32_t pw[kPartWords];
+        quantize_piece_words<F, kBits, kWide, kEnc>(v, d[j], divisor_is_tame(d[j]), qp, pw);
+        uint32_t* row_run = run + j * a.vrow;
+        if (kPartWords == 8 && whole_quad && (reinterpret_cast<uintptr_t>(row_run) & 15u) == 0)
+            store_quad_run(row_run, pw, s);
+        else
+            store_words<kPartWords>(row_run + s * kPartWords, pw, kPartWords);
     }
 }
 
 // Block abs-max -> scale typed `out_dtype` (what cq_compute_scales produces), same mapping.
 template <class F>
 __global__ __launch_bounds__(kThreads) void scales_transposed_kernel(TransposedArgs a, int out_dtype, QuantParams qp) {
-    const uint32_t r = blockIdx.x * kWave + (threadIdx.x & (kWave - 1));
-    const uint32_t seg = blockIdx.y * kSegmentsPerGroup + threadIdx.x / kWave;
-    if (r >= a.rows || seg >= a.segments) return;
+    const Lane t = lane_of<F>(a);
+    if (!t.live) return;
+    const uint32_t r = t.r, seg = t.seg;
     const BatchPos b = batch_pos(a, blockIdx.z);
-    const uint64_t f0 = b.f + r + static_cast<uint64_t>(seg) * a.segment * a.pitch_f;
+    const char* in0 = wave_base<F>(a.input, a, b.f, seg * a.segment);
     constexpr uint32_t kPiece = 32;
     float amax = 0.0f;
     for (uint32_t c = 0; c < a.segment; c += kPiece) {
         float v[kPiece];
+        if (c + kPiece <= a.segment) {
 #pragma unroll
-        for (uint32_t i = 0; i < kPiece; i++) {
-            v[i] = 0.0f;
-            if (c + i < a.segment) v[i] = F::load(a.input, f0 + static_cast<uint64_t>(c + i) * a.pitch_f);
+            for (uint32_t i = 0; i < kPiece; i++) v[i] = F::load(column<F>(in0, a, c + i) + t.byte, 0);
+        } else {
+#pragma unroll
+            for (uint32_t i = 0; i < kPiece; i++) {
+                v[i] = 0.0f;
+                if (c + i < a.segment) v[i] = F::load(column<F>(in0, a, c + i) + t.byte, 0);
+            }
         }
 #pragma unroll
         for (uint32_t i = 0; i < kPiece; i++) amax = fmaxf(amax, fabsf(v[i]));  // NaN elements drop out
@@ -205,12 +394,12 @@ __global__ __launch_bounds__(kThreads) void scales_transposed_kernel(TransposedA
 template <class F, int kBits, int kEnc>
 __global__ __launch_bounds__(kThreads) void dequantize_transposed_kernel(TransposedArgs a) {
     using U = Unit<F, kBits>;
-    const uint32_t r = blockIdx.x * kWave + (threadIdx.x & (kWave - 1));
-    const uint32_t seg = blockIdx.y * kSegmentsPerGroup + threadIdx.x / kWave;
-    if (r >= a.rows || seg >= a.segments) return;
+    const Lane t = lane_of<F>(a);
+    if (!t.live) return;
+    const uint32_t r = t.r, seg = t.seg;
     const BatchPos b = batch_pos(a, blockIdx.z);
     const uint32_t c0 = seg * a.segment;
-    const uint64_t f0 = b.f + r + static_cast<uint64_t>(c0) * a.pitch_f;
+    char* out0 = const_cast<char*>(wave_base<F>(a.output, a, b.f, c0));
     const uint64_t si = a.tensor_level ? 0 : b.sa + static_cast<uint64_t>(r) * a.sa_row + static_cast<uint64_t>(seg) * a.sa_col;
     const float s = F::round(load_dtype(a.param_dtype, a.scale_in, si));  // Line::cast_from(scale)
     const uint32_t* in = static_cast<const uint32_t*>(a.input) + b.v + static_cast<uint64_t>(r) * a.vrow + c0 / U::kNq;
@@ -228,7 +417,7 @@ __global__ __launch_bounds__(kThreads) void dequantize_transposed_kernel(Transpo
             decode_fields<kEnc, kBits, U::kNq>(w[k], y);
 #pragma unroll
             for (uint32_t i = 0; i < U::kNq; i++)
-                F::store(a.output, f0 + static_cast<uint64_t>(c + k * U::kNq + i) * a.pitch_f, s * y[i]);  // store rounds to F
+                F::store(const_cast<char*>(column<F>(out0, a, c + k * U::kNq + i)) + t.byte, 0, s * y[i]);  // store rounds to F
         }
     }
 }
@@ -253,10 +442,30 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
     qp.width = a.range.hi - a.range.lo;
     qp.rwidth = 1.0f / qp.width;  // IEEE division on the host: correctly rounded
     const bool wide = a.range.hi > 127.0f || a.range.lo < -128.0f;
-#define CQ_LAUNCH(B, W, E)                                                                                       \
-    {                                                                                                            \
-        hipLaunchKernelGGL((quantize_transposed_kernel<F, B, W, E, kScale>), grid_of(a), dim3(kThreads), 0, s, a, qp); \
-        return hipGetLastError();                                                                                \
+    // blocks of 64 or 128 columns on 8-byte aligned runs: the kernel whose lanes share a block
+    constexpr uint32_t kR = kRowsPerLane<F>;
+    bool quads = !a.tensor_level && (a.segment == 64 || a.segment == 128) && a.rows % kR == 0 &&
+                 (reinterpret_cast<uintptr_t>(a.input) & 7u) == 0 && (a.pitch_f * F::kBytes) % 8 == 0 &&
+                 a.pitch_f * F::kBytes * 128 < (1ull << 31);
+    for (uint32_t k = 0; k < a.num_batch_dims; k++) quads = quads && (a.batch_f[k] * F::kBytes) % 8 == 0;
+    dim3 grid = grid_of(a);
+    if (quads) {
+        constexpr uint32_t kWaveRows = kWave / kQuad * kR;
+        const uint32_t parts = a.segments * (a.segment / 32);
+        grid.x = (a.rows + kWaveRows - 1) / kWaveRows;
+        grid.y = (parts + kQuad * kSegmentsPerGroup - 1) / (kQuad * kSegmentsPerGroup);
+        if (grid.y > 65535) {
+            quads = false;
+            grid = grid_of(a);
+        }
+    }
+#define CQ_LAUNCH(B, W, E)                                                                                        \
+    {                                                                                                             \
+        if (quads)                                                                                                \
+            hipLaunchKernelGGL((quantize_transposed_quads_kernel<F, B, W, E, kScale>), grid, dim3(kThreads), 0, s, a, qp); \
+        else                                                                                                      \
+            hipLaunchKernelGGL((quantize_transposed_kernel<F, B, W, E, kScale>), grid, dim3(kThreads), 0, s, a, qp); \
+        return hipGetLastError();                                                                                 \
     }
     switch (a.encoding) {
         case kEncInt:

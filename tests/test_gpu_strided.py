@@ -87,6 +87,11 @@ SCHEMES = [
     ("e4m3_native_tensor", QuantScheme.default().with_value(QuantValue.E4M3).with_store(QuantStore.Native)),
     ("e2m1_native_block32", QuantScheme.default().with_value(QuantValue.E2M1).with_store(QuantStore.Native)
      .with_level(QuantLevel.block([32]))),
+    # blocks of 64 / 128 columns: on transposed floats, lanes share a block
+    ("q8s_block64", QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([64]))),
+    ("q4s_block128", QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([128]))),
+    ("e4m3_native_block64", QuantScheme.default().with_value(QuantValue.E4M3).with_store(QuantStore.Native)
+     .with_level(QuantLevel.block([64]))),
 ]
 
 
@@ -100,7 +105,9 @@ def test_strided_value_tensors(gpu, oracle, elem, name, scheme):
     per = scheme.num_quants()
     stored_np = np.uint32 if scheme.store == QuantStore.U32 else np.uint8
     pe = gpu.param_elem(scheme)
-    for shape in ((6, 64), (2, 4, 96), (3, 70, 128)):
+    for shape in ((6, 64), (2, 4, 96), (3, 70, 128), (2, 72, 256)):
+        if scheme.level.block_size is not None and shape[-1] % scheme.level.block_size.dims[-1]:
+            continue
         pshape, cases = layouts(shape, per)
         sshape = scheme.scales_shape(shape)
         for case, fstr, vstr in cases:
