@@ -92,6 +92,18 @@ __device__ __forceinline__ const char* column(const char* base, const Transposed
     return scalar_address(base + static_cast<uint64_t>(c) * a.pitch_f * F::kBytes);
 }
 
+// f32 value -> the bits of an element of F (rounded to nearest even)
+template <class F>
+__device__ __forceinline__ uint32_t element_bits(float v) {
+    if constexpr (F::kBytes == 4) {
+        return f32_bits(v);
+    } else if constexpr (F::kDtype == CQ_BF16) {
+        return BF16::pack2(v, 0.0f) & 0xffffu;
+    } else {
+        return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, F16::narrow(v)));
+    }
+}
+
 // kCount consecutive words of one thread, as one 16- or 8-byte access when the address allows:
 // threads of a wave sit in different rows, so every access is a transaction of its own.
 template <int kCount>
@@ -242,14 +254,18 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_kernel(Transpose
     }
 }
 
-// Blocks of 64 or 128 columns: the lane-per-row kernel above would read them twice (abs-max, then
-// quantize, 32 columns at a time).  Here 2 or 4 neighbouring lanes share a block, 32 columns
-// each, and combine their maxima through DPP, so a block is read once and stays in registers.
+// Quads of lanes, for 8-byte aligned runs.  Blocks of 64 or 128 columns: the lane-per-row kernel
+// above would read them twice (abs-max, then quantize, 32 columns at a time); here 2 or 4
+// neighbouring lanes share a block, 32 columns each, and combine their maxima through DPP, so a
+// block is read once and stays in registers.  Blocks of 32 columns: four neighbouring lanes hold
+// four neighbouring blocks of the same rows, so the words and scales of a row leave as one
+// contiguous run per quad (64 bytes of 4-bit codes, 16 bytes of f32 scales) and the memory
+// system sees a quarter of the store requests.
 // To keep the float runs long with fewer lanes along r, a lane holds kR = 2 (f32) or 4 (16-bit
-// types) consecutive r through one 8-byte load: a wave covers 16 * kR rows by 128 columns, a
-// load instruction fetches four runs of 128 bytes, and the words of a row leave as one
-// contiguous run per quad of lanes.  Needs 8-byte aligned runs (base address, pitch, batch
-// strides), a row count that is a multiple of kR and 128 columns within 2 GiB of each other.
+// types) consecutive r through one 8-byte load: a wave covers 16 * kR rows by 128 columns and a
+// load instruction fetches four runs of 128 bytes.  Needs 8-byte aligned runs (base address,
+// pitch, batch strides), a row count that is a multiple of kR and 128 columns within 2 GiB of
+// each other.
 template <class F>
 constexpr int kRowsPerLane = 8 / F::kBytes;
 constexpr int kQuad = 4;
@@ -301,7 +317,7 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_quads_kernel(Tra
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t s = lane & (kQuad - 1);
     const uint32_t r0 = (blockIdx.x * kLaneRows + lane / kQuad) * kR;
-    // parts of 32 columns: the quad's first, the lane's own; a block is 2 or 4 parts, so the lanes of a block sit in one quad
+    // parts of 32 columns: the quad's first, the lane's own; a block is 1, 2 or 4 parts, so the lanes of a block sit in one quad
     const uint32_t part0 = __builtin_amdgcn_readfirstlane((blockIdx.y * kSegmentsPerGroup + threadIdx.x / kWave) * kQuad);
     const uint32_t parts_per_block = a.segment / kPart;
     const uint32_t parts = a.segments * parts_per_block;
@@ -329,19 +345,24 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_quads_kernel(Tra
 #pragma unroll
             for (uint32_t i = 0; i < kPart; i++) amax = fmaxf(amax, fabsf(lane_row<F>(raw[i], j)));  // NaN elements drop out
             uint32_t bits = f32_bits(amax);  // non-negative floats order like their bits
-            bits = max(bits, dpp<kDppXor1>(bits));
-            if (parts_per_block == kQuad) bits = max(bits, dpp<kDppXor2>(bits));
+            if (parts_per_block >= 2) bits = max(bits, dpp<kDppXor1>(bits));
+            if (parts_per_block >= kQuad) bits = max(bits, dpp<kDppXor2>(bits));
             amax = bits_f32(bits);
             const float s32 = absmax_is_tame(amax) ? scale_from_absmax_tame(amax, qp) : scale_from_absmax(amax, qp.width);
             s_f = F::round(s32);
         } else {
-            s_f = load_dtype(a.scale_in_dtype, a.scale_in,
-                             b.sa + static_cast<uint64_t>(r0 + j) * a.sa_row + static_cast<uint64_t>(seg) * a.sa_col);
+            const uint64_t si = a.tensor_level ? 0 : b.sa + static_cast<uint64_t>(r0 + j) * a.sa_row + static_cast<uint64_t>(seg) * a.sa_col;
+            s_f = load_dtype(a.scale_in_dtype, a.scale_in, si);
         }
         const float s_fs = round_to_dtype(a.param_dtype, s_f);  // write_scale (src/quantize.rs:83-98)
-        if (a.scale_out != nullptr && first_part)
-            store_dtype(a.param_dtype, a.scale_out,
-                        b.sb + static_cast<uint64_t>(r0 + j) * a.sb_row + static_cast<uint64_t>(seg) * a.sb_col, s_fs);
+        if (a.scale_out != nullptr && first_part) {
+            if (a.tensor_level) {
+                if (b.first && r0 + j == 0 && part0 + s == 0) store_dtype(a.param_dtype, a.scale_out, 0, s_fs);
+            } else {
+                store_dtype(a.param_dtype, a.scale_out,
+                            b.sb + static_cast<uint64_t>(r0 + j) * a.sb_row + static_cast<uint64_t>(seg) * a.sb_col, s_fs);
+            }
+        }
         d[j] = F::round(s_fs);
     }
 
@@ -422,6 +443,58 @@ __global__ __launch_bounds__(kThreads) void dequantize_transposed_kernel(Transpo
     }
 }
 
+// Dequantize on 8-byte aligned runs.  The 2-byte stores of the lane-per-row kernel reach memory
+// through the L2 in no particular order, which holds a tensor that does not sit in the Infinity
+// Cache at half the HBM rate; here a lane writes its kR consecutive r of a column as one 8-byte
+// non-temporal store (a run of 512 bytes per wave and column) and walks 32 columns.  With 4-bit
+// codes, inputs and outputs rotated out of the cache: bf16 [8192, 8192] 32 us against 44 us,
+// [28672, 8192] 138 us against 150 us.  Blocks of any multiple of 32 columns, or per tensor.
+template <class F, int kBits, int kEnc>
+__global__ __launch_bounds__(kThreads) void dequantize_transposed_wide_kernel(TransposedArgs a) {
+    using U = Unit<F, kBits>;
+    constexpr int kR = kRowsPerLane<F>;
+    constexpr uint32_t kPart = 32;
+    constexpr uint32_t kPartWords = kPart / U::kNq;
+    constexpr int kPerWord = 4 / F::kBytes;  // elements of F per 32-bit word of the 8-byte store
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t r0 = (blockIdx.x * kWave + lane) * kR;
+    const uint32_t part = __builtin_amdgcn_readfirstlane(blockIdx.y * kSegmentsPerGroup + threadIdx.x / kWave);  // 32 columns
+    const uint32_t parts_per_block = a.segment / kPart;
+    if (r0 >= a.rows || part >= a.segments * parts_per_block) return;  // rows is a multiple of kR: a lane's rows all exist
+    const uint32_t seg = part / parts_per_block;
+    const BatchPos b = batch_pos(a, blockIdx.z);
+    const char* out0 = scalar_address(static_cast<const char*>(a.output) +
+                                      (b.f + static_cast<uint64_t>(blockIdx.x) * kWave * kR +
+                                       static_cast<uint64_t>(part) * kPart * a.pitch_f) * F::kBytes);
+
+    uint32_t w[kR][kPartWords];
+    float sc[kR];
+    const uint32_t* in = static_cast<const uint32_t*>(a.input) + b.v + static_cast<uint64_t>(r0) * a.vrow + part * kPartWords;
+#pragma unroll
+    for (int j = 0; j < kR; j++) {
+        load_words<kPartWords>(in + j * a.vrow, w[j], kPartWords);
+        const uint64_t si = a.tensor_level ? 0 : b.sa + static_cast<uint64_t>(r0 + j) * a.sa_row + static_cast<uint64_t>(seg) * a.sa_col;
+        sc[j] = F::round(load_dtype(a.param_dtype, a.scale_in, si));  // Line::cast_from(scale)
+    }
+    u32x2 raw[kPart];
+#pragma unroll
+    for (uint32_t i = 0; i < kPart; i++) raw[i] = u32x2{0u, 0u};
+#pragma unroll
+    for (int j = 0; j < kR; j++) {
+#pragma unroll
+        for (uint32_t k = 0; k < kPartWords; k++) {
+            float y[U::kNq];
+            decode_fields<kEnc, kBits, U::kNq>(w[j][k], y);
+#pragma unroll
+            for (uint32_t i = 0; i < U::kNq; i++)
+                raw[k * U::kNq + i][j / kPerWord] |= element_bits<F>(sc[j] * y[i]) << (32 / kPerWord * (j % kPerWord));
+        }
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < kPart; i++)
+        stream_store(raw[i], reinterpret_cast<u32x2*>(const_cast<char*>(column<F>(out0, a, i)) + lane * 8));
+}
+
 #define CQ_SWITCH_DTYPE(D, ...)                              \
     switch (D) {                                             \
         case CQ_F32: { using kF = F32; __VA_ARGS__; }        \
@@ -434,6 +507,13 @@ inline dim3 grid_of(const TransposedArgs& a) {
     return dim3((a.rows + kWave - 1) / kWave, (a.segments + kSegmentsPerGroup - 1) / kSegmentsPerGroup, a.batches);
 }
 
+// 8-byte runs along r for the kernels that hold kR rows per lane
+template <class F>
+bool runs_of_8_bytes(const TransposedArgs& a, const void* floats) {
+    bool ok = a.rows % kRowsPerLane<F> == 0 && (reinterpret_cast<uintptr_t>(floats) & 7u) == 0 && (a.pitch_f * F::kBytes) % 8 == 0;
+    for (uint32_t k = 0; k < a.num_batch_dims; k++) ok = ok && (a.batch_f[k] * F::kBytes) % 8 == 0;
+    return ok;
+}
 template <class F, int kScale>
 hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a) {
     QuantParams qp;
@@ -442,23 +522,18 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
     qp.width = a.range.hi - a.range.lo;
     qp.rwidth = 1.0f / qp.width;  // IEEE division on the host: correctly rounded
     const bool wide = a.range.hi > 127.0f || a.range.lo < -128.0f;
-    // blocks of 64 or 128 columns on 8-byte aligned runs: the kernel whose lanes share a block
-    constexpr uint32_t kR = kRowsPerLane<F>;
-    bool quads = !a.tensor_level && (a.segment == 64 || a.segment == 128) && a.rows % kR == 0 &&
-                 (reinterpret_cast<uintptr_t>(a.input) & 7u) == 0 && (a.pitch_f * F::kBytes) % 8 == 0 &&
-                 a.pitch_f * F::kBytes * 128 < (1ull << 31);
-    for (uint32_t k = 0; k < a.num_batch_dims; k++) quads = quads && (a.batch_f[k] * F::kBytes) % 8 == 0;
+    // Quads of lanes wherever the runs are 8-byte aligned: blocks of 64 / 128 columns are read once
+    // instead of twice, blocks of 32 cost a quarter of the store requests (4-bit codes of a transposed
+    // bf16 view [28672, 8192]: 161 us against 214 us; when the tensor sits in the Infinity Cache the
+    // lane-per-row kernel is up to 10 % faster, which is given up).  A fused per-tensor launch does
+    // not exist: that scale comes from the two-pass reduction.
+    constexpr uint32_t kWaveRows = kWave / kQuad * kRowsPerLane<F>;
+    const uint32_t parts = a.segments * (a.segment / 32);
     dim3 grid = grid_of(a);
-    if (quads) {
-        constexpr uint32_t kWaveRows = kWave / kQuad * kR;
-        const uint32_t parts = a.segments * (a.segment / 32);
-        grid.x = (a.rows + kWaveRows - 1) / kWaveRows;
-        grid.y = (parts + kQuad * kSegmentsPerGroup - 1) / (kQuad * kSegmentsPerGroup);
-        if (grid.y > 65535) {
-            quads = false;
-            grid = grid_of(a);
-        }
-    }
+    bool quads = (kScale == 1 || !a.tensor_level) && runs_of_8_bytes<F>(a, a.input) &&
+                 (a.segment == 32 || a.segment == 64 || a.segment == 128) &&
+                 a.pitch_f * F::kBytes * 128 < (1ull << 31) && (parts + 15) / 16 <= 65535;
+    if (quads) grid = dim3((a.rows + kWaveRows - 1) / kWaveRows, (parts + 15) / 16, a.batches);
 #define CQ_LAUNCH(B, W, E)                                                                                        \
     {                                                                                                             \
         if (quads)                                                                                                \
@@ -484,9 +559,20 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
 
 template <class F>
 hipError_t dequantize_transposed(hipStream_t s, int bits, const TransposedArgs& a) {
+    constexpr uint32_t kWaveRows = kWave * kRowsPerLane<F>;
+    const uint64_t parts = static_cast<uint64_t>(a.segments) * (a.segment / 32);
+    dim3 grid = grid_of(a);
+    const bool wide_rows = a.segment % 32 == 0 && runs_of_8_bytes<F>(a, a.output) &&
+                           (parts + kSegmentsPerGroup - 1) / kSegmentsPerGroup <= 65535;
+    if (wide_rows)
+        grid = dim3((a.rows + kWaveRows - 1) / kWaveRows, static_cast<uint32_t>((parts + kSegmentsPerGroup - 1) / kSegmentsPerGroup),
+                    a.batches);
 #define CQ_LAUNCH(B, E)                                                                                       \
     {                                                                                                         \
-        hipLaunchKernelGGL((dequantize_transposed_kernel<F, B, E>), grid_of(a), dim3(kThreads), 0, s, a);     \
+        if (wide_rows)                                                                                        \
+            hipLaunchKernelGGL((dequantize_transposed_wide_kernel<F, B, E>), grid, dim3(kThreads), 0, s, a);  \
+        else                                                                                                  \
+            hipLaunchKernelGGL((dequantize_transposed_kernel<F, B, E>), grid, dim3(kThreads), 0, s, a);       \
         return hipGetLastError();                                                                             \
     }
     switch (a.encoding) {

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 from numpy.lib.stride_tricks import as_strided
 
-from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantScheme, QuantStore, QuantValue)
+from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantScheme, QuantStore, QuantValue, TensorHandleRef)
 from cubek_amd import dequantize as dq
 from cubek_amd import quantize as qz
 
@@ -170,3 +170,63 @@ def test_strided_value_tensors(gpu, oracle, elem, name, scheme):
             mask = np.ones(got.size, dtype=bool)
             view(mask, shape, fstr)[...] = False
             assert np.all(got[mask] == fill), tag + ("dequantize wrote outside the view",)
+
+
+@pytest.mark.parametrize("elem,rows,cols", [(ElemType.BF16, 12288, 8192), (ElemType.F32, 6144, 8192)],
+                         ids=["bf16", "f32"])
+def test_large_transposed_floats_match_the_contiguous_path(gpu, elem, rows, cols):
+    """A transposed float tensor of 192 MiB (grids of thousands of workgroups, offsets beyond
+    32 bits in bytes): codes, scales and dequantized values must equal what the contiguous
+    kernels, checked against the oracle elsewhere, give for the same logical tensor."""
+    import torch
+
+    client = ComputeClient.current()
+    tdt = torch.float32 if elem == ElemType.F32 else torch.bfloat16
+    eb = 4 if elem == ElemType.F32 else 2
+    g = torch.Generator(device="cuda")
+    g.manual_seed(rows + int(elem))
+    x = torch.randn((rows, cols), generator=g, device="cuda", dtype=torch.float32).mul_(0.05).to(tdt)
+    x[5, 7] = -0.0
+    xt = x.t().contiguous()                      # memory [cols, rows]
+    h = TensorHandleRef.from_torch
+    h_x = h(x)
+    h_xt = TensorHandleRef(h(xt).handle, (rows, cols), (1, rows), eb)
+    for name, scheme in (("q4s_block32", QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([32]))),
+                         ("q8s_tensor", QuantScheme.default().with_value(QuantValue.Q8S)),
+                         ("e4m3_native_block32", QuantScheme.default().with_value(QuantValue.E4M3)
+                          .with_store(QuantStore.Native).with_level(QuantLevel.block([32])))):
+        print(name, elem.name, flush=True)
+        native = scheme.store == QuantStore.Native
+        pshape = scheme.packed_shape((rows, cols)) if not native else (rows, cols)
+        sshape = scheme.scales_shape((rows, cols))
+        ws, nbytes = gpu.workspace(scheme, rows * cols)
+        outs = []
+        for hx in (h_x, h_xt):
+            codes = torch.full(pshape, 0x5A, dtype=torch.uint8 if native else torch.int32, device="cuda")
+            scales = torch.zeros(sshape, dtype=torch.float32, device="cuda")
+            qz.launch_dynamic(client, hx, h(codes), h(scales), scheme, elem, ws.data_ptr(), nbytes)
+            outs.append((codes, scales))
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0][0], outs[1][0]), (name, "codes")
+        assert torch.equal(outs[0][1].view(torch.int32), outs[1][1].view(torch.int32)), (name, "scales")
+        # given scales (the launch_ref form), transposed input
+        codes2 = torch.zeros_like(outs[0][0])
+        os2 = torch.zeros_like(outs[0][1])
+        s_in = outs[0][1].to(tdt)
+        qz.launch_ref(client, h_xt, h(codes2), h(s_in), h(os2), scheme, elem)
+        codes3 = torch.zeros_like(outs[0][0])
+        os3 = torch.zeros_like(outs[0][1])
+        qz.launch_ref(client, h_x, h(codes3), h(s_in), h(os3), scheme, elem)
+        torch.cuda.synchronize()
+        assert torch.equal(codes2, codes3), (name, "codes, given scales")
+        assert torch.equal(os2.view(torch.int32), os3.view(torch.int32)), (name, "out_scale, given scales")
+        # dequantize into a transposed and into a contiguous tensor
+        y = torch.empty_like(x)
+        yt = torch.empty_like(xt)
+        dq.launch_ref(client, h(outs[0][0]), h(y), h(outs[0][1]), scheme, elem)
+        dq.launch_ref(client, h(outs[0][0]), TensorHandleRef(h(yt).handle, (rows, cols), (1, rows), eb), h(outs[0][1]),
+                      scheme, elem)
+        torch.cuda.synchronize()
+        bits = torch.int32 if elem == ElemType.F32 else torch.int16
+        assert torch.equal(yt.t().contiguous().view(bits), y.view(bits)), (name, "dequantize")
+        del outs, codes2, codes3, y, yt
