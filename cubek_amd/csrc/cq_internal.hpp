@@ -166,6 +166,7 @@ struct TransposedArgs {
     uint64_t vrow;           // stored stride of the second to last dimension, in 32-bit words
     uint64_t sa_row, sa_col, sb_row, sb_col;  // scale strides along the two dimensions
     uint32_t num_batch_dims;
+    uint32_t staged;         // quads kernel, set by its launcher: 1 words, 2 scales leave through LDS as whole runs
     uint32_t batch_shape[CQ_MAX_RANK];
     uint64_t batch_f[CQ_MAX_RANK], batch_v[CQ_MAX_RANK], batch_sa[CQ_MAX_RANK], batch_sb[CQ_MAX_RANK];
 };

@@ -258,9 +258,11 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_kernel(Transpose
 // above would read them twice (abs-max, then quantize, 32 columns at a time); here 2 or 4
 // neighbouring lanes share a block, 32 columns each, and combine their maxima through DPP, so a
 // block is read once and stays in registers.  Blocks of 32 columns: four neighbouring lanes hold
-// four neighbouring blocks of the same rows, so the words and scales of a row leave as one
-// contiguous run per quad (64 bytes of 4-bit codes, 16 bytes of f32 scales) and the memory
-// system sees a quarter of the store requests.
+// four neighbouring blocks of the same rows, so the words and scales of a row sit side by side.
+// The four waves of a workgroup sit side by side along the columns too and hand their words and
+// f32 scales over through LDS, from where a tile's rows leave as whole runs (256 bytes of 4-bit
+// codes, 64 bytes of scales per row) rather than one request per lane; outputs that are not
+// 16-byte aligned are stored by each quad for itself.
 // To keep the float runs long with fewer lanes along r, a lane holds kR = 2 (f32) or 4 (16-bit
 // types) consecutive r through one 8-byte load: a wave covers 16 * kR rows by 128 columns and a
 // load instruction fetches four runs of 128 bytes.  Needs 8-byte aligned runs (base address,
@@ -314,71 +316,117 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_quads_kernel(Tra
     constexpr uint32_t kPart = 32;                 // columns per lane
     constexpr uint32_t kLaneRows = kWave / kQuad;  // lanes along r
     constexpr uint32_t kPartWords = kPart / U::kNq;
+    // the workgroup's tile: its four waves sit side by side along the columns
+    constexpr uint32_t kTileRows = kLaneRows * kR;
+    constexpr uint32_t kTileParts = kQuad * kSegmentsPerGroup;
+    constexpr uint32_t kRowWords = kTileParts * kPartWords;
+    constexpr uint32_t kRowPitch = kRowWords + 4;  // rows start four banks apart
+    __shared__ __attribute__((aligned(16))) uint32_t lds_words[kTileRows * kRowPitch];
+    __shared__ uint32_t lds_scales[kTileRows * kTileParts];
+
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t s = lane & (kQuad - 1);
-    const uint32_t r0 = (blockIdx.x * kLaneRows + lane / kQuad) * kR;
-    // parts of 32 columns: the quad's first, the lane's own; a block is 1, 2 or 4 parts, so the lanes of a block sit in one quad
-    const uint32_t part0 = __builtin_amdgcn_readfirstlane((blockIdx.y * kSegmentsPerGroup + threadIdx.x / kWave) * kQuad);
+    const uint32_t lr = lane / kQuad;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t r0 = (blockIdx.x * kLaneRows + lr) * kR;
+    // parts of 32 columns: the tile's first, the quad's first, the lane's own; a block is 1, 2 or 4
+    // parts, so the lanes of a block sit in one quad
+    const uint32_t tile_part0 = blockIdx.y * kTileParts;
+    const uint32_t part0 = tile_part0 + wave * kQuad;
     const uint32_t parts_per_block = a.segment / kPart;
     const uint32_t parts = a.segments * parts_per_block;
-    if (r0 >= a.rows || part0 + s >= parts) return;  // rows is a multiple of kR: a lane's rows all exist
-    const bool whole_quad = part0 + kQuad <= parts;  // else blocks of two parts, and only the first is here
-    const uint32_t seg = (part0 + s) / parts_per_block;
-    const bool first_part = (s & (parts_per_block - 1)) == 0;
     const BatchPos b = batch_pos(a, blockIdx.z);
-    const char* in0 = scalar_address(static_cast<const char*>(a.input) +
-                                     (b.f + static_cast<uint64_t>(blockIdx.x) * kLaneRows * kR +
-                                      static_cast<uint64_t>(part0) * kPart * a.pitch_f) * F::kBytes);
-    // the lane's own corner: its part's first column, its first r (below 2 GiB, the launcher checks)
-    const uint32_t corner = s * kPart * static_cast<uint32_t>(a.pitch_f) * F::kBytes + (lane / kQuad) * 8;
+    if (r0 < a.rows && part0 + s < parts) {  // rows is a multiple of kR: a lane's rows all exist
+        const bool whole_quad = part0 + kQuad <= parts;  // else blocks of two parts, and only the first is here
+        const uint32_t seg = (part0 + s) / parts_per_block;
+        const bool first_part = (s & (parts_per_block - 1)) == 0;
+        const char* in0 = scalar_address(static_cast<const char*>(a.input) +
+                                         (b.f + static_cast<uint64_t>(blockIdx.x) * kLaneRows * kR +
+                                          static_cast<uint64_t>(part0) * kPart * a.pitch_f) * F::kBytes);
+        // the lane's own corner: its part's first column, its first r (below 2 GiB, the launcher checks)
+        const uint32_t corner = s * kPart * static_cast<uint32_t>(a.pitch_f) * F::kBytes + lr * 8;
 
-    u32x2 raw[kPart];
+        u32x2 raw[kPart];
 #pragma unroll
-    for (uint32_t i = 0; i < kPart; i++) raw[i] = *reinterpret_cast<const u32x2*>(column<F>(in0, a, i) + corner);
+        for (uint32_t i = 0; i < kPart; i++) raw[i] = *reinterpret_cast<const u32x2*>(column<F>(in0, a, i) + corner);
 
-    float d[kR];
+        float d[kR];
 #pragma unroll
-    for (int j = 0; j < kR; j++) {
-        float s_f;
-        if constexpr (kScale == 0) {
-            float amax = 0.0f;
+        for (int j = 0; j < kR; j++) {
+            float s_f;
+            if constexpr (kScale == 0) {
+                float amax = 0.0f;
 #pragma unroll
-            for (uint32_t i = 0; i < kPart; i++) amax = fmaxf(amax, fabsf(lane_row<F>(raw[i], j)));  // NaN elements drop out
-            uint32_t bits = f32_bits(amax);  // non-negative floats order like their bits
-            if (parts_per_block >= 2) bits = max(bits, dpp<kDppXor1>(bits));
-            if (parts_per_block >= kQuad) bits = max(bits, dpp<kDppXor2>(bits));
-            amax = bits_f32(bits);
-            const float s32 = absmax_is_tame(amax) ? scale_from_absmax_tame(amax, qp) : scale_from_absmax(amax, qp.width);
-            s_f = F::round(s32);
-        } else {
-            const uint64_t si = a.tensor_level ? 0 : b.sa + static_cast<uint64_t>(r0 + j) * a.sa_row + static_cast<uint64_t>(seg) * a.sa_col;
-            s_f = load_dtype(a.scale_in_dtype, a.scale_in, si);
-        }
-        const float s_fs = round_to_dtype(a.param_dtype, s_f);  // write_scale (src/quantize.rs:83-98)
-        if (a.scale_out != nullptr && first_part) {
-            if (a.tensor_level) {
-                if (b.first && r0 + j == 0 && part0 + s == 0) store_dtype(a.param_dtype, a.scale_out, 0, s_fs);
+                for (uint32_t i = 0; i < kPart; i++) amax = fmaxf(amax, fabsf(lane_row<F>(raw[i], j)));  // NaN elements drop out
+                uint32_t bits = f32_bits(amax);  // non-negative floats order like their bits
+                if (parts_per_block >= 2) bits = max(bits, dpp<kDppXor1>(bits));
+                if (parts_per_block >= kQuad) bits = max(bits, dpp<kDppXor2>(bits));
+                amax = bits_f32(bits);
+                const float s32 = absmax_is_tame(amax) ? scale_from_absmax_tame(amax, qp) : scale_from_absmax(amax, qp.width);
+                s_f = F::round(s32);
             } else {
-                store_dtype(a.param_dtype, a.scale_out,
-                            b.sb + static_cast<uint64_t>(r0 + j) * a.sb_row + static_cast<uint64_t>(seg) * a.sb_col, s_fs);
+                const uint64_t si = a.tensor_level ? 0 : b.sa + static_cast<uint64_t>(r0 + j) * a.sa_row + static_cast<uint64_t>(seg) * a.sa_col;
+                s_f = load_dtype(a.scale_in_dtype, a.scale_in, si);
             }
+            const float s_fs = round_to_dtype(a.param_dtype, s_f);  // write_scale (src/quantize.rs:83-98)
+            if (a.scale_out != nullptr && first_part) {
+                if (a.tensor_level) {
+                    if (b.first && r0 + j == 0 && part0 + s == 0) store_dtype(a.param_dtype, a.scale_out, 0, s_fs);
+                } else if (a.staged & 2u) {
+                    lds_scales[(lr * kR + j) * kTileParts + (wave * kQuad + s) / parts_per_block] = f32_bits(s_fs);
+                } else {
+                    store_dtype(a.param_dtype, a.scale_out,
+                                b.sb + static_cast<uint64_t>(r0 + j) * a.sb_row + static_cast<uint64_t>(seg) * a.sb_col, s_fs);
+                }
+            }
+            d[j] = F::round(s_fs);
         }
-        d[j] = F::round(s_fs);
-    }
 
-    uint32_t* run = static_cast<uint32_t*>(a.output) + b.v + static_cast<uint64_t>(r0) * a.vrow + part0 * kPartWords;
+        uint32_t* run = static_cast<uint32_t*>(a.output) + b.v + static_cast<uint64_t>(r0) * a.vrow + part0 * kPartWords;
 #pragma unroll
-    for (int j = 0; j < kR; j++) {
-        float v[kPart];
+        for (int j = 0; j < kR; j++) {
+            float v[kPart];
 #pragma unroll
-        for (uint32_t i = 0; i < kPart; i++) v[i] = lane_row<F>(raw[i], j);
-        uint32_t pw[kPartWords];
-        quantize_piece_words<F, kBits, kWide, kEnc>(v, d[j], divisor_is_tame(d[j]), qp, pw);
-        uint32_t* row_run = run + j * a.vrow;
-        if (kPartWords == 8 && whole_quad && (reinterpret_cast<uintptr_t>(row_run) & 15u) == 0)
-            store_quad_run(row_run, pw, s);
-        else
-            store_words<kPartWords>(row_run + s * kPartWords, pw, kPartWords);
+            for (uint32_t i = 0; i < kPart; i++) v[i] = lane_row<F>(raw[i], j);
+            uint32_t pw[kPartWords];
+            quantize_piece_words<F, kBits, kWide, kEnc>(v, d[j], divisor_is_tame(d[j]), qp, pw);
+            uint32_t* row_run = run + j * a.vrow;
+            if (a.staged & 1u)
+                store_words<kPartWords>(&lds_words[(lr * kR + j) * kRowPitch + (wave * kQuad + s) * kPartWords], pw, kPartWords);
+            else if (kPartWords == 8 && whole_quad && (reinterpret_cast<uintptr_t>(row_run) & 15u) == 0)
+                store_quad_run(row_run, pw, s);
+            else
+                store_words<kPartWords>(row_run + s * kPartWords, pw, kPartWords);
+        }
+    }
+    if (a.staged == 0) return;  // the same for every thread of the launch
+
+    // the tile's words and scales leave as whole rows of the tile: 16-byte pieces side by side
+    __syncthreads();
+    const uint32_t tile_r0 = blockIdx.x * kTileRows;
+    const uint32_t rows_here = a.rows - tile_r0 < kTileRows ? a.rows - tile_r0 : kTileRows;
+    if (a.staged & 1u) {
+        const uint32_t words_here = (parts - tile_part0) * kPartWords < kRowWords ? (parts - tile_part0) * kPartWords : kRowWords;
+        uint32_t* tile_out = static_cast<uint32_t*>(a.output) + b.v + static_cast<uint64_t>(tile_r0) * a.vrow + tile_part0 * kPartWords;
+#pragma unroll
+        for (uint32_t idx = threadIdx.x; idx < kTileRows * (kRowWords / 4); idx += kThreads) {
+            const uint32_t row = idx / (kRowWords / 4), q = idx % (kRowWords / 4);
+            if (row < rows_here && q * 4 < words_here)  // the launcher checked: rows hold a multiple of four words
+                stream_store(*reinterpret_cast<const u32x4*>(&lds_words[row * kRowPitch + q * 4]),
+                             reinterpret_cast<u32x4*>(tile_out + static_cast<uint64_t>(row) * a.vrow + q * 4));
+        }
+    }
+    if (a.staged & 2u) {
+        const uint32_t tile_seg0 = tile_part0 / parts_per_block;
+        const uint32_t tile_segs = kTileParts / parts_per_block;
+        const uint32_t segs_here = a.segments - tile_seg0 < tile_segs ? a.segments - tile_seg0 : tile_segs;
+        float* tile_scales = static_cast<float*>(a.scale_out) + b.sb + tile_seg0;  // f32, contiguous along the blocks of a row
+#pragma unroll
+        for (uint32_t idx = threadIdx.x; idx < kTileRows * kTileParts; idx += kThreads) {
+            const uint32_t row = idx / kTileParts, i = idx % kTileParts;
+            if (row < rows_here && i < segs_here)
+                tile_scales[static_cast<uint64_t>(tile_r0 + row) * a.sb_row + i] = bits_f32(lds_scales[row * kTileParts + i]);
+        }
     }
 }
 
@@ -533,11 +581,20 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
     bool quads = (kScale == 1 || !a.tensor_level) && runs_of_8_bytes<F>(a, a.input) &&
                  (a.segment == 32 || a.segment == 64 || a.segment == 128) &&
                  a.pitch_f * F::kBytes * 128 < (1ull << 31) && (parts + 15) / 16 <= 65535;
-    if (quads) grid = dim3((a.rows + kWaveRows - 1) / kWaveRows, (parts + 15) / 16, a.batches);
+    TransposedArgs q = a;
+    if (quads) {
+        grid = dim3((a.rows + kWaveRows - 1) / kWaveRows, (parts + 15) / 16, a.batches);
+        // words and scales through LDS when their runs can be written as 16-byte / 4-byte pieces side by side
+        const uint32_t row_words = a.segments * a.segment / (32u / static_cast<uint32_t>(bits));
+        bool words = (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0 && a.vrow % 4 == 0 && row_words % 4 == 0;
+        for (uint32_t k = 0; k < a.num_batch_dims; k++) words = words && a.batch_v[k] % 4 == 0;
+        const bool scales = a.scale_out != nullptr && !a.tensor_level && a.param_dtype == CQ_F32 && a.sb_col == 1;
+        q.staged = (words ? 1u : 0u) | (scales ? 2u : 0u);
+    }
 #define CQ_LAUNCH(B, W, E)                                                                                        \
     {                                                                                                             \
         if (quads)                                                                                                \
-            hipLaunchKernelGGL((quantize_transposed_quads_kernel<F, B, W, E, kScale>), grid, dim3(kThreads), 0, s, a, qp); \
+            hipLaunchKernelGGL((quantize_transposed_quads_kernel<F, B, W, E, kScale>), grid, dim3(kThreads), 0, s, q, qp); \
         else                                                                                                      \
             hipLaunchKernelGGL((quantize_transposed_kernel<F, B, W, E, kScale>), grid, dim3(kThreads), 0, s, a, qp); \
         return hipGetLastError();                                                                                 \
