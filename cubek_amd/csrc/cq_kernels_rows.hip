@@ -401,31 +401,37 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
     }
 }
 
-// Per-tensor abs-max, pass 1, over strided rows: gridDim.x <= kMaxPartials workgroups
-// stride over the (row tile, chunk tile) pairs; one f32 partial per workgroup.
+// Per-tensor abs-max, pass 1, over strided rows: gridDim.x <= kMaxPartials workgroups of 1024
+// threads stride over the (row tile, chunk tile) pairs; one f32 partial per workgroup.  A
+// maximum does not mind seeing an element twice: indices beyond the end are clamped to the
+// last tile / row / chunk instead of guarding every load.
+constexpr int kAbsmaxThreads = 1024;
 template <class F>
-__global__ __launch_bounds__(kThreads) void absmax_rows_kernel(RowArgs a, float* __restrict__ partials,
-                                                               uint32_t row_tiles, uint32_t col_tiles) {
+__global__ __launch_bounds__(kAbsmaxThreads) void absmax_rows_kernel(RowArgs a, float* __restrict__ partials,
+                                                                     uint32_t row_tiles, uint32_t col_tiles) {
     constexpr int kN = F::kPerChunk;
-    __shared__ float lds[kThreads / kWave];
+    __shared__ float lds[kAbsmaxThreads / kWave];
     const int last = static_cast<int>(a.rank) - 1;
     const uint32_t tj = 1u << a.tj_log2;
     const uint32_t chunks_per_row = a.shape[last] / kN;
+    const uint32_t last_row = static_cast<uint32_t>(a.rows - 1);
     const u32x4* in = static_cast<const u32x4*>(a.input);
     constexpr int kUnroll = 4;  // tiles in flight per thread
-    const uint64_t tiles = static_cast<uint64_t>(row_tiles) * col_tiles;
+    const uint32_t tiles = row_tiles * col_tiles;  // the launcher keeps it below 2^32
     float amax = 0.0f;
-    for (uint64_t t0 = blockIdx.x; t0 < tiles; t0 += static_cast<uint64_t>(gridDim.x) * kUnroll) {
+    for (uint32_t t0 = blockIdx.x; t0 < tiles; t0 += gridDim.x * kUnroll) {
         u32x4 raw[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
-            const uint64_t t = t0 + static_cast<uint64_t>(u) * gridDim.x;
-            const uint32_t rt = static_cast<uint32_t>(t / col_tiles), ct = static_cast<uint32_t>(t % col_tiles);
-            const uint32_t row = rt * (kThreads >> a.tj_log2) + (threadIdx.x >> a.tj_log2);
-            const uint32_t jc = ct * tj + (threadIdx.x & (tj - 1));
+            uint32_t t = t0 + u * gridDim.x;
+            t = t < tiles ? t : tiles - 1;
+            const uint32_t rt = t / col_tiles, ct = t - rt * col_tiles;
+            uint32_t row = rt * (kAbsmaxThreads >> a.tj_log2) + (threadIdx.x >> a.tj_log2);
+            uint32_t jc = ct * tj + (threadIdx.x & (tj - 1));
+            row = row < last_row ? row : last_row;
+            jc = jc < chunks_per_row ? jc : chunks_per_row - 1;
             const RowPos r = row_pos(a, row);
-            raw[u] = u32x4{0, 0, 0, 0};
-            if (t < tiles && r.live && jc < chunks_per_row) raw[u] = stream_load(in + r.f / kN + jc);
+            raw[u] = stream_load(in + r.f / kN + jc);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
@@ -439,7 +445,7 @@ __global__ __launch_bounds__(kThreads) void absmax_rows_kernel(RowArgs a, float*
     if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = amax;
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < kThreads / kWave; w++) amax = fmaxf(amax, lds[w]);
+        for (int w = 1; w < kAbsmaxThreads / kWave; w++) amax = fmaxf(amax, lds[w]);
         partials[blockIdx.x] = amax;
     }
 }
@@ -676,13 +682,14 @@ hipError_t launch_absmax_partials_rows(hipStream_t s, int dtype, const RowArgs& 
     const uint32_t per_chunk = dtype == CQ_F32 ? 4 : 8;
     const uint32_t chunks_per_row = a.shape[a.rank - 1] / per_chunk;
     a.tj_log2 = lanes_log2(chunks_per_row);
-    const uint32_t tr = kThreads >> a.tj_log2;
+    const uint32_t tr = kAbsmaxThreads >> a.tj_log2;
     const uint32_t row_tiles = static_cast<uint32_t>((a.rows + tr - 1) / tr);
     const uint32_t col_tiles = (chunks_per_row + (1u << a.tj_log2) - 1) >> a.tj_log2;
     const uint64_t tiles = static_cast<uint64_t>(row_tiles) * col_tiles;
+    if (tiles >= (1ull << 32)) return hipErrorInvalidValue;  // cannot happen below 2^48 elements: a tile holds 4096 of them or more
     const uint32_t grid = static_cast<uint32_t>(tiles < 1 ? 1 : (tiles > kMaxPartials ? kMaxPartials : tiles));
     *num_partials = grid;
-    CQ_SWITCH_DTYPE(dtype, hipLaunchKernelGGL((absmax_rows_kernel<kF>), dim3(grid), dim3(kThreads), 0, s, a, partials,
+    CQ_SWITCH_DTYPE(dtype, hipLaunchKernelGGL((absmax_rows_kernel<kF>), dim3(grid), dim3(kAbsmaxThreads), 0, s, a, partials,
                                               row_tiles, col_tiles);
                     return hipGetLastError())
 }
