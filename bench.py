@@ -188,13 +188,13 @@ def cpu_baseline(torch, w, path, budget_s=12.0):
             return xs.cpu().numpy()
         return xs.view(torch.int16).cpu().numpy().view(np.uint16)
 
-    def run(nrows):
+    def run(nrows, nthreads=threads):
         xs = host_rows(nrows)
         shape = (nrows, cols)
         scales = oracle.compute_scales(xs, elem, shape, path.scheme)  # not timed: the reference takes scales as input
         t0 = time.perf_counter()
-        words, out_scale = oracle.quantize(xs, elem, shape, scales, path.scheme, threads=threads)
-        oracle.dequantize(words, shape, out_scale, elem, path.scheme, threads=threads)
+        words, out_scale = oracle.quantize(xs, elem, shape, scales, path.scheme, threads=nthreads)
+        oracle.dequantize(words, shape, out_scale, elem, path.scheme, threads=nthreads)
         return time.perf_counter() - t0
 
     probe_rows = max(threads, min(rows, (1 << 21) // cols))
@@ -203,11 +203,17 @@ def cpu_baseline(torch, w, path, budget_s=12.0):
     nrows = max(threads, nrows // threads * threads)
     t = min(run(nrows) for _ in range(3 if nrows == rows else 1))
     sample_bytes = 2 * algorithmic_bytes(dict(w, shape=(nrows, cols)))
+    # the same on one thread, on a sample an eighth as long
+    rows1 = max(1, nrows // 8)
+    t1 = run(rows1, 1)
+    bytes1 = 2 * algorithmic_bytes(dict(w, shape=(rows1, cols)))
     return {
         "value": sample_bytes / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
         "sample": f"first {nrows} of {rows} rows of the headline tensor ({nrows * cols} elements), "
                   f"quantize with given scales + dequantize, {t:.2f} s on {threads} threads",
         "elements_per_s": nrows * cols / t,
+        "one_thread": {"value": round(bytes1 / t1 / 1e9, 3), "unit": "GB/s", "cores": 1,
+                       "sample": f"first {rows1} rows, {t1:.2f} s"},
     }
 
 
