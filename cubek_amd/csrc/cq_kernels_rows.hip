@@ -233,12 +233,9 @@ __global__ __launch_bounds__(kThreads) void scales_rows_kernel(RowArgs a, int ou
 // several block rows into one tile.  The abs-max meets across the chunk columns of a
 // block by DPP (power-of-two widths; other widths use only the lanes that hold whole
 // blocks and meet in LDS) and across the phases in LDS.
-// kPipeline (tall tiles): as many workgroups as the GPU holds at once walk the tiles
-// with a stride of gridDim.x and load tile i+1 before they work on tile i, so every
-// wave has loads in flight while it computes, whatever the other workgroups of its CU
-// are doing (one-shot workgroups of equal length fall into step, all loading and then
-// all computing: 53 us against 40 us on 128 x 128 blocks of a bf16 [8192, 8192]).
-// Flat tiles (one or two rows per thread) are cheaper as one workgroup per tile.
+// One workgroup per tile.  (A persistent variant that loaded tile i+1 before working on tile i
+// was slower at every block shape: 44 us against 39-41 us on 128 x 128 blocks of a bf16
+// [8192, 8192], 144 us against 129 us on [28672, 8192].)
 template <int kLog2>
 __device__ __forceinline__ float group_max_log2(float v, uint32_t log2) {
     if constexpr (kLog2 > 5) {
@@ -256,11 +253,11 @@ struct BlocksGeom {
     uint32_t num_block_rows, col_groups, tiles;
 };
 
-template <class F, int kBits, bool kWide, int kEnc, int kRows, int kCols, bool kPipeline>
+template <class F, int kBits, bool kWide, int kEnc, int kRows, int kCols>
 __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, BlocksGeom g, QuantParams qp) {
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;
-    __shared__ float lds[2][kCols][kThreads];
+    __shared__ float lds[kCols][kThreads];
     const int last = static_cast<int>(a.rank) - 1;
     const uint32_t tj = 1u << g.tj_log2;
     const uint32_t ph = threadIdx.x >> g.tj_log2, jl = threadIdx.x & (tj - 1);
@@ -303,24 +300,10 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
         }
     };
 
-    Pos pos = locate(blockIdx.x);
+    const Pos pos = locate(blockIdx.x);
     u32x4 raw[kCols][kRows];
     load(pos, raw);
-    uint32_t buf = 0;
-    for (uint32_t t = blockIdx.x; t < g.tiles; t += gridDim.x, buf ^= 1) {  // the same trip count for the whole workgroup
-        Pos next_pos = pos;
-        u32x4 next_raw[kPipeline ? kCols : 1][kPipeline ? kRows : 1];
-        if constexpr (kPipeline) {
-#pragma unroll
-            for (int c = 0; c < kCols; c++)
-#pragma unroll
-                for (int k = 0; k < kRows; k++) next_raw[c][k] = u32x4{0, 0, 0, 0};
-            if (t + gridDim.x < g.tiles) {
-                next_pos = locate(t + gridDim.x);
-                load(next_pos, next_raw);
-            }
-        }
-
+    {
         float amax[kCols];
 #pragma unroll
         for (int c = 0; c < kCols; c++) {
@@ -333,11 +316,9 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
                 for (int i = 0; i < kN; i++) amax[c] = fmaxf(amax[c], fabsf(v[i]));  // NaN elements drop out
             }
             amax[c] = group_max_log2<0>(amax[c], g.cpb_log2);  // over the chunk columns of a power-of-two block
-            lds[buf][c][threadIdx.x] = amax[c];
+            lds[c][threadIdx.x] = amax[c];
         }
-        // LDS writes done, then the barrier; no wait for the global loads in flight.  The two LDS
-        // buffers alternate, so one barrier per tile orders everything.
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        __syncthreads();
 
 #pragma unroll
         for (int c = 0; c < kCols; c++) {
@@ -351,7 +332,7 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
             if (bsub < g.per_group)  // phases beyond the last whole block row hold nothing
                 for (uint32_t p = 0; p < g.ph_per_block; p++)
                     for (uint32_t k = 0; k < entries; k++)
-                        amax[c] = fmaxf(amax[c], lds[buf][c][((bsub * g.ph_per_block + p) << g.tj_log2) + lane0 + k]);
+                        amax[c] = fmaxf(amax[c], lds[c][((bsub * g.ph_per_block + p) << g.tj_log2) + lane0 + k]);
             const float s32 =
                 absmax_is_tame(amax[c]) ? scale_from_absmax_tame(amax[c], qp) : scale_from_absmax(amax[c], qp.width);
             const float s_fs = round_to_dtype(a.param_dtype, F::round(s32));
@@ -390,13 +371,6 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
                     if (row_live && sub == 0) stream_store(word, dst + jc / kLanesPerWord);
                 }
             }
-        }
-        if constexpr (kPipeline) {
-            pos = next_pos;
-#pragma unroll
-            for (int c = 0; c < kCols; c++)
-#pragma unroll
-                for (int k = 0; k < kRows; k++) raw[c][k] = next_raw[c][k];
         }
     }
 }
@@ -570,24 +544,8 @@ bool blocks_geom(uint32_t per_chunk, uint32_t bits, const RowArgs& a, BlocksGeom
 
 template <class F, int kBits, bool kWide, int kEnc, int kRows, int kCols>
 hipError_t quantize_blocks_variant(hipStream_t s, const RowArgs& a, const BlocksGeom& g, const QuantParams& qp) {
-    constexpr bool kPipeline = kRows >= 4;
-    auto kernel = quantize_blocks_kernel<F, kBits, kWide, kEnc, kRows, kCols, kPipeline>;
-    uint32_t grid = g.tiles;
-    if constexpr (kPipeline) {
-        // workgroups of this kernel the GPU holds at once (a property of the code object and the
-        // device model, looked up once)
-        static const uint32_t resident = [&] {
-            int per_cu = 0, cus = 0, dev = 0;
-            if (hipGetDevice(&dev) != hipSuccess ||
-                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-                hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, 0) != hipSuccess ||
-                per_cu <= 0 || cus <= 0)
-                return 768u;
-            return static_cast<uint32_t>(per_cu) * static_cast<uint32_t>(cus);
-        }();
-        if (grid > resident) grid = resident;
-    }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, a, g, qp);
+    hipLaunchKernelGGL((quantize_blocks_kernel<F, kBits, kWide, kEnc, kRows, kCols>), dim3(g.tiles), dim3(kThreads), 0, s, a,
+                       g, qp);
     return hipGetLastError();
 }
 
