@@ -192,6 +192,66 @@ bool flat_ok(const Plan& p, int dtype, const cq_tensor* floats, const cq_tensor*
     return cq::flat_block_supported(dtype, p.block_last);
 }
 
+// Rows of a tensor as the flat kernels take them: the last dimension contiguous, everything
+// in front of it one uniform run of rows `*pitch` elements apart (pitched, sliced along the
+// last dimension; 0 when there is a single row).
+bool uniform_rows(const cq_tensor* t, uint64_t* rows, uint64_t* pitch) {
+    const uint32_t last = t->rank - 1;
+    if (t->shape[last] != 1 && t->strides[last] != 1) return false;
+    *rows = 1;
+    *pitch = 0;
+    uint64_t expect = 0;
+    for (int d = static_cast<int>(last) - 1; d >= 0; d--) {
+        if (t->shape[d] == 1) continue;
+        if (expect == 0) {
+            *pitch = t->strides[d];
+        } else if (t->strides[d] != expect) {
+            return false;
+        }
+        expect = t->strides[d] * t->shape[d];
+        *rows *= t->shape[d];
+    }
+    return true;
+}
+
+// Can the flat kernels take this launch row by row?  (value tensors with a contiguous last
+// dimension and a uniform row pitch, rows long enough to fill their tiles, no ragged row end,
+// 1-D blocks that map onto lane groups, scales with a contiguous last dimension.)  Fills the
+// row fields of `a` and a.num_chunks = chunks per row.
+bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
+                  const cq_tensor* scale_a, uint32_t scale_a_size, const cq_tensor* scale_b, uint32_t scale_b_size,
+                  cq::FlatArgs* a) {
+    if (p.rank < 2) return false;
+    const uint32_t last = p.rank - 1;
+    const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
+    const uint32_t stored = s->store == CQ_STORE_U32 ? 4u : 1u;
+    uint64_t rows_f, rows_v, pitch_f, pitch_v;
+    if (!uniform_rows(floats, &rows_f, &pitch_f) || !uniform_rows(values, &rows_v, &pitch_v) || rows_f != rows_v) return false;
+    if (!aligned(floats->ptr, 16) || !aligned(values->ptr, 8) || (pitch_f * elem) % 16 || (pitch_v * stored) % 8) return false;
+    const uint64_t cols = p.shape[last];
+    const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+    if (cols == 0 || cols % chunk_elems) return false;
+    const uint64_t row_chunks = cols / per_chunk;
+    if (row_chunks < 2048 && row_chunks % 1024) return false;  // tiles of up to 1024 chunks: little of a row's last one idle
+    if (rows_f > 65535ull * 65535ull) return false;
+    a->scale_in_pitch = a->scale_out_pitch = 0;
+    if (!p.tensor_level) {
+        if (!p.last_dim_blocks || !cq::flat_block_supported(dtype, p.block_last)) return false;
+        uint64_t rows_s, pitch_s;
+        if (!uniform_rows(scale_a, &rows_s, &pitch_s) || rows_s != rows_f) return false;
+        a->scale_in_pitch = pitch_s * scale_a_size;
+        if (scale_b) {
+            if (!uniform_rows(scale_b, &rows_s, &pitch_s) || rows_s != rows_f) return false;
+            a->scale_out_pitch = pitch_s * scale_b_size;
+        }
+    }
+    a->rows = rows_f;
+    a->num_chunks = row_chunks;
+    a->in_pitch = pitch_f * elem;      // quantize: floats in, stored out; dequantize swaps them
+    a->out_pitch = pitch_v * stored;
+    return true;
+}
+
 // Stored encoding of the flat kernels (cq::Encoding) and the field width they see.
 int flat_encoding(const cq_scheme* s) {
     if (s->store == CQ_STORE_U32) return 0;
@@ -428,6 +488,20 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         if (st != CQ_OK) return st;
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
+    cq::FlatArgs fr{};
+    if (flat_words == 0 && flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
+                                        dtype_size(pd), &fr)) {
+        fr.input = input->ptr;
+        fr.output = output->ptr;
+        fr.scale_in = scale->ptr;
+        fr.scale_in_dtype = input_dtype;
+        fr.scale_out = out_scale->ptr;
+        fr.block = p.tensor_level ? 0 : p.block_last;
+        fr.param_dtype = pd;
+        fr.encoding = flat_encoding(scheme);
+        fr.range = p.range;
+        return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, fr));
+    }
     cq::RowArgs r;
     if (flat_words == 0 && rows_args(p, scheme, input_dtype, input, output, &r)) {
         r.input = input->ptr;
@@ -489,6 +563,20 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         if (st != CQ_OK) return st;
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
+    cq::FlatArgs fr{};
+    if (flat_words == 0 && flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, &fr)) {
+        fr.input = values->ptr;
+        fr.output = output->ptr;
+        fr.scale_in = params->ptr;
+        const uint64_t floats_pitch = fr.in_pitch;  // the float tensor is the output here
+        fr.in_pitch = fr.out_pitch;
+        fr.out_pitch = floats_pitch;
+        fr.block = p.tensor_level ? 0 : p.block_last;
+        fr.param_dtype = pd;
+        fr.encoding = flat_encoding(scheme);
+        fr.range = p.range;
+        return hip_status(cq::launch_dequantize_flat(stream, output_dtype, p.bits, fr));
+    }
     cq::RowArgs r;
     if (flat_words == 0 && rows_args(p, scheme, output_dtype, output, values, &r)) {
         r.input = values->ptr;
@@ -518,33 +606,38 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
 
 // Shared by cq_compute_scales and cq_quantize_dynamic: scale of every block (or
 // of the tensor) as out_dtype(F(2*absmax/(hi-lo))), written into `scales`.
+// Pass 1 of the per-tensor reduction for any layout of the float tensor: `*num_partials` f32
+// abs-max partials in the workspace.
+static cq_status absmax_partials(cq_stream_t stream, const Plan& p, const cq_scheme* scheme, const cq_tensor* input,
+                                 int input_dtype, void* workspace, size_t workspace_bytes, uint32_t* num_partials) {
+    if (!workspace || workspace_bytes < cq::kMaxPartials * sizeof(float)) return CQ_ERR_WORKSPACE_TOO_SMALL;
+    if (!aligned(workspace, 4)) return CQ_ERR_INVALID_ARGUMENT;
+    cq::RowArgs r;
+    if (p.vs.on && is_dense_permutation(input)) {
+        // the order does not matter for a maximum: read the buffer front to back
+        return hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n, static_cast<float*>(workspace),
+                                                     num_partials));
+    }
+    if (p.vs.on && rows_args(p, scheme, input_dtype, input, nullptr, &r)) {
+        r.input = input->ptr;
+        return hip_status(cq::launch_absmax_partials_rows(stream, input_dtype, r, static_cast<float*>(workspace), num_partials));
+    }
+    if (p.vs.on) {
+        cq::GenericArgs g = generic_args(p, scheme);
+        g.input = input->ptr;
+        return hip_status(cq::launch_absmax_partials_strided(stream, input_dtype, g, p.n, static_cast<float*>(workspace),
+                                                             num_partials));
+    }
+    return hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n, static_cast<float*>(workspace),
+                                                 num_partials));
+}
+
 static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_scheme* scheme,
                                 const cq_tensor* input, int input_dtype, const cq_tensor* scales,
                                 int out_dtype, void* workspace, size_t workspace_bytes) {
     if (p.tensor_level) {
-        if (!workspace || workspace_bytes < cq::kMaxPartials * sizeof(float))
-            return CQ_ERR_WORKSPACE_TOO_SMALL;
-        if (!aligned(workspace, 4)) return CQ_ERR_INVALID_ARGUMENT;
         uint32_t num_partials = 0;
-        cq_status st;
-        cq::RowArgs r;
-        if (p.vs.on && is_dense_permutation(input)) {
-            // the order does not matter for a maximum: read the buffer front to back
-            st = hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n,
-                                                       static_cast<float*>(workspace), &num_partials));
-        } else if (p.vs.on && rows_args(p, scheme, input_dtype, input, nullptr, &r)) {
-            r.input = input->ptr;
-            st = hip_status(cq::launch_absmax_partials_rows(stream, input_dtype, r, static_cast<float*>(workspace),
-                                                            &num_partials));
-        } else if (p.vs.on) {
-            cq::GenericArgs g = generic_args(p, scheme);
-            g.input = input->ptr;
-            st = hip_status(cq::launch_absmax_partials_strided(stream, input_dtype, g, p.n,
-                                                               static_cast<float*>(workspace), &num_partials));
-        } else {
-            st = hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n,
-                                                       static_cast<float*>(workspace), &num_partials));
-        }
+        const cq_status st = absmax_partials(stream, p, scheme, input, input_dtype, workspace, workspace_bytes, &num_partials);
         if (st != CQ_OK) return st;
         return hip_status(cq::launch_tensor_scale(stream, input_dtype, out_dtype,
                                                   static_cast<const float*>(workspace), num_partials,
@@ -633,6 +726,21 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
     }
 
+    // pitched rows with 1-D blocks: the same fused kernel, row by row
+    cq::FlatArgs fr{};
+    if (!p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, &fr)) {
+        fr.input = input->ptr;
+        fr.output = output->ptr;
+        fr.scale_out = out_scale->ptr;
+        fr.scale_out_pitch = fr.scale_in_pitch;  // the only scale tensor of this call is the output
+        fr.scale_in_pitch = 0;
+        fr.block = p.block_last;
+        fr.param_dtype = pd;
+        fr.encoding = flat_encoding(scheme);
+        fr.range = p.range;
+        return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, fr));
+    }
+
     // blocks over the last two dimensions (or 1-D blocks on layouts the flat kernel refuses): one
     // launch that owns whole blocks
     cq::RowArgs rb;
@@ -680,6 +788,21 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, a));
         if (st != CQ_OK) return st;
         flat_words = flat_chunks * per_chunk / p.nq;
+    } else if (p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, &fr)) {
+        // per tensor on pitched rows: the same two passes, the second one row by row
+        uint32_t num_partials = 0;
+        st = absmax_partials(stream, p, scheme, input, input_dtype, workspace, workspace_bytes, &num_partials);
+        if (st != CQ_OK) return st;
+        fr.input = input->ptr;
+        fr.output = output->ptr;
+        fr.scale_in = workspace;
+        fr.num_partials = num_partials;
+        fr.scale_out = out_scale->ptr;
+        fr.block = 0;
+        fr.param_dtype = pd;
+        fr.encoding = flat_encoding(scheme);
+        fr.range = p.range;
+        return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, fr));
     } else {
         // scales as FS(F(scale)) into out_scale first, then quantize reading them back
         // (the divisor F(FS(scale)) is the same either way)

@@ -33,7 +33,10 @@ struct FlatArgs {
     int scale_in_dtype;   // cq_dtype of scale_in (quantize only)
     void* scale_out;      // quantize: out_scale typed as param dtype, NULL = do not write;
                           // launch_scales_flat: scales typed like the input
-    uint64_t num_chunks;  // 16-byte chunks of the float tensor handled by this launch
+    uint64_t num_chunks;  // 16-byte chunks of the float tensor handled by this launch (per row when rows > 1)
+    // rows > 1: the launch covers `rows` runs of num_chunks chunks whose starts lie this many bytes apart in
+    // the four tensors (pitched rows); 0 or 1: one contiguous run
+    uint64_t rows, in_pitch, out_pitch, scale_in_pitch, scale_out_pitch;
     uint32_t block;       // elements per block, 0 = per-tensor
     int param_dtype;      // cq_dtype of the stored scales
     int encoding;         // 0 two's-complement fields (U32 store, native i8); 1 e4m3, 2 e5m2 bytes; 3 e2m1 nibbles

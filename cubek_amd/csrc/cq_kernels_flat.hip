@@ -1,151 +1,11 @@
-// Launchers of the flat (contiguous) quantize / dequantize kernels: map
-// (dtype, bits, block size, param dtype) onto the kernel templates of
-// cq_kernels_flat.hpp and pick the launch shape.
-#include "cq_internal.hpp"
-#include "cq_kernels_flat.hpp"
+// Launchers of the flat (contiguous) kernels: quantize with the scale produced in the launch
+// (fused abs-max, or pass 2 of the per-tensor reduction), block scales, the per-tensor abs-max.
+// Quantize with given scales and dequantize are in cq_kernels_flat_given.hip and
+// cq_kernels_flat_dequantize.hip.
+#include "cq_kernels_flat_launch.hpp"
 
 namespace cq {
 namespace {
-
-constexpr int kThreads = 256;
-
-inline uint32_t grid_for(uint64_t num_chunks, int unroll) {
-    uint64_t per = static_cast<uint64_t>(kThreads) * unroll;
-    return static_cast<uint32_t>((num_chunks + per - 1) / per);
-}
-
-int group_of(int dtype, uint32_t block) {
-    if (block == 0) return 0;
-    uint32_t per_chunk = dtype == CQ_F32 ? 4u : 8u;
-    if (block % per_chunk) return -1;
-    uint32_t g = block / per_chunk;
-    if (g & (g - 1)) return -1;
-    return g <= 32 ? static_cast<int>(g) : -1;
-}
-
-// Launch shapes from a sweep on MI355X (batches of back-to-back launches,
-// 117 MB - 470 MB tensors): quantize is best with four 16-byte loads in flight
-// per lane; dequantize, which is store-dominated, with two 16-byte stores per lane
-// for 16-bit outputs.  For f32 outputs the best depth follows the share of reads:
-// four stores per lane where the codes and scales are under ~15 % of the bytes
-// written (measured 87-91 % of HBM peak against 78-87 % with two), two stores
-// where they are more (8-bit codes, 4-bit codes with blocks of 32: 81-83 % against 73-75 %).
-constexpr int kUnrollQ = 4;
-template <class F, int kBits, int kGroup>
-constexpr int kUnrollD = F::kBytes != 4 ? 2 : ((kBits == 8 || (kBits == 4 && kGroup > 0 && kGroup <= 8)) ? 2 : 4);
-
-QuantParams quant_params(const Range& r) {
-    QuantParams p;
-    p.lo = r.lo;
-    p.hi = r.hi;
-    p.width = r.hi - r.lo;
-    p.rwidth = 1.0f / p.width;  // IEEE division on the host: correctly rounded
-    return p;
-}
-
-// Launches `kernel(false)` over the full tiles and `kernel(true)` (bounds-checked)
-// over the ragged rest; a tile is kThreads*unroll chunks.
-template <class LaunchFn>
-hipError_t launch_tiles(uint64_t num_chunks, int unroll, LaunchFn launch) {
-    const uint64_t tile = static_cast<uint64_t>(kThreads) * unroll;
-    const uint64_t full = num_chunks / tile;
-    if (full > 0) {
-        launch(false, static_cast<uint32_t>(full), 0, full * tile);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
-    if (full * tile < num_chunks) {
-        launch(true, 1u, full * tile, num_chunks);
-        return hipGetLastError();
-    }
-    return hipSuccess;
-}
-
-template <class F, int kBits, int kGroup, int kSrc, bool kWide, int kEnc>
-hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
-    // scale sources that exist: per-block launches compute the scale or read the
-    // input-typed tensor; per-tensor launches read it or finish the grid reduction
-    if constexpr ((kGroup == 0 && kSrc == kScaleDynamic) || (kGroup != 0 && kSrc == kScalePartials)) {
-        return hipErrorInvalidValue;
-    } else {
-        auto in = static_cast<const u32x4*>(a.input);
-        auto out = static_cast<uint32_t*>(a.output);
-        const QuantParams qp = quant_params(a.range);
-        const bool p32 = a.param_dtype == CQ_F32;
-        return launch_tiles(a.num_chunks, kUnrollQ, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
-            auto kernel =
-                checked ? (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, true, kEnc>
-                               : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, true, kEnc>)
-                        : (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false, kEnc>
-                               : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false, kEnc>);
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
-                               a.param_dtype, begin, end, qp, a.num_partials);
-        });
-    }
-}
-
-template <class F, int kBits, int kGroup, bool kWide, int kEnc>
-hipError_t quantize_launch_enc(hipStream_t s, ScaleSource src, const FlatArgs& a) {
-    if (src == ScaleSource::Dynamic) return quantize_launch_src<F, kBits, kGroup, kScaleDynamic, kWide, kEnc>(s, a);
-    if (src == ScaleSource::Partials) return quantize_launch_src<F, kBits, kGroup, kScalePartials, kWide, kEnc>(s, a);
-    if (a.scale_in_dtype == F::kDtype) return quantize_launch_src<F, kBits, kGroup, kScaleGivenF, kWide, kEnc>(s, a);
-    return hipErrorInvalidValue;  // given scales are typed like the input
-}
-
-template <class F, int kBits, int kGroup>
-hipError_t quantize_launch(hipStream_t s, ScaleSource src, const FlatArgs& a) {
-    switch (a.encoding) {
-        case kEncInt: {
-            // only 8-bit fields can be narrower than their value range (E4M3, E5M2)
-            const bool wide = kBits == 8 && (a.range.hi > 127.0f || a.range.lo < -128.0f);
-            if constexpr (kBits == 8)
-                if (wide) return quantize_launch_enc<F, kBits, kGroup, true, kEncInt>(s, src, a);
-            return quantize_launch_enc<F, kBits, kGroup, false, kEncInt>(s, src, a);
-        }
-        case kEncE4M3:
-            if constexpr (kBits == 8) return quantize_launch_enc<F, 8, kGroup, false, kEncE4M3>(s, src, a);
-            break;
-        case kEncE5M2:
-            if constexpr (kBits == 8) return quantize_launch_enc<F, 8, kGroup, false, kEncE5M2>(s, src, a);
-            break;
-        case kEncE2M1:
-            if constexpr (kBits == 4) return quantize_launch_enc<F, 4, kGroup, false, kEncE2M1>(s, src, a);
-            break;
-    }
-    return hipErrorInvalidValue;
-}
-
-template <class F, int kBits, int kGroup, int kEnc>
-hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
-    auto in = static_cast<const uint32_t*>(a.input);
-    auto out = static_cast<u32x4*>(a.output);
-    const bool p32 = a.param_dtype == CQ_F32;
-    return launch_tiles(a.num_chunks, kUnrollD<F, kBits, kGroup>, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
-        auto kernel =
-            checked ? (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F, kBits, kGroup>, kThreads, true, kEnc>
-                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F, kBits, kGroup>, kThreads, true, kEnc>)
-                    : (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F, kBits, kGroup>, kThreads, false, kEnc>
-                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F, kBits, kGroup>, kThreads, false, kEnc>);
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, begin, end);
-    });
-}
-
-template <class F, int kBits, int kGroup>
-hipError_t dequantize_launch(hipStream_t s, const FlatArgs& a) {
-    switch (a.encoding) {
-        case kEncInt: return dequantize_launch_enc<F, kBits, kGroup, kEncInt>(s, a);
-        case kEncE4M3:
-            if constexpr (kBits == 8) return dequantize_launch_enc<F, 8, kGroup, kEncE4M3>(s, a);
-            break;
-        case kEncE5M2:
-            if constexpr (kBits == 8) return dequantize_launch_enc<F, 8, kGroup, kEncE5M2>(s, a);
-            break;
-        case kEncE2M1:
-            if constexpr (kBits == 4) return dequantize_launch_enc<F, 4, kGroup, kEncE2M1>(s, a);
-            break;
-    }
-    return hipErrorInvalidValue;
-}
 
 template <class F, int kGroup>
 hipError_t scales_launch(hipStream_t s, const FlatArgs& a) {
@@ -156,48 +16,15 @@ hipError_t scales_launch(hipStream_t s, const FlatArgs& a) {
     return hipGetLastError();
 }
 
-#define CQ_SWITCH_GROUP(G, ...)                          \
-    switch (G) {                                         \
-        case 0: { constexpr int kG = 0; __VA_ARGS__; }   \
-        case 1: { constexpr int kG = 1; __VA_ARGS__; }   \
-        case 2: { constexpr int kG = 2; __VA_ARGS__; }   \
-        case 4: { constexpr int kG = 4; __VA_ARGS__; }   \
-        case 8: { constexpr int kG = 8; __VA_ARGS__; }   \
-        case 16: { constexpr int kG = 16; __VA_ARGS__; } \
-        case 32: { constexpr int kG = 32; __VA_ARGS__; } \
-        default: return hipErrorInvalidValue;            \
-    }
-
-#define CQ_SWITCH_BITS(B, ...)                          \
-    switch (B) {                                        \
-        case 2: { constexpr int kB = 2; __VA_ARGS__; }  \
-        case 4: { constexpr int kB = 4; __VA_ARGS__; }  \
-        case 8: { constexpr int kB = 8; __VA_ARGS__; }  \
-        default: return hipErrorInvalidValue;           \
-    }
-
-#define CQ_SWITCH_DTYPE(D, ...)                              \
-    switch (D) {                                             \
-        case CQ_F32: { using kF = F32; __VA_ARGS__; }        \
-        case CQ_BF16: { using kF = BF16; __VA_ARGS__; }      \
-        case CQ_F16: { using kF = F16; __VA_ARGS__; }        \
-        default: return hipErrorInvalidValue;                \
-    }
-
 }  // namespace
 
 bool flat_block_supported(int dtype, uint32_t block) { return group_of(dtype, block) >= 0; }
 
 hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource src, const FlatArgs& a) {
     if (a.num_chunks == 0) return hipSuccess;
+    if (src == ScaleSource::Given) return launch_quantize_flat_given(s, dtype, bits, a);
     int g = group_of(dtype, a.block);
-    CQ_SWITCH_DTYPE(dtype, CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return quantize_launch<kF, kB, kG>(s, src, a))))
-}
-
-hipError_t launch_dequantize_flat(hipStream_t s, int dtype, int bits, const FlatArgs& a) {
-    if (a.num_chunks == 0) return hipSuccess;
-    int g = group_of(dtype, a.block);
-    CQ_SWITCH_DTYPE(dtype, CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return dequantize_launch<kF, kB, kG>(s, a))))
+    CQ_SWITCH_DTYPE(dtype, CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (quantize_launch<kF, kB, kG, false>(s, src, a)))))
 }
 
 hipError_t launch_scales_flat(hipStream_t s, int dtype, const FlatArgs& a) {

@@ -9,6 +9,9 @@
 // its abs-max is a DPP butterfly, no LDS.  Codes narrower than a word
 // (chunk bits 16 or 8) are OR-combined across 2 or 4 lanes before one store.
 //
+// quantize_flat_rows_kernel / dequantize_flat_rows_kernel run the same bodies over pitched rows
+// (grid y, z = the row), each row a run of chunks of its own.
+//
 // HBM traffic per element is the algorithmic minimum: the input once, the
 // codes once, one scale per block.  Loads and stores carry the non-temporal
 // hint: nothing is re-read.
@@ -33,12 +36,14 @@ enum ScaleSrc : int {
 //            are clamped and stores masked.  Full tiles use the unchecked variant.
 // kEnc     : stored encoding (kEncInt for the U32 store and native i8; e4m3 / e5m2 /
 //            e2m1 for the native float stores, where kBits is the stored width).
+// `first_row`: false in the launches over pitched rows (quantize_flat_rows_kernel) for every row but
+// the first; only the per-tensor scale store looks at it.
 template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
-          int kThreads, bool kChecked, int kEnc = kEncInt>
-__global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
+          int kThreads, bool kChecked, int kEnc>
+__device__ __forceinline__ void quantize_flat_body(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
     void* __restrict__ scale_out, int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end,
-    QuantParams qp, uint32_t num_partials) {
+    const QuantParams& qp, uint32_t num_partials, bool first_row) {
     constexpr bool kDynamic = kScaleSrc == kScaleDynamic;
     static_assert(kScaleSrc != kScalePartials || kGroup == 0, "partials feed the per-tensor scale only");
     constexpr int kDiv = kGroup == 0 ? 1 : kGroup;
@@ -114,7 +119,7 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
         // write_scale (src/quantize.rs:83-98): FS(scale), stored by the block's first lane
         const float s_fs = round_to_dtype(param_dtype, s_f);
         const uint64_t si = kGroup == 0 ? 0 : c / kDiv;
-        const bool block_start = kGroup == 0 ? c == 0 : (c % kDiv) == 0;
+        const bool block_start = kGroup == 0 ? (c == 0 && first_row) : (c % kDiv) == 0;
         if (scale_out != nullptr && live && block_start) store_dtype(param_dtype, scale_out, si, s_fs);
         // divisor F(FS(scale)); s_f is an F value, so f32 params leave it unchanged
         float d = s_fs;
@@ -142,9 +147,41 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
     }
 }
 
-template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked,
-          int kEnc = kEncInt>
-__global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
+template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
+          int kThreads, bool kChecked, int kEnc = kEncInt>
+__global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
+    const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
+    void* __restrict__ scale_out, int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end,
+    QuantParams qp, uint32_t num_partials) {
+    quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParamF32, kWide, kUnroll, kThreads, kChecked, kEnc>(
+        in, out, scale_in, scale_out, param_dtype_rt, chunk_begin, chunk_end, qp, num_partials, true);
+}
+
+// Pitched rows: grid y, z = the row; a row is a run of chunks [chunk_begin, chunk_end) of its own, and
+// the rows of the four tensors start `rows.*` bytes apart.  A kernel of its own so that the launches
+// over one contiguous run carry none of this in their prologue.
+struct FlatRows {
+    uint32_t count;
+    uint64_t in, out, scale_in, scale_out;
+};
+template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
+          int kThreads, bool kChecked, int kEnc = kEncInt>
+__global__ __launch_bounds__(kThreads) void quantize_flat_rows_kernel(
+    const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
+    void* __restrict__ scale_out, int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end,
+    QuantParams qp, uint32_t num_partials, FlatRows rows) {
+    const uint32_t row = blockIdx.y + blockIdx.z * gridDim.y;
+    if (row >= rows.count) return;
+    quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParamF32, kWide, kUnroll, kThreads, kChecked, kEnc>(
+        reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(in) + row * rows.in),
+        reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(out) + row * rows.out),
+        static_cast<const char*>(scale_in) + row * rows.scale_in,
+        scale_out == nullptr ? nullptr : static_cast<char*>(scale_out) + row * rows.scale_out, param_dtype_rt,
+        chunk_begin, chunk_end, qp, num_partials, row == 0);
+}
+
+template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked, int kEnc>
+__device__ __forceinline__ void dequantize_flat_body(
     const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params,
     int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end) {
     const int param_dtype = kParamF32 ? static_cast<int>(CQ_F32) : param_dtype_rt;
@@ -189,6 +226,27 @@ __global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
         for (int i = 0; i < kN; i++) y[i] = sc[u] * y[i];
         if (!kChecked || c < chunk_end) stream_store(F::pack(y), out + c);  // pack rounds to F
     }
+}
+
+template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked,
+          int kEnc = kEncInt>
+__global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
+    const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params,
+    int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end) {
+    dequantize_flat_body<F, kBits, kGroup, kParamF32, kUnroll, kThreads, kChecked, kEnc>(in, out, params, param_dtype_rt,
+                                                                                         chunk_begin, chunk_end);
+}
+template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked,
+          int kEnc = kEncInt>
+__global__ __launch_bounds__(kThreads) void dequantize_flat_rows_kernel(
+    const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params,
+    int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end, FlatRows rows) {
+    const uint32_t row = blockIdx.y + blockIdx.z * gridDim.y;
+    if (row >= rows.count) return;
+    dequantize_flat_body<F, kBits, kGroup, kParamF32, kUnroll, kThreads, kChecked, kEnc>(
+        reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(in) + row * rows.in),
+        reinterpret_cast<u32x4*>(reinterpret_cast<char*>(out) + row * rows.out),
+        static_cast<const char*>(params) + row * rows.scale_in, param_dtype_rt, chunk_begin, chunk_end);
 }
 
 // Block abs-max -> scale typed like the input (what quantize takes as `scale`).

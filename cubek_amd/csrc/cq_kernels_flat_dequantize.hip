@@ -1,0 +1,57 @@
+// Launchers of the flat (contiguous) dequantize kernels.
+#include "cq_kernels_flat_launch.hpp"
+
+namespace cq {
+namespace {
+
+template <class F, int kBits, int kGroup, int kEnc>
+hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
+    auto in = static_cast<const uint32_t*>(a.input);
+    auto out = static_cast<u32x4*>(a.output);
+    const bool p32 = a.param_dtype == CQ_F32;
+    return launch_tiles(a.num_chunks, kUnrollD<F, kBits, kGroup>, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
+        auto kernel =
+            checked ? (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F, kBits, kGroup>, kThreads, true, kEnc>
+                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F, kBits, kGroup>, kThreads, true, kEnc>)
+                    : (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F, kBits, kGroup>, kThreads, false, kEnc>
+                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F, kBits, kGroup>, kThreads, false, kEnc>);
+        if (a.rows > 1) {
+            constexpr int kU = kUnrollD<F, kBits, kGroup>;
+            auto rows_kernel = checked ? (p32 ? dequantize_flat_rows_kernel<F, kBits, kGroup, true, kU, kThreads, true, kEnc>
+                                              : dequantize_flat_rows_kernel<F, kBits, kGroup, false, kU, kThreads, true, kEnc>)
+                                       : (p32 ? dequantize_flat_rows_kernel<F, kBits, kGroup, true, kU, kThreads, false, kEnc>
+                                              : dequantize_flat_rows_kernel<F, kBits, kGroup, false, kU, kThreads, false, kEnc>);
+            hipLaunchKernelGGL(rows_kernel, rows_grid(grid, a), dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, begin,
+                               end, flat_rows(a));
+            return;
+        }
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, begin, end);
+    });
+}
+
+template <class F, int kBits, int kGroup>
+hipError_t dequantize_launch(hipStream_t s, const FlatArgs& a) {
+    switch (a.encoding) {
+        case kEncInt: return dequantize_launch_enc<F, kBits, kGroup, kEncInt>(s, a);
+        case kEncE4M3:
+            if constexpr (kBits == 8) return dequantize_launch_enc<F, 8, kGroup, kEncE4M3>(s, a);
+            break;
+        case kEncE5M2:
+            if constexpr (kBits == 8) return dequantize_launch_enc<F, 8, kGroup, kEncE5M2>(s, a);
+            break;
+        case kEncE2M1:
+            if constexpr (kBits == 4) return dequantize_launch_enc<F, 4, kGroup, kEncE2M1>(s, a);
+            break;
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+hipError_t launch_dequantize_flat(hipStream_t s, int dtype, int bits, const FlatArgs& a) {
+    if (a.num_chunks == 0) return hipSuccess;
+    int g = group_of(dtype, a.block);
+    CQ_SWITCH_DTYPE(dtype, CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (dequantize_launch<kF, kB, kG>(s, a)))))
+}
+
+}  // namespace cq

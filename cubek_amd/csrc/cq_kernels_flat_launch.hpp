@@ -1,0 +1,178 @@
+// Shared by the translation units that launch the flat kernels (cq_kernels_flat*.hip): launch
+// shapes, tile splitting, the dispatch macros, and the quantize launch chain, which each unit
+// instantiates for its own scale sources.
+#pragma once
+
+#include "cq_internal.hpp"
+#include "cq_kernels_flat.hpp"
+
+namespace cq {
+
+// quantize with given scales, defined in cq_kernels_flat_given.hip
+hipError_t launch_quantize_flat_given(hipStream_t s, int dtype, int bits, const FlatArgs& a);
+
+namespace {
+
+constexpr int kThreads = 256;
+
+inline uint32_t grid_for(uint64_t num_chunks, int unroll) {
+    uint64_t per = static_cast<uint64_t>(kThreads) * unroll;
+    return static_cast<uint32_t>((num_chunks + per - 1) / per);
+}
+
+int group_of(int dtype, uint32_t block) {
+    if (block == 0) return 0;
+    uint32_t per_chunk = dtype == CQ_F32 ? 4u : 8u;
+    if (block % per_chunk) return -1;
+    uint32_t g = block / per_chunk;
+    if (g & (g - 1)) return -1;
+    return g <= 32 ? static_cast<int>(g) : -1;
+}
+
+// Launch shapes from a sweep on MI355X (batches of back-to-back launches,
+// 117 MB - 470 MB tensors): quantize is best with four 16-byte loads in flight
+// per lane; dequantize, which is store-dominated, with two 16-byte stores per lane
+// for 16-bit outputs.  For f32 outputs the best depth follows the share of reads:
+// four stores per lane where the codes and scales are under ~15 % of the bytes
+// written (measured 87-91 % of HBM peak against 78-87 % with two), two stores
+// where they are more (8-bit codes, 4-bit codes with blocks of 32: 81-83 % against 73-75 %).
+constexpr int kUnrollQ = 4;
+template <class F, int kBits, int kGroup>
+constexpr int kUnrollD = F::kBytes != 4 ? 2 : ((kBits == 8 || (kBits == 4 && kGroup > 0 && kGroup <= 8)) ? 2 : 4);
+
+// grid of a launch of `tiles` workgroups per row, and the rows as the kernels take them
+dim3 rows_grid(uint32_t tiles, const FlatArgs& a) {
+    const uint32_t y = a.rows < 65535 ? static_cast<uint32_t>(a.rows) : 65535u;
+    return dim3(tiles, y, static_cast<uint32_t>((a.rows + y - 1) / y));
+}
+FlatRows flat_rows(const FlatArgs& a) {
+    return FlatRows{static_cast<uint32_t>(a.rows), a.in_pitch, a.out_pitch, a.scale_in_pitch, a.scale_out_pitch};
+}
+
+QuantParams quant_params(const Range& r) {
+    QuantParams p;
+    p.lo = r.lo;
+    p.hi = r.hi;
+    p.width = r.hi - r.lo;
+    p.rwidth = 1.0f / p.width;  // IEEE division on the host: correctly rounded
+    return p;
+}
+
+// Launches `kernel(false)` over the full tiles and `kernel(true)` (bounds-checked)
+// over the ragged rest; a tile is kThreads*unroll chunks.
+template <class LaunchFn>
+hipError_t launch_tiles(uint64_t num_chunks, int unroll, LaunchFn launch) {
+    const uint64_t tile = static_cast<uint64_t>(kThreads) * unroll;
+    const uint64_t full = num_chunks / tile;
+    if (full > 0) {
+        launch(false, static_cast<uint32_t>(full), 0, full * tile);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (full * tile < num_chunks) {
+        launch(true, 1u, full * tile, num_chunks);
+        return hipGetLastError();
+    }
+    return hipSuccess;
+}
+
+template <class F, int kBits, int kGroup, int kSrc, bool kWide, int kEnc>
+hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
+    // scale sources that exist: per-block launches compute the scale or read the
+    // input-typed tensor; per-tensor launches read it or finish the grid reduction
+    if constexpr ((kGroup == 0 && kSrc == kScaleDynamic) || (kGroup != 0 && kSrc == kScalePartials)) {
+        return hipErrorInvalidValue;
+    } else {
+        auto in = static_cast<const u32x4*>(a.input);
+        auto out = static_cast<uint32_t*>(a.output);
+        const QuantParams qp = quant_params(a.range);
+        const bool p32 = a.param_dtype == CQ_F32;
+        return launch_tiles(a.num_chunks, kUnrollQ, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
+            auto kernel =
+                checked ? (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, true, kEnc>
+                               : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, true, kEnc>)
+                        : (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false, kEnc>
+                               : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false, kEnc>);
+            if (a.rows > 1) {
+                auto rows_kernel =
+                    checked ? (p32 ? quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, true, kEnc>
+                                   : quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, true, kEnc>)
+                            : (p32 ? quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false, kEnc>
+                                   : quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false, kEnc>);
+                hipLaunchKernelGGL(rows_kernel, rows_grid(grid, a), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
+                                   a.param_dtype, begin, end, qp, a.num_partials, flat_rows(a));
+                return;
+            }
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
+                               a.param_dtype, begin, end, qp, a.num_partials);
+        });
+    }
+}
+
+// kGiven: the translation unit holds the kernels that read given scales, or those that produce
+// the scale themselves (the two sets are compiled apart: together they take minutes).
+template <class F, int kBits, int kGroup, bool kWide, int kEnc, bool kGiven>
+hipError_t quantize_launch_enc(hipStream_t s, ScaleSource src, const FlatArgs& a) {
+    if constexpr (kGiven) {
+        if (src == ScaleSource::Given && a.scale_in_dtype == F::kDtype)  // given scales are typed like the input
+            return quantize_launch_src<F, kBits, kGroup, kScaleGivenF, kWide, kEnc>(s, a);
+    } else {
+        if (src == ScaleSource::Dynamic) return quantize_launch_src<F, kBits, kGroup, kScaleDynamic, kWide, kEnc>(s, a);
+        if (src == ScaleSource::Partials) return quantize_launch_src<F, kBits, kGroup, kScalePartials, kWide, kEnc>(s, a);
+    }
+    return hipErrorInvalidValue;
+}
+
+template <class F, int kBits, int kGroup, bool kGiven>
+hipError_t quantize_launch(hipStream_t s, ScaleSource src, const FlatArgs& a) {
+    switch (a.encoding) {
+        case kEncInt: {
+            // only 8-bit fields can be narrower than their value range (E4M3, E5M2)
+            const bool wide = kBits == 8 && (a.range.hi > 127.0f || a.range.lo < -128.0f);
+            if constexpr (kBits == 8)
+                if (wide) return quantize_launch_enc<F, kBits, kGroup, true, kEncInt, kGiven>(s, src, a);
+            return quantize_launch_enc<F, kBits, kGroup, false, kEncInt, kGiven>(s, src, a);
+        }
+        case kEncE4M3:
+            if constexpr (kBits == 8) return quantize_launch_enc<F, 8, kGroup, false, kEncE4M3, kGiven>(s, src, a);
+            break;
+        case kEncE5M2:
+            if constexpr (kBits == 8) return quantize_launch_enc<F, 8, kGroup, false, kEncE5M2, kGiven>(s, src, a);
+            break;
+        case kEncE2M1:
+            if constexpr (kBits == 4) return quantize_launch_enc<F, 4, kGroup, false, kEncE2M1, kGiven>(s, src, a);
+            break;
+    }
+    return hipErrorInvalidValue;
+}
+
+#define CQ_SWITCH_GROUP(G, ...)                          \
+    switch (G) {                                         \
+        case 0: { constexpr int kG = 0; __VA_ARGS__; }   \
+        case 1: { constexpr int kG = 1; __VA_ARGS__; }   \
+        case 2: { constexpr int kG = 2; __VA_ARGS__; }   \
+        case 4: { constexpr int kG = 4; __VA_ARGS__; }   \
+        case 8: { constexpr int kG = 8; __VA_ARGS__; }   \
+        case 16: { constexpr int kG = 16; __VA_ARGS__; } \
+        case 32: { constexpr int kG = 32; __VA_ARGS__; } \
+        default: return hipErrorInvalidValue;            \
+    }
+
+#define CQ_SWITCH_BITS(B, ...)                          \
+    switch (B) {                                        \
+        case 2: { constexpr int kB = 2; __VA_ARGS__; }  \
+        case 4: { constexpr int kB = 4; __VA_ARGS__; }  \
+        case 8: { constexpr int kB = 8; __VA_ARGS__; }  \
+        default: return hipErrorInvalidValue;           \
+    }
+
+#define CQ_SWITCH_DTYPE(D, ...)                              \
+    switch (D) {                                             \
+        case CQ_F32: { using kF = F32; __VA_ARGS__; }        \
+        case CQ_BF16: { using kF = BF16; __VA_ARGS__; }      \
+        case CQ_F16: { using kF = F16; __VA_ARGS__; }        \
+        default: return hipErrorInvalidValue;                \
+    }
+
+}  // namespace
+}  // namespace cq

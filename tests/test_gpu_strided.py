@@ -54,6 +54,7 @@ def layouts(shape, per):
         return tuple(st)
 
     out = [("pitched", contiguous(shape, 5), contiguous(pshape, 3)),
+           ("pitched_aligned", contiguous(shape, 64), contiguous(pshape, 8)),
            ("transposed_floats", permuted(shape), contiguous(pshape)),
            ("transposed_stored", contiguous(shape), permuted(pshape)),
            ("both", permuted(shape), permuted(pshape))]
@@ -98,6 +99,18 @@ SCHEMES = [
 @pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
 @pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
 def test_strided_value_tensors(gpu, oracle, elem, name, scheme):
+    check_layouts(gpu, oracle, elem, name, scheme, ((6, 64), (2, 4, 96), (3, 70, 128), (2, 72, 256)), None)
+
+
+@pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
+@pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
+def test_long_pitched_rows(gpu, oracle, elem, name, scheme):
+    """Rows long enough for the streaming kernels to take them one by one (whole tiles, and a
+    ragged last tile per row)."""
+    check_layouts(gpu, oracle, elem, name, scheme, ((3, 16384), (2, 2, 16384 + 4096 + 512)), ("pitched_aligned", "every_other_row"))
+
+
+def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
     import torch
 
     rng = np.random.default_rng(zlib.crc32(name.encode()) % 1000 + int(elem))
@@ -105,12 +118,16 @@ def test_strided_value_tensors(gpu, oracle, elem, name, scheme):
     per = scheme.num_quants()
     stored_np = np.uint32 if scheme.store == QuantStore.U32 else np.uint8
     pe = gpu.param_elem(scheme)
-    for shape in ((6, 64), (2, 4, 96), (3, 70, 128), (2, 72, 256)):
+    for shape in shapes:
         if scheme.level.block_size is not None and shape[-1] % scheme.level.block_size.dims[-1]:
+            continue
+        if scheme.level.block_size is not None and len(scheme.level.block_size.dims) > 1 and only is not None:
             continue
         pshape, cases = layouts(shape, per)
         sshape = scheme.scales_shape(shape)
         for case, fstr, vstr in cases:
+            if only is not None and case not in only:
+                continue
             fbuf = oracle.to_bits(rng.normal(0, 1, reach(shape, fstr)).astype(np.float32), elem)
             xc = np.ascontiguousarray(view(fbuf, shape, fstr))
             s_ref = oracle.compute_scales(xc, elem, shape, scheme)
