@@ -107,7 +107,7 @@ def test_strided_value_tensors(gpu, oracle, elem, name, scheme):
 def test_long_pitched_rows(gpu, oracle, elem, name, scheme):
     """Rows long enough for the streaming kernels to take them one by one (whole tiles, and a
     ragged last tile per row)."""
-    check_layouts(gpu, oracle, elem, name, scheme, ((3, 16384), (2, 2, 16384 + 4096 + 512)), ("pitched_aligned", "every_other_row"))
+    check_layouts(gpu, oracle, elem, name, scheme, ((3, 16384), (2, 2, 16384 + 4096 + 512)), ("pitched", "pitched_aligned", "every_other_row"))
 
 
 def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
