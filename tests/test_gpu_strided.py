@@ -247,3 +247,37 @@ def test_large_transposed_floats_match_the_contiguous_path(gpu, elem, rows, cols
         bits = torch.int32 if elem == ElemType.F32 else torch.int16
         assert torch.equal(yt.t().contiguous().view(bits), y.view(bits)), (name, "dequantize")
         del outs, codes2, codes3, y, yt
+
+
+def test_more_pitched_rows_than_one_grid_dimension_holds(gpu):
+    """70000 pitched rows: the row index of the streaming kernels spills from the grid's y into z.
+    Codes, scales and dequantized values must equal those of the contiguous copy."""
+    import torch
+
+    client = ComputeClient.current()
+    h = TensorHandleRef.from_torch
+    rows, cols, pad = 70000, 8192, 64
+    scheme = QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([32]))
+    g = torch.Generator(device="cuda")
+    g.manual_seed(9)
+    buf = torch.empty((rows, cols + pad), dtype=torch.bfloat16, device="cuda")
+    for r0 in range(0, rows, 10000):
+        buf[r0:r0 + 10000] = torch.randn((min(10000, rows - r0), cols + pad), generator=g, device="cuda").mul_(0.1).to(torch.bfloat16)
+    xc = buf[:, :cols].contiguous()
+    hp = TensorHandleRef(h(buf).handle, (rows, cols), (cols + pad, 1), 2)
+    outs = []
+    for hx in (h(xc), hp):
+        codes = torch.zeros((rows, cols // 8), dtype=torch.int32, device="cuda")
+        scales = torch.zeros((rows, cols // 32), dtype=torch.float32, device="cuda")
+        qz.launch_dynamic(client, hx, h(codes), h(scales), scheme, ElemType.BF16)
+        outs.append((codes, scales))
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    y = torch.empty_like(xc)
+    dq.launch_ref(client, h(outs[0][0]), h(y), h(outs[0][1]), scheme, ElemType.BF16)
+    ybuf = torch.full_like(buf, 7.0)
+    dq.launch_ref(client, h(outs[0][0]), TensorHandleRef(h(ybuf).handle, (rows, cols), (cols + pad, 1), 2), h(outs[0][1]),
+                  scheme, ElemType.BF16)
+    torch.cuda.synchronize()
+    assert torch.equal(ybuf[:, :cols].contiguous().view(torch.int16), y.view(torch.int16))
+    assert bool((ybuf[:, cols:] == 7.0).all())
