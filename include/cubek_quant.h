@@ -12,8 +12,8 @@
  *   - calls are asynchronous and ordered on the given HIP stream (NULL = the
  *     default stream); nothing here synchronises the device;
  *   - every function returns a cq_status (0 = success) and never aborts;
- *   - calls are re-entrant and thread safe: the library keeps no state besides a few
- *     device properties it looks up once.
+ *   - calls are re-entrant and thread safe: the library keeps no state besides the
+ *     per-thread code behind cq_last_hip_error().
  */
 #ifndef CUBEK_QUANT_H
 #define CUBEK_QUANT_H
