@@ -215,7 +215,7 @@ bool uniform_rows(const cq_tensor* t, uint64_t* rows, uint64_t* pitch) {
 }
 
 // Can the flat kernels take this launch row by row?  (value tensors with a contiguous last
-// dimension and a uniform row pitch, rows long enough to fill their tiles, no ragged row end,
+// dimension and a uniform row pitch, rows of at least one tile, whole chunks,
 // 1-D blocks that map onto lane groups, scales with a contiguous last dimension.)  Fills the
 // row fields of `a` and a.num_chunks = chunks per row.
 bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
@@ -232,7 +232,8 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
     if (cols == 0 || cols % chunk_elems) return false;
     const uint64_t row_chunks = cols / per_chunk;
-    if (row_chunks < 2048 && row_chunks % 1024) return false;  // tiles of up to 1024 chunks: little of a row's last one idle
+    // tiles of up to 1024 chunks; a row's ragged last one is a launch of its own, mostly idle: at most 1/8 on top
+    if (row_chunks < 1024 || (row_chunks + 1023) / 1024 * 1024 > row_chunks + row_chunks / 8) return false;
     if (rows_f > 65535ull * 65535ull) return false;
     a->scale_in_pitch = a->scale_out_pitch = 0;
     if (!p.tensor_level) {

@@ -519,6 +519,20 @@ bool blocks_geom(uint32_t per_chunk, uint32_t bits, const RowArgs& a, BlocksGeom
     uint32_t tj_log2 = lanes_log2(chunks_per_row);
     if (tj_log2 < min_log2) tj_log2 = min_log2;
     while (tj_log2 > min_log2 && br > kPreferredRowsPerThread * (kThreads >> tj_log2)) tj_log2--;
+    // A thread takes 1-4 column tiles: narrower lanes (more rows per workgroup) while half the lanes
+    // would still cover the row, and while that leaves clearly fewer idle lanes in the last column
+    // group (rows of 128 chunks ran at a quarter of the lanes, rows of 1152 chunks at 56 %).
+    const auto cols_at = [&](uint32_t log2) {
+        const uint32_t phases = kThreads >> log2, ppb = br >= phases ? phases : br;
+        return blocks_cols_per_thread((br + ppb - 1) / ppb) << log2;  // chunks one column group covers (all lanes in use)
+    };
+    const auto covered_at = [&](uint32_t log2) {
+        const uint64_t per = cols_at(log2);
+        return (chunks_per_row + per - 1) / per * per;
+    };
+    while (tj_log2 > min_log2 && cols_at(tj_log2 - 1) >= chunks_per_row) tj_log2--;
+    for (uint32_t l = tj_log2; l > min_log2 && l > 6; l--)  // not below 64 lanes: runs of 1 KiB
+        if (covered_at(l - 1) * 10 <= covered_at(tj_log2) * 9) tj_log2 = l - 1;
     const uint32_t phases = kThreads >> tj_log2;
     g->tj_log2 = tj_log2;
     // whole blocks and whole stored words only (lanes that share a word exchange their parts by lane number)
