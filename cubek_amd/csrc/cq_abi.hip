@@ -694,6 +694,25 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
         a.range = p.range;
         return hip_status(cq::launch_scales_flat(stream, input_dtype, a));
     }
+    // pitched rows of at least one tile, 1-D blocks: the same kernel row by row
+    uint64_t rows_f, rows_s, pitch_f, pitch_s;
+    const uint64_t row_chunks = input->shape[input->rank - 1] / (16 / dtype_size(input_dtype));
+    if (!p.tensor_level && p.last_dim_blocks && p.rank >= 2 && cq::flat_block_supported(input_dtype, p.block_last) &&
+        uniform_rows(input, &rows_f, &pitch_f) && uniform_rows(scales, &rows_s, &pitch_s) && rows_f == rows_s &&
+        rows_f <= 65535ull * 65535ull && aligned(input->ptr, 16) && (pitch_f * dtype_size(input_dtype)) % 16 == 0 &&
+        input->shape[input->rank - 1] % (16 / dtype_size(input_dtype)) == 0 && row_chunks >= 1024 &&
+        (row_chunks + 1023) / 1024 * 1024 <= row_chunks + row_chunks / 8) {
+        cq::FlatArgs a{};
+        a.input = input->ptr;
+        a.scale_out = scales->ptr;
+        a.num_chunks = row_chunks;
+        a.rows = rows_f;
+        a.in_pitch = pitch_f * dtype_size(input_dtype);
+        a.scale_out_pitch = pitch_s * dtype_size(input_dtype);
+        a.block = p.block_last;
+        a.range = p.range;
+        return hip_status(cq::launch_scales_flat(stream, input_dtype, a));
+    }
     return produce_scales(stream, p, scheme, input, input_dtype, scales, input_dtype, workspace, workspace_bytes);
 }
 

@@ -251,9 +251,8 @@ __global__ __launch_bounds__(kThreads) void dequantize_flat_rows_kernel(
 
 // Block abs-max -> scale typed like the input (what quantize takes as `scale`).
 template <class F, int kGroup, int kUnroll, int kThreads>
-__global__ __launch_bounds__(kThreads) void scales_flat_kernel(const u32x4* __restrict__ in,
-                                                               void* __restrict__ scales,
-                                                               uint64_t num_chunks, QuantParams qp) {
+__device__ __forceinline__ void scales_flat_body(const u32x4* __restrict__ in, void* __restrict__ scales,
+                                                 uint64_t num_chunks, const QuantParams& qp) {
     constexpr int kN = F::kPerChunk;
     const uint64_t first = static_cast<uint64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
     const uint64_t last = num_chunks - 1;
@@ -277,6 +276,24 @@ __global__ __launch_bounds__(kThreads) void scales_flat_kernel(const u32x4* __re
                                                : scale_from_absmax(amax, qp.width);
         if (c < num_chunks && (c % kGroup) == 0) F::store(scales, c / kGroup, s32);
     }
+}
+
+template <class F, int kGroup, int kUnroll, int kThreads>
+__global__ __launch_bounds__(kThreads) void scales_flat_kernel(const u32x4* __restrict__ in,
+                                                               void* __restrict__ scales,
+                                                               uint64_t num_chunks, QuantParams qp) {
+    scales_flat_body<F, kGroup, kUnroll, kThreads>(in, scales, num_chunks, qp);
+}
+// pitched rows (grid y, z = the row): rows.in / rows.scale_out bytes between the rows of the two tensors
+template <class F, int kGroup, int kUnroll, int kThreads>
+__global__ __launch_bounds__(kThreads) void scales_flat_rows_kernel(const u32x4* __restrict__ in,
+                                                                    void* __restrict__ scales,
+                                                                    uint64_t num_chunks, QuantParams qp, FlatRows rows) {
+    const uint32_t row = blockIdx.y + blockIdx.z * gridDim.y;
+    if (row >= rows.count) return;
+    scales_flat_body<F, kGroup, kUnroll, kThreads>(
+        reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(in) + row * rows.in),
+        static_cast<char*>(scales) + row * rows.scale_out, num_chunks, qp);
 }
 
 // Per-tensor abs-max, pass 1: grid-stride over chunks with kUnroll 16-byte loads

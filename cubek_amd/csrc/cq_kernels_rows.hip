@@ -205,7 +205,10 @@ __global__ __launch_bounds__(kThreads) void scales_rows_kernel(RowArgs a, int ou
         for (uint32_t r0 = 0; r0 < br; r0 += kUnroll) {
             u32x4 raw[kUnroll];
 #pragma unroll
-            for (int u = 0; u < kUnroll; u++) raw[u] = stream_load(p + (r0 + u < br ? r0 + u : br - 1) * pitch);
+            for (int u = 0; u < kUnroll; u++) {
+                raw[u] = u32x4{0, 0, 0, 0};
+                if (r0 + u < br) raw[u] = stream_load(p + (r0 + u) * pitch);  // the same for the whole workgroup
+            }
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
                 float v[kN];
@@ -444,6 +447,13 @@ dim3 unit_grid(RowArgs* a) {
     using U = Unit<F, kBits>;
     a->units_per_row = a->shape[a->rank - 1] / U::kV;
     a->tj_log2 = lanes_log2((a->units_per_row + U::kUnits - 1) / U::kUnits);
+    // fewer lanes along the row (not below 64) where that leaves clearly fewer of them idle past the row end
+    const auto covered = [&](uint32_t log2) {
+        const uint64_t per = static_cast<uint64_t>(U::kUnits) << log2;
+        return (a->units_per_row + per - 1) / per * per;
+    };
+    for (uint32_t l = a->tj_log2; l > 6; l--)
+        if (covered(l - 1) * 10 <= covered(a->tj_log2) * 9) a->tj_log2 = l - 1;
     const uint32_t tr = kThreads >> a->tj_log2;
     const uint32_t per_group = U::kUnits << a->tj_log2;
     return dim3(static_cast<uint32_t>((a->rows + tr - 1) / tr), (a->units_per_row + per_group - 1) / per_group);
