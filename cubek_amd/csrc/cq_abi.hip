@@ -200,9 +200,10 @@ bool uniform_rows(const cq_tensor* t, uint64_t* rows, uint64_t* pitch) {
     if (t->shape[last] != 1 && t->strides[last] != 1) return false;
     *rows = 1;
     *pitch = 0;
-    uint64_t expect = 0;
+    uint64_t expect = 0;  // 0: no dimension with more than one entry seen yet
     for (int d = static_cast<int>(last) - 1; d >= 0; d--) {
         if (t->shape[d] == 1) continue;
+        if (t->strides[d] == 0) return false;  // broadcast rows: not for these kernels
         if (expect == 0) {
             *pitch = t->strides[d];
         } else if (t->strides[d] != expect) {

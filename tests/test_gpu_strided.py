@@ -281,3 +281,33 @@ def test_more_pitched_rows_than_one_grid_dimension_holds(gpu):
     torch.cuda.synchronize()
     assert torch.equal(ybuf[:, :cols].contiguous().view(torch.int16), y.view(torch.int16))
     assert bool((ybuf[:, cols:] == 7.0).all())
+
+
+@pytest.mark.parametrize("cols", [64, 16384], ids=["short_rows", "long_rows"])
+def test_broadcast_rows_read_like_their_copies(gpu, cols):
+    """A float input whose rows are one row repeated (row stride 0) quantizes like its materialised copy."""
+    import torch
+
+    client = ComputeClient.current()
+    h = TensorHandleRef.from_torch
+    rows = 6
+    scheme = QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([32]))
+    g = torch.Generator(device="cuda")
+    g.manual_seed(cols)
+    row = torch.randn((1, cols), generator=g, device="cuda").to(torch.bfloat16)
+    full = row.expand(rows, cols).contiguous()
+    outs = []
+    for hx in (h(full), TensorHandleRef(h(row).handle, (rows, cols), (0, 1), 2)):
+        codes = torch.zeros((rows, cols // 4), dtype=torch.int32, device="cuda")
+        scales = torch.zeros((rows, cols // 32), dtype=torch.float32, device="cuda")
+        qz.launch_dynamic(client, hx, h(codes), h(scales), scheme, ElemType.BF16)
+        in_scales = torch.zeros((rows, cols // 32), dtype=torch.bfloat16, device="cuda")
+        qz.compute_scales(client, hx, h(in_scales), scheme, ElemType.BF16)
+        codes2 = torch.zeros_like(codes)
+        scales2 = torch.zeros_like(scales)
+        qz.launch_ref(client, hx, h(codes2), h(in_scales), h(scales2), scheme, ElemType.BF16)
+        outs.append((codes, scales, codes2, scales2))
+    torch.cuda.synchronize()
+    for a, b in zip(outs[0], outs[1]):
+        assert torch.equal(a, b)
+    assert torch.equal(outs[0][0], outs[0][2])
