@@ -215,13 +215,15 @@ bool uniform_rows(const cq_tensor* t, uint64_t* rows, uint64_t* pitch) {
     return true;
 }
 
+bool scales_rows_ok(const Plan& p);
+
 // Can the flat kernels take this launch row by row?  (value tensors with a contiguous last
 // dimension and a uniform row pitch, rows of at least one tile, whole chunks,
 // 1-D blocks that map onto lane groups, scales with a contiguous last dimension.)  Fills the
 // row fields of `a` and a.num_chunks = chunks per row.
 bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
                   const cq_tensor* scale_a, uint32_t scale_a_size, const cq_tensor* scale_b, uint32_t scale_b_size,
-                  cq::FlatArgs* a) {
+                  bool block_rows_allowed, cq::FlatArgs* a) {
     if (p.rank < 2) return false;
     const uint32_t last = p.rank - 1;
     const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
@@ -237,15 +239,20 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     if (row_chunks < 1024 || (row_chunks + 1023) / 1024 * 1024 > row_chunks + row_chunks / 8) return false;
     if (rows_f > 65535ull * 65535ull) return false;
     a->scale_in_pitch = a->scale_out_pitch = 0;
+    a->scale_rows = 1;
     if (!p.tensor_level) {
-        if (!p.last_dim_blocks || !cq::flat_block_supported(dtype, p.block_last)) return false;
+        // blocks along the last dimension, or (where the scales are given) over the last two: a block of
+        // br rows is br rows of the launch that read the same row of scales
+        const uint32_t br = p.layout.block[last - 1];
+        if (!cq::flat_block_supported(dtype, p.block_last) || !scales_rows_ok(p) || (br != 1 && !block_rows_allowed)) return false;
         uint64_t rows_s, pitch_s;
-        if (!uniform_rows(scale_a, &rows_s, &pitch_s) || rows_s != rows_f) return false;
+        if (!uniform_rows(scale_a, &rows_s, &pitch_s) || rows_s * br != rows_f) return false;
         a->scale_in_pitch = pitch_s * scale_a_size;
         if (scale_b) {
-            if (!uniform_rows(scale_b, &rows_s, &pitch_s) || rows_s != rows_f) return false;
+            if (!uniform_rows(scale_b, &rows_s, &pitch_s) || rows_s * br != rows_f) return false;
             a->scale_out_pitch = pitch_s * scale_b_size;
         }
+        a->scale_rows = br;
     }
     a->rows = rows_f;
     a->num_chunks = row_chunks;
@@ -492,7 +499,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     }
     cq::FlatArgs fr{};
     if (flat_words == 0 && flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
-                                        dtype_size(pd), &fr)) {
+                                        dtype_size(pd), true, &fr)) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_in = scale->ptr;
@@ -566,7 +573,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
     cq::FlatArgs fr{};
-    if (flat_words == 0 && flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, &fr)) {
+    if (flat_words == 0 && flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr)) {
         fr.input = values->ptr;
         fr.output = output->ptr;
         fr.scale_in = params->ptr;
@@ -749,7 +756,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
 
     // pitched rows with 1-D blocks: the same fused kernel, row by row
     cq::FlatArgs fr{};
-    if (!p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, &fr)) {
+    if (!p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr)) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_out = out_scale->ptr;
@@ -809,7 +816,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, a));
         if (st != CQ_OK) return st;
         flat_words = flat_chunks * per_chunk / p.nq;
-    } else if (p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, &fr)) {
+    } else if (p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr)) {
         // per tensor on pitched rows: the same two passes, the second one row by row
         uint32_t num_partials = 0;
         st = absmax_partials(stream, p, scheme, input, input_dtype, workspace, workspace_bytes, &num_partials);

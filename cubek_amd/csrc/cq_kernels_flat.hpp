@@ -36,8 +36,8 @@ enum ScaleSrc : int {
 //            are clamped and stores masked.  Full tiles use the unchecked variant.
 // kEnc     : stored encoding (kEncInt for the U32 store and native i8; e4m3 / e5m2 /
 //            e2m1 for the native float stores, where kBits is the stored width).
-// `first_row`: false in the launches over pitched rows (quantize_flat_rows_kernel) for every row but
-// the first; only the per-tensor scale store looks at it.
+// `first_row`: false in the launches over rows (quantize_flat_rows_kernel) for rows that do not start a
+// block (per tensor: every row but the first); only the scale store looks at it.
 template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
           int kThreads, bool kChecked, int kEnc>
 __device__ __forceinline__ void quantize_flat_body(
@@ -119,7 +119,7 @@ __device__ __forceinline__ void quantize_flat_body(
         // write_scale (src/quantize.rs:83-98): FS(scale), stored by the block's first lane
         const float s_fs = round_to_dtype(param_dtype, s_f);
         const uint64_t si = kGroup == 0 ? 0 : c / kDiv;
-        const bool block_start = kGroup == 0 ? (c == 0 && first_row) : (c % kDiv) == 0;
+        const bool block_start = first_row && (kGroup == 0 ? c == 0 : (c % kDiv) == 0);
         if (scale_out != nullptr && live && block_start) store_dtype(param_dtype, scale_out, si, s_fs);
         // divisor F(FS(scale)); s_f is an F value, so f32 params leave it unchanged
         float d = s_fs;
@@ -158,10 +158,12 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
 }
 
 // Pitched rows: grid y, z = the row; a row is a run of chunks [chunk_begin, chunk_end) of its own, and
-// the rows of the four tensors start `rows.*` bytes apart.  A kernel of its own so that the launches
-// over one contiguous run carry none of this in their prologue.
+// the rows of the four tensors start `rows.*` bytes apart; blocks of rows.scale_rows rows by a lane group
+// of columns share their scale (given scales only: a fused abs-max sees one row).  A kernel of its own so
+// that the launches over one contiguous run carry none of this in their prologue.
 struct FlatRows {
     uint32_t count;
+    uint32_t scale_rows;  // rows that share a row of scales (blocks of that many rows); >= 1
     uint64_t in, out, scale_in, scale_out;
 };
 template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
@@ -175,9 +177,9 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_rows_kernel(
     quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParamF32, kWide, kUnroll, kThreads, kChecked, kEnc>(
         reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(in) + row * rows.in),
         reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(out) + row * rows.out),
-        static_cast<const char*>(scale_in) + row * rows.scale_in,
-        scale_out == nullptr ? nullptr : static_cast<char*>(scale_out) + row * rows.scale_out, param_dtype_rt,
-        chunk_begin, chunk_end, qp, num_partials, row == 0);
+        static_cast<const char*>(scale_in) + (row / rows.scale_rows) * rows.scale_in,
+        scale_out == nullptr ? nullptr : static_cast<char*>(scale_out) + (row / rows.scale_rows) * rows.scale_out,
+        param_dtype_rt, chunk_begin, chunk_end, qp, num_partials, kGroup == 0 ? row == 0 : row % rows.scale_rows == 0);
 }
 
 template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked, int kEnc>
@@ -246,7 +248,7 @@ __global__ __launch_bounds__(kThreads) void dequantize_flat_rows_kernel(
     dequantize_flat_body<F, kBits, kGroup, kParamF32, kUnroll, kThreads, kChecked, kEnc>(
         reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(in) + row * rows.in),
         reinterpret_cast<u32x4*>(reinterpret_cast<char*>(out) + row * rows.out),
-        static_cast<const char*>(params) + row * rows.scale_in, param_dtype_rt, chunk_begin, chunk_end);
+        static_cast<const char*>(params) + (row / rows.scale_rows) * rows.scale_in, param_dtype_rt, chunk_begin, chunk_end);
 }
 
 // Block abs-max -> scale typed like the input (what quantize takes as `scale`).
@@ -293,7 +295,7 @@ __global__ __launch_bounds__(kThreads) void scales_flat_rows_kernel(const u32x4*
     if (row >= rows.count) return;
     scales_flat_body<F, kGroup, kUnroll, kThreads>(
         reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(in) + row * rows.in),
-        static_cast<char*>(scales) + row * rows.scale_out, num_chunks, qp);
+        static_cast<char*>(scales) + (row / rows.scale_rows) * rows.scale_out, num_chunks, qp);
 }
 
 // Per-tensor abs-max, pass 1: grid-stride over chunks with kUnroll 16-byte loads

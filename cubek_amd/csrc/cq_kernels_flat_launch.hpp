@@ -46,7 +46,8 @@ dim3 rows_grid(uint32_t tiles, const FlatArgs& a) {
     return dim3(tiles, y, static_cast<uint32_t>((a.rows + y - 1) / y));
 }
 FlatRows flat_rows(const FlatArgs& a) {
-    return FlatRows{static_cast<uint32_t>(a.rows), a.in_pitch, a.out_pitch, a.scale_in_pitch, a.scale_out_pitch};
+    return FlatRows{static_cast<uint32_t>(a.rows), a.scale_rows > 1 ? a.scale_rows : 1u, a.in_pitch, a.out_pitch,
+                    a.scale_in_pitch, a.scale_out_pitch};
 }
 
 QuantParams quant_params(const Range& r) {

@@ -53,7 +53,8 @@ def layouts(shape, per):
             acc *= n
         return tuple(st)
 
-    out = [("pitched", contiguous(shape, 5), contiguous(pshape, 3)),
+    out = [("contiguous", contiguous(shape), contiguous(pshape)),
+           ("pitched", contiguous(shape, 5), contiguous(pshape, 3)),
            ("pitched_aligned", contiguous(shape, 64), contiguous(pshape, 8)),
            ("transposed_floats", permuted(shape), contiguous(pshape)),
            ("transposed_stored", contiguous(shape), permuted(pshape)),
@@ -106,8 +107,9 @@ def test_strided_value_tensors(gpu, oracle, elem, name, scheme):
 @pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
 def test_long_pitched_rows(gpu, oracle, elem, name, scheme):
     """Rows long enough for the streaming kernels to take them one by one (whole tiles, and a
-    ragged last tile per row)."""
-    check_layouts(gpu, oracle, elem, name, scheme, ((3, 16384), (2, 2, 16384 + 4096 + 512)), ("pitched", "pitched_aligned", "every_other_row"))
+    ragged last tile per row), with 1-D blocks and with blocks over the last two dimensions."""
+    check_layouts(gpu, oracle, elem, name, scheme, ((4, 16384), (2, 2, 16384 + 4096 + 512)),
+                  ("contiguous", "pitched", "pitched_aligned", "every_other_row"))
 
 
 def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
@@ -120,8 +122,6 @@ def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
     pe = gpu.param_elem(scheme)
     for shape in shapes:
         if scheme.level.block_size is not None and shape[-1] % scheme.level.block_size.dims[-1]:
-            continue
-        if scheme.level.block_size is not None and len(scheme.level.block_size.dims) > 1 and only is not None:
             continue
         pshape, cases = layouts(shape, per)
         sshape = scheme.scales_shape(shape)
