@@ -217,13 +217,18 @@ bool uniform_rows(const cq_tensor* t, uint64_t* rows, uint64_t* pitch) {
 
 bool scales_rows_ok(const Plan& p);
 
+// How much of a row the idle lanes of its ragged last tile may add before the row kernels are the
+// better choice: the quantize kernels lose to them beyond an eighth (rows of 1152 - 2304 chunks:
+// 45 / 43 / 41 us against 50 / 48 / 41 us), the dequantize kernels never did (38 - 43 us against 41 - 49 us).
+constexpr double kRaggedQuantize = 0.125;
+
 // Can the flat kernels take this launch row by row?  (value tensors with a contiguous last
 // dimension and a uniform row pitch, rows of at least one tile, whole chunks,
 // 1-D blocks that map onto lane groups, scales with a contiguous last dimension.)  Fills the
 // row fields of `a` and a.num_chunks = chunks per row.
 bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
                   const cq_tensor* scale_a, uint32_t scale_a_size, const cq_tensor* scale_b, uint32_t scale_b_size,
-                  bool block_rows_allowed, cq::FlatArgs* a) {
+                  bool given_scales, cq::FlatArgs* a) {
     if (p.rank < 2) return false;
     const uint32_t last = p.rank - 1;
     const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
@@ -235,8 +240,9 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
     if (cols == 0 || cols % chunk_elems) return false;
     const uint64_t row_chunks = cols / per_chunk;
-    // tiles of up to 1024 chunks; a row's ragged last one is a launch of its own, mostly idle: at most 1/8 on top
-    if (row_chunks < 1024 || (row_chunks + 1023) / 1024 * 1024 > row_chunks + row_chunks / 8) return false;
+    // tiles of up to 1024 chunks; a row's ragged last one is a launch of its own with idle lanes
+    if (row_chunks < 1024) return false;
+    a->ragged_share = static_cast<double>((row_chunks + 1023) / 1024 * 1024 - row_chunks) / static_cast<double>(row_chunks);
     if (rows_f > 65535ull * 65535ull) return false;
     a->scale_in_pitch = a->scale_out_pitch = 0;
     a->scale_rows = 1;
@@ -244,7 +250,7 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
         // blocks along the last dimension, or (where the scales are given) over the last two: a block of
         // br rows is br rows of the launch that read the same row of scales
         const uint32_t br = p.layout.block[last - 1];
-        if (!cq::flat_block_supported(dtype, p.block_last) || !scales_rows_ok(p) || (br != 1 && !block_rows_allowed)) return false;
+        if (!cq::flat_block_supported(dtype, p.block_last) || !scales_rows_ok(p) || (br != 1 && !given_scales)) return false;
         uint64_t rows_s, pitch_s;
         if (!uniform_rows(scale_a, &rows_s, &pitch_s) || rows_s * br != rows_f) return false;
         a->scale_in_pitch = pitch_s * scale_a_size;
@@ -499,7 +505,8 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     }
     cq::FlatArgs fr{};
     if (flat_words == 0 && flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
-                                        dtype_size(pd), true, &fr)) {
+                                        dtype_size(pd), true, &fr) &&
+        fr.ragged_share <= kRaggedQuantize) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_in = scale->ptr;
@@ -756,7 +763,8 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
 
     // pitched rows with 1-D blocks: the same fused kernel, row by row
     cq::FlatArgs fr{};
-    if (!p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr)) {
+    if (!p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) &&
+        fr.ragged_share <= kRaggedQuantize) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_out = out_scale->ptr;
@@ -816,7 +824,8 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, a));
         if (st != CQ_OK) return st;
         flat_words = flat_chunks * per_chunk / p.nq;
-    } else if (p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr)) {
+    } else if (p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) &&
+               fr.ragged_share <= kRaggedQuantize) {
         // per tensor on pitched rows: the same two passes, the second one row by row
         uint32_t num_partials = 0;
         st = absmax_partials(stream, p, scheme, input, input_dtype, workspace, workspace_bytes, &num_partials);
