@@ -217,13 +217,20 @@ bool uniform_rows(const cq_tensor* t, uint64_t* rows, uint64_t* pitch) {
 
 bool scales_rows_ok(const Plan& p);
 
-// How much of a row the idle lanes of its ragged last tile may add before the row kernels are the
-// better choice: the quantize kernels lose to them beyond an eighth (rows of 1152 - 2304 chunks:
-// 45 / 43 / 41 us against 50 / 48 / 41 us), the dequantize kernels never did (38 - 43 us against 41 - 49 us).
-constexpr double kRaggedQuantize = 0.125;
+// Do the flat kernels beat the row kernels on rows of this length?  Measured on pitched bf16 rows with
+// rotated buffers.  Quantize (tiles of 1024 chunks): rows of several tiles lose once the idle lanes of
+// the ragged last tile add more than an eighth (1152 - 2304 chunks: 45 / 43 / 41 us against 50 / 48 / 41 us);
+// rows of one partial tile win from five eighths of a tile on (640 / 768 / 896 chunks: 44.5 / 26 / 28 us
+// against 50 / 29 / 34.5 us; 512 chunks: 39.5 against 38 us).  Dequantize (tiles of 512 chunks for 16-bit
+// floats): any row of at least 1024 chunks wins (38 - 43 us against 41 - 49 us); below that only the
+// whole tile does (512 chunks: 29 against 33 us; 640 / 896 chunks: 44 / 31 against 42 / 28 us).
+bool flat_rows_pay(const cq::FlatArgs& a, int dtype, bool quantize) {
+    if (quantize) return a.num_chunks >= 1024 ? a.ragged_share <= 0.125 : a.num_chunks >= 640;
+    return a.num_chunks >= 1024 || (a.num_chunks == 512 && dtype_size(dtype) == 2);
+}
 
 // Can the flat kernels take this launch row by row?  (value tensors with a contiguous last
-// dimension and a uniform row pitch, rows of at least one tile, whole chunks,
+// dimension and a uniform row pitch, rows of at least half a tile, whole chunks,
 // 1-D blocks that map onto lane groups, scales with a contiguous last dimension.)  Fills the
 // row fields of `a` and a.num_chunks = chunks per row.
 bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
@@ -241,7 +248,7 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     if (cols == 0 || cols % chunk_elems) return false;
     const uint64_t row_chunks = cols / per_chunk;
     // tiles of up to 1024 chunks; a row's ragged last one is a launch of its own with idle lanes
-    if (row_chunks < 1024) return false;
+    if (row_chunks < 512) return false;  // callers narrow this further with flat_rows_pay()
     a->ragged_share = static_cast<double>((row_chunks + 1023) / 1024 * 1024 - row_chunks) / static_cast<double>(row_chunks);
     if (rows_f > 65535ull * 65535ull) return false;
     a->scale_in_pitch = a->scale_out_pitch = 0;
@@ -506,7 +513,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     cq::FlatArgs fr{};
     if (flat_words == 0 && flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
                                         dtype_size(pd), true, &fr) &&
-        fr.ragged_share <= kRaggedQuantize) {
+        flat_rows_pay(fr, input_dtype, true)) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_in = scale->ptr;
@@ -580,7 +587,8 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
     cq::FlatArgs fr{};
-    if (flat_words == 0 && flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr)) {
+    if (flat_words == 0 && flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr) &&
+        flat_rows_pay(fr, output_dtype, false)) {
         fr.input = values->ptr;
         fr.output = output->ptr;
         fr.scale_in = params->ptr;
@@ -764,7 +772,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
     // pitched rows with 1-D blocks: the same fused kernel, row by row
     cq::FlatArgs fr{};
     if (!p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) &&
-        fr.ragged_share <= kRaggedQuantize) {
+        flat_rows_pay(fr, input_dtype, true)) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_out = out_scale->ptr;
@@ -825,7 +833,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         if (st != CQ_OK) return st;
         flat_words = flat_chunks * per_chunk / p.nq;
     } else if (p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) &&
-               fr.ragged_share <= kRaggedQuantize) {
+               flat_rows_pay(fr, input_dtype, true)) {
         // per tensor on pitched rows: the same two passes, the second one row by row
         uint32_t num_partials = 0;
         st = absmax_partials(stream, p, scheme, input, input_dtype, workspace, workspace_bytes, &num_partials);

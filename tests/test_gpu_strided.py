@@ -112,6 +112,16 @@ def test_long_pitched_rows(gpu, oracle, elem, name, scheme):
                   ("contiguous", "pitched", "pitched_aligned", "every_other_row"))
 
 
+@pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
+@pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
+def test_pitched_rows_of_less_than_a_tile(gpu, oracle, elem, name, scheme):
+    """Rows of 512 - 896 sixteen-byte chunks: at 640 and more the streaming quantize kernels take
+    them as one partial tile per row, at exactly 512 (16-bit floats) the dequantize kernels do; the
+    other lengths go to the row kernels."""
+    check_layouts(gpu, oracle, elem, name, scheme, ((4, 4096), (6, 5120), (2, 2, 7168), (4, 2560), (4, 2048)),
+                  ("pitched", "pitched_aligned", "every_other_row"))
+
+
 def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
     import torch
 
