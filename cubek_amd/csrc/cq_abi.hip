@@ -217,18 +217,6 @@ bool uniform_rows(const cq_tensor* t, uint64_t* rows, uint64_t* pitch) {
 
 bool scales_rows_ok(const Plan& p);
 
-// Do the flat kernels beat the row kernels on rows of this length?  Measured on pitched bf16 rows with
-// rotated buffers.  Quantize (tiles of 1024 chunks): rows of several tiles lose once the idle lanes of
-// the ragged last tile add more than an eighth (1152 - 2304 chunks: 45 / 43 / 41 us against 50 / 48 / 41 us);
-// rows of one partial tile win from five eighths of a tile on (640 / 768 / 896 chunks: 44.5 / 26 / 28 us
-// against 50 / 29 / 34.5 us; 512 chunks: 39.5 against 38 us).  Dequantize (tiles of 512 chunks for 16-bit
-// floats): any row of at least 1024 chunks wins (38 - 43 us against 41 - 49 us); below that only the
-// whole tile does (512 chunks: 29 against 33 us; 640 / 896 chunks: 44 / 31 against 42 / 28 us).
-bool flat_rows_pay(const cq::FlatArgs& a, int dtype, bool quantize) {
-    if (quantize) return a.num_chunks >= 1024 ? a.ragged_share <= 0.125 : a.num_chunks >= 640;
-    return a.num_chunks >= 1024 || (a.num_chunks == 512 && dtype_size(dtype) == 2);
-}
-
 // Can the flat kernels take this launch row by row?  (value tensors with a contiguous last
 // dimension and a uniform row pitch, rows of at least half a tile, whole chunks,
 // 1-D blocks that map onto lane groups, scales with a contiguous last dimension.)  Fills the
@@ -247,10 +235,13 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
     if (cols == 0 || cols % chunk_elems) return false;
     const uint64_t row_chunks = cols / per_chunk;
-    // tiles of up to 1024 chunks; a row's ragged last one is a launch of its own with idle lanes
-    if (row_chunks < 512) return false;  // callers narrow this further with flat_rows_pay()
-    a->ragged_share = static_cast<double>((row_chunks + 1023) / 1024 * 1024 - row_chunks) / static_cast<double>(row_chunks);
-    if (rows_f > 65535ull * 65535ull) return false;
+    // steps of 256 chunks, a row's last one with idle lanes where 256 does not divide the row.  Measured on
+    // pitched bf16 rows against the row kernels: ahead or level down to rows of 320 chunks (idle lanes 60 % of
+    // the row: quantize 21 against 29 us, dequantize 21.5 against 21.7 us); shorter ragged rows stay there.
+    if (row_chunks < 256) return false;
+    const uint64_t row_steps = (row_chunks + 255) / 256;
+    if ((row_steps * 256 - row_chunks) * 10 > row_chunks * 6) return false;
+    if (rows_f * row_steps >= (1ull << 31)) return false;
     a->scale_in_pitch = a->scale_out_pitch = 0;
     a->scale_rows = 1;
     if (!p.tensor_level) {
@@ -512,8 +503,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     }
     cq::FlatArgs fr{};
     if (flat_words == 0 && flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
-                                        dtype_size(pd), true, &fr) &&
-        flat_rows_pay(fr, input_dtype, true)) {
+                                        dtype_size(pd), true, &fr)) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_in = scale->ptr;
@@ -587,8 +577,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
     cq::FlatArgs fr{};
-    if (flat_words == 0 && flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr) &&
-        flat_rows_pay(fr, output_dtype, false)) {
+    if (flat_words == 0 && flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr)) {
         fr.input = values->ptr;
         fr.output = output->ptr;
         fr.scale_in = params->ptr;
@@ -717,14 +706,15 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
         a.range = p.range;
         return hip_status(cq::launch_scales_flat(stream, input_dtype, a));
     }
-    // pitched rows of at least one tile, 1-D blocks: the same kernel row by row
+    // pitched rows of at least a step of 256 chunks, 1-D blocks: the same kernel over the rows' steps
     uint64_t rows_f, rows_s, pitch_f, pitch_s;
     const uint64_t row_chunks = input->shape[input->rank - 1] / (16 / dtype_size(input_dtype));
     if (!p.tensor_level && p.last_dim_blocks && p.rank >= 2 && cq::flat_block_supported(input_dtype, p.block_last) &&
         uniform_rows(input, &rows_f, &pitch_f) && uniform_rows(scales, &rows_s, &pitch_s) && rows_f == rows_s &&
-        rows_f <= 65535ull * 65535ull && aligned(input->ptr, 16) && (pitch_f * dtype_size(input_dtype)) % 16 == 0 &&
-        input->shape[input->rank - 1] % (16 / dtype_size(input_dtype)) == 0 && row_chunks >= 1024 &&
-        (row_chunks + 1023) / 1024 * 1024 <= row_chunks + row_chunks / 8) {
+        aligned(input->ptr, 16) && (pitch_f * dtype_size(input_dtype)) % 16 == 0 &&
+        input->shape[input->rank - 1] % (16 / dtype_size(input_dtype)) == 0 && row_chunks >= 256 &&
+        ((row_chunks + 255) / 256 * 256 - row_chunks) * 10 <= row_chunks * 6 &&
+        rows_f * ((row_chunks + 255) / 256) < (1ull << 31)) {
         cq::FlatArgs a{};
         a.input = input->ptr;
         a.scale_out = scales->ptr;
@@ -771,8 +761,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
 
     // pitched rows with 1-D blocks: the same fused kernel, row by row
     cq::FlatArgs fr{};
-    if (!p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) &&
-        flat_rows_pay(fr, input_dtype, true)) {
+    if (!p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr)) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_out = out_scale->ptr;
@@ -832,8 +821,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, a));
         if (st != CQ_OK) return st;
         flat_words = flat_chunks * per_chunk / p.nq;
-    } else if (p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) &&
-               flat_rows_pay(fr, input_dtype, true)) {
+    } else if (p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr)) {
         // per tensor on pitched rows: the same two passes, the second one row by row
         uint32_t num_partials = 0;
         st = absmax_partials(stream, p, scheme, input, input_dtype, workspace, workspace_bytes, &num_partials);

@@ -38,7 +38,6 @@ struct FlatArgs {
     // the four tensors (pitched rows); 0 or 1: one contiguous run
     uint64_t rows, in_pitch, out_pitch, scale_in_pitch, scale_out_pitch;
     uint32_t scale_rows;  // rows > 1, given scales: blocks of this many rows share a row of scales (0 or 1: one)
-    double ragged_share;  // filled by the planner: idle share of a row's last tile, relative to the row
     uint32_t block;       // elements per block, 0 = per-tensor
     int param_dtype;      // cq_dtype of the stored scales
     int encoding;         // 0 two's-complement fields (U32 store, native i8); 1 e4m3, 2 e5m2 bytes; 3 e2m1 nibbles

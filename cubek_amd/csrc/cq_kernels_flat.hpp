@@ -9,8 +9,9 @@
 // its abs-max is a DPP butterfly, no LDS.  Codes narrower than a word
 // (chunk bits 16 or 8) are OR-combined across 2 or 4 lanes before one store.
 //
-// quantize_flat_rows_kernel / dequantize_flat_rows_kernel run the same bodies over pitched rows
-// (grid y, z = the row), each row a run of chunks of its own.
+// quantize_flat_rows_kernel / dequantize_flat_rows_kernel run the same bodies over pitched rows: a
+// row is a whole number of steps (kThreads chunks, the last one of a row may be partial), and a
+// workgroup's kUnroll steps may lie in different rows.
 //
 // HBM traffic per element is the algorithmic minimum: the input once, the
 // codes once, one scale per block.  Loads and stores carry the non-temporal
@@ -29,6 +30,157 @@ enum ScaleSrc : int {
                            // kernel (pass 2) finishes the reduction, derives the scale and quantizes
 };
 
+// ---- where the steps of a workgroup's tile lie -------------------------------------------------
+// A tile is kUnroll steps of kThreads consecutive chunks, one per lane.  The kernel bodies ask a
+// geometry, for each step u, for the (wave-uniform) base pointers of the tensors, the lane's chunk
+// index relative to them (`chunk`; `load_chunk` is the same clamped into the data, for lanes past
+// the end), whether the lane holds data (`live`) and whether the step's row starts its blocks
+// (`first_row`).  Scale i of a base pointer belongs to chunks [i * kDiv, (i + 1) * kDiv).
+
+// One contiguous run of chunks [chunk_begin, chunk_end): the same pointers for every step.
+template <int kUnroll, int kThreads, bool kChecked>
+struct RunSteps;
+struct RunGeo {
+    const void* in;
+    void* out;
+    const void* scale_in;
+    void* scale_out;
+    uint64_t chunk_begin, chunk_end;
+    template <int kUnroll, int kThreads, bool kChecked>
+    using Steps = RunSteps<kUnroll, kThreads, kChecked>;
+};
+template <int kUnroll, int kThreads, bool kChecked>
+struct RunSteps {
+    using Index = uint64_t;
+    const RunGeo& g;
+    const uint64_t first;
+    __device__ __forceinline__ RunSteps(const RunGeo& geo, uint32_t tile)
+        : g(geo), first(geo.chunk_begin + static_cast<uint64_t>(tile) * (kThreads * kUnroll) + threadIdx.x) {}
+    __device__ __forceinline__ Index chunk(int u) const { return first + static_cast<uint64_t>(u) * kThreads; }
+    // checked launches let out-of-range lanes re-read the last chunk instead of branching
+    __device__ __forceinline__ Index load_chunk(int u) const {
+        const Index c = chunk(u);
+        return kChecked ? (c < g.chunk_end ? c : g.chunk_end - 1) : c;
+    }
+    __device__ __forceinline__ bool live(int u) const { return !kChecked || chunk(u) < g.chunk_end; }
+    __device__ __forceinline__ bool first_row(int) const { return true; }
+    __device__ __forceinline__ const void* in(int) const { return g.in; }
+    __device__ __forceinline__ void* out(int) const { return g.out; }
+    __device__ __forceinline__ const void* scale_in(int) const { return g.scale_in; }
+    __device__ __forceinline__ void* scale_out(int) const { return g.scale_out; }
+};
+
+// Pitched rows.  A row of `row_chunks` chunks is `steps_per_row` steps, the last one partial where
+// kThreads does not divide the row; step g of the launch is step g % steps_per_row of row
+// g / steps_per_row.  The rows of the four tensors start `in` / `out` / `scale_in` / `scale_out`
+// bytes apart, and blocks of `scale_rows` rows (by a lane group of columns) share a row of scales
+// (given scales only: a fused abs-max sees one row).
+struct FlatRows {
+    uint32_t row_chunks, steps_per_row, total_steps;  // total_steps < 2^31
+    uint32_t scale_rows;  // >= 1
+    // n / steps_per_row and n / scale_rows for n < 2^31 as (n * magic) >> shift (see magic_of())
+    uint32_t steps_magic, steps_shift, scale_magic, scale_shift;
+    uint64_t in, out, scale_in, scale_out;
+};
+// Division by an invariant d >= 1 of any n < 2^31: with s = ceil(log2 d) and
+// magic = floor(2^(31+s) / d) + 1 (which fits 32 bits), n / d == (n * magic) >> (31 + s).
+inline void magic_of(uint32_t d, uint32_t* magic, uint32_t* shift) {
+    uint32_t s = 0;
+    while ((1ull << s) < d) s++;
+    *magic = static_cast<uint32_t>((1ull << (31 + s)) / d + 1);
+    *shift = 31 + s;
+}
+__device__ __forceinline__ uint32_t magic_div(uint32_t n, uint32_t magic, uint32_t shift) {
+    return static_cast<uint32_t>((static_cast<uint64_t>(n) * magic) >> shift);
+}
+template <int kUnroll, int kThreads, bool kChecked, int kInBytes, int kOutBytes, int kDiv>
+struct RowSteps;
+// kInBytes / kOutBytes: bytes of a chunk in `in` / `out`; kDiv: chunks per scale, 0 = one scale per tensor
+template <int kInBytes, int kOutBytes, int kDiv>
+struct RowsGeo {
+    const void* in;
+    void* out;
+    const void* scale_in;
+    void* scale_out;
+    uint32_t step_begin;  // first step of the launch
+    uint32_t scale_in_bytes, scale_out_bytes;  // bytes per scale
+    FlatRows rows;
+    template <int kUnroll, int kThreads, bool kChecked>
+    using Steps = RowSteps<kUnroll, kThreads, kChecked, kInBytes, kOutBytes, kDiv>;
+};
+// The row and column of a step are wave-uniform, so each step's pointers are scalar arithmetic on
+// the base pointers (the first step's by a multiplication, the following ones count on from it),
+// and the lane's index is just its number in the workgroup.
+template <int kUnroll, int kThreads, bool kChecked, int kInBytes, int kOutBytes, int kDiv>
+struct RowSteps {
+    using Index = uint32_t;
+    const char* in_[kUnroll];
+    char* out_[kUnroll];
+    const char* scale_in_[kUnroll];
+    char* scale_out_[kUnroll];
+    uint32_t last_[kUnroll];  // last lane of the step that holds a chunk of its row
+    bool valid_[kUnroll];     // the step exists (a checked launch may run past the last step)
+    bool first_[kUnroll];
+    __device__ __forceinline__ RowSteps(const RowsGeo<kInBytes, kOutBytes, kDiv>& g, uint32_t tile) {
+        const FlatRows& r = g.rows;
+        const uint32_t step = g.step_begin + tile * kUnroll;
+        const uint32_t row = magic_div(step, r.steps_magic, r.steps_shift);
+        uint32_t col = step - row * r.steps_per_row;
+        const uint32_t scale_row = magic_div(row, r.scale_magic, r.scale_shift);
+        uint32_t sub = row - scale_row * r.scale_rows;
+        bool first = kDiv == 0 ? step == 0 : sub == 0;
+        // bytes from one step to the next one of the same row, and back to the row's first step
+        constexpr uint64_t kScalesPerStep = kDiv == 0 ? 0 : kThreads / (kDiv == 0 ? 1 : kDiv);
+        const uint64_t scale_in_step = kScalesPerStep * g.scale_in_bytes, scale_out_step = kScalesPerStep * g.scale_out_bytes;
+        const uint64_t back = r.steps_per_row - 1;
+        const char* in = static_cast<const char*>(g.in) + row * r.in + static_cast<uint64_t>(col) * (kThreads * kInBytes);
+        char* out = static_cast<char*>(g.out) + row * r.out + static_cast<uint64_t>(col) * (kThreads * kOutBytes);
+        const char* scale_in = static_cast<const char*>(g.scale_in) + scale_row * r.scale_in + col * scale_in_step;
+        char* scale_out = static_cast<char*>(g.scale_out) + scale_row * r.scale_out + col * scale_out_step;
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            valid_[u] = !kChecked || u == 0 || step + u < r.total_steps;
+            in_[u] = in;
+            out_[u] = out;
+            scale_in_[u] = scale_in;
+            scale_out_[u] = g.scale_out == nullptr ? nullptr : scale_out;
+            const uint32_t left = r.row_chunks - col * kThreads;
+            last_[u] = left < kThreads ? left - 1 : kThreads - 1;
+            first_[u] = first && valid_[u];
+            // past the launch's last step the addresses stay where they are: on data
+            if (kChecked && step + u + 1 >= r.total_steps) continue;
+            if (++col != r.steps_per_row) {
+                in += kThreads * kInBytes;
+                out += kThreads * kOutBytes;
+                scale_in += scale_in_step;
+                scale_out += scale_out_step;
+            } else {  // on to the next row
+                col = 0;
+                in += r.in - back * (kThreads * kInBytes);
+                out += r.out - back * (kThreads * kOutBytes);
+                scale_in -= back * scale_in_step;
+                scale_out -= back * scale_out_step;
+                if (++sub == r.scale_rows) {
+                    sub = 0;
+                    scale_in += r.scale_in;
+                    scale_out += r.scale_out;
+                }
+                first = kDiv == 0 ? false : sub == 0;
+            }
+        }
+    }
+    __device__ __forceinline__ Index chunk(int) const { return threadIdx.x; }
+    __device__ __forceinline__ Index load_chunk(int u) const {
+        return kChecked ? (threadIdx.x < last_[u] ? threadIdx.x : last_[u]) : threadIdx.x;
+    }
+    __device__ __forceinline__ bool live(int u) const { return !kChecked || (valid_[u] && threadIdx.x <= last_[u]); }
+    __device__ __forceinline__ bool first_row(int u) const { return first_[u]; }
+    __device__ __forceinline__ const void* in(int u) const { return in_[u]; }
+    __device__ __forceinline__ void* out(int u) const { return out_[u]; }
+    __device__ __forceinline__ const void* scale_in(int u) const { return scale_in_[u]; }
+    __device__ __forceinline__ void* scale_out(int u) const { return scale_out_[u]; }
+};
+
 // kParamF32: the stored scales are f32 (the common case, resolved at compile
 //            time); otherwise `param_dtype_rt` selects f16 / bf16 at run time.
 // kWide    : the value range does not fit its field (E4M3 / E5M2 in 8 bits).
@@ -36,21 +188,16 @@ enum ScaleSrc : int {
 //            are clamped and stores masked.  Full tiles use the unchecked variant.
 // kEnc     : stored encoding (kEncInt for the U32 store and native i8; e4m3 / e5m2 /
 //            e2m1 for the native float stores, where kBits is the stored width).
-// `first_row`: false in the launches over rows (quantize_flat_rows_kernel) for rows that do not start a
-// block (per tensor: every row but the first); only the scale store looks at it.
 template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
-          int kThreads, bool kChecked, int kEnc>
-__device__ __forceinline__ void quantize_flat_body(
-    const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
-    void* __restrict__ scale_out, int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end,
-    const QuantParams& qp, uint32_t num_partials, bool first_row) {
+          int kThreads, bool kChecked, int kEnc, class Geo>
+__device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dtype_rt, const QuantParams& qp,
+                                                   uint32_t num_partials) {
     constexpr bool kDynamic = kScaleSrc == kScaleDynamic;
     static_assert(kScaleSrc != kScalePartials || kGroup == 0, "partials feed the per-tensor scale only");
     constexpr int kDiv = kGroup == 0 ? 1 : kGroup;
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;  // 64, 32, 16 or 8
     const int param_dtype = kParamF32 ? static_cast<int>(CQ_F32) : param_dtype_rt;
-    const auto load_scale = [&](uint64_t i) { return F::load(scale_in, i); };
     // Pass 2 of the per-tensor reduction walks the tiles last to first: pass 1 has just read the
     // tensor first to last, so what it read last is what the L2 caches still hold.  Groups of
     // eight consecutive tiles keep their places, because workgroup i runs on XCD i % 8 and tile
@@ -60,23 +207,21 @@ __device__ __forceinline__ void quantize_flat_body(
         const uint32_t whole = gridDim.x & ~7u;
         if (tile < whole) tile = (whole - 8 - (tile & ~7u)) + (tile & 7u);
     }
-    const uint64_t first = chunk_begin + static_cast<uint64_t>(tile) * (kThreads * kUnroll) + threadIdx.x;
+    const typename Geo::template Steps<kUnroll, kThreads, kChecked> at(geo, tile);
 
-    // All kUnroll loads are issued back to back.  Checked launches let
-    // out-of-range lanes re-read the last chunk instead of branching.
+    // All kUnroll loads are issued back to back.
     u32x4 raw[kUnroll];
     float s_given[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-        uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
-        if (kChecked) c = c < chunk_end ? c : chunk_end - 1;
-        raw[u] = stream_load(in + c);
-        if constexpr (!kDynamic && kGroup != 0 && kScaleSrc != kScalePartials) s_given[u] = load_scale(c / kDiv);
+        const auto c = at.load_chunk(u);
+        raw[u] = stream_load(static_cast<const u32x4*>(at.in(u)) + c);
+        if constexpr (!kDynamic && kGroup != 0 && kScaleSrc != kScalePartials) s_given[u] = F::load(at.scale_in(u), c / kDiv);
     }
     if constexpr (kScaleSrc == kScalePartials) {
         // second pass of the grid reduction: every workgroup reduces the (<= a few
         // hundred) partial maxima again — max is exact, so all agree bit for bit
-        const float* partials = static_cast<const float*>(scale_in);
+        const float* partials = static_cast<const float*>(geo.scale_in);
         float amax = 0.0f;
         for (uint32_t i = threadIdx.x; i < num_partials; i += kThreads) amax = fmaxf(amax, partials[i]);
         amax = group_max<64>(amax);
@@ -90,7 +235,7 @@ __device__ __forceinline__ void quantize_flat_body(
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) s_given[u] = s;
     } else if constexpr (!kDynamic && kGroup == 0) {
-        const float s = load_scale(0);  // one scale for the whole tensor
+        const float s = F::load(geo.scale_in, 0);  // one scale for the whole tensor
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) s_given[u] = s;
     }
@@ -98,8 +243,10 @@ __device__ __forceinline__ void quantize_flat_body(
 
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-        const uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
-        const bool live = !kChecked || c < chunk_end;
+        const auto c = at.chunk(u);
+        const bool live = at.live(u);
+        uint32_t* const out = static_cast<uint32_t*>(at.out(u));
+        void* const scale_out = at.scale_out(u);
         float v[kN];
         F::unpack(raw[u], v);
 
@@ -118,8 +265,8 @@ __device__ __forceinline__ void quantize_flat_body(
         }
         // write_scale (src/quantize.rs:83-98): FS(scale), stored by the block's first lane
         const float s_fs = round_to_dtype(param_dtype, s_f);
-        const uint64_t si = kGroup == 0 ? 0 : c / kDiv;
-        const bool block_start = first_row && (kGroup == 0 ? c == 0 : (c % kDiv) == 0);
+        const auto si = kGroup == 0 ? 0 : c / kDiv;
+        const bool block_start = at.first_row(u) && (kGroup == 0 ? c == 0 : (c % kDiv) == 0);
         if (scale_out != nullptr && live && block_start) store_dtype(param_dtype, scale_out, si, s_fs);
         // divisor F(FS(scale)); s_f is an F value, so f32 params leave it unchanged
         float d = s_fs;
@@ -153,51 +300,40 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
     void* __restrict__ scale_out, int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end,
     QuantParams qp, uint32_t num_partials) {
+    const RunGeo geo{in, out, scale_in, scale_out, chunk_begin, chunk_end};
     quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParamF32, kWide, kUnroll, kThreads, kChecked, kEnc>(
-        in, out, scale_in, scale_out, param_dtype_rt, chunk_begin, chunk_end, qp, num_partials, true);
+        geo, param_dtype_rt, qp, num_partials);
 }
 
-// Pitched rows: grid y, z = the row; a row is a run of chunks [chunk_begin, chunk_end) of its own, and
-// the rows of the four tensors start `rows.*` bytes apart; blocks of rows.scale_rows rows by a lane group
-// of columns share their scale (given scales only: a fused abs-max sees one row).  A kernel of its own so
-// that the launches over one contiguous run carry none of this in their prologue.
-struct FlatRows {
-    uint32_t count;
-    uint32_t scale_rows;  // rows that share a row of scales (blocks of that many rows); >= 1
-    uint64_t in, out, scale_in, scale_out;
-};
+// Pitched rows, from step `step_begin` of the launch on.  A kernel of its own so that the launches
+// over one contiguous run carry none of the row arithmetic in their prologue.
 template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
           int kThreads, bool kChecked, int kEnc = kEncInt>
 __global__ __launch_bounds__(kThreads) void quantize_flat_rows_kernel(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
-    void* __restrict__ scale_out, int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end,
-    QuantParams qp, uint32_t num_partials, FlatRows rows) {
-    const uint32_t row = blockIdx.y + blockIdx.z * gridDim.y;
-    if (row >= rows.count) return;
+    void* __restrict__ scale_out, int param_dtype_rt, uint32_t step_begin, QuantParams qp, uint32_t num_partials,
+    FlatRows rows) {
+    const uint32_t out_scale_bytes = (kParamF32 || param_dtype_rt == CQ_F32) ? 4 : 2;
+    const RowsGeo<16, F::kPerChunk * kBits / 8, kGroup> geo{in, out, scale_in, scale_out, step_begin,
+                                                            F::kBytes, out_scale_bytes, rows};
     quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParamF32, kWide, kUnroll, kThreads, kChecked, kEnc>(
-        reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(in) + row * rows.in),
-        reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(out) + row * rows.out),
-        static_cast<const char*>(scale_in) + (row / rows.scale_rows) * rows.scale_in,
-        scale_out == nullptr ? nullptr : static_cast<char*>(scale_out) + (row / rows.scale_rows) * rows.scale_out,
-        param_dtype_rt, chunk_begin, chunk_end, qp, num_partials, kGroup == 0 ? row == 0 : row % rows.scale_rows == 0);
+        geo, param_dtype_rt, qp, num_partials);
 }
 
-template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked, int kEnc>
-__device__ __forceinline__ void dequantize_flat_body(
-    const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params,
-    int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end) {
+// `scale_in` of the geometry holds the stored scales
+template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked, int kEnc, class Geo>
+__device__ __forceinline__ void dequantize_flat_body(const Geo& geo, int param_dtype_rt) {
     const int param_dtype = kParamF32 ? static_cast<int>(CQ_F32) : param_dtype_rt;
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;
-    const uint64_t first =
-        chunk_begin + static_cast<uint64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+    const typename Geo::template Steps<kUnroll, kThreads, kChecked> at(geo, blockIdx.x);
 
     uint32_t w0[kUnroll], w1[kUnroll];
     float sc[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-        uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
-        if (kChecked) c = c < chunk_end ? c : chunk_end - 1;  // clamp instead of branching
+        const auto c = at.load_chunk(u);
+        const uint32_t* const in = static_cast<const uint32_t*>(at.in(u));
         w1[u] = 0;
         if constexpr (kChunkBits == 64) {
             u32x2 w = stream_load(reinterpret_cast<const u32x2*>(in) + c);
@@ -210,13 +346,12 @@ __device__ __forceinline__ void dequantize_flat_body(
             uint32_t w = in[c / kLanesPerWord];  // neighbouring lanes share the word
             w0[u] = w >> ((static_cast<uint32_t>(c) & (kLanesPerWord - 1)) * kChunkBits);
         }
-        const uint64_t si = kGroup == 0 ? 0 : c / (kGroup == 0 ? 1 : kGroup);
-        sc[u] = F::round(load_dtype(param_dtype, params, si));  // Line::cast_from(scale)
+        const auto si = kGroup == 0 ? 0 : c / (kGroup == 0 ? 1 : kGroup);
+        sc[u] = F::round(load_dtype(param_dtype, at.scale_in(u), si));  // Line::cast_from(scale)
     }
     __builtin_amdgcn_sched_barrier(0);  // keep every load ahead of the arithmetic
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-        const uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
         float y[kN];
         if constexpr (kChunkBits == 64) {
             decode_fields<kEnc, kBits, 4>(w0[u], y);
@@ -226,7 +361,7 @@ __device__ __forceinline__ void dequantize_flat_body(
         }
 #pragma unroll
         for (int i = 0; i < kN; i++) y[i] = sc[u] * y[i];
-        if (!kChecked || c < chunk_end) stream_store(F::pack(y), out + c);  // pack rounds to F
+        if (at.live(u)) stream_store(F::pack(y), static_cast<u32x4*>(at.out(u)) + at.chunk(u));  // pack rounds to F
     }
 }
 
@@ -235,39 +370,31 @@ template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThre
 __global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
     const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params,
     int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end) {
-    dequantize_flat_body<F, kBits, kGroup, kParamF32, kUnroll, kThreads, kChecked, kEnc>(in, out, params, param_dtype_rt,
-                                                                                         chunk_begin, chunk_end);
+    const RunGeo geo{in, out, params, nullptr, chunk_begin, chunk_end};
+    dequantize_flat_body<F, kBits, kGroup, kParamF32, kUnroll, kThreads, kChecked, kEnc>(geo, param_dtype_rt);
 }
 template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked,
           int kEnc = kEncInt>
 __global__ __launch_bounds__(kThreads) void dequantize_flat_rows_kernel(
     const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params,
-    int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end, FlatRows rows) {
-    const uint32_t row = blockIdx.y + blockIdx.z * gridDim.y;
-    if (row >= rows.count) return;
-    dequantize_flat_body<F, kBits, kGroup, kParamF32, kUnroll, kThreads, kChecked, kEnc>(
-        reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(in) + row * rows.in),
-        reinterpret_cast<u32x4*>(reinterpret_cast<char*>(out) + row * rows.out),
-        static_cast<const char*>(params) + (row / rows.scale_rows) * rows.scale_in, param_dtype_rt, chunk_begin, chunk_end);
+    int param_dtype_rt, uint32_t step_begin, FlatRows rows) {
+    const uint32_t param_bytes = (kParamF32 || param_dtype_rt == CQ_F32) ? 4 : 2;
+    const RowsGeo<F::kPerChunk * kBits / 8, 16, kGroup> geo{in, out, params, nullptr, step_begin, param_bytes, 0, rows};
+    dequantize_flat_body<F, kBits, kGroup, kParamF32, kUnroll, kThreads, kChecked, kEnc>(geo, param_dtype_rt);
 }
 
 // Block abs-max -> scale typed like the input (what quantize takes as `scale`).
-template <class F, int kGroup, int kUnroll, int kThreads>
-__device__ __forceinline__ void scales_flat_body(const u32x4* __restrict__ in, void* __restrict__ scales,
-                                                 uint64_t num_chunks, const QuantParams& qp) {
+template <class F, int kGroup, int kUnroll, int kThreads, class Geo>
+__device__ __forceinline__ void scales_flat_body(const Geo& geo, const QuantParams& qp) {
     constexpr int kN = F::kPerChunk;
-    const uint64_t first = static_cast<uint64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
-    const uint64_t last = num_chunks - 1;
+    const typename Geo::template Steps<kUnroll, kThreads, true> at(geo, blockIdx.x);
     u32x4 raw[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; u++) {
-        uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
-        raw[u] = stream_load(in + (c < num_chunks ? c : last));
-    }
+    for (int u = 0; u < kUnroll; u++) raw[u] = stream_load(static_cast<const u32x4*>(at.in(u)) + at.load_chunk(u));
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-        const uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
+        const auto c = at.chunk(u);
         float v[kN];
         F::unpack(raw[u], v);
         float amax = 0.0f;
@@ -276,7 +403,7 @@ __device__ __forceinline__ void scales_flat_body(const u32x4* __restrict__ in, v
         amax = group_max<kGroup>(amax);
         const float s32 = absmax_is_tame(amax) ? scale_from_absmax_tame(amax, qp)
                                                : scale_from_absmax(amax, qp.width);
-        if (c < num_chunks && (c % kGroup) == 0) F::store(scales, c / kGroup, s32);
+        if (at.live(u) && (c % kGroup) == 0) F::store(at.scale_out(u), c / kGroup, s32);
     }
 }
 
@@ -284,18 +411,16 @@ template <class F, int kGroup, int kUnroll, int kThreads>
 __global__ __launch_bounds__(kThreads) void scales_flat_kernel(const u32x4* __restrict__ in,
                                                                void* __restrict__ scales,
                                                                uint64_t num_chunks, QuantParams qp) {
-    scales_flat_body<F, kGroup, kUnroll, kThreads>(in, scales, num_chunks, qp);
+    const RunGeo geo{in, nullptr, nullptr, scales, 0, num_chunks};
+    scales_flat_body<F, kGroup, kUnroll, kThreads>(geo, qp);
 }
-// pitched rows (grid y, z = the row): rows.in / rows.scale_out bytes between the rows of the two tensors
+// pitched rows: rows.in / rows.scale_out bytes between the rows of the two tensors
 template <class F, int kGroup, int kUnroll, int kThreads>
 __global__ __launch_bounds__(kThreads) void scales_flat_rows_kernel(const u32x4* __restrict__ in,
-                                                                    void* __restrict__ scales,
-                                                                    uint64_t num_chunks, QuantParams qp, FlatRows rows) {
-    const uint32_t row = blockIdx.y + blockIdx.z * gridDim.y;
-    if (row >= rows.count) return;
-    scales_flat_body<F, kGroup, kUnroll, kThreads>(
-        reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(in) + row * rows.in),
-        static_cast<char*>(scales) + (row / rows.scale_rows) * rows.scale_out, num_chunks, qp);
+                                                                    void* __restrict__ scales, QuantParams qp,
+                                                                    FlatRows rows) {
+    const RowsGeo<16, 0, kGroup> geo{in, nullptr, nullptr, scales, 0, 0, F::kBytes, rows};
+    scales_flat_body<F, kGroup, kUnroll, kThreads>(geo, qp);
 }
 
 // Per-tensor abs-max, pass 1: grid-stride over chunks with kUnroll 16-byte loads

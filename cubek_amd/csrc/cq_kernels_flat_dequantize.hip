@@ -9,22 +9,21 @@ hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
     auto in = static_cast<const uint32_t*>(a.input);
     auto out = static_cast<u32x4*>(a.output);
     const bool p32 = a.param_dtype == CQ_F32;
-    return launch_tiles(a.num_chunks, kUnrollD<F, kBits, kGroup>, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
-        auto kernel =
-            checked ? (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F, kBits, kGroup>, kThreads, true, kEnc>
-                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F, kBits, kGroup>, kThreads, true, kEnc>)
-                    : (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kUnrollD<F, kBits, kGroup>, kThreads, false, kEnc>
-                           : dequantize_flat_kernel<F, kBits, kGroup, false, kUnrollD<F, kBits, kGroup>, kThreads, false, kEnc>);
-        if (a.rows > 1) {
-            constexpr int kU = kUnrollD<F, kBits, kGroup>;
-            auto rows_kernel = checked ? (p32 ? dequantize_flat_rows_kernel<F, kBits, kGroup, true, kU, kThreads, true, kEnc>
-                                              : dequantize_flat_rows_kernel<F, kBits, kGroup, false, kU, kThreads, true, kEnc>)
-                                       : (p32 ? dequantize_flat_rows_kernel<F, kBits, kGroup, true, kU, kThreads, false, kEnc>
-                                              : dequantize_flat_rows_kernel<F, kBits, kGroup, false, kU, kThreads, false, kEnc>);
-            hipLaunchKernelGGL(rows_kernel, rows_grid(grid, a), dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, begin,
-                               end, flat_rows(a));
-            return;
-        }
+    constexpr int kU = kUnrollD<F, kBits, kGroup>;
+    if (a.rows > 1)
+        return launch_row_steps(a, kU, [&](bool checked, uint32_t grid, uint32_t step_begin) {
+            auto kernel = checked ? (p32 ? dequantize_flat_rows_kernel<F, kBits, kGroup, true, kU, kThreads, true, kEnc>
+                                         : dequantize_flat_rows_kernel<F, kBits, kGroup, false, kU, kThreads, true, kEnc>)
+                                  : (p32 ? dequantize_flat_rows_kernel<F, kBits, kGroup, true, kU, kThreads, false, kEnc>
+                                         : dequantize_flat_rows_kernel<F, kBits, kGroup, false, kU, kThreads, false, kEnc>);
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, step_begin,
+                               flat_rows(a));
+        });
+    return launch_tiles(a.num_chunks, kU, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
+        auto kernel = checked ? (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kU, kThreads, true, kEnc>
+                                     : dequantize_flat_kernel<F, kBits, kGroup, false, kU, kThreads, true, kEnc>)
+                              : (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kU, kThreads, false, kEnc>
+                                     : dequantize_flat_kernel<F, kBits, kGroup, false, kU, kThreads, false, kEnc>);
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, begin, end);
     });
 }

@@ -40,14 +40,20 @@ constexpr int kUnrollQ = 4;
 template <class F, int kBits, int kGroup>
 constexpr int kUnrollD = F::kBytes != 4 ? 2 : ((kBits == 8 || (kBits == 4 && kGroup > 0 && kGroup <= 8)) ? 2 : 4);
 
-// grid of a launch of `tiles` workgroups per row, and the rows as the kernels take them
-dim3 rows_grid(uint32_t tiles, const FlatArgs& a) {
-    const uint32_t y = a.rows < 65535 ? static_cast<uint32_t>(a.rows) : 65535u;
-    return dim3(tiles, y, static_cast<uint32_t>((a.rows + y - 1) / y));
-}
+// the rows of a launch as the kernels take them: steps of kThreads chunks, a row's last one partial
 FlatRows flat_rows(const FlatArgs& a) {
-    return FlatRows{static_cast<uint32_t>(a.rows), a.scale_rows > 1 ? a.scale_rows : 1u, a.in_pitch, a.out_pitch,
-                    a.scale_in_pitch, a.scale_out_pitch};
+    FlatRows r;
+    r.row_chunks = static_cast<uint32_t>(a.num_chunks);
+    r.steps_per_row = static_cast<uint32_t>((a.num_chunks + kThreads - 1) / kThreads);
+    r.total_steps = static_cast<uint32_t>(a.rows * r.steps_per_row);
+    r.scale_rows = a.scale_rows > 1 ? a.scale_rows : 1u;
+    magic_of(r.steps_per_row, &r.steps_magic, &r.steps_shift);
+    magic_of(r.scale_rows, &r.scale_magic, &r.scale_shift);
+    r.in = a.in_pitch;
+    r.out = a.out_pitch;
+    r.scale_in = a.scale_in_pitch;
+    r.scale_out = a.scale_out_pitch;
+    return r;
 }
 
 QuantParams quant_params(const Range& r) {
@@ -77,6 +83,28 @@ hipError_t launch_tiles(uint64_t num_chunks, int unroll, LaunchFn launch) {
     return hipSuccess;
 }
 
+// The same over pitched rows: `launch(checked, grid, step_begin)`.  Rows of whole steps run
+// unchecked but for the workgroup that holds the launch's last steps; other rows run checked throughout.
+template <class LaunchFn>
+hipError_t launch_row_steps(const FlatArgs& a, int unroll, LaunchFn launch) {
+    const uint32_t total = flat_rows(a).total_steps;
+    if (a.num_chunks % kThreads != 0) {
+        launch(true, (total + unroll - 1) / unroll, 0u);
+        return hipGetLastError();
+    }
+    const uint32_t full = total / unroll;
+    if (full > 0) {
+        launch(false, full, 0u);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (full * unroll < total) {
+        launch(true, 1u, full * unroll);
+        return hipGetLastError();
+    }
+    return hipSuccess;
+}
+
 template <class F, int kBits, int kGroup, int kSrc, bool kWide, int kEnc>
 hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
     // scale sources that exist: per-block launches compute the scale or read the
@@ -88,22 +116,22 @@ hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
         auto out = static_cast<uint32_t*>(a.output);
         const QuantParams qp = quant_params(a.range);
         const bool p32 = a.param_dtype == CQ_F32;
+        if (a.rows > 1)
+            return launch_row_steps(a, kUnrollQ, [&](bool checked, uint32_t grid, uint32_t step_begin) {
+                auto kernel =
+                    checked ? (p32 ? quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, true, kEnc>
+                                   : quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, true, kEnc>)
+                            : (p32 ? quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false, kEnc>
+                                   : quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false, kEnc>);
+                hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out, a.param_dtype,
+                                   step_begin, qp, a.num_partials, flat_rows(a));
+            });
         return launch_tiles(a.num_chunks, kUnrollQ, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
             auto kernel =
                 checked ? (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, true, kEnc>
                                : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, true, kEnc>)
                         : (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false, kEnc>
                                : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false, kEnc>);
-            if (a.rows > 1) {
-                auto rows_kernel =
-                    checked ? (p32 ? quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, true, kEnc>
-                                   : quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, true, kEnc>)
-                            : (p32 ? quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false, kEnc>
-                                   : quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false, kEnc>);
-                hipLaunchKernelGGL(rows_kernel, rows_grid(grid, a), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
-                                   a.param_dtype, begin, end, qp, a.num_partials, flat_rows(a));
-                return;
-            }
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
                                a.param_dtype, begin, end, qp, a.num_partials);
         });

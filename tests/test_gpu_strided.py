@@ -106,19 +106,20 @@ def test_strided_value_tensors(gpu, oracle, elem, name, scheme):
 @pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
 @pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
 def test_long_pitched_rows(gpu, oracle, elem, name, scheme):
-    """Rows long enough for the streaming kernels to take them one by one (whole tiles, and a
-    ragged last tile per row), with 1-D blocks and with blocks over the last two dimensions."""
+    """Rows of many steps of the streaming kernels (whole steps, and a partial last step per row),
+    with 1-D blocks and with blocks over the last two dimensions."""
     check_layouts(gpu, oracle, elem, name, scheme, ((4, 16384), (2, 2, 16384 + 4096 + 512)),
                   ("contiguous", "pitched", "pitched_aligned", "every_other_row"))
 
 
 @pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
 @pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
-def test_pitched_rows_of_less_than_a_tile(gpu, oracle, elem, name, scheme):
-    """Rows of 512 - 896 sixteen-byte chunks: at 640 and more the streaming quantize kernels take
-    them as one partial tile per row, at exactly 512 (16-bit floats) the dequantize kernels do; the
-    other lengths go to the row kernels."""
-    check_layouts(gpu, oracle, elem, name, scheme, ((4, 4096), (6, 5120), (2, 2, 7168), (4, 2560), (4, 2048)),
+def test_pitched_rows_of_a_few_steps(gpu, oracle, elem, name, scheme):
+    """Rows of 256 - 896 sixteen-byte chunks: the streaming kernels take them as steps of 256 chunks,
+    so one workgroup's steps lie in up to four rows (also rows of a block that share their scales),
+    a row's last step may be partial, and the launch ends on a workgroup with fewer steps than the others."""
+    check_layouts(gpu, oracle, elem, name, scheme,
+                  ((4, 4096), (6, 5120), (2, 2, 7168), (4, 2560), (6, 2048), (6, 1024), (10, 1280)),
                   ("pitched", "pitched_aligned", "every_other_row"))
 
 
