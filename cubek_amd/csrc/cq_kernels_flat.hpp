@@ -19,6 +19,7 @@
 #pragma once
 
 #include "cq_device.hpp"
+#include "cq_magic_div.hpp"
 
 namespace cq {
 
@@ -78,21 +79,10 @@ struct RunSteps {
 struct FlatRows {
     uint32_t row_chunks, steps_per_row, total_steps;  // total_steps < 2^31
     uint32_t scale_rows;  // >= 1
-    // n / steps_per_row and n / scale_rows for n < 2^31 as (n * magic) >> shift (see magic_of())
+    // n / steps_per_row and n / scale_rows for n < 2^31 as (n * magic) >> shift (cq_magic_div.hpp)
     uint32_t steps_magic, steps_shift, scale_magic, scale_shift;
     uint64_t in, out, scale_in, scale_out;
 };
-// Division by an invariant d >= 1 of any n < 2^31: with s = ceil(log2 d) and
-// magic = floor(2^(31+s) / d) + 1 (which fits 32 bits), n / d == (n * magic) >> (31 + s).
-inline void magic_of(uint32_t d, uint32_t* magic, uint32_t* shift) {
-    uint32_t s = 0;
-    while ((1ull << s) < d) s++;
-    *magic = static_cast<uint32_t>((1ull << (31 + s)) / d + 1);
-    *shift = 31 + s;
-}
-__device__ __forceinline__ uint32_t magic_div(uint32_t n, uint32_t magic, uint32_t shift) {
-    return static_cast<uint32_t>((static_cast<uint64_t>(n) * magic) >> shift);
-}
 template <int kUnroll, int kThreads, bool kChecked, int kInBytes, int kOutBytes, int kDiv>
 struct RowSteps;
 // kInBytes / kOutBytes: bytes of a chunk in `in` / `out`; kDiv: chunks per scale, 0 = one scale per tensor
