@@ -285,27 +285,29 @@ def adjacent_kernels(torch):
                     "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
     del xs, codes, scales, ys, hx, hc, hs, hy, words, bscales, hxt, hyt, hw, hb
     torch.cuda.empty_cache()
-    # the headline scheme on pitched rows: [rows, cols] views of [rows, cols + 64] buffers
+    # the headline scheme on pitched rows: [rows, cols] views of [rows, cols + 64] buffers, at the headline
+    # row length and with the same elements in rows a quarter as long
     pad = 64
-    xp = [torch.randn((rows, cols + pad), device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
-    yp = [torch.empty((rows, cols + pad), device="cuda", dtype=torch.bfloat16) for _ in range(2)]
-    words = [torch.empty((rows, cols // 8), dtype=torch.int32, device="cuda") for _ in range(2)]
-    bscales = [torch.empty((rows, cols // 32), dtype=torch.float32, device="cuda") for _ in range(2)]
-    pitched = lambda t: TensorHandleRef(h(t).handle, (rows, cols), (cols + pad, 1), 2)
-    hxp, hyp = [pitched(t) for t in xp], [pitched(t) for t in yp]
-    hw, hb = [h(t) for t in words], [h(t) for t in bscales]
-    b = rows * cols * 2 + rows * cols // 2 + bscales[0].numel() * 4
-    for label, fn in (
-            ("quantize_dynamic", lambda i: cq_quantize.launch_dynamic(client, hxp[i % sets], hw[i % 2], hb[i % 2], scheme,
-                                                                       ElemType.BF16)),
-            ("dequantize", lambda i: cq_dequantize.launch_ref(client, hw[i % 2], hyp[i % 2], hb[i % 2], scheme,
-                                                              ElemType.BF16))):
-        ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
-        out.append({"kernel": f"{label}, e2m1 blocks of 32, pitched bf16 rows: [{rows}, {cols}] view of a [{rows}, {cols + pad}] buffer",
-                    "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
-                    "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
-    del xp, yp, words, bscales, hxp, hyp, hw, hb
-    torch.cuda.empty_cache()
+    for pr, pc in ((rows, cols), (rows * 4, cols // 4)):
+        xp = [torch.randn((pr, pc + pad), device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
+        yp = [torch.empty((pr, pc + pad), device="cuda", dtype=torch.bfloat16) for _ in range(2)]
+        words = [torch.empty((pr, pc // 8), dtype=torch.int32, device="cuda") for _ in range(2)]
+        bscales = [torch.empty((pr, pc // 32), dtype=torch.float32, device="cuda") for _ in range(2)]
+        pitched = lambda t: TensorHandleRef(h(t).handle, (pr, pc), (pc + pad, 1), 2)
+        hxp, hyp = [pitched(t) for t in xp], [pitched(t) for t in yp]
+        hw, hb = [h(t) for t in words], [h(t) for t in bscales]
+        b = pr * pc * 2 + pr * pc // 2 + bscales[0].numel() * 4
+        for label, fn in (
+                ("quantize_dynamic", lambda i: cq_quantize.launch_dynamic(client, hxp[i % sets], hw[i % 2], hb[i % 2], scheme,
+                                                                           ElemType.BF16)),
+                ("dequantize", lambda i: cq_dequantize.launch_ref(client, hw[i % 2], hyp[i % 2], hb[i % 2], scheme,
+                                                                  ElemType.BF16))):
+            ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
+            out.append({"kernel": f"{label}, e2m1 blocks of 32, pitched bf16 rows: [{pr}, {pc}] view of a [{pr}, {pc + pad}] buffer",
+                        "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                        "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+        del xp, yp, words, bscales, hxp, hyp, hw, hb
+        torch.cuda.empty_cache()
     # 4-bit codes of a [rows, cols] weight, 8 per u32 word along cols, viewed transposed as [cols, rows]
     packing = 8
     srcs = [torch.randint(-2**31, 2**31 - 1, (rows, cols // packing), dtype=torch.int32, device="cuda")
