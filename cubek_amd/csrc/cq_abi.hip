@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <utility>
 
 #include "../../include/cubek_quant.h"
 #include "cq_internal.hpp"
@@ -215,6 +216,38 @@ bool uniform_rows(const cq_tensor* t, uint64_t* rows, uint64_t* pitch) {
     return true;
 }
 
+// The same with one more level: the rows in front of the last dimension as `outer_rows` groups of
+// `inner_rows` rows, `inner` elements between the rows of a group and `outer` between groups (a slice
+// along the second to last dimension, a batch of pitched matrices).  levels = 0 (a single row), 1 (one
+// uniform run: inner_rows = all rows) or 2.
+struct RowLevels {
+    int levels;
+    uint64_t rows, inner_rows, inner, outer;
+};
+bool row_levels(const cq_tensor* t, RowLevels* l) {
+    const uint32_t last = t->rank - 1;
+    if (t->shape[last] != 1 && t->strides[last] != 1) return false;
+    *l = RowLevels{0, 1, 1, 0, 0};
+    uint64_t expect = 0;
+    for (int d = static_cast<int>(last) - 1; d >= 0; d--) {
+        if (t->shape[d] == 1) continue;
+        if (t->strides[d] == 0) return false;  // broadcast rows: not for these kernels
+        if (l->levels == 0) {
+            l->levels = 1;
+            l->inner = t->strides[d];
+        } else if (t->strides[d] != expect) {
+            if (l->levels == 2) return false;
+            l->levels = 2;
+            l->inner_rows = l->rows;
+            l->outer = t->strides[d];
+        }
+        expect = t->strides[d] * t->shape[d];
+        l->rows *= t->shape[d];
+    }
+    if (l->levels < 2) l->inner_rows = l->rows;
+    return true;
+}
+
 bool scales_rows_ok(const Plan& p);
 
 // Can the flat kernels take this launch row by row?  (value tensors with a contiguous last
@@ -228,9 +261,9 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     const uint32_t last = p.rank - 1;
     const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
     const uint32_t stored = s->store == CQ_STORE_U32 ? 4u : 1u;
-    uint64_t rows_f, rows_v, pitch_f, pitch_v;
-    if (!uniform_rows(floats, &rows_f, &pitch_f) || !uniform_rows(values, &rows_v, &pitch_v) || rows_f != rows_v) return false;
-    if (!aligned(floats->ptr, 16) || !aligned(values->ptr, 8) || (pitch_f * elem) % 16 || (pitch_v * stored) % 8) return false;
+    RowLevels lf, lv, la{}, lb{};
+    if (!row_levels(floats, &lf) || !row_levels(values, &lv) || lf.rows != lv.rows) return false;
+    const uint64_t rows_f = lf.rows;
     const uint64_t cols = p.shape[last];
     const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
     if (cols == 0 || cols % chunk_elems) return false;
@@ -242,26 +275,40 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     const uint64_t row_steps = (row_chunks + 255) / 256;
     if ((row_steps * 256 - row_chunks) * 10 > row_chunks * 6) return false;
     if (rows_f * row_steps >= (1ull << 31)) return false;
-    a->scale_in_pitch = a->scale_out_pitch = 0;
     a->scale_rows = 1;
     if (!p.tensor_level) {
         // blocks along the last dimension, or (where the scales are given) over the last two: a block of
         // br rows is br rows of the launch that read the same row of scales
         const uint32_t br = p.layout.block[last - 1];
         if (!cq::flat_block_supported(dtype, p.block_last) || !scales_rows_ok(p) || (br != 1 && !given_scales)) return false;
-        uint64_t rows_s, pitch_s;
-        if (!uniform_rows(scale_a, &rows_s, &pitch_s) || rows_s * br != rows_f) return false;
-        a->scale_in_pitch = pitch_s * scale_a_size;
-        if (scale_b) {
-            if (!uniform_rows(scale_b, &rows_s, &pitch_s) || rows_s * br != rows_f) return false;
-            a->scale_out_pitch = pitch_s * scale_b_size;
-        }
+        if (!row_levels(scale_a, &la) || la.rows * br != rows_f) return false;
+        if (scale_b && (!row_levels(scale_b, &lb) || lb.rows * br != rows_f)) return false;
         a->scale_rows = br;
     }
+    // one split into groups of rows must serve all tensors; uniform ones fit any
+    uint64_t inner_rows = 0;
+    for (const RowLevels* l : {&lf, &lv, &la, &lb}) {
+        if (l->levels != 2) continue;
+        if (inner_rows != 0 && inner_rows != l->inner_rows) return false;
+        inner_rows = l->inner_rows;
+    }
+    if (inner_rows == 0) inner_rows = rows_f;
+    if (inner_rows != rows_f && a->scale_rows != 1) return false;  // blocks of rows: uniform rows only
+    const auto outer_of = [&](const RowLevels& l) { return l.levels == 2 ? l.outer : l.inner * inner_rows; };
+    if (!aligned(floats->ptr, 16) || !aligned(values->ptr, 8) || (lf.inner * elem) % 16 || (outer_of(lf) * elem) % 16 ||
+        (lv.inner * stored) % 8 || (outer_of(lv) * stored) % 8)
+        return false;
     a->rows = rows_f;
+    a->inner_rows = inner_rows;
     a->num_chunks = row_chunks;
-    a->in_pitch = pitch_f * elem;      // quantize: floats in, stored out; dequantize swaps them
-    a->out_pitch = pitch_v * stored;
+    a->in_pitch = lf.inner * elem;  // quantize: floats in, stored out; dequantize swaps them
+    a->in_outer = outer_of(lf) * elem;
+    a->out_pitch = lv.inner * stored;
+    a->out_outer = outer_of(lv) * stored;
+    a->scale_in_pitch = la.inner * scale_a_size;
+    a->scale_in_outer = outer_of(la) * scale_a_size;
+    a->scale_out_pitch = lb.inner * scale_b_size;
+    a->scale_out_outer = outer_of(lb) * scale_b_size;
     return true;
 }
 
@@ -581,9 +628,8 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         fr.input = values->ptr;
         fr.output = output->ptr;
         fr.scale_in = params->ptr;
-        const uint64_t floats_pitch = fr.in_pitch;  // the float tensor is the output here
-        fr.in_pitch = fr.out_pitch;
-        fr.out_pitch = floats_pitch;
+        std::swap(fr.in_pitch, fr.out_pitch);  // the float tensor is the output here
+        std::swap(fr.in_outer, fr.out_outer);
         fr.block = p.tensor_level ? 0 : p.block_last;
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
@@ -766,7 +812,8 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         fr.output = output->ptr;
         fr.scale_out = out_scale->ptr;
         fr.scale_out_pitch = fr.scale_in_pitch;  // the only scale tensor of this call is the output
-        fr.scale_in_pitch = 0;
+        fr.scale_out_outer = fr.scale_in_outer;
+        fr.scale_in_pitch = fr.scale_in_outer = 0;
         fr.block = p.block_last;
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);

@@ -34,9 +34,11 @@ struct FlatArgs {
     void* scale_out;      // quantize: out_scale typed as param dtype, NULL = do not write;
                           // launch_scales_flat: scales typed like the input
     uint64_t num_chunks;  // 16-byte chunks of the float tensor handled by this launch (per row when rows > 1)
-    // rows > 1: the launch covers `rows` runs of num_chunks chunks whose starts lie this many bytes apart in
-    // the four tensors (pitched rows); 0 or 1: one contiguous run
-    uint64_t rows, in_pitch, out_pitch, scale_in_pitch, scale_out_pitch;
+    // rows > 1: the launch covers `rows` runs of num_chunks chunks, in groups of `inner_rows` (0: one group);
+    // the rows of a group start *_pitch bytes apart in the four tensors, the groups *_outer bytes.  rows 0 or 1:
+    // one contiguous run
+    uint64_t rows, inner_rows, in_pitch, out_pitch, scale_in_pitch, scale_out_pitch;
+    uint64_t in_outer, out_outer, scale_in_outer, scale_out_outer;
     uint32_t scale_rows;  // rows > 1, given scales: blocks of this many rows share a row of scales (0 or 1: one)
     uint32_t block;       // elements per block, 0 = per-tensor
     int param_dtype;      // cq_dtype of the stored scales

@@ -73,15 +73,20 @@ struct RunSteps {
 
 // Pitched rows.  A row of `row_chunks` chunks is `steps_per_row` steps, the last one partial where
 // kThreads does not divide the row; step g of the launch is step g % steps_per_row of row
-// g / steps_per_row.  The rows of the four tensors start `in` / `out` / `scale_in` / `scale_out`
-// bytes apart, and blocks of `scale_rows` rows (by a lane group of columns) share a row of scales
-// (given scales only: a fused abs-max sees one row).
+// g / steps_per_row.  The rows come in groups of `inner_rows`: the rows of a group start `in` / `out` /
+// `scale_in` / `scale_out` bytes apart in the four tensors, the groups `*_outer` bytes (`*_wrap` =
+// outer - inner_rows * inner, the step from a group's last row to the next group's first minus one row
+// pitch).  Blocks of `scale_rows` rows (by a lane group of columns) share a row of scales (given scales
+// only: a fused abs-max sees one row; one group of rows only).
 struct FlatRows {
     uint32_t row_chunks, steps_per_row, total_steps;  // total_steps < 2^31
     uint32_t scale_rows;  // >= 1
-    // n / steps_per_row and n / scale_rows for n < 2^31 as (n * magic) >> shift (cq_magic_div.hpp)
-    uint32_t steps_magic, steps_shift, scale_magic, scale_shift;
+    uint32_t inner_rows;
+    // n / steps_per_row, n / inner_rows and n / scale_rows for n < 2^31 as (n * magic) >> shift (cq_magic_div.hpp)
+    uint32_t steps_magic, steps_shift, inner_magic, inner_shift, scale_magic, scale_shift;
     uint64_t in, out, scale_in, scale_out;
+    uint64_t in_outer, out_outer, scale_in_outer, scale_out_outer;
+    uint64_t in_wrap, out_wrap, scale_in_wrap, scale_out_wrap;
 };
 template <int kUnroll, int kThreads, bool kChecked, int kInBytes, int kOutBytes, int kDiv>
 struct RowSteps;
@@ -116,17 +121,23 @@ struct RowSteps {
         const uint32_t step = g.step_begin + tile * kUnroll;
         const uint32_t row = magic_div(step, r.steps_magic, r.steps_shift);
         uint32_t col = step - row * r.steps_per_row;
-        const uint32_t scale_row = magic_div(row, r.scale_magic, r.scale_shift);
-        uint32_t sub = row - scale_row * r.scale_rows;
+        const uint32_t group = magic_div(row, r.inner_magic, r.inner_shift);
+        uint32_t lo = row - group * r.inner_rows;  // row within its group
+        const uint32_t scale_row = magic_div(lo, r.scale_magic, r.scale_shift);
+        uint32_t sub = lo - scale_row * r.scale_rows;
         bool first = kDiv == 0 ? step == 0 : sub == 0;
         // bytes from one step to the next one of the same row, and back to the row's first step
         constexpr uint64_t kScalesPerStep = kDiv == 0 ? 0 : kThreads / (kDiv == 0 ? 1 : kDiv);
         const uint64_t scale_in_step = kScalesPerStep * g.scale_in_bytes, scale_out_step = kScalesPerStep * g.scale_out_bytes;
         const uint64_t back = r.steps_per_row - 1;
-        const char* in = static_cast<const char*>(g.in) + row * r.in + static_cast<uint64_t>(col) * (kThreads * kInBytes);
-        char* out = static_cast<char*>(g.out) + row * r.out + static_cast<uint64_t>(col) * (kThreads * kOutBytes);
-        const char* scale_in = static_cast<const char*>(g.scale_in) + scale_row * r.scale_in + col * scale_in_step;
-        char* scale_out = static_cast<char*>(g.scale_out) + scale_row * r.scale_out + col * scale_out_step;
+        const char* in = static_cast<const char*>(g.in) + group * r.in_outer + lo * r.in +
+                         static_cast<uint64_t>(col) * (kThreads * kInBytes);
+        char* out = static_cast<char*>(g.out) + group * r.out_outer + lo * r.out +
+                    static_cast<uint64_t>(col) * (kThreads * kOutBytes);
+        const char* scale_in = static_cast<const char*>(g.scale_in) + group * r.scale_in_outer + scale_row * r.scale_in +
+                               col * scale_in_step;
+        char* scale_out = static_cast<char*>(g.scale_out) + group * r.scale_out_outer + scale_row * r.scale_out +
+                          col * scale_out_step;
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             valid_[u] = !kChecked || u == 0 || step + u < r.total_steps;
@@ -140,6 +151,7 @@ struct RowSteps {
             // past the launch's last step the addresses stay where they are: on data
             if (kChecked && step + u + 1 >= r.total_steps) continue;
             if (++col != r.steps_per_row) {
+                if (kDiv == 0) first = false;  // one scale per tensor: the launch's first step stores it
                 in += kThreads * kInBytes;
                 out += kThreads * kOutBytes;
                 scale_in += scale_in_step;
@@ -154,6 +166,13 @@ struct RowSteps {
                     sub = 0;
                     scale_in += r.scale_in;
                     scale_out += r.scale_out;
+                }
+                if (++lo == r.inner_rows) {  // on to the next group of rows (scale_rows is 1 where there are several)
+                    lo = 0;
+                    in += r.in_wrap;
+                    out += r.out_wrap;
+                    scale_in += r.scale_in_wrap;
+                    scale_out += r.scale_out_wrap;
                 }
                 first = kDiv == 0 ? false : sub == 0;
             }

@@ -47,12 +47,23 @@ FlatRows flat_rows(const FlatArgs& a) {
     r.steps_per_row = static_cast<uint32_t>((a.num_chunks + kThreads - 1) / kThreads);
     r.total_steps = static_cast<uint32_t>(a.rows * r.steps_per_row);
     r.scale_rows = a.scale_rows > 1 ? a.scale_rows : 1u;
+    r.inner_rows = static_cast<uint32_t>(a.inner_rows == 0 ? a.rows : a.inner_rows);
     magic_of(r.steps_per_row, &r.steps_magic, &r.steps_shift);
+    magic_of(r.inner_rows, &r.inner_magic, &r.inner_shift);
     magic_of(r.scale_rows, &r.scale_magic, &r.scale_shift);
     r.in = a.in_pitch;
     r.out = a.out_pitch;
     r.scale_in = a.scale_in_pitch;
     r.scale_out = a.scale_out_pitch;
+    r.in_outer = a.in_outer;
+    r.out_outer = a.out_outer;
+    r.scale_in_outer = a.scale_in_outer;
+    r.scale_out_outer = a.scale_out_outer;
+    // unsigned wrap-around is meant: an outer pitch may be smaller than a group of rows (permuted dimensions)
+    r.in_wrap = a.in_outer - r.inner_rows * a.in_pitch;
+    r.out_wrap = a.out_outer - r.inner_rows * a.out_pitch;
+    r.scale_in_wrap = a.scale_in_outer - r.inner_rows * a.scale_in_pitch;
+    r.scale_out_wrap = a.scale_out_outer - r.inner_rows * a.scale_out_pitch;
     return r;
 }
 

@@ -76,6 +76,14 @@ def layouts(shape, per):
         out.append(("last_two_swapped_pitched", swapped(shape, 6), contiguous(pshape, 3)))
         out.append(("every_other_row", tuple(s * (2 if d == 0 else 1) for d, s in enumerate(contiguous(shape))),
                     tuple(s * (2 if d == 0 else 1) for d, s in enumerate(contiguous(pshape)))))
+    if rank >= 3:
+        # the first two dimensions swapped in memory, pitched rows: groups of rows with a pitch of their own
+        def leading_swapped(sh, pad):
+            st = contiguous((sh[1], sh[0]) + tuple(sh[2:]), pad)
+            return (st[1], st[0]) + tuple(st[2:])
+
+        out.append(("leading_swapped", leading_swapped(shape, 64), leading_swapped(pshape, 8)))
+        out.append(("leading_swapped_floats", leading_swapped(shape, 0), contiguous(pshape)))
     return pshape, out
 
 
@@ -109,7 +117,7 @@ def test_long_pitched_rows(gpu, oracle, elem, name, scheme):
     """Rows of many steps of the streaming kernels (whole steps, and a partial last step per row),
     with 1-D blocks and with blocks over the last two dimensions."""
     check_layouts(gpu, oracle, elem, name, scheme, ((4, 16384), (2, 2, 16384 + 4096 + 512)),
-                  ("contiguous", "pitched", "pitched_aligned", "every_other_row"))
+                  ("contiguous", "pitched", "pitched_aligned", "every_other_row", "leading_swapped", "leading_swapped_floats"))
 
 
 @pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
@@ -119,8 +127,8 @@ def test_pitched_rows_of_a_few_steps(gpu, oracle, elem, name, scheme):
     so one workgroup's steps lie in up to four rows (also rows of a block that share their scales),
     a row's last step may be partial, and the launch ends on a workgroup with fewer steps than the others."""
     check_layouts(gpu, oracle, elem, name, scheme,
-                  ((4, 4096), (6, 5120), (2, 2, 7168), (4, 2560), (6, 2048), (6, 1024), (10, 1280)),
-                  ("pitched", "pitched_aligned", "every_other_row"))
+                  ((4, 4096), (6, 5120), (2, 2, 7168), (4, 2560), (6, 2048), (6, 1024), (10, 1280), (3, 2, 2048), (2, 3, 2, 2560)),
+                  ("pitched", "pitched_aligned", "every_other_row", "leading_swapped", "leading_swapped_floats"))
 
 
 def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
