@@ -193,33 +193,10 @@ bool flat_ok(const Plan& p, int dtype, const cq_tensor* floats, const cq_tensor*
     return cq::flat_block_supported(dtype, p.block_last);
 }
 
-// Rows of a tensor as the flat kernels take them: the last dimension contiguous, everything
-// in front of it one uniform run of rows `*pitch` elements apart (pitched, sliced along the
-// last dimension; 0 when there is a single row).
-bool uniform_rows(const cq_tensor* t, uint64_t* rows, uint64_t* pitch) {
-    const uint32_t last = t->rank - 1;
-    if (t->shape[last] != 1 && t->strides[last] != 1) return false;
-    *rows = 1;
-    *pitch = 0;
-    uint64_t expect = 0;  // 0: no dimension with more than one entry seen yet
-    for (int d = static_cast<int>(last) - 1; d >= 0; d--) {
-        if (t->shape[d] == 1) continue;
-        if (t->strides[d] == 0) return false;  // broadcast rows: not for these kernels
-        if (expect == 0) {
-            *pitch = t->strides[d];
-        } else if (t->strides[d] != expect) {
-            return false;
-        }
-        expect = t->strides[d] * t->shape[d];
-        *rows *= t->shape[d];
-    }
-    return true;
-}
-
-// The same with one more level: the rows in front of the last dimension as `outer_rows` groups of
-// `inner_rows` rows, `inner` elements between the rows of a group and `outer` between groups (a slice
-// along the second to last dimension, a batch of pitched matrices).  levels = 0 (a single row), 1 (one
-// uniform run: inner_rows = all rows) or 2.
+// Rows of a tensor as the flat kernels take them: the last dimension contiguous, the rows in front of
+// it as groups of `inner_rows` rows, `inner` elements between the rows of a group and `outer` between
+// groups (pitched rows; a slice along the second to last dimension, a batch of pitched matrices).
+// levels = 0 (a single row), 1 (one uniform run: inner_rows = all rows) or 2.
 struct RowLevels {
     int levels;
     uint64_t rows, inner_rows, inner, outer;
@@ -753,24 +730,33 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
         return hip_status(cq::launch_scales_flat(stream, input_dtype, a));
     }
     // pitched rows of at least a step of 256 chunks, 1-D blocks: the same kernel over the rows' steps
-    uint64_t rows_f, rows_s, pitch_f, pitch_s;
-    const uint64_t row_chunks = input->shape[input->rank - 1] / (16 / dtype_size(input_dtype));
+    // (rows in one uniform run or in groups with a pitch of their own, as in flat_rows_ok())
+    const uint32_t elem = dtype_size(input_dtype);
+    const uint64_t row_chunks = input->shape[input->rank - 1] / (16 / elem);
+    RowLevels lf, ls;
     if (!p.tensor_level && p.last_dim_blocks && p.rank >= 2 && cq::flat_block_supported(input_dtype, p.block_last) &&
-        uniform_rows(input, &rows_f, &pitch_f) && uniform_rows(scales, &rows_s, &pitch_s) && rows_f == rows_s &&
-        aligned(input->ptr, 16) && (pitch_f * dtype_size(input_dtype)) % 16 == 0 &&
-        input->shape[input->rank - 1] % (16 / dtype_size(input_dtype)) == 0 && row_chunks >= 256 &&
+        row_levels(input, &lf) && row_levels(scales, &ls) && lf.rows == ls.rows &&
+        !(lf.levels == 2 && ls.levels == 2 && lf.inner_rows != ls.inner_rows) &&
+        input->shape[input->rank - 1] % (16 / elem) == 0 && row_chunks >= 256 &&
         ((row_chunks + 255) / 256 * 256 - row_chunks) * 10 <= row_chunks * 6 &&
-        rows_f * ((row_chunks + 255) / 256) < (1ull << 31)) {
-        cq::FlatArgs a{};
-        a.input = input->ptr;
-        a.scale_out = scales->ptr;
-        a.num_chunks = row_chunks;
-        a.rows = rows_f;
-        a.in_pitch = pitch_f * dtype_size(input_dtype);
-        a.scale_out_pitch = pitch_s * dtype_size(input_dtype);
-        a.block = p.block_last;
-        a.range = p.range;
-        return hip_status(cq::launch_scales_flat(stream, input_dtype, a));
+        lf.rows * ((row_chunks + 255) / 256) < (1ull << 31)) {
+        const uint64_t inner_rows = lf.levels == 2 ? lf.inner_rows : (ls.levels == 2 ? ls.inner_rows : lf.rows);
+        const auto outer_of = [&](const RowLevels& l) { return l.levels == 2 ? l.outer : l.inner * inner_rows; };
+        if (aligned(input->ptr, 16) && (lf.inner * elem) % 16 == 0 && (outer_of(lf) * elem) % 16 == 0) {
+            cq::FlatArgs a{};
+            a.input = input->ptr;
+            a.scale_out = scales->ptr;
+            a.num_chunks = row_chunks;
+            a.rows = lf.rows;
+            a.inner_rows = inner_rows;
+            a.in_pitch = lf.inner * elem;
+            a.in_outer = outer_of(lf) * elem;
+            a.scale_out_pitch = ls.inner * elem;
+            a.scale_out_outer = outer_of(ls) * elem;
+            a.block = p.block_last;
+            a.range = p.range;
+            return hip_status(cq::launch_scales_flat(stream, input_dtype, a));
+        }
     }
     return produce_scales(stream, p, scheme, input, input_dtype, scales, input_dtype, workspace, workspace_bytes);
 }
