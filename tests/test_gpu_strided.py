@@ -330,3 +330,69 @@ def test_broadcast_rows_read_like_their_copies(gpu, cols):
     for a, b in zip(outs[0], outs[1]):
         assert torch.equal(a, b)
     assert torch.equal(outs[0][0], outs[0][2])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("elem", [ElemType.BF16, ElemType.F32], ids=lambda e: e.name)
+def test_large_sliced_batches_match_the_contiguous_path(gpu, elem):
+    """A [4, 3584, 8192] slice of a [4, 4096, 8256] buffer (rows in groups with a pitch of their own, the
+    grid numbered through all of them): codes, scales and dequantized values must equal what the contiguous
+    kernels, checked against the oracle elsewhere, give for a contiguous copy; what lies between the rows
+    and between the groups stays as it was."""
+    import torch
+
+    client = ComputeClient.current()
+    tdt = torch.float32 if elem == ElemType.F32 else torch.bfloat16
+    eb = 4 if elem == ElemType.F32 else 2
+    b, r, c, rb, cb = 4, 3584, 8192, 4096, 8256
+    g = torch.Generator(device="cuda")
+    g.manual_seed(77 + int(elem))
+    buf = torch.randn((b, rb, cb), generator=g, device="cuda", dtype=torch.float32).mul_(0.05).to(tdt)
+    x = buf[:, :r, :c].contiguous()
+    h = TensorHandleRef.from_torch
+    sliced = lambda t: TensorHandleRef(h(t).handle, (b, r, c), (rb * cb, cb, 1), eb)
+    for name, scheme in (("e2m1_block32", QuantScheme.default().with_value(QuantValue.E2M1).with_level(QuantLevel.block([32]))),
+                         ("q8s_tensor", QuantScheme.default().with_value(QuantValue.Q8S)),
+                         ("e4m3_native_block64", QuantScheme.default().with_value(QuantValue.E4M3)
+                          .with_store(QuantStore.Native).with_level(QuantLevel.block([64])))):
+        print(name, elem.name, flush=True)
+        native = scheme.store == QuantStore.Native
+        pshape = scheme.packed_shape((b, r, c)) if not native else (b, r, c)
+        sshape = scheme.scales_shape((b, r, c))
+        ws, nbytes = gpu.workspace(scheme, b * r * c)
+        outs = []
+        for hx in (h(x), sliced(buf)):
+            codes = torch.full(pshape, 0x5A, dtype=torch.uint8 if native else torch.int32, device="cuda")
+            scales = torch.zeros(sshape, dtype=torch.float32, device="cuda")
+            qz.launch_dynamic(client, hx, h(codes), h(scales), scheme, elem, ws.data_ptr(), nbytes)
+            outs.append((codes, scales))
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0][0], outs[1][0]), (name, "codes")
+        assert torch.equal(outs[0][1].view(torch.int32), outs[1][1].view(torch.int32)), (name, "scales")
+        # block scales from the sliced tensor, then quantize with them given
+        if scheme.level.block_size is not None:
+            s_in = [torch.zeros(sshape, dtype=tdt, device="cuda") for _ in range(2)]
+            qz.compute_scales(client, h(x), h(s_in[0]), scheme, elem)
+            qz.compute_scales(client, sliced(buf), h(s_in[1]), scheme, elem)
+            torch.cuda.synchronize()
+            assert torch.equal(s_in[0].view(torch.int16 if eb == 2 else torch.int32),
+                               s_in[1].view(torch.int16 if eb == 2 else torch.int32)), (name, "compute_scales")
+        else:
+            s_in = [outs[0][1].to(tdt)] * 2
+        codes2, os2 = torch.zeros_like(outs[0][0]), torch.zeros_like(outs[0][1])
+        qz.launch_ref(client, sliced(buf), h(codes2), h(s_in[1]), h(os2), scheme, elem)
+        codes3, os3 = torch.zeros_like(outs[0][0]), torch.zeros_like(outs[0][1])
+        qz.launch_ref(client, h(x), h(codes3), h(s_in[0]), h(os3), scheme, elem)
+        torch.cuda.synchronize()
+        assert torch.equal(codes2, codes3), (name, "codes, given scales")
+        assert torch.equal(os2.view(torch.int32), os3.view(torch.int32)), (name, "out_scale, given scales")
+        # dequantize into a contiguous tensor and into the slice of a buffer full of a sentinel
+        y = torch.empty_like(x)
+        ybuf = torch.full((b, rb, cb), 3.0, dtype=tdt, device="cuda")
+        dq.launch_ref(client, h(outs[0][0]), h(y), h(outs[0][1]), scheme, elem)
+        dq.launch_ref(client, h(outs[0][0]), sliced(ybuf), h(outs[0][1]), scheme, elem)
+        torch.cuda.synchronize()
+        bits = torch.int16 if eb == 2 else torch.int32
+        assert torch.equal(ybuf[:, :r, :c].contiguous().view(bits), y.view(bits)), (name, "dequantized")
+        assert bool((ybuf[:, :, c:] == 3.0).all()) and bool((ybuf[:, r:, :] == 3.0).all()), (name, "padding")
+        del outs, codes2, codes3, os2, os3, y, ybuf
