@@ -227,10 +227,10 @@ bool row_levels(const cq_tensor* t, RowLevels* l) {
 
 bool scales_rows_ok(const Plan& p);
 
-// Can the flat kernels take this launch row by row?  (value tensors with a contiguous last
-// dimension and a uniform row pitch, rows of at least half a tile, whole chunks,
-// 1-D blocks that map onto lane groups, scales with a contiguous last dimension.)  Fills the
-// row fields of `a` and a.num_chunks = chunks per row.
+// Can the flat kernels take this launch over the steps of its rows?  (value tensors with a contiguous last
+// dimension whose rows form one uniform run or groups with a pitch of their own, rows of at least a step
+// of 256 whole chunks, 1-D blocks that map onto lane groups (given scales: also blocks of rows), scales
+// with a contiguous last dimension.)  Fills the row fields of `a` and a.num_chunks = chunks per row.
 bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
                   const cq_tensor* scale_a, uint32_t scale_a_size, const cq_tensor* scale_b, uint32_t scale_b_size,
                   bool given_scales, cq::FlatArgs* a) {
@@ -791,7 +791,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
     }
 
-    // pitched rows with 1-D blocks: the same fused kernel, row by row
+    // pitched rows with 1-D blocks: the same fused kernel over the rows' steps
     cq::FlatArgs fr{};
     if (!p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr)) {
         fr.input = input->ptr;
@@ -855,7 +855,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         if (st != CQ_OK) return st;
         flat_words = flat_chunks * per_chunk / p.nq;
     } else if (p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr)) {
-        // per tensor on pitched rows: the same two passes, the second one row by row
+        // per tensor on pitched rows: the same two passes, the second one over the rows' steps
         uint32_t num_partials = 0;
         st = absmax_partials(stream, p, scheme, input, input_dtype, workspace, workspace_bytes, &num_partials);
         if (st != CQ_OK) return st;
