@@ -289,6 +289,79 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     return true;
 }
 
+// Can the flat kernels take this launch with every lane finding its own row?  (Every tensor with a
+// contiguous last dimension, rows of whole chunks, aligned strides, one scale per tensor or 1-D blocks that
+// map onto lane groups.)  Fills a.rows, a.num_chunks = chunks per row and a.lanes: the leading dimensions
+// innermost first, neighbours merged where all four tensors step uniformly through them.
+bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
+                  const cq_tensor* scale_a, uint32_t scale_a_size, const cq_tensor* scale_b, uint32_t scale_b_size,
+                  cq::FlatArgs* a) {
+    if (p.rank < 2) return false;
+    const uint32_t last = p.rank - 1;
+    const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
+    const uint32_t stored = s->store == CQ_STORE_U32 ? 4u : 1u;
+    const auto rows_contiguous = [&](const cq_tensor* t) { return t->shape[last] == 1 || t->strides[last] == 1; };
+    if (!rows_contiguous(floats) || !rows_contiguous(values) || !aligned(floats->ptr, 16) || !aligned(values->ptr, 8)) return false;
+    const uint64_t cols = p.shape[last];
+    const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+    if (cols == 0 || cols % chunk_elems) return false;
+    const bool scales = !p.tensor_level;
+    if (scales && (!p.last_dim_blocks || !cq::flat_block_supported(dtype, p.block_last) || !rows_contiguous(scale_a) ||
+                   (scale_b && !rows_contiguous(scale_b))))
+        return false;
+    cq::LaneLevels& l = a->lanes;
+    l = cq::LaneLevels{};
+    uint64_t rows = 1;
+    for (int d = static_cast<int>(last) - 1; d >= 0; d--) {
+        const uint64_t n = p.shape[d];
+        if (n == 1) continue;
+        const uint64_t in = floats->strides[d] * elem, out = values->strides[d] * stored;
+        const uint64_t scale_in = scales ? scale_a->strides[d] * scale_a_size : 0;
+        const uint64_t scale_out = scales && scale_b ? scale_b->strides[d] * scale_b_size : 0;
+        if (in == 0 || out == 0 || in % 16 || out % 8) return false;  // broadcast or misaligned rows
+        const uint32_t k = l.levels;
+        if (k > 0 && in == l.in[k - 1] * l.count[k - 1] && out == l.out[k - 1] * l.count[k - 1] &&
+            scale_in == l.scale_in[k - 1] * l.count[k - 1] && scale_out == l.scale_out[k - 1] * l.count[k - 1] &&
+            l.count[k - 1] * n < (1ull << 31)) {
+            l.count[k - 1] *= static_cast<uint32_t>(n);
+        } else {
+            l.count[k] = static_cast<uint32_t>(n);
+            l.in[k] = in;
+            l.out[k] = out;
+            l.scale_in[k] = scale_in;
+            l.scale_out[k] = scale_out;
+            l.levels = k + 1;
+        }
+        rows *= n;
+    }
+    if (l.levels == 0) {  // a single row
+        l.levels = 1;
+        l.count[0] = 1;
+    }
+    const uint64_t row_chunks = cols / per_chunk;
+    if (rows * row_chunks >= (1ull << 31)) return false;
+    a->rows = rows;
+    a->num_chunks = row_chunks;
+    return true;
+}
+
+// The float tensor is the output (dequantize): the planners fill `in` with it.
+void swap_value_roles(cq::FlatArgs* a) {
+    std::swap(a->in_pitch, a->out_pitch);
+    std::swap(a->in_outer, a->out_outer);
+    for (uint32_t l = 0; l < a->lanes.levels; l++) std::swap(a->lanes.in[l], a->lanes.out[l]);
+}
+// The only scale tensor of the call is an output (fused abs-max): the planners fill `scale_in` with it.
+void scale_in_to_out(cq::FlatArgs* a) {
+    a->scale_out_pitch = a->scale_in_pitch;
+    a->scale_out_outer = a->scale_in_outer;
+    a->scale_in_pitch = a->scale_in_outer = 0;
+    for (uint32_t l = 0; l < a->lanes.levels; l++) {
+        a->lanes.scale_out[l] = a->lanes.scale_in[l];
+        a->lanes.scale_in[l] = 0;
+    }
+}
+
 // Stored encoding of the flat kernels (cq::Encoding) and the field width they see.
 int flat_encoding(const cq_scheme* s) {
     if (s->store == CQ_STORE_U32) return 0;
@@ -526,8 +599,10 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
     cq::FlatArgs fr{};
-    if (flat_words == 0 && flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
-                                        dtype_size(pd), true, &fr)) {
+    if (flat_words == 0 && (flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
+                                         dtype_size(pd), true, &fr) ||
+                            lane_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
+                                         dtype_size(pd), &fr))) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_in = scale->ptr;
@@ -601,12 +676,12 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
     cq::FlatArgs fr{};
-    if (flat_words == 0 && flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr)) {
+    if (flat_words == 0 && (flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr) ||
+                            lane_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, &fr))) {
         fr.input = values->ptr;
         fr.output = output->ptr;
         fr.scale_in = params->ptr;
-        std::swap(fr.in_pitch, fr.out_pitch);  // the float tensor is the output here
-        std::swap(fr.in_outer, fr.out_outer);
+        swap_value_roles(&fr);
         fr.block = p.tensor_level ? 0 : p.block_last;
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
@@ -793,13 +868,12 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
 
     // pitched rows with 1-D blocks: the same fused kernel over the rows' steps
     cq::FlatArgs fr{};
-    if (!p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr)) {
+    if (!p.tensor_level && (flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) ||
+                            lane_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, &fr))) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_out = out_scale->ptr;
-        fr.scale_out_pitch = fr.scale_in_pitch;  // the only scale tensor of this call is the output
-        fr.scale_out_outer = fr.scale_in_outer;
-        fr.scale_in_pitch = fr.scale_in_outer = 0;
+        scale_in_to_out(&fr);
         fr.block = p.block_last;
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
@@ -854,7 +928,8 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, a));
         if (st != CQ_OK) return st;
         flat_words = flat_chunks * per_chunk / p.nq;
-    } else if (p.tensor_level && flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr)) {
+    } else if (p.tensor_level && (flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) ||
+                                  lane_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, &fr))) {
         // per tensor on pitched rows: the same two passes, the second one over the rows' steps
         uint32_t num_partials = 0;
         st = absmax_partials(stream, p, scheme, input, input_dtype, workspace, workspace_bytes, &num_partials);

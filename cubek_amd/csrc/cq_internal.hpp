@@ -22,6 +22,14 @@ struct Range {
     float lo, hi;
 };
 
+// Rows that each lane finds for itself (short rows, leading dimensions with strides of their own):
+// the leading dimensions innermost first, `count` entries each, and the bytes per entry in the four tensors.
+struct LaneLevels {
+    uint32_t levels;  // 0: not used
+    uint32_t count[CQ_MAX_RANK - 1];
+    uint64_t in[CQ_MAX_RANK - 1], out[CQ_MAX_RANK - 1], scale_in[CQ_MAX_RANK - 1], scale_out[CQ_MAX_RANK - 1];
+};
+
 // Flat fast path: contiguous tensors, scales contiguous, blocks are runs of
 // `block` consecutive elements (block == 0: one scale for the whole tensor).
 struct FlatArgs {
@@ -39,6 +47,7 @@ struct FlatArgs {
     // one contiguous run
     uint64_t rows, inner_rows, in_pitch, out_pitch, scale_in_pitch, scale_out_pitch;
     uint64_t in_outer, out_outer, scale_in_outer, scale_out_outer;
+    LaneLevels lanes;     // lanes.levels > 0: `rows` rows of num_chunks chunks addressed lane by lane instead
     uint32_t scale_rows;  // rows > 1, given scales: blocks of this many rows share a row of scales (0 or 1: one)
     uint32_t block;       // elements per block, 0 = per-tensor
     int param_dtype;      // cq_dtype of the stored scales

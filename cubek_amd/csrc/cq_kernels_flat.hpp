@@ -35,8 +35,9 @@ enum ScaleSrc : int {
 // A tile is kUnroll steps of kThreads consecutive chunks, one per lane.  The kernel bodies ask a
 // geometry, for each step u, for the (wave-uniform) base pointers of the tensors, the lane's chunk
 // index relative to them (`chunk`; `load_chunk` is the same clamped into the data, for lanes past
-// the end), whether the lane holds data (`live`) and whether the step's row starts its blocks
-// (`first_row`).  Scale i of a base pointer belongs to chunks [i * kDiv, (i + 1) * kDiv).
+// the end), whether the lane holds data (`live`), whether the step's row starts its blocks
+// (`first_row`) and whether the lane holds the tensor's first chunk (`tensor_start`).  Scale i of a
+// base pointer belongs to chunks [i * kDiv, (i + 1) * kDiv).
 
 // One contiguous run of chunks [chunk_begin, chunk_end): the same pointers for every step.
 template <int kUnroll, int kThreads, bool kChecked>
@@ -65,6 +66,7 @@ struct RunSteps {
     }
     __device__ __forceinline__ bool live(int u) const { return !kChecked || chunk(u) < g.chunk_end; }
     __device__ __forceinline__ bool first_row(int) const { return true; }
+    __device__ __forceinline__ bool tensor_start(int u) const { return chunk(u) == 0; }
     __device__ __forceinline__ const void* in(int) const { return g.in; }
     __device__ __forceinline__ void* out(int) const { return g.out; }
     __device__ __forceinline__ const void* scale_in(int) const { return g.scale_in; }
@@ -184,6 +186,83 @@ struct RowSteps {
     }
     __device__ __forceinline__ bool live(int u) const { return !kChecked || (valid_[u] && threadIdx.x <= last_[u]); }
     __device__ __forceinline__ bool first_row(int u) const { return first_[u]; }
+    __device__ __forceinline__ bool tensor_start(int u) const { return first_[u] && threadIdx.x == 0; }
+    __device__ __forceinline__ const void* in(int u) const { return in_[u]; }
+    __device__ __forceinline__ void* out(int u) const { return out_[u]; }
+    __device__ __forceinline__ const void* scale_in(int u) const { return scale_in_[u]; }
+    __device__ __forceinline__ void* scale_out(int u) const { return scale_out_[u]; }
+};
+
+// Short or irregularly strided rows (a head dimension behind permuted leading dimensions): the chunks
+// of the launch are numbered through all rows, a step is kThreads consecutive ones, so the lanes of a
+// step lie in several rows.  Each lane finds its row (chunk / row_chunks) and from it, dimension by
+// dimension (innermost first, `count` entries each, multiply-and-shift divisions), the byte offsets of
+// that row in the four tensors.  Blocks lie along the row (or one scale per tensor).
+constexpr int kMaxLaneLevels = 7;
+struct LaneRows {
+    uint32_t row_chunks, row_magic, row_shift;
+    uint32_t total_chunks;  // < 2^31
+    uint32_t levels;        // leading dimensions, 1 .. kMaxLaneLevels
+    uint32_t count[kMaxLaneLevels], magic[kMaxLaneLevels], shift[kMaxLaneLevels];
+    uint64_t in[kMaxLaneLevels], out[kMaxLaneLevels], scale_in[kMaxLaneLevels], scale_out[kMaxLaneLevels];
+};
+template <int kUnroll, int kThreads>
+struct LaneSteps;
+struct LanesGeo {
+    const void* in;
+    void* out;
+    const void* scale_in;
+    void* scale_out;
+    LaneRows rows;
+    template <int kUnroll, int kThreads, bool kChecked>
+    using Steps = LaneSteps<kUnroll, kThreads>;  // always checked
+};
+template <int kUnroll, int kThreads>
+struct LaneSteps {
+    using Index = uint32_t;
+    const char* in_[kUnroll];
+    char* out_[kUnroll];
+    const char* scale_in_[kUnroll];
+    char* scale_out_[kUnroll];
+    uint32_t col_[kUnroll];  // the lane's chunk within its row
+    bool live_[kUnroll], first_[kUnroll];
+    __device__ __forceinline__ LaneSteps(const LanesGeo& g, uint32_t tile) {
+        const LaneRows& r = g.rows;
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const uint32_t chunk = (tile * kUnroll + u) * kThreads + threadIdx.x;
+            live_[u] = chunk < r.total_chunks;
+            const uint32_t c = live_[u] ? chunk : r.total_chunks - 1;  // lanes past the end re-read the last chunk
+            uint32_t row = magic_div(c, r.row_magic, r.row_shift);
+            col_[u] = c - row * r.row_chunks;
+            first_[u] = row == 0;
+            uint64_t in = 0, out = 0, scale_in = 0, scale_out = 0;
+#pragma unroll
+            for (int l = 0; l < kMaxLaneLevels; l++) {
+                if (l < static_cast<int>(r.levels)) {
+                    uint32_t index = row;
+                    if (l + 1 < static_cast<int>(r.levels)) {
+                        const uint32_t q = magic_div(row, r.magic[l], r.shift[l]);
+                        index = row - q * r.count[l];
+                        row = q;
+                    }
+                    in += index * r.in[l];
+                    out += index * r.out[l];
+                    scale_in += index * r.scale_in[l];
+                    scale_out += index * r.scale_out[l];
+                }
+            }
+            in_[u] = static_cast<const char*>(g.in) + in;
+            out_[u] = static_cast<char*>(g.out) + out;
+            scale_in_[u] = static_cast<const char*>(g.scale_in) + scale_in;
+            scale_out_[u] = g.scale_out == nullptr ? nullptr : static_cast<char*>(g.scale_out) + scale_out;
+        }
+    }
+    __device__ __forceinline__ Index chunk(int u) const { return col_[u]; }
+    __device__ __forceinline__ Index load_chunk(int u) const { return col_[u]; }
+    __device__ __forceinline__ bool live(int u) const { return live_[u]; }
+    __device__ __forceinline__ bool first_row(int) const { return true; }
+    __device__ __forceinline__ bool tensor_start(int u) const { return first_[u] && col_[u] == 0; }
     __device__ __forceinline__ const void* in(int u) const { return in_[u]; }
     __device__ __forceinline__ void* out(int u) const { return out_[u]; }
     __device__ __forceinline__ const void* scale_in(int u) const { return scale_in_[u]; }
@@ -275,7 +354,7 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         // write_scale (src/quantize.rs:83-98): FS(scale), stored by the block's first lane
         const float s_fs = round_to_dtype(param_dtype, s_f);
         const auto si = kGroup == 0 ? 0 : c / kDiv;
-        const bool block_start = at.first_row(u) && (kGroup == 0 ? c == 0 : (c % kDiv) == 0);
+        const bool block_start = kGroup == 0 ? at.tensor_start(u) : (at.first_row(u) && (c % kDiv) == 0);
         if (scale_out != nullptr && live && block_start) store_dtype(param_dtype, scale_out, si, s_fs);
         // divisor F(FS(scale)); s_f is an F value, so f32 params leave it unchanged
         float d = s_fs;
@@ -327,6 +406,16 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_rows_kernel(
                                                             F::kBytes, out_scale_bytes, rows};
     quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParamF32, kWide, kUnroll, kThreads, kChecked, kEnc>(
         geo, param_dtype_rt, qp, num_partials);
+}
+
+// Rows found lane by lane (LaneSteps); the scale type is read at run time.
+template <class F, int kBits, int kGroup, int kScaleSrc, bool kWide, int kUnroll, int kThreads, int kEnc = kEncInt>
+__global__ __launch_bounds__(kThreads) void quantize_flat_lanes_kernel(
+    const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
+    void* __restrict__ scale_out, int param_dtype_rt, QuantParams qp, uint32_t num_partials, LaneRows rows) {
+    const LanesGeo geo{in, out, scale_in, scale_out, rows};
+    quantize_flat_body<F, kBits, kGroup, kScaleSrc, false, kWide, kUnroll, kThreads, true, kEnc>(geo, param_dtype_rt, qp,
+                                                                                               num_partials);
 }
 
 // `scale_in` of the geometry holds the stored scales
@@ -392,6 +481,14 @@ __global__ __launch_bounds__(kThreads) void dequantize_flat_rows_kernel(
     dequantize_flat_body<F, kBits, kGroup, kParamF32, kUnroll, kThreads, kChecked, kEnc>(geo, param_dtype_rt);
 }
 
+template <class F, int kBits, int kGroup, int kUnroll, int kThreads, int kEnc = kEncInt>
+__global__ __launch_bounds__(kThreads) void dequantize_flat_lanes_kernel(
+    const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params, int param_dtype_rt,
+    LaneRows rows) {
+    const LanesGeo geo{in, out, params, nullptr, rows};
+    dequantize_flat_body<F, kBits, kGroup, false, kUnroll, kThreads, true, kEnc>(geo, param_dtype_rt);
+}
+
 // Block abs-max -> scale typed like the input (what quantize takes as `scale`).
 template <class F, int kGroup, int kUnroll, int kThreads, class Geo>
 __device__ __forceinline__ void scales_flat_body(const Geo& geo, const QuantParams& qp) {
@@ -429,6 +526,14 @@ __global__ __launch_bounds__(kThreads) void scales_flat_rows_kernel(const u32x4*
                                                                     void* __restrict__ scales, QuantParams qp,
                                                                     FlatRows rows) {
     const RowsGeo<16, 0, kGroup> geo{in, nullptr, nullptr, scales, 0, 0, F::kBytes, rows};
+    scales_flat_body<F, kGroup, kUnroll, kThreads>(geo, qp);
+}
+
+template <class F, int kGroup, int kUnroll, int kThreads>
+__global__ __launch_bounds__(kThreads) void scales_flat_lanes_kernel(const u32x4* __restrict__ in,
+                                                                     void* __restrict__ scales, QuantParams qp,
+                                                                     LaneRows rows) {
+    const LanesGeo geo{in, nullptr, nullptr, scales, rows};
     scales_flat_body<F, kGroup, kUnroll, kThreads>(geo, qp);
 }
 

@@ -10,6 +10,11 @@ hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
     auto out = static_cast<u32x4*>(a.output);
     const bool p32 = a.param_dtype == CQ_F32;
     constexpr int kU = kUnrollD<F, kBits, kGroup>;
+    if (a.lanes.levels > 0) {
+        hipLaunchKernelGGL((dequantize_flat_lanes_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(lanes_grid(a, kU)),
+                           dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, lane_rows(a));
+        return hipGetLastError();
+    }
     if (a.rows > 1)
         return launch_row_steps(a, kU, [&](bool checked, uint32_t grid, uint32_t step_begin) {
             auto kernel = checked ? (p32 ? dequantize_flat_rows_kernel<F, kBits, kGroup, true, kU, kThreads, true, kEnc>

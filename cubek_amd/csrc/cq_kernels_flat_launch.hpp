@@ -67,6 +67,29 @@ FlatRows flat_rows(const FlatArgs& a) {
     return r;
 }
 
+// the same for the kernels that find each lane's row
+static_assert(kMaxLaneLevels == CQ_MAX_RANK - 1, "one level per leading dimension");
+LaneRows lane_rows(const FlatArgs& a) {
+    LaneRows r{};
+    r.row_chunks = static_cast<uint32_t>(a.num_chunks);
+    magic_of(r.row_chunks, &r.row_magic, &r.row_shift);
+    r.total_chunks = static_cast<uint32_t>(a.rows * a.num_chunks);
+    r.levels = a.lanes.levels;
+    for (uint32_t l = 0; l < r.levels; l++) {
+        r.count[l] = a.lanes.count[l];
+        magic_of(r.count[l], &r.magic[l], &r.shift[l]);
+        r.in[l] = a.lanes.in[l];
+        r.out[l] = a.lanes.out[l];
+        r.scale_in[l] = a.lanes.scale_in[l];
+        r.scale_out[l] = a.lanes.scale_out[l];
+    }
+    return r;
+}
+inline uint32_t lanes_grid(const FlatArgs& a, int unroll) {
+    const uint64_t per = static_cast<uint64_t>(kThreads) * unroll;
+    return static_cast<uint32_t>((a.rows * a.num_chunks + per - 1) / per);
+}
+
 QuantParams quant_params(const Range& r) {
     QuantParams p;
     p.lo = r.lo;
@@ -127,6 +150,12 @@ hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
         auto out = static_cast<uint32_t*>(a.output);
         const QuantParams qp = quant_params(a.range);
         const bool p32 = a.param_dtype == CQ_F32;
+        if (a.lanes.levels > 0) {
+            hipLaunchKernelGGL((quantize_flat_lanes_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
+                               dim3(lanes_grid(a, kUnrollQ)), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
+                               a.param_dtype, qp, a.num_partials, lane_rows(a));
+            return hipGetLastError();
+        }
         if (a.rows > 1)
             return launch_row_steps(a, kUnrollQ, [&](bool checked, uint32_t grid, uint32_t step_begin) {
                 auto kernel =

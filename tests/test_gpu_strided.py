@@ -84,6 +84,15 @@ def layouts(shape, per):
 
         out.append(("leading_swapped", leading_swapped(shape, 64), leading_swapped(pshape, 8)))
         out.append(("leading_swapped_floats", leading_swapped(shape, 0), contiguous(pshape)))
+    if rank >= 4:
+        # dimensions 1 and 2 swapped in memory (heads and positions of an attention tensor): short rows
+        # behind three levels of strides
+        def middle_swapped(sh):
+            st = contiguous((sh[0], sh[2], sh[1]) + tuple(sh[3:]))
+            return (st[0], st[2], st[1]) + tuple(st[3:])
+
+        out.append(("middle_swapped", middle_swapped(shape), middle_swapped(pshape)))
+        out.append(("middle_swapped_floats", middle_swapped(shape), contiguous(pshape)))
     return pshape, out
 
 
@@ -129,6 +138,15 @@ def test_pitched_rows_of_a_few_steps(gpu, oracle, elem, name, scheme):
     check_layouts(gpu, oracle, elem, name, scheme,
                   ((4, 4096), (6, 5120), (2, 2, 7168), (4, 2560), (6, 2048), (6, 1024), (10, 1280), (3, 2, 2048), (2, 3, 2, 2560)),
                   ("pitched", "pitched_aligned", "every_other_row", "leading_swapped", "leading_swapped_floats"))
+
+
+@pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
+@pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
+def test_short_rows_behind_permuted_dimensions(gpu, oracle, elem, name, scheme):
+    """[batch, heads, positions, head dimension] views of [batch, positions, heads, head dimension] buffers,
+    and short pitched rows: every lane of the streaming kernels finds its own row."""
+    check_layouts(gpu, oracle, elem, name, scheme, ((2, 3, 6, 128), (2, 5, 8, 64), (1, 2, 300, 256), (3, 2, 2, 1024)),
+                  ("middle_swapped", "middle_swapped_floats", "pitched_aligned", "every_other_row", "leading_swapped"))
 
 
 def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
@@ -332,36 +350,46 @@ def test_broadcast_rows_read_like_their_copies(gpu, cols):
     assert torch.equal(outs[0][0], outs[0][2])
 
 
+LARGE_VIEWS = {
+    # a [4, 3584, 8192] slice of a [4, 4096, 8256] buffer: rows in groups with a pitch of their own
+    "sliced_batches": ((4, 3584, 8192), (4, 4096, 8256), (4096 * 8256, 8256, 1)),
+    # [batch, heads, positions, head dimension] out of [batch, positions, heads, head dimension]
+    "permuted_heads": ((8, 32, 2048, 128), (8, 2048, 32, 128), (2048 * 32 * 128, 128, 32 * 128, 1)),
+    # short pitched rows
+    "short_pitched_rows": ((65536, 512), (65536, 576), (576, 1)),
+}
+
+
 @pytest.mark.gpu
+@pytest.mark.parametrize("case", sorted(LARGE_VIEWS))
 @pytest.mark.parametrize("elem", [ElemType.BF16, ElemType.F32], ids=lambda e: e.name)
-def test_large_sliced_batches_match_the_contiguous_path(gpu, elem):
-    """A [4, 3584, 8192] slice of a [4, 4096, 8256] buffer (rows in groups with a pitch of their own, the
-    grid numbered through all of them): codes, scales and dequantized values must equal what the contiguous
-    kernels, checked against the oracle elsewhere, give for a contiguous copy; what lies between the rows
-    and between the groups stays as it was."""
+def test_large_strided_views_match_the_contiguous_path(gpu, elem, case):
+    """Strided views with a contiguous last dimension at sizes of thousands of workgroups: codes, scales and
+    dequantized values must equal what the contiguous kernels, checked against the oracle elsewhere, give for
+    a contiguous copy; what the view does not cover stays as it was."""
     import torch
 
     client = ComputeClient.current()
     tdt = torch.float32 if elem == ElemType.F32 else torch.bfloat16
     eb = 4 if elem == ElemType.F32 else 2
-    b, r, c, rb, cb = 4, 3584, 8192, 4096, 8256
+    shape, bufshape, strides = LARGE_VIEWS[case]
     g = torch.Generator(device="cuda")
     g.manual_seed(77 + int(elem))
-    buf = torch.randn((b, rb, cb), generator=g, device="cuda", dtype=torch.float32).mul_(0.05).to(tdt)
-    x = buf[:, :r, :c].contiguous()
+    buf = torch.randn(bufshape, generator=g, device="cuda", dtype=torch.float32).mul_(0.05).to(tdt)
+    x = torch.as_strided(buf, shape, strides).contiguous()
     h = TensorHandleRef.from_torch
-    sliced = lambda t: TensorHandleRef(h(t).handle, (b, r, c), (rb * cb, cb, 1), eb)
+    strided = lambda t: TensorHandleRef(h(t).handle, shape, strides, eb)
     for name, scheme in (("e2m1_block32", QuantScheme.default().with_value(QuantValue.E2M1).with_level(QuantLevel.block([32]))),
                          ("q8s_tensor", QuantScheme.default().with_value(QuantValue.Q8S)),
                          ("e4m3_native_block64", QuantScheme.default().with_value(QuantValue.E4M3)
                           .with_store(QuantStore.Native).with_level(QuantLevel.block([64])))):
-        print(name, elem.name, flush=True)
+        print(case, name, elem.name, flush=True)
         native = scheme.store == QuantStore.Native
-        pshape = scheme.packed_shape((b, r, c)) if not native else (b, r, c)
-        sshape = scheme.scales_shape((b, r, c))
-        ws, nbytes = gpu.workspace(scheme, b * r * c)
+        pshape = scheme.packed_shape(shape) if not native else shape
+        sshape = scheme.scales_shape(shape)
+        ws, nbytes = gpu.workspace(scheme, x.numel())
         outs = []
-        for hx in (h(x), sliced(buf)):
+        for hx in (h(x), strided(buf)):
             codes = torch.full(pshape, 0x5A, dtype=torch.uint8 if native else torch.int32, device="cuda")
             scales = torch.zeros(sshape, dtype=torch.float32, device="cuda")
             qz.launch_dynamic(client, hx, h(codes), h(scales), scheme, elem, ws.data_ptr(), nbytes)
@@ -369,30 +397,32 @@ def test_large_sliced_batches_match_the_contiguous_path(gpu, elem):
         torch.cuda.synchronize()
         assert torch.equal(outs[0][0], outs[1][0]), (name, "codes")
         assert torch.equal(outs[0][1].view(torch.int32), outs[1][1].view(torch.int32)), (name, "scales")
-        # block scales from the sliced tensor, then quantize with them given
+        bits = torch.int16 if eb == 2 else torch.int32
+        # block scales from the strided tensor, then quantize with them given
         if scheme.level.block_size is not None:
             s_in = [torch.zeros(sshape, dtype=tdt, device="cuda") for _ in range(2)]
             qz.compute_scales(client, h(x), h(s_in[0]), scheme, elem)
-            qz.compute_scales(client, sliced(buf), h(s_in[1]), scheme, elem)
+            qz.compute_scales(client, strided(buf), h(s_in[1]), scheme, elem)
             torch.cuda.synchronize()
-            assert torch.equal(s_in[0].view(torch.int16 if eb == 2 else torch.int32),
-                               s_in[1].view(torch.int16 if eb == 2 else torch.int32)), (name, "compute_scales")
+            assert torch.equal(s_in[0].view(bits), s_in[1].view(bits)), (name, "compute_scales")
         else:
             s_in = [outs[0][1].to(tdt)] * 2
         codes2, os2 = torch.zeros_like(outs[0][0]), torch.zeros_like(outs[0][1])
-        qz.launch_ref(client, sliced(buf), h(codes2), h(s_in[1]), h(os2), scheme, elem)
+        qz.launch_ref(client, strided(buf), h(codes2), h(s_in[1]), h(os2), scheme, elem)
         codes3, os3 = torch.zeros_like(outs[0][0]), torch.zeros_like(outs[0][1])
         qz.launch_ref(client, h(x), h(codes3), h(s_in[0]), h(os3), scheme, elem)
         torch.cuda.synchronize()
         assert torch.equal(codes2, codes3), (name, "codes, given scales")
         assert torch.equal(os2.view(torch.int32), os3.view(torch.int32)), (name, "out_scale, given scales")
-        # dequantize into a contiguous tensor and into the slice of a buffer full of a sentinel
+        # dequantize into a contiguous tensor and into the view of a buffer full of a sentinel
         y = torch.empty_like(x)
-        ybuf = torch.full((b, rb, cb), 3.0, dtype=tdt, device="cuda")
+        ybuf = torch.full(bufshape, 3.0, dtype=tdt, device="cuda")
         dq.launch_ref(client, h(outs[0][0]), h(y), h(outs[0][1]), scheme, elem)
-        dq.launch_ref(client, h(outs[0][0]), sliced(ybuf), h(outs[0][1]), scheme, elem)
+        dq.launch_ref(client, h(outs[0][0]), strided(ybuf), h(outs[0][1]), scheme, elem)
         torch.cuda.synchronize()
-        bits = torch.int16 if eb == 2 else torch.int32
-        assert torch.equal(ybuf[:, :r, :c].contiguous().view(bits), y.view(bits)), (name, "dequantized")
-        assert bool((ybuf[:, :, c:] == 3.0).all()) and bool((ybuf[:, r:, :] == 3.0).all()), (name, "padding")
-        del outs, codes2, codes3, os2, os3, y, ybuf
+        yv = torch.as_strided(ybuf, shape, strides)
+        assert torch.equal(yv.contiguous().view(bits), y.view(bits)), (name, "dequantized")
+        covered = torch.zeros(bufshape, dtype=torch.bool, device="cuda")
+        torch.as_strided(covered, shape, strides).fill_(True)
+        assert bool((ybuf[~covered] == 3.0).all()), (name, "wrote outside the view")
+        del outs, codes2, codes3, os2, os3, y, ybuf, yv, covered
