@@ -1,6 +1,5 @@
-// Launchers of the flat (contiguous) kernels: quantize with the scale produced in the launch
-// (fused abs-max, or pass 2 of the per-tensor reduction), block scales, the per-tensor abs-max.
-// Quantize with given scales and dequantize are in cq_kernels_flat_given.hip and
+// Launchers of the flat (contiguous) kernels: block scales, the per-tensor abs-max, and the dispatch of
+// quantize to the per-type launchers of cq_kernels_flat_quantize.hip.  Dequantize is in
 // cq_kernels_flat_dequantize.hip.
 #include "cq_kernels_flat_launch.hpp"
 
@@ -31,9 +30,13 @@ bool flat_block_supported(int dtype, uint32_t block) { return group_of(dtype, bl
 
 hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource src, const FlatArgs& a) {
     if (a.num_chunks == 0) return hipSuccess;
-    if (src == ScaleSource::Given) return launch_quantize_flat_given(s, dtype, bits, a);
-    int g = group_of(dtype, a.block);
-    CQ_SWITCH_DTYPE(dtype, CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (quantize_launch<kF, kB, kG, false>(s, src, a)))))
+    const bool given = src == ScaleSource::Given;
+    switch (dtype) {
+        case CQ_F32: return given ? CQ_QUANTIZE_FLAT_TU(F32, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(F32, 0)(s, bits, src, a);
+        case CQ_BF16: return given ? CQ_QUANTIZE_FLAT_TU(BF16, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(BF16, 0)(s, bits, src, a);
+        case CQ_F16: return given ? CQ_QUANTIZE_FLAT_TU(F16, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(F16, 0)(s, bits, src, a);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 hipError_t launch_scales_flat(hipStream_t s, int dtype, const FlatArgs& a) {

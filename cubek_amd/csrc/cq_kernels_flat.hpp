@@ -11,7 +11,9 @@
 //
 // quantize_flat_rows_kernel / dequantize_flat_rows_kernel run the same bodies over pitched rows: a
 // row is a whole number of steps (kThreads chunks, the last one of a row may be partial), and a
-// workgroup's kUnroll steps may lie in different rows.
+// workgroup's kUnroll steps may lie in different rows.  quantize_flat_lanes_kernel /
+// dequantize_flat_lanes_kernel do so for short rows and rows behind several levels of strides: there
+// the lanes of one step lie in different rows and each finds its own.
 //
 // HBM traffic per element is the algorithmic minimum: the input once, the
 // codes once, one scale per block.  Loads and stores carry the non-temporal

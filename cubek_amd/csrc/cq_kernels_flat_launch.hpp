@@ -8,8 +8,16 @@
 
 namespace cq {
 
-// quantize with given scales, defined in cq_kernels_flat_given.hip
-hipError_t launch_quantize_flat_given(hipStream_t s, int dtype, int bits, const FlatArgs& a);
+// The quantize launchers, one per float type and family of scale sources (0: produced in the launch,
+// 1: given), each compiled from cq_kernels_flat_quantize.hip into an object of its own.
+#define CQ_QUANTIZE_FLAT_TU_(f, g) launch_quantize_flat_##f##_##g
+#define CQ_QUANTIZE_FLAT_TU(f, g) CQ_QUANTIZE_FLAT_TU_(f, g)
+hipError_t CQ_QUANTIZE_FLAT_TU(F32, 0)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
+hipError_t CQ_QUANTIZE_FLAT_TU(F32, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
+hipError_t CQ_QUANTIZE_FLAT_TU(BF16, 0)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
+hipError_t CQ_QUANTIZE_FLAT_TU(BF16, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
+hipError_t CQ_QUANTIZE_FLAT_TU(F16, 0)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
+hipError_t CQ_QUANTIZE_FLAT_TU(F16, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
 
 namespace {
 

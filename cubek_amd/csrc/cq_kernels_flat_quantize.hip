@@ -1,0 +1,21 @@
+// Launchers of the flat quantize kernels of one float type and one family of scale sources.  The
+// Makefile compiles this file six times (-DCQ_TU_FLOAT=F32|BF16|F16, -DCQ_TU_GIVEN=0|1: scales produced
+// in the launch, or given), each into an object of its own, so that the build runs in parallel: in
+// one translation unit the instantiations take minutes.
+#include "cq_kernels_flat_launch.hpp"
+
+#ifndef CQ_TU_FLOAT
+#define CQ_TU_FLOAT F32
+#endif
+#ifndef CQ_TU_GIVEN
+#define CQ_TU_GIVEN 0
+#endif
+
+namespace cq {
+
+hipError_t CQ_QUANTIZE_FLAT_TU(CQ_TU_FLOAT, CQ_TU_GIVEN)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a) {
+    int g = group_of(CQ_TU_FLOAT::kDtype, a.block);
+    CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (quantize_launch<CQ_TU_FLOAT, kB, kG, CQ_TU_GIVEN != 0>(s, src, a))))
+}
+
+}  // namespace cq
