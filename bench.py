@@ -219,8 +219,8 @@ def cpu_baseline(torch, w, path, budget_s=12.0):
 
 def adjacent_kernels(torch):
     """The steps either side of the path on the headline tensor: abs-max along an axis
-    (cq_reduce_max_abs) in front of it, 2-D blocks, a transposed float tensor and pitched rows
-    through the path itself, re-packing of a transposed quantized tensor (cq_into_contiguous_packed)
+    (cq_reduce_max_abs) in front of it, 2-D blocks, a transposed float tensor, pitched rows and an
+    attention layout through the path itself, re-packing of a transposed quantized tensor (cq_into_contiguous_packed)
     behind it.  Reported only; `value` does not include them."""
     from cubek_amd import ComputeClient, ElemType, TensorHandleRef
     from cubek_amd import contiguous as cq_contiguous
@@ -308,6 +308,28 @@ def adjacent_kernels(torch):
                         "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
         del xp, yp, words, bscales, hxp, hyp, hw, hb
         torch.cuda.empty_cache()
+    # the headline scheme on an attention layout: the [batch, heads, positions, head dimension] view of a
+    # [batch, positions, heads, head dimension] buffer (rows of 128 elements behind permuted dimensions)
+    nb, nh, ns, nd = 8, 32, 4096, 128
+    xa = [torch.randn((nb, ns, nh, nd), device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
+    ya = [torch.empty((nb, ns, nh, nd), device="cuda", dtype=torch.bfloat16) for _ in range(2)]
+    words = [torch.empty((nb, nh, ns, nd // 8), dtype=torch.int32, device="cuda") for _ in range(2)]
+    bscales = [torch.empty((nb, nh, ns, nd // 32), dtype=torch.float32, device="cuda") for _ in range(2)]
+    heads = lambda t: TensorHandleRef(h(t).handle, (nb, nh, ns, nd), (ns * nh * nd, nd, nh * nd, 1), 2)
+    hxa, hya = [heads(t) for t in xa], [heads(t) for t in ya]
+    hw, hb = [h(t) for t in words], [h(t) for t in bscales]
+    b = nb * nh * ns * nd * 2 + words[0].numel() * 4 + bscales[0].numel() * 4
+    for label, fn in (
+            ("quantize_dynamic", lambda i: cq_quantize.launch_dynamic(client, hxa[i % sets], hw[i % 2], hb[i % 2], scheme,
+                                                                       ElemType.BF16)),
+            ("dequantize", lambda i: cq_dequantize.launch_ref(client, hw[i % 2], hya[i % 2], hb[i % 2], scheme,
+                                                              ElemType.BF16))):
+        ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
+        out.append({"kernel": f"{label}, e2m1 blocks of 32, bf16 [{nb}, {nh}, {ns}, {nd}] view of a [{nb}, {ns}, {nh}, {nd}] buffer",
+                    "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                    "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+    del xa, ya, words, bscales, hxa, hya, hw, hb
+    torch.cuda.empty_cache()
     # 4-bit codes of a [rows, cols] weight, 8 per u32 word along cols, viewed transposed as [cols, rows]
     packing = 8
     srcs = [torch.randint(-2**31, 2**31 - 1, (rows, cols // packing), dtype=torch.int32, device="cuda")
