@@ -145,7 +145,7 @@ def test_pitched_rows_of_a_few_steps(gpu, oracle, elem, name, scheme):
 def test_short_rows_behind_permuted_dimensions(gpu, oracle, elem, name, scheme):
     """[batch, heads, positions, head dimension] views of [batch, positions, heads, head dimension] buffers,
     and short pitched rows: every lane of the streaming kernels finds its own row."""
-    check_layouts(gpu, oracle, elem, name, scheme, ((2, 3, 6, 128), (2, 5, 8, 64), (1, 2, 300, 256), (3, 2, 2, 1024)),
+    check_layouts(gpu, oracle, elem, name, scheme, ((2, 3, 6, 128), (2, 5, 8, 64), (2, 4, 8, 128), (1, 12, 24, 64), (1, 2, 300, 256), (3, 2, 2, 1024)),
                   ("middle_swapped", "middle_swapped_floats", "pitched_aligned", "every_other_row", "leading_swapped"))
 
 
