@@ -313,16 +313,17 @@ def adjacent_kernels(torch):
     nb, nh, ns, nd = 8, 32, 4096, 128
     xa = [torch.randn((nb, ns, nh, nd), device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
     ya = [torch.empty((nb, ns, nh, nd), device="cuda", dtype=torch.bfloat16) for _ in range(2)]
-    words = [torch.empty((nb, nh, ns, nd // 8), dtype=torch.int32, device="cuda") for _ in range(2)]
-    bscales = [torch.empty((nb, nh, ns, nd // 32), dtype=torch.float32, device="cuda") for _ in range(2)]
+    # four output sets as well: two (168 MB) would stay in the 256 MB Infinity Cache and never reach HBM
+    words = [torch.empty((nb, nh, ns, nd // 8), dtype=torch.int32, device="cuda") for _ in range(sets)]
+    bscales = [torch.empty((nb, nh, ns, nd // 32), dtype=torch.float32, device="cuda") for _ in range(sets)]
     heads = lambda t: TensorHandleRef(h(t).handle, (nb, nh, ns, nd), (ns * nh * nd, nd, nh * nd, 1), 2)
     hxa, hya = [heads(t) for t in xa], [heads(t) for t in ya]
     hw, hb = [h(t) for t in words], [h(t) for t in bscales]
     b = nb * nh * ns * nd * 2 + words[0].numel() * 4 + bscales[0].numel() * 4
     for label, fn in (
-            ("quantize_dynamic", lambda i: cq_quantize.launch_dynamic(client, hxa[i % sets], hw[i % 2], hb[i % 2], scheme,
+            ("quantize_dynamic", lambda i: cq_quantize.launch_dynamic(client, hxa[i % sets], hw[i % sets], hb[i % sets], scheme,
                                                                        ElemType.BF16)),
-            ("dequantize", lambda i: cq_dequantize.launch_ref(client, hw[i % 2], hya[i % 2], hb[i % 2], scheme,
+            ("dequantize", lambda i: cq_dequantize.launch_ref(client, hw[i % sets], hya[i % 2], hb[i % sets], scheme,
                                                               ElemType.BF16))):
         ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
         out.append({"kernel": f"{label}, e2m1 blocks of 32, bf16 [{nb}, {nh}, {ns}, {nd}] view of a [{nb}, {ns}, {nh}, {nd}] buffer",
