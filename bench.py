@@ -52,8 +52,8 @@ WORKLOADS = {
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); filled from
 # the summaries under profiles/.  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/quantize_dequantize_flat_bf16_e2m1_b32_cfg5.md: (229419.5*2.0 + 143360.1) KiB
-    "cfg5": 616651878,
+    # profiles/quantize_dequantize_flat_bf16_e2m1_b32_cfg5.md: (229432.5*2.0 + 143360.0) KiB
+    "cfg5": 616678400,
 }
 
 
