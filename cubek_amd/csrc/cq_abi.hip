@@ -1054,7 +1054,8 @@ cq_status cq_reduce_max_abs(cq_stream_t stream, const cq_tensor* input, const cq
     a.workspace_bytes = a.workspace ? workspace_bytes : 0;
     a.rank = input->rank;
     a.axis = axis;
-    a.contiguous = is_contiguous(input) && is_contiguous(output);
+    a.out_contiguous = is_contiguous(output);
+    a.contiguous = is_contiguous(input) && a.out_contiguous;
     reduce_view(input, axis, &a.outer, &a.len, &a.inner);
     if (a.outer == 0 || a.inner == 0) return CQ_OK;  // no outputs
     return hip_status(cq::launch_reduce_max_abs(stream, dtype, a));

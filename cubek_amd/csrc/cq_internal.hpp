@@ -120,6 +120,7 @@ struct ReduceArgs {
     uint64_t shape[CQ_MAX_RANK];
     uint64_t in_strides[CQ_MAX_RANK], out_strides[CQ_MAX_RANK];
     bool contiguous;         // input and output are contiguous row-major
+    bool out_contiguous;     // the output is
     uint64_t outer, len, inner;  // the contiguous view [outer, len, inner] around the axis
 };
 hipError_t launch_reduce_max_abs(hipStream_t s, int dtype, const ReduceArgs& a);

@@ -20,6 +20,7 @@
 // one-wave-per-output (long axis) or one-thread-per-output fallback.
 #include "cq_device.hpp"
 #include "cq_internal.hpp"
+#include "cq_magic_div.hpp"
 
 namespace cq {
 namespace {
@@ -215,6 +216,131 @@ __global__ __launch_bounds__(kT) void reduce_tile_kernel(const u32x4* __restrict
     }
 }
 
+// ---- strided inputs with a contiguous last dimension ------------------------------------
+// The dimensions that are not reduced, innermost first (`count` entries each, multiply-and-shift
+// divisions), with their input strides in 16-byte chunks; the outputs are contiguous.
+struct ReduceLevels {
+    uint32_t levels;
+    uint32_t count[CQ_MAX_RANK], magic[CQ_MAX_RANK], shift[CQ_MAX_RANK];
+    uint64_t in[CQ_MAX_RANK];
+};
+__device__ __forceinline__ uint64_t level_offset(const ReduceLevels& r, uint32_t n) {
+    uint64_t off = 0;
+#pragma unroll
+    for (int l = 0; l < CQ_MAX_RANK; l++) {
+        if (l < static_cast<int>(r.levels)) {
+            uint32_t index = n;
+            if (l + 1 < static_cast<int>(r.levels)) {
+                const uint32_t q = magic_div(n, r.magic[l], r.shift[l]);
+                index = n - q * r.count[l];
+                n = q;
+            }
+            off += index * r.in[l];
+        }
+    }
+    return off;
+}
+
+// reduce_rows_grouped_kernel with the rows (all dimensions but the last) found through `r`
+template <class F, int kGroup, int kUnroll>
+__global__ __launch_bounds__(kThreads) void reduce_rows_grouped_strided_kernel(const u32x4* __restrict__ in,
+                                                                               void* __restrict__ out, ReduceLevels r,
+                                                                               uint64_t num_chunks) {
+    const uint64_t first = static_cast<uint64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+    u32x4 raw[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+        uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
+        c = c < num_chunks ? c : num_chunks - 1;
+        raw[u] = stream_load(in + level_offset(r, static_cast<uint32_t>(c / kGroup)) + c % kGroup);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+        const uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
+        float amax = group_max<kGroup>(chunk_absmax<F>(raw[u], 0.0f));
+        if (c < num_chunks && (c % kGroup) == 0) F::store(out, c / kGroup, amax);
+    }
+}
+
+// reduce_rows_wave_kernel with the rows found through `r`
+template <class F, bool kPartial>
+__global__ __launch_bounds__(kThreads) void reduce_rows_wave_strided_kernel(const u32x4* __restrict__ in,
+                                                                            void* __restrict__ out, ReduceLevels r,
+                                                                            uint64_t rows, uint64_t chunks_per_row,
+                                                                            uint32_t slices, uint64_t pitch) {
+    constexpr int kUnroll = 4;
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint64_t job = static_cast<uint64_t>(blockIdx.x) * (kThreads / kWave) + threadIdx.x / kWave;
+    if (job >= rows * slices) return;  // whole waves leave together
+    const uint64_t row = job / slices;
+    const uint32_t slice = static_cast<uint32_t>(job % slices);
+    const uint64_t per_slice = (chunks_per_row + slices - 1) / slices;
+    const uint64_t begin = slice * per_slice;
+    const uint64_t end = begin + per_slice < chunks_per_row ? begin + per_slice : chunks_per_row;
+    const u32x4* p = in + level_offset(r, static_cast<uint32_t>(row));
+    float amax = 0.0f;
+    for (uint64_t c0 = begin + lane; c0 < end; c0 += kWave * kUnroll) {
+        u32x4 raw[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const uint64_t c = c0 + static_cast<uint64_t>(u) * kWave;
+            raw[u] = stream_load(p + (c < end ? c : end - 1));
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) amax = chunk_absmax<F>(raw[u], amax);
+    }
+    amax = group_max<64>(amax);
+    if (lane == 0) {
+        if constexpr (kPartial)
+            static_cast<float*>(out)[static_cast<uint64_t>(slice) * pitch + row] = amax;
+        else
+            F::store(out, row, amax);
+    }
+}
+
+// reduce_cols_kernel with the output chunks (the last dimension in chunks, then the other kept
+// dimensions) found through `r`; the reduced axis steps `len_stride` chunks
+template <class F, bool kPartial>
+__global__ __launch_bounds__(kThreads) void reduce_cols_strided_kernel(const u32x4* __restrict__ in, void* __restrict__ out,
+                                                                       ReduceLevels r, uint64_t cols, uint64_t len,
+                                                                       uint64_t len_stride, uint32_t slices) {
+    constexpr int kN = F::kPerChunk;
+    constexpr int kUnroll = 4;
+    const uint64_t t = static_cast<uint64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (t >= cols * slices) return;
+    const uint32_t slice = static_cast<uint32_t>(t / cols);
+    const uint64_t col = t % cols;
+    const uint64_t per_slice = (len + slices - 1) / slices;
+    const uint64_t begin = slice * per_slice;
+    const uint64_t end = begin + per_slice < len ? begin + per_slice : len;
+    const u32x4* p = in + level_offset(r, static_cast<uint32_t>(col));
+    float amax[kN];
+#pragma unroll
+    for (int i = 0; i < kN; i++) amax[i] = 0.0f;
+    for (uint64_t l0 = begin; l0 < end; l0 += kUnroll) {
+        u32x4 raw[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const uint64_t l = l0 + u < end ? l0 + u : end - 1;
+            raw[u] = stream_load(p + l * len_stride);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            float v[kN];
+            F::unpack(raw[u], v);
+#pragma unroll
+            for (int i = 0; i < kN; i++) amax[i] = fmaxf(amax[i], fabsf(v[i]));
+        }
+    }
+    if constexpr (kPartial) {
+        float* dst = static_cast<float*>(out) + (static_cast<uint64_t>(slice) * cols + col) * kN;
+#pragma unroll
+        for (int i = 0; i < kN; i++) dst[i] = amax[i];
+    } else {
+        static_cast<u32x4*>(out)[col] = F::pack(amax);
+    }
+}
+
 // ---- fallbacks: any strides -----------------------------------------------------------
 struct StridedReduce {
     uint32_t rank, axis;
@@ -266,6 +392,7 @@ struct ReducePlan {
     uint64_t chunks_per_row = 0, inner_chunks = 0;
     uint32_t cw = 1, col_tiles = 1;
     uint64_t slices = 1;  // wanted; the launcher lowers it to what the workspace holds
+    uint64_t lane_slices = 1;  // kTile on a strided input (one lane per output chunk and slice instead): wanted there
     uint64_t pitch = 0;   // floats per slice of partials
 };
 
@@ -305,6 +432,10 @@ ReducePlan plan_reduce(uint64_t outer, uint64_t len, uint64_t inner, uint64_t kN
         return p;
     }
     p.kind = ReducePlan::kTile;
+    p.lane_slices = kTargetLanes / cols;
+    if (p.lane_slices > (len + 15) / 16) p.lane_slices = (len + 15) / 16;
+    if (p.lane_slices > traffic_cap) p.lane_slices = traffic_cap;
+    if (p.lane_slices < 1) p.lane_slices = 1;
     p.cw = pow2_at_least(p.inner_chunks, kWave);
     p.col_tiles = static_cast<uint32_t>((p.inner_chunks + p.cw - 1) / p.cw);
     p.pitch = outer * inner;  // a multiple of kN, hence of 4
@@ -342,11 +473,102 @@ void launch_fold(hipStream_t s, const void* partials, void* out, uint64_t slices
     launch_tile<F32, F, kFoldThreads, kTileFinalChecked>(s, cw, tiles, partials, out, slices, chunks, tiles, 1u, 0, count);
 }
 
+// The levels of a strided input with a contiguous last dimension of whole chunks, aligned strides and
+// fewer than 2^31 rows and output chunks; false: not such a tensor.
+template <class F>
+bool strided_levels(const ReduceArgs& a, ReduceLevels* r, uint64_t* len_stride) {
+    constexpr uint64_t kN = F::kPerChunk;
+    if (a.rank < 2 || (reinterpret_cast<uintptr_t>(a.input) & 15u) != 0) return false;
+    const uint32_t last = a.rank - 1;
+    if (a.in_strides[last] != 1 || a.shape[last] % kN != 0) return false;
+    *r = ReduceLevels{};
+    *len_stride = 0;
+    uint64_t total = 1;
+    const auto push = [&](uint64_t count, uint64_t stride) {
+        const uint32_t k = r->levels;
+        if (k > 0 && stride == r->in[k - 1] * r->count[k - 1] && r->count[k - 1] * count < (1ull << 31)) {
+            r->count[k - 1] *= static_cast<uint32_t>(count);  // steps on uniformly from the level inside it
+        } else {
+            r->count[k] = static_cast<uint32_t>(count);
+            r->in[k] = stride;
+            r->levels = k + 1;
+        }
+        total *= count;
+    };
+    if (a.axis != last) push(a.shape[last] / kN, 1);
+    for (int d = static_cast<int>(last) - 1; d >= 0; d--) {
+        if (a.in_strides[d] % kN != 0 && a.shape[d] > 1) return false;
+        if (static_cast<uint32_t>(d) == a.axis) {
+            *len_stride = a.in_strides[d] / kN;
+            continue;
+        }
+        if (a.shape[d] == 1) continue;
+        push(a.shape[d], a.in_strides[d] / kN);
+    }
+    if (r->levels == 0) push(1, 0);
+    if (total >= (1ull << 31)) return false;
+    for (uint32_t l = 0; l < r->levels; l++) magic_of(r->count[l], &r->magic[l], &r->shift[l]);
+    return true;
+}
+
 template <class F>
 hipError_t reduce_dispatch(hipStream_t s, const ReduceArgs& a) {
     constexpr uint64_t kN = F::kPerChunk;
     ReducePlan p;
     if (a.contiguous && (reinterpret_cast<uintptr_t>(a.input) & 15u) == 0) p = plan_reduce(a.outer, a.len, a.inner, kN);
+    ReduceLevels levels;
+    uint64_t len_stride = 0;
+    if (!a.contiguous && a.out_contiguous && strided_levels<F>(a, &levels, &len_stride)) {
+        // the plan of the contiguous tensor of this shape, with kernels that look up where rows and columns lie
+        p = plan_reduce(a.outer, a.len, a.inner, kN);
+        const bool rows = p.kind == ReducePlan::kRowsGrouped || p.kind == ReducePlan::kRowsWave;
+        const bool cols = p.kind == ReducePlan::kCols || p.kind == ReducePlan::kTile;
+        if ((rows && a.axis != a.rank - 1) || (cols && (a.axis == a.rank - 1 || (reinterpret_cast<uintptr_t>(a.output) & 15u) != 0)))
+            p.kind = ReducePlan::kFallback;
+        uint64_t slices = p.kind == ReducePlan::kTile ? p.lane_slices : p.slices;
+        if (slices > 1) {
+            const uint64_t fit = a.workspace == nullptr ? 0 : a.workspace_bytes / (p.pitch * sizeof(float));
+            if (slices > fit) slices = fit > 1 ? fit : 1;
+        }
+        auto in = static_cast<const u32x4*>(a.input);
+        if (p.kind == ReducePlan::kRowsGrouped) {
+            const uint64_t num_chunks = a.outer * p.chunks_per_row;
+            constexpr int kU = 4;
+            dim3 grid = blocks(num_chunks, kThreads * kU);
+            switch (p.chunks_per_row) {
+#define CQ_CASE(G) case G: hipLaunchKernelGGL((reduce_rows_grouped_strided_kernel<F, G, kU>), grid, dim3(kThreads), 0, s, in, a.output, levels, num_chunks); break;
+                CQ_CASE(1) CQ_CASE(2) CQ_CASE(4) CQ_CASE(8) CQ_CASE(16) CQ_CASE(32) CQ_CASE(64)
+#undef CQ_CASE
+            }
+            return hipGetLastError();
+        }
+        if (p.kind == ReducePlan::kRowsWave) {
+            dim3 grid = blocks(a.outer * slices, kThreads / kWave);
+            if (slices > 1) {
+                hipLaunchKernelGGL((reduce_rows_wave_strided_kernel<F, true>), grid, dim3(kThreads), 0, s, in, a.workspace,
+                                   levels, a.outer, p.chunks_per_row, static_cast<uint32_t>(slices), p.pitch);
+                launch_fold<F>(s, a.workspace, a.output, slices, p.pitch, a.outer);
+            } else {
+                hipLaunchKernelGGL((reduce_rows_wave_strided_kernel<F, false>), grid, dim3(kThreads), 0, s, in, a.output,
+                                   levels, a.outer, p.chunks_per_row, 1u, 0);
+            }
+            return hipGetLastError();
+        }
+        if (cols && p.kind != ReducePlan::kFallback) {
+            const uint64_t out_chunks = a.outer * p.inner_chunks;
+            dim3 grid = blocks(out_chunks * slices, kThreads);
+            if (slices > 1) {
+                hipLaunchKernelGGL((reduce_cols_strided_kernel<F, true>), grid, dim3(kThreads), 0, s, in, a.workspace, levels,
+                                   out_chunks, a.len, len_stride, static_cast<uint32_t>(slices));
+                launch_fold<F>(s, a.workspace, a.output, slices, p.pitch, p.pitch);
+            } else {
+                hipLaunchKernelGGL((reduce_cols_strided_kernel<F, false>), grid, dim3(kThreads), 0, s, in, a.output, levels,
+                                   out_chunks, a.len, len_stride, 1u);
+            }
+            return hipGetLastError();
+        }
+        p = ReducePlan{};
+    }
     if ((p.kind == ReducePlan::kCols || p.kind == ReducePlan::kTile) && (reinterpret_cast<uintptr_t>(a.output) & 15u) != 0)
         p.kind = ReducePlan::kFallback;
     uint64_t slices = p.slices;
@@ -429,7 +651,8 @@ hipError_t reduce_dispatch(hipStream_t s, const ReduceArgs& a) {
 
 uint64_t reduce_workspace_bytes(uint64_t outer, uint64_t len, uint64_t inner, int dtype) {
     const ReducePlan p = plan_reduce(outer, len, inner, dtype == CQ_F32 ? 4 : 8);
-    return p.slices > 1 ? p.slices * p.pitch * sizeof(float) : 0;
+    const uint64_t slices = p.slices > p.lane_slices ? p.slices : p.lane_slices;  // either kernel set may run
+    return slices > 1 ? slices * p.pitch * sizeof(float) : 0;
 }
 
 hipError_t launch_reduce_max_abs(hipStream_t s, int dtype, const ReduceArgs& a) {

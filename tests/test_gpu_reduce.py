@@ -167,6 +167,71 @@ def test_reduce_random_shapes_axes_and_layouts(gpu, oracle, seed):
             assert np.array_equal(got[:n_out].view(np.uint8), want.view(np.uint8)), (shape, strides, axis, elem.name, use_ws)
 
 
+# shape, input strides (elements): strided inputs whose last dimension is contiguous
+ROWWISE_STRIDED = [
+    ((96, 4096), (4160, 1)),                                   # pitched rows, long
+    ((2048, 64), (72, 1)),                                     # pitched rows, short
+    ((300, 1024), (2048, 1)),                                  # every other row
+    ((2, 6, 40, 128), (6 * 40 * 128, 128, 6 * 128, 1)),        # heads and positions swapped in memory
+    ((3, 5, 2048), (2048, 3 * 2048, 1)),                       # leading dimensions swapped
+    ((4, 700, 256), (1024 * 320, 320, 1)),                     # a slice of a larger batch, pitched
+    ((1, 9000, 8), (0, 16, 1)),                                # rows of one 16-byte chunk (two for f32) at a pitch
+]
+
+
+@pytest.mark.parametrize("elem", ELEMS, ids=lambda e: e.name)
+def test_reduce_strided_inputs_with_contiguous_rows(gpu, oracle, elem):
+    """Every axis of pitched, sliced and permuted inputs (the kernels that look up each row or column
+    dimension by dimension), with and without the workspace for partial maxima, NaN elements ignored."""
+    import torch
+
+    rng = np.random.default_rng(4242 + int(elem))
+    for shape, strides in ROWWISE_STRIDED:
+        reach = 1 + sum((n - 1) * st for n, st in zip(shape, strides))
+        x32 = rng.normal(0, 1, reach).astype(np.float32)
+        x32[rng.random(reach) < 0.01] = np.nan
+        x = oracle.to_bits(x32, elem)
+        for axis in range(len(shape)):
+            want = oracle.reduce_max_abs(x, elem, shape, axis, in_strides=strides).reshape(-1)
+            for use_ws in (True, False):
+                got, n_out = run(torch, gpu, x, elem, shape, axis, use_workspace=use_ws, in_strides=strides)
+                assert np.array_equal(got[:n_out].view(np.uint8), want.view(np.uint8)), (shape, strides, axis, use_ws)
+
+
+@pytest.mark.parametrize("case", ["permuted_heads", "pitched_rows"])
+def test_reduce_large_strided_views_match_their_contiguous_copies(gpu, case):
+    """Full-size strided inputs (thousands of workgroups, sliced reductions with a fold) against the
+    contiguous kernels, which the other tests check against the oracle, on a contiguous copy."""
+    import torch
+
+    from cubek_amd import TensorHandleRef
+
+    shape, bufshape, strides = {
+        "permuted_heads": ((8, 32, 2048, 128), (8, 2048, 32, 128), (2048 * 32 * 128, 128, 32 * 128, 1)),
+        "pitched_rows": ((14336, 8192), (14336, 8256), (8256, 1)),
+    }[case]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    buf = torch.randn(bufshape, generator=g, device="cuda", dtype=torch.bfloat16)
+    buf.view(-1)[::4099] = float("nan")
+    x = torch.as_strided(buf, shape, strides).contiguous()
+    h = TensorHandleRef.from_torch
+    client = ComputeClient.current()
+    for axis in range(len(shape)):
+        oshape = tuple(1 if d == axis else n for d, n in enumerate(shape))
+        outs = []
+        for hin in (h(x), TensorHandleRef(h(buf).handle, shape, strides, 2)):
+            o = torch.full(oshape, -1.0, device="cuda", dtype=torch.bfloat16)
+            nbytes = cq_reduce.workspace_bytes(hin, axis, ElemType.BF16)
+            ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+            cq_reduce.max_abs(client, hin, h(o), axis, ElemType.BF16, ws.data_ptr() if nbytes else 0, nbytes)
+            torch.cuda.synchronize()
+            outs.append(o)
+        assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16)), (case, axis)
+        ref = torch.nan_to_num(x.float(), nan=0.0).abs().amax(dim=axis, keepdim=True).to(torch.bfloat16)
+        assert torch.equal(outs[1].view(torch.int16), ref.view(torch.int16)), (case, axis, "torch")
+
+
 def test_reduce_over_an_empty_axis_writes_the_identity(gpu):
     """No elements along the axis: every output is the identity of max-abs, 0."""
     import torch
