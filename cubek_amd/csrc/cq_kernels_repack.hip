@@ -5,7 +5,9 @@
 // (P values per stored element, value 0 in the low bits); the input holds P values
 // per element along `packed_dim` and is addressed through its strides.
 #include "cq_device.hpp"
+#include "cq_device.hpp"
 #include "cq_internal.hpp"
+#include "cq_magic_div.hpp"
 
 #include <cstring>
 
@@ -48,6 +50,76 @@ __global__ __launch_bounds__(kThreads) void repack_generic_kernel(RepackArgs a) 
             out |= ((static_cast<uint32_t>(in[base + k * a.strides[last]]) >> (sub * a.bits)) & mask) << (k * a.bits);
     }
     static_cast<W*>(a.output)[pos] = static_cast<W>(out);
+}
+
+// ---- packed along the last dimension, which is contiguous: a copy of strided rows ----
+// One lane per unit of the output (16 bytes where rows, strides and pointers allow, else one stored
+// element), four units in flight per lane.  The unit number, taken apart dimension by dimension
+// (innermost first: the row in units, then the other dimensions; multiply-and-shift divisions), gives
+// the unit's place in the input.
+struct CopyLevels {
+    uint32_t levels;
+    uint32_t count[CQ_MAX_RANK], magic[CQ_MAX_RANK], shift[CQ_MAX_RANK];
+    uint64_t in[CQ_MAX_RANK];  // input stride of the level, in units
+};
+template <class V>
+__global__ __launch_bounds__(kThreads) void repack_rows_kernel(const V* __restrict__ in, V* __restrict__ out, CopyLevels r,
+                                                               uint32_t total) {
+    constexpr int kUnroll = 4;
+    const uint32_t first = blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+    V v[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+        uint32_t n = first + u * kThreads;
+        n = n < total ? n : total - 1;
+        uint64_t off = 0;
+#pragma unroll
+        for (int l = 0; l < CQ_MAX_RANK; l++) {
+            if (l < static_cast<int>(r.levels)) {
+                uint32_t index = n;
+                if (l + 1 < static_cast<int>(r.levels)) {
+                    const uint32_t q = magic_div(n, r.magic[l], r.shift[l]);
+                    index = n - q * r.count[l];
+                    n = q;
+                }
+                off += index * r.in[l];
+            }
+        }
+        v[u] = __builtin_nontemporal_load(in + off);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+        const uint32_t n = first + u * kThreads;
+        if (n < total) __builtin_nontemporal_store(v[u], out + n);
+    }
+}
+
+// Fills `r` for units of `unit` stored elements and returns true when the copy kernel can take the launch.
+bool plan_rows_copy(const RepackArgs& a, uint32_t unit, CopyLevels* r, uint32_t* total) {
+    const uint32_t last = a.rank - 1;
+    if (a.packed_dim != last || a.strides[last] != 1) return false;
+    const uint64_t row = a.shape[last] / a.packing;  // stored elements per row
+    if (row % unit != 0 || a.num_out / unit >= (1ull << 31)) return false;
+    *r = CopyLevels{};
+    const auto push = [&](uint64_t count, uint64_t stride) {
+        const uint32_t k = r->levels;
+        if (k > 0 && stride == r->in[k - 1] * r->count[k - 1] && r->count[k - 1] * count < (1ull << 31)) {
+            r->count[k - 1] *= static_cast<uint32_t>(count);
+        } else {
+            r->count[k] = static_cast<uint32_t>(count);
+            r->in[k] = stride;
+            r->levels = k + 1;
+        }
+    };
+    push(row / unit, 1);
+    for (int d = static_cast<int>(last) - 1; d >= 0; d--) {
+        if (a.shape[d] == 1) continue;
+        if (a.strides[d] % unit != 0) return false;
+        push(a.shape[d], a.strides[d] / unit);
+    }
+    for (uint32_t l = 0; l < r->levels; l++) magic_of(r->count[l], &r->magic[l], &r->shift[l]);
+    *total = static_cast<uint32_t>(a.num_out / unit);
+    return true;
 }
 
 // ---- tiled transposition: packed along a stride-1 dimension that is not the last ----
@@ -222,6 +294,20 @@ hipError_t launch_repack(hipStream_t s, const RepackArgs& bytes_or_words) {
             case 8: hipLaunchKernelGGL((repack_tile_kernel<8, 32, 32>), tile_grid, dim3(256), 0, s, t); break;
             default: hipLaunchKernelGGL((repack_tile_kernel<16, 32, 32>), tile_grid, dim3(256), 0, s, t); break;
         }
+        return hipGetLastError();
+    }
+    // the same packing on both sides: strided rows, copied in 16-byte units where everything is aligned
+    CopyLevels levels;
+    uint32_t total = 0;
+    const uint32_t per16 = 16 / g.elem_bytes;
+    if (aligned16(g.input) && aligned16(g.output) && plan_rows_copy(g, per16, &levels, &total)) {
+        hipLaunchKernelGGL((repack_rows_kernel<u32x4>), dim3((total + kThreads * 4 - 1) / (kThreads * 4)), dim3(kThreads), 0, s,
+                           static_cast<const u32x4*>(g.input), static_cast<u32x4*>(g.output), levels, total);
+        return hipGetLastError();
+    }
+    if (g.elem_bytes == 4 && plan_rows_copy(g, 1, &levels, &total)) {
+        hipLaunchKernelGGL((repack_rows_kernel<uint32_t>), dim3((total + kThreads * 4 - 1) / (kThreads * 4)), dim3(kThreads), 0, s,
+                           static_cast<const uint32_t*>(g.input), static_cast<uint32_t*>(g.output), levels, total);
         return hipGetLastError();
     }
     const dim3 grid(static_cast<uint32_t>((g.num_out + kThreads - 1) / kThreads));

@@ -22,6 +22,11 @@ BIG = [
     ("u8x2_transposed_ragged_tiles", np.uint8, 2, (2080, 1312), 0, (1, 0)),
     ("u8x2_batched_transposed_big", np.uint8, 2, (3, 256, 640), 1, (0, 2, 1)),
     ("u8x2_transposed_not_word_multiple", np.uint8, 2, (516, 388), 0, (1, 0)),
+    # packed along the contiguous last dimension: copies of strided rows
+    ("u32x8_rows_heads_swapped", np.uint32, 8, (2, 6, 40, 128), 3, (0, 2, 1, 3)),
+    ("u32x8_rows_leading_swapped", np.uint32, 8, (5, 3, 2048), 2, (1, 0, 2)),
+    ("u8x2_rows_pitched_big", np.uint8, 2, (300, 4096), 1, (0, 1)),
+    ("u8x2_rows_heads_swapped", np.uint8, 2, (2, 6, 40, 96), 3, (0, 2, 1, 3)),
 ]
 
 
