@@ -301,7 +301,8 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
     const uint32_t stored = s->store == CQ_STORE_U32 ? 4u : 1u;
     const auto rows_contiguous = [&](const cq_tensor* t) { return t->shape[last] == 1 || t->strides[last] == 1; };
-    if (!rows_contiguous(floats) || !rows_contiguous(values) || !aligned(floats->ptr, 16) || !aligned(values->ptr, 8)) return false;
+    if (!rows_contiguous(floats) || !aligned(floats->ptr, 16)) return false;
+    if (values && (!rows_contiguous(values) || !aligned(values->ptr, 8))) return false;  // NULL: scales only
     const uint64_t cols = p.shape[last];
     const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
     if (cols == 0 || cols % chunk_elems) return false;
@@ -315,7 +316,7 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     for (int d = static_cast<int>(last) - 1; d >= 0; d--) {
         const uint64_t n = p.shape[d];
         if (n == 1) continue;
-        const uint64_t in = floats->strides[d] * elem, out = values->strides[d] * stored;
+        const uint64_t in = floats->strides[d] * elem, out = values ? values->strides[d] * stored : in;
         const uint64_t scale_in = scales ? scale_a->strides[d] * scale_a_size : 0;
         const uint64_t scale_out = scales && scale_b ? scale_b->strides[d] * scale_b_size : 0;
         if (in == 0 || out == 0 || in % 16 || out % 8) return false;  // broadcast or misaligned rows
@@ -832,6 +833,16 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
             a.range = p.range;
             return hip_status(cq::launch_scales_flat(stream, input_dtype, a));
         }
+    }
+    // short rows, rows behind several levels of strides: every lane finds its row
+    cq::FlatArgs fl{};
+    if (!p.tensor_level && lane_rows_ok(p, scheme, input_dtype, input, nullptr, scales, elem, nullptr, 0, &fl)) {
+        scale_in_to_out(&fl);
+        fl.input = input->ptr;
+        fl.scale_out = scales->ptr;
+        fl.block = p.block_last;
+        fl.range = p.range;
+        return hip_status(cq::launch_scales_flat(stream, input_dtype, fl));
     }
     return produce_scales(stream, p, scheme, input, input_dtype, scales, input_dtype, workspace, workspace_bytes);
 }
