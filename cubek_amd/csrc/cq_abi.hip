@@ -1037,8 +1037,52 @@ static bool reduce_view(const cq_tensor* input, uint32_t axis, uint64_t* outer, 
     return true;
 }
 
+// A reduction does not care about the order of the dimensions.  Where the input's last dimension is not the
+// contiguous one (a transposed view), the dimensions are put in the order of the input's strides, slowest
+// first, if the output, permuted the same way, is still contiguous (always so for matrices): the kernels
+// for contiguous rows then apply.  `out_strides` NULL: the output is taken to be contiguous.  Returns
+// the tensors to launch with (the caller's, or the permuted copies in `store`) and the axis among them.
+struct PermutedReduce {
+    uint64_t shape[CQ_MAX_RANK], in_strides[CQ_MAX_RANK], out_shape[CQ_MAX_RANK], out_strides[CQ_MAX_RANK];
+    cq_tensor input, output;
+};
+static uint32_t canonical_reduce(const cq_tensor* input, const cq_tensor* output, uint32_t axis, PermutedReduce* store,
+                                 const cq_tensor** in_used, const cq_tensor** out_used) {
+    *in_used = input;
+    *out_used = output;
+    const uint32_t rank = input->rank;
+    if (rank < 2 || input->shape[rank - 1] == 1 || input->strides[rank - 1] == 1) return axis;
+    uint32_t order[CQ_MAX_RANK];
+    for (uint32_t d = 0; d < rank; d++) order[d] = d;
+    for (uint32_t i = 1; i < rank; i++)  // insertion sort, stable: strides descending
+        for (uint32_t j = i; j > 0 && input->strides[order[j - 1]] < input->strides[order[j]]; j--) std::swap(order[j - 1], order[j]);
+    uint64_t contiguous_out[CQ_MAX_RANK], expect = 1;
+    for (int d = static_cast<int>(rank) - 1; d >= 0; d--) {
+        contiguous_out[d] = expect;
+        expect *= static_cast<uint32_t>(d) == axis ? 1 : input->shape[d];
+    }
+    uint32_t new_axis = axis;
+    for (uint32_t i = 0; i < rank; i++) {
+        const uint32_t d = order[i];
+        store->shape[i] = input->shape[d];
+        store->in_strides[i] = input->strides[d];
+        store->out_shape[i] = d == axis ? 1 : input->shape[d];
+        store->out_strides[i] = output ? output->strides[d] : contiguous_out[d];
+        if (d == axis) new_axis = i;
+    }
+    store->input = cq_tensor{input->ptr, store->shape, store->in_strides, rank, input->elem_size};
+    store->output = cq_tensor{output ? output->ptr : nullptr, store->out_shape, store->out_strides, rank, input->elem_size};
+    if (!is_contiguous(&store->output)) return axis;
+    *in_used = &store->input;
+    *out_used = &store->output;
+    return new_axis;
+}
+
 size_t cq_reduce_workspace_bytes(const cq_tensor* input, uint32_t axis, cq_dtype dtype) {
     if (!tensor_ok(input) || axis >= input->rank || !valid_dtype(dtype)) return 0;
+    PermutedReduce store;
+    const cq_tensor* out_unused;
+    axis = canonical_reduce(input, nullptr, axis, &store, &input, &out_unused);
     uint64_t outer, len, inner;
     reduce_view(input, axis, &outer, &len, &inner);
     if (outer == 0 || inner == 0) return 0;
@@ -1051,10 +1095,14 @@ cq_status cq_reduce_max_abs(cq_stream_t stream, const cq_tensor* input, const cq
     if (axis >= input->rank) return CQ_ERR_INVALID_AXIS;
     if (input->elem_size != dtype_size(dtype) || output->elem_size != dtype_size(dtype)) return CQ_ERR_SHAPE_MISMATCH;
     if (output->rank != input->rank) return CQ_ERR_SHAPE_MISMATCH;
-    cq::ReduceArgs a{};
     for (uint32_t d = 0; d < input->rank; d++) {
         if (output->shape[d] != (d == axis ? 1 : input->shape[d])) return CQ_ERR_SHAPE_MISMATCH;
         if (input->shape[d] > 0xffffffffull) return CQ_ERR_TOO_LARGE;
+    }
+    PermutedReduce store;
+    axis = canonical_reduce(input, output, axis, &store, &input, &output);
+    cq::ReduceArgs a{};
+    for (uint32_t d = 0; d < input->rank; d++) {
         a.shape[d] = input->shape[d];
         a.in_strides[d] = input->strides[d];
         a.out_strides[d] = output->strides[d];
