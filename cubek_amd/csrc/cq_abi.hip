@@ -301,8 +301,10 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
     const uint32_t stored = s->store == CQ_STORE_U32 ? 4u : 1u;
     const auto rows_contiguous = [&](const cq_tensor* t) { return t->shape[last] == 1 || t->strides[last] == 1; };
-    if (!rows_contiguous(floats) || !aligned(floats->ptr, 16)) return false;
-    if (values && (!rows_contiguous(values) || !aligned(values->ptr, 8))) return false;  // NULL: scales only
+    // 16-byte loads and 8-byte stores at any multiple of 4 bytes: the hardware takes them, at some cost in
+    // cache lines crossed, and whole-chunk alignment is what the other flat launches are for
+    if (!rows_contiguous(floats) || !aligned(floats->ptr, 4)) return false;
+    if (values && (!rows_contiguous(values) || !aligned(values->ptr, 4))) return false;  // NULL: scales only
     const uint64_t cols = p.shape[last];
     const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
     if (cols == 0 || cols % chunk_elems) return false;
@@ -319,7 +321,7 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
         const uint64_t in = floats->strides[d] * elem, out = values ? values->strides[d] * stored : in;
         const uint64_t scale_in = scales ? scale_a->strides[d] * scale_a_size : 0;
         const uint64_t scale_out = scales && scale_b ? scale_b->strides[d] * scale_b_size : 0;
-        if (in == 0 || out == 0 || in % 16 || out % 8) return false;  // broadcast or misaligned rows
+        if (in == 0 || out == 0 || in % 4 || out % 4) return false;  // broadcast or misaligned rows
         const uint32_t k = l.levels;
         if (k > 0 && in == l.in[k - 1] * l.count[k - 1] && out == l.out[k - 1] * l.count[k - 1] &&
             scale_in == l.scale_in[k - 1] * l.count[k - 1] && scale_out == l.scale_out[k - 1] * l.count[k - 1] &&

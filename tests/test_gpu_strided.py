@@ -56,6 +56,8 @@ def layouts(shape, per):
     out = [("contiguous", contiguous(shape), contiguous(pshape)),
            ("pitched", contiguous(shape, 5), contiguous(pshape, 3)),
            ("pitched_aligned", contiguous(shape, 64), contiguous(pshape, 8)),
+           # rows that start on multiples of 4 bytes only: 16-byte loads and 8-byte stores off their alignment
+           ("pitched_words", contiguous(shape, 6), contiguous(pshape, 1)),
            ("transposed_floats", permuted(shape), contiguous(pshape)),
            ("transposed_stored", contiguous(shape), permuted(pshape)),
            ("both", permuted(shape), permuted(pshape))]
@@ -137,7 +139,7 @@ def test_pitched_rows_of_a_few_steps(gpu, oracle, elem, name, scheme):
     a row's last step may be partial, and the launch ends on a workgroup with fewer steps than the others."""
     check_layouts(gpu, oracle, elem, name, scheme,
                   ((4, 4096), (6, 5120), (2, 2, 7168), (4, 2560), (6, 2048), (6, 1024), (10, 1280), (3, 2, 2048), (2, 3, 2, 2560)),
-                  ("pitched", "pitched_aligned", "every_other_row", "leading_swapped", "leading_swapped_floats"))
+                  ("pitched", "pitched_aligned", "pitched_words", "every_other_row", "leading_swapped", "leading_swapped_floats"))
 
 
 @pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
@@ -146,7 +148,7 @@ def test_short_rows_behind_permuted_dimensions(gpu, oracle, elem, name, scheme):
     """[batch, heads, positions, head dimension] views of [batch, positions, heads, head dimension] buffers,
     and short pitched rows: every lane of the streaming kernels finds its own row."""
     check_layouts(gpu, oracle, elem, name, scheme, ((2, 3, 6, 128), (2, 5, 8, 64), (2, 4, 8, 128), (1, 12, 24, 64), (1, 2, 300, 256), (3, 2, 2, 1024)),
-                  ("middle_swapped", "middle_swapped_floats", "pitched_aligned", "every_other_row", "leading_swapped"))
+                  ("middle_swapped", "middle_swapped_floats", "pitched_aligned", "pitched_words", "every_other_row", "leading_swapped"))
 
 
 def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
