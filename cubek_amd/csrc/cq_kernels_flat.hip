@@ -1,5 +1,5 @@
 // Launchers of the flat (contiguous) kernels: block scales, the per-tensor abs-max, and the dispatch of
-// quantize to the per-type launchers of cq_kernels_flat_quantize.hip.  Dequantize is in
+// quantize and dequantize to the per-type launchers of cq_kernels_flat_quantize.hip and
 // cq_kernels_flat_dequantize.hip.
 #include "cq_kernels_flat_launch.hpp"
 
@@ -35,6 +35,16 @@ hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource 
         case CQ_F32: return given ? CQ_QUANTIZE_FLAT_TU(F32, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(F32, 0)(s, bits, src, a);
         case CQ_BF16: return given ? CQ_QUANTIZE_FLAT_TU(BF16, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(BF16, 0)(s, bits, src, a);
         case CQ_F16: return given ? CQ_QUANTIZE_FLAT_TU(F16, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(F16, 0)(s, bits, src, a);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_dequantize_flat(hipStream_t s, int dtype, int bits, const FlatArgs& a) {
+    if (a.num_chunks == 0) return hipSuccess;
+    switch (dtype) {
+        case CQ_F32: return CQ_DEQUANTIZE_FLAT_TU(F32)(s, bits, a);
+        case CQ_BF16: return CQ_DEQUANTIZE_FLAT_TU(BF16)(s, bits, a);
+        case CQ_F16: return CQ_DEQUANTIZE_FLAT_TU(F16)(s, bits, a);
         default: return hipErrorInvalidValue;
     }
 }

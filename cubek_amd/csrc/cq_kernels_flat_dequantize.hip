@@ -1,5 +1,11 @@
-// Launchers of the flat (contiguous) dequantize kernels.
+// Launchers of the flat dequantize kernels of one float type.  The Makefile compiles this file three
+// times (-DCQ_TU_FLOAT=F32|BF16|F16), each into an object of its own: the build runs in parallel, and a
+// process loads the kernels of the float types it uses only.
 #include "cq_kernels_flat_launch.hpp"
+
+#ifndef CQ_TU_FLOAT
+#define CQ_TU_FLOAT F32
+#endif
 
 namespace cq {
 namespace {
@@ -52,10 +58,9 @@ hipError_t dequantize_launch(hipStream_t s, const FlatArgs& a) {
 
 }  // namespace
 
-hipError_t launch_dequantize_flat(hipStream_t s, int dtype, int bits, const FlatArgs& a) {
-    if (a.num_chunks == 0) return hipSuccess;
-    int g = group_of(dtype, a.block);
-    CQ_SWITCH_DTYPE(dtype, CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (dequantize_launch<kF, kB, kG>(s, a)))))
+hipError_t CQ_DEQUANTIZE_FLAT_TU(CQ_TU_FLOAT)(hipStream_t s, int bits, const FlatArgs& a) {
+    int g = group_of(CQ_TU_FLOAT::kDtype, a.block);
+    CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (dequantize_launch<CQ_TU_FLOAT, kB, kG>(s, a))))
 }
 
 }  // namespace cq

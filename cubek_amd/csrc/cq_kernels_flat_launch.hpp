@@ -18,6 +18,12 @@ hipError_t CQ_QUANTIZE_FLAT_TU(BF16, 0)(hipStream_t s, int bits, ScaleSource src
 hipError_t CQ_QUANTIZE_FLAT_TU(BF16, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
 hipError_t CQ_QUANTIZE_FLAT_TU(F16, 0)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
 hipError_t CQ_QUANTIZE_FLAT_TU(F16, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
+// the dequantize launchers, one per float type, each compiled from cq_kernels_flat_dequantize.hip
+#define CQ_DEQUANTIZE_FLAT_TU_(f) launch_dequantize_flat_##f
+#define CQ_DEQUANTIZE_FLAT_TU(f) CQ_DEQUANTIZE_FLAT_TU_(f)
+hipError_t CQ_DEQUANTIZE_FLAT_TU(F32)(hipStream_t s, int bits, const FlatArgs& a);
+hipError_t CQ_DEQUANTIZE_FLAT_TU(BF16)(hipStream_t s, int bits, const FlatArgs& a);
+hipError_t CQ_DEQUANTIZE_FLAT_TU(F16)(hipStream_t s, int bits, const FlatArgs& a);
 
 namespace {
 
