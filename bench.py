@@ -244,6 +244,20 @@ def adjacent_kernels(torch):
         out.append({"kernel": f"reduce_max_abs axis {axis} of bf16 [{rows}, {cols}]", "algorithmic_bytes": b,
                     "workspace_bytes": nbytes, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+    # the same buffers seen transposed ([cols, rows] with strides (1, cols)): reduced in the order of their strides
+    for axis in (0, 1):
+        o = torch.zeros((1, rows) if axis == 0 else (cols, 1), device="cuda", dtype=torch.bfloat16)
+        hs = [TensorHandleRef(h(x).handle, (cols, rows), (1, cols), 2) for x in xs]
+        nbytes = cq_reduce.workspace_bytes(hs[0], axis, ElemType.BF16)
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+        ho = h(o)
+        fn = lambda i: cq_reduce.max_abs(client, hs[i % sets], ho, axis, ElemType.BF16, ws.data_ptr() if nbytes else 0,
+                                         nbytes)
+        ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
+        b = rows * cols * 2
+        out.append({"kernel": f"reduce_max_abs axis {axis} of the transposed bf16 view [{cols}, {rows}]", "algorithmic_bytes": b,
+                    "workspace_bytes": nbytes, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                    "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
     # weight-style 128 x 128 blocks, fp8 e4m3 bytes: the fused block kernel (one launch, one read)
     from cubek_amd import QuantLevel, QuantScheme, QuantStore, QuantValue
     from cubek_amd import dequantize as cq_dequantize
@@ -306,6 +320,19 @@ def adjacent_kernels(torch):
             out.append({"kernel": f"{label}, e2m1 blocks of 32, pitched bf16 rows: [{pr}, {pc}] view of a [{pr}, {pc + pad}] buffer",
                         "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                         "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+        if pc == cols:  # abs-max along both axes of the same pitched rows
+            for axis in (1, 0):
+                o = torch.zeros((pr, 1) if axis == 1 else (1, pc), device="cuda", dtype=torch.bfloat16)
+                nbytes = cq_reduce.workspace_bytes(hxp[0], axis, ElemType.BF16)
+                ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+                ho = h(o)
+                fn = lambda i: cq_reduce.max_abs(client, hxp[i % sets], ho, axis, ElemType.BF16,
+                                                 ws.data_ptr() if nbytes else 0, nbytes)
+                ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
+                out.append({"kernel": f"reduce_max_abs axis {axis} of pitched bf16 rows: [{pr}, {pc}] view of a [{pr}, {pc + pad}] buffer",
+                            "algorithmic_bytes": pr * pc * 2, "workspace_bytes": nbytes, "ms": round(ms, 4),
+                            "GBps": round(pr * pc * 2 / (ms * 1e-3) / 1e9, 1),
+                            "frac_hbm_peak": round(pr * pc * 2 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
         del xp, yp, words, bscales, hxp, hyp, hw, hb
         torch.cuda.empty_cache()
     # the headline scheme on an attention layout: the [batch, heads, positions, head dimension] view of a
@@ -342,6 +369,16 @@ def adjacent_kernels(torch):
     ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
     b = 2 * rows * cols // packing * 4
     out.append({"kernel": f"into_contiguous_packed of transposed 4-bit [{cols}, {rows}] (u32 x 8)",
+                "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+    # the same codes with pitched rows ([rows, cols/8 - 8] words out of every row of cols/8): a copy of strided rows
+    wcols = cols // packing - 8
+    hs = [TensorHandleRef(h(t).handle, (rows, wcols), (cols // packing, 1), 4) for t in srcs]
+    hd = TensorHandleRef(h(dst).handle, (rows, wcols), (wcols, 1), 4)
+    fn = lambda i: cq_contiguous.into_contiguous_packed_ref(client, hs[i % len(hs)], hd, (rows, wcols * packing), packing)
+    ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
+    b = 2 * rows * wcols * 4
+    out.append({"kernel": f"into_contiguous_packed of 4-bit rows with a pitch: [{rows}, {wcols}] words out of [{rows}, {cols // packing}]",
                 "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                 "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
     return out
