@@ -295,7 +295,7 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
 // innermost first, neighbours merged where all four tensors step uniformly through them.
 bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
                   const cq_tensor* scale_a, uint32_t scale_a_size, const cq_tensor* scale_b, uint32_t scale_b_size,
-                  cq::FlatArgs* a) {
+                  bool given_scales, cq::FlatArgs* a) {
     if (p.rank < 2) return false;
     const uint32_t last = p.rank - 1;
     const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
@@ -309,9 +309,13 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
     if (cols == 0 || cols % chunk_elems) return false;
     const bool scales = !p.tensor_level;
-    if (scales && (!p.last_dim_blocks || !cq::flat_block_supported(dtype, p.block_last) || !rows_contiguous(scale_a) ||
-                   (scale_b && !rows_contiguous(scale_b))))
+    // blocks along the last dimension, or (where the scales are given) over the last two: the rows of a block
+    // read the same row of scales
+    const uint32_t br = scales ? p.layout.block[last - 1] : 1;
+    if (scales && (!(p.last_dim_blocks || (given_scales && scales_rows_ok(p))) || !cq::flat_block_supported(dtype, p.block_last) ||
+                   !rows_contiguous(scale_a) || (scale_b && !rows_contiguous(scale_b))))
         return false;
+    a->scale_rows = br;
     cq::LaneLevels& l = a->lanes;
     l = cq::LaneLevels{};
     uint64_t rows = 1;
@@ -323,8 +327,10 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
         const uint64_t scale_out = scales && scale_b ? scale_b->strides[d] * scale_b_size : 0;
         if (in == 0 || out == 0 || in % 4 || out % 4) return false;  // broadcast or misaligned rows
         const uint32_t k = l.levels;
+        // entries of the level inside this one as the scales count them: blocks of rows at the innermost level
+        const uint64_t scale_count = k == 1 && br > 1 ? l.count[0] / br : (k > 0 ? l.count[k - 1] : 0);
         if (k > 0 && in == l.in[k - 1] * l.count[k - 1] && out == l.out[k - 1] * l.count[k - 1] &&
-            scale_in == l.scale_in[k - 1] * l.count[k - 1] && scale_out == l.scale_out[k - 1] * l.count[k - 1] &&
+            scale_in == l.scale_in[k - 1] * scale_count && scale_out == l.scale_out[k - 1] * scale_count &&
             l.count[k - 1] * n < (1ull << 31)) {
             l.count[k - 1] *= static_cast<uint32_t>(n);
         } else {
@@ -605,7 +611,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     if (flat_words == 0 && (flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
                                          dtype_size(pd), true, &fr) ||
                             lane_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
-                                         dtype_size(pd), &fr))) {
+                                         dtype_size(pd), true, &fr))) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_in = scale->ptr;
@@ -680,7 +686,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
     }
     cq::FlatArgs fr{};
     if (flat_words == 0 && (flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr) ||
-                            lane_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, &fr))) {
+                            lane_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr))) {
         fr.input = values->ptr;
         fr.output = output->ptr;
         fr.scale_in = params->ptr;
@@ -838,7 +844,7 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
     }
     // short rows, rows behind several levels of strides: every lane finds its row
     cq::FlatArgs fl{};
-    if (!p.tensor_level && lane_rows_ok(p, scheme, input_dtype, input, nullptr, scales, elem, nullptr, 0, &fl)) {
+    if (!p.tensor_level && lane_rows_ok(p, scheme, input_dtype, input, nullptr, scales, elem, nullptr, 0, false, &fl)) {
         scale_in_to_out(&fl);
         fl.input = input->ptr;
         fl.scale_out = scales->ptr;
@@ -882,7 +888,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
     // pitched rows with 1-D blocks: the same fused kernel over the rows' steps
     cq::FlatArgs fr{};
     if (!p.tensor_level && (flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) ||
-                            lane_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, &fr))) {
+                            lane_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr))) {
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_out = out_scale->ptr;
@@ -942,7 +948,7 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
         if (st != CQ_OK) return st;
         flat_words = flat_chunks * per_chunk / p.nq;
     } else if (p.tensor_level && (flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) ||
-                                  lane_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, &fr))) {
+                                  lane_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr))) {
         // per tensor on pitched rows: the same two passes, the second one over the rows' steps
         uint32_t num_partials = 0;
         st = absmax_partials(stream, p, scheme, input, input_dtype, workspace, workspace_bytes, &num_partials);

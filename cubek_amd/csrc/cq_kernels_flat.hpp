@@ -199,12 +199,16 @@ struct RowSteps {
 // of the launch are numbered through all rows, a step is kThreads consecutive ones, so the lanes of a
 // step lie in several rows.  Each lane finds its row (chunk / row_chunks) and from it, dimension by
 // dimension (innermost first, `count` entries each, multiply-and-shift divisions), the byte offsets of
-// that row in the four tensors.  Blocks lie along the row (or one scale per tensor).
+// that row in the four tensors.  Blocks lie along the row, or (given scales) over rows of the innermost
+// level as well, or there is one scale per tensor.
 constexpr int kMaxLaneLevels = 7;
 struct LaneRows {
     uint32_t row_chunks, row_magic, row_shift;
     uint32_t total_chunks;  // < 2^31
     uint32_t levels;        // leading dimensions, 1 .. kMaxLaneLevels
+    // blocks of `scale_rows` entries of the innermost level (by a lane group of columns) share their scale
+    // (given scales only); the scale strides of that level are per block of rows
+    uint32_t scale_rows, scale_magic, scale_shift;
     uint32_t count[kMaxLaneLevels], magic[kMaxLaneLevels], shift[kMaxLaneLevels];
     uint64_t in[kMaxLaneLevels], out[kMaxLaneLevels], scale_in[kMaxLaneLevels], scale_out[kMaxLaneLevels];
 };
@@ -227,7 +231,7 @@ struct LaneSteps {
     const char* scale_in_[kUnroll];
     char* scale_out_[kUnroll];
     uint32_t col_[kUnroll];  // the lane's chunk within its row
-    bool live_[kUnroll], first_[kUnroll];
+    bool live_[kUnroll], first_[kUnroll], block_row_[kUnroll];
     __device__ __forceinline__ LaneSteps(const LanesGeo& g, uint32_t tile) {
         const LaneRows& r = g.rows;
 #pragma unroll
@@ -238,6 +242,7 @@ struct LaneSteps {
             uint32_t row = magic_div(c, r.row_magic, r.row_shift);
             col_[u] = c - row * r.row_chunks;
             first_[u] = row == 0;
+            block_row_[u] = true;
             uint64_t in = 0, out = 0, scale_in = 0, scale_out = 0;
 #pragma unroll
             for (int l = 0; l < kMaxLaneLevels; l++) {
@@ -250,8 +255,13 @@ struct LaneSteps {
                     }
                     in += index * r.in[l];
                     out += index * r.out[l];
-                    scale_in += index * r.scale_in[l];
-                    scale_out += index * r.scale_out[l];
+                    uint32_t scale_index = index;
+                    if (l == 0 && r.scale_rows > 1) {
+                        scale_index = magic_div(index, r.scale_magic, r.scale_shift);
+                        block_row_[u] = index == scale_index * r.scale_rows;
+                    }
+                    scale_in += scale_index * r.scale_in[l];
+                    scale_out += scale_index * r.scale_out[l];
                 }
             }
             in_[u] = static_cast<const char*>(g.in) + in;
@@ -263,7 +273,7 @@ struct LaneSteps {
     __device__ __forceinline__ Index chunk(int u) const { return col_[u]; }
     __device__ __forceinline__ Index load_chunk(int u) const { return col_[u]; }
     __device__ __forceinline__ bool live(int u) const { return live_[u]; }
-    __device__ __forceinline__ bool first_row(int) const { return true; }
+    __device__ __forceinline__ bool first_row(int u) const { return block_row_[u]; }
     __device__ __forceinline__ bool tensor_start(int u) const { return first_[u] && col_[u] == 0; }
     __device__ __forceinline__ const void* in(int u) const { return in_[u]; }
     __device__ __forceinline__ void* out(int u) const { return out_[u]; }

@@ -89,6 +89,8 @@ LaneRows lane_rows(const FlatArgs& a) {
     magic_of(r.row_chunks, &r.row_magic, &r.row_shift);
     r.total_chunks = static_cast<uint32_t>(a.rows * a.num_chunks);
     r.levels = a.lanes.levels;
+    r.scale_rows = a.scale_rows > 1 ? a.scale_rows : 1u;
+    magic_of(r.scale_rows, &r.scale_magic, &r.scale_shift);
     for (uint32_t l = 0; l < r.levels; l++) {
         r.count[l] = a.lanes.count[l];
         magic_of(r.count[l], &r.magic[l], &r.shift[l]);

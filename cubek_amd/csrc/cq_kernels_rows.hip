@@ -578,7 +578,9 @@ hipError_t quantize_blocks_rows(hipStream_t s, const RowArgs& a, const BlocksGeo
     if (g.rows_per_thread <= 1) return quantize_blocks_variant<F, kBits, kWide, kEnc, 1, 4>(s, a, g, qp);
     if (g.rows_per_thread <= 2) return quantize_blocks_variant<F, kBits, kWide, kEnc, 2, 4>(s, a, g, qp);
     if (g.rows_per_thread <= 4) return quantize_blocks_variant<F, kBits, kWide, kEnc, 4, 2>(s, a, g, qp);
-    if (g.rows_per_thread <= 8) return quantize_blocks_variant<F, kBits, kWide, kEnc, 8, 1>(s, a, g, qp);
+    // f32: the eight-row variant compiles to 120 registers (half the waves per SIMD: 29 % of HBM peak), the
+    // sixteen-row one to 52, and rows beyond a block's are neither loaded nor stored
+    if (g.rows_per_thread <= 8 && F::kBytes != 4) return quantize_blocks_variant<F, kBits, kWide, kEnc, 8, 1>(s, a, g, qp);
     return quantize_blocks_variant<F, kBits, kWide, kEnc, 16, 1>(s, a, g, qp);
 }
 
