@@ -902,6 +902,26 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
 
     // blocks over the last two dimensions (or 1-D blocks on layouts the flat kernel refuses): one
     // launch that owns whole blocks
+    // Blocks of 8 - 64 rows on rows of at most 1 KiB leave the fused block kernel too few lanes along the row
+    // (18 - 35 % of HBM peak).  Two launches take half the time there: the blocks' scales as FS(F(scale)) into
+    // out_scale, then the flat body, lane by lane, reading them back (the divisor F(FS(scale)) is the same either way).
+    if (!p.tensor_level && p.rank >= 2 && scales_rows_ok(p) && p.layout.block[p.rank - 2] >= 8 && p.layout.block[p.rank - 2] <= 64 &&
+        p.shape[p.rank - 1] * dtype_size(input_dtype) <= 1024) {
+        cq::FlatArgs f2{};
+        if (lane_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, true, &f2)) {
+            st = produce_scales(stream, p, scheme, input, input_dtype, out_scale, pd, workspace, workspace_bytes);
+            if (st != CQ_OK) return st;
+            f2.input = input->ptr;
+            f2.output = output->ptr;
+            f2.scale_in = out_scale->ptr;
+            f2.block = p.block_last;
+            f2.param_dtype = pd;
+            f2.encoding = flat_encoding(scheme);
+            f2.range = p.range;
+            return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Stored, f2));
+        }
+    }
+
     cq::RowArgs rb;
     if (!p.tensor_level && scales_rows_ok(p) && rows_args(p, scheme, input_dtype, input, output, &rb) &&
         cq::blocks_dynamic_supported(input_dtype, static_cast<int>(p.bits), rb)) {

@@ -55,7 +55,7 @@ struct FlatArgs {
     Range range;
 };
 
-enum class ScaleSource { Given, Dynamic, Partials };
+enum class ScaleSource { Given, Dynamic, Partials, Stored };  // Stored: lane-wise launches only (FlatArgs::lanes)
 
 // every launcher returns hipGetLastError() of its launch
 hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource src, const FlatArgs& a);

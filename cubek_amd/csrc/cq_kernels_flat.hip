@@ -30,7 +30,7 @@ bool flat_block_supported(int dtype, uint32_t block) { return group_of(dtype, bl
 
 hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource src, const FlatArgs& a) {
     if (a.num_chunks == 0) return hipSuccess;
-    const bool given = src == ScaleSource::Given;
+    const bool given = src == ScaleSource::Given || src == ScaleSource::Stored;  // the objects that read scales
     switch (dtype) {
         case CQ_F32: return given ? CQ_QUANTIZE_FLAT_TU(F32, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(F32, 0)(s, bits, src, a);
         case CQ_BF16: return given ? CQ_QUANTIZE_FLAT_TU(BF16, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(BF16, 0)(s, bits, src, a);

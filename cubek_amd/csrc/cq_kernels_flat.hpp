@@ -31,6 +31,9 @@ enum ScaleSrc : int {
     kScaleGivenF = 1,      // `scale_in`, typed like the input (the reference's `scale` argument)
     kScalePartials = 2,    // per tensor: `scale_in` holds the f32 abs-max partials of pass 1; this
                            // kernel (pass 2) finishes the reduction, derives the scale and quantizes
+    kScaleStored = 3,      // `scale_in` holds the stored scales FS(F(scale)) of every block, written by an
+                           // earlier launch and typed like the parameters: the divisor is F(stored), and
+                           // nothing is written back (second pass of a two-launch dynamic quantize)
 };
 
 // ---- where the steps of a workgroup's tile lie -------------------------------------------------
@@ -294,6 +297,7 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
                                                    uint32_t num_partials) {
     constexpr bool kDynamic = kScaleSrc == kScaleDynamic;
     static_assert(kScaleSrc != kScalePartials || kGroup == 0, "partials feed the per-tensor scale only");
+    static_assert(kScaleSrc != kScaleStored || kGroup != 0, "stored scales are read back per block only");
     constexpr int kDiv = kGroup == 0 ? 1 : kGroup;
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;  // 64, 32, 16 or 8
@@ -316,7 +320,10 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
     for (int u = 0; u < kUnroll; u++) {
         const auto c = at.load_chunk(u);
         raw[u] = stream_load(static_cast<const u32x4*>(at.in(u)) + c);
-        if constexpr (!kDynamic && kGroup != 0 && kScaleSrc != kScalePartials) s_given[u] = F::load(at.scale_in(u), c / kDiv);
+        if constexpr (kScaleSrc == kScaleStored)
+            s_given[u] = F::round(load_dtype(param_dtype, at.scale_in(u), c / kDiv));
+        else if constexpr (!kDynamic && kGroup != 0 && kScaleSrc != kScalePartials)
+            s_given[u] = F::load(at.scale_in(u), c / kDiv);
     }
     if constexpr (kScaleSrc == kScalePartials) {
         // second pass of the grid reduction: every workgroup reduces the (<= a few
@@ -334,7 +341,7 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         const float s = F::round(scale_from_absmax(amax, qp.width));
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) s_given[u] = s;
-    } else if constexpr (!kDynamic && kGroup == 0) {
+    } else if constexpr (!kDynamic && kGroup == 0 && kScaleSrc != kScaleStored) {
         const float s = F::load(geo.scale_in, 0);  // one scale for the whole tensor
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) s_given[u] = s;
@@ -367,10 +374,12 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         const float s_fs = round_to_dtype(param_dtype, s_f);
         const auto si = kGroup == 0 ? 0 : c / kDiv;
         const bool block_start = kGroup == 0 ? at.tensor_start(u) : (at.first_row(u) && (c % kDiv) == 0);
-        if (scale_out != nullptr && live && block_start) store_dtype(param_dtype, scale_out, si, s_fs);
+        if constexpr (kScaleSrc != kScaleStored)
+            if (scale_out != nullptr && live && block_start) store_dtype(param_dtype, scale_out, si, s_fs);
         // divisor F(FS(scale)); s_f is an F value, so f32 params leave it unchanged
         float d = s_fs;
         if constexpr (!kParamF32) d = F::round(s_fs);
+        if constexpr (kScaleSrc == kScaleStored) d = s_f;  // F(stored) as loaded
         if constexpr (!(kDynamic && kParamF32 && F::kDtype != CQ_F16)) tame = divisor_is_tame(d);
 
         float qn[kN];  // negated codes

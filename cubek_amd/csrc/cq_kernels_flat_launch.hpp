@@ -159,8 +159,16 @@ template <class F, int kBits, int kGroup, int kSrc, bool kWide, int kEnc>
 hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
     // scale sources that exist: per-block launches compute the scale or read the
     // input-typed tensor; per-tensor launches read it or finish the grid reduction
-    if constexpr ((kGroup == 0 && kSrc == kScaleDynamic) || (kGroup != 0 && kSrc == kScalePartials)) {
+    if constexpr ((kGroup == 0 && (kSrc == kScaleDynamic || kSrc == kScaleStored)) || (kGroup != 0 && kSrc == kScalePartials)) {
         return hipErrorInvalidValue;
+    } else if constexpr (kSrc == kScaleStored) {
+        // read back by the second pass of a two-launch dynamic quantize, which runs lane by lane only
+        if (a.lanes.levels == 0) return hipErrorInvalidValue;
+        hipLaunchKernelGGL((quantize_flat_lanes_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
+                           dim3(lanes_grid(a, kUnrollQ)), dim3(kThreads), 0, s, static_cast<const u32x4*>(a.input),
+                           static_cast<uint32_t*>(a.output), a.scale_in, a.scale_out, a.param_dtype, quant_params(a.range),
+                           a.num_partials, lane_rows(a));
+        return hipGetLastError();
     } else {
         auto in = static_cast<const u32x4*>(a.input);
         auto out = static_cast<uint32_t*>(a.output);
@@ -201,6 +209,7 @@ hipError_t quantize_launch_enc(hipStream_t s, ScaleSource src, const FlatArgs& a
     if constexpr (kGiven) {
         if (src == ScaleSource::Given && a.scale_in_dtype == F::kDtype)  // given scales are typed like the input
             return quantize_launch_src<F, kBits, kGroup, kScaleGivenF, kWide, kEnc>(s, a);
+        if (src == ScaleSource::Stored) return quantize_launch_src<F, kBits, kGroup, kScaleStored, kWide, kEnc>(s, a);
     } else {
         if (src == ScaleSource::Dynamic) return quantize_launch_src<F, kBits, kGroup, kScaleDynamic, kWide, kEnc>(s, a);
         if (src == ScaleSource::Partials) return quantize_launch_src<F, kBits, kGroup, kScalePartials, kWide, kEnc>(s, a);

@@ -151,6 +151,25 @@ def test_short_rows_behind_permuted_dimensions(gpu, oracle, elem, name, scheme):
                   ("middle_swapped", "middle_swapped_floats", "pitched_aligned", "pitched_words", "every_other_row", "leading_swapped"))
 
 
+BLOCKS_OF_ROWS = [
+    ("q8s_block_16x32", QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([16, 32]))),
+    ("q4s_block_8x64", QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([8, 64]))),
+    ("e4m3_native_block_32x32", QuantScheme.default().with_value(QuantValue.E4M3).with_store(QuantStore.Native)
+     .with_level(QuantLevel.block([32, 32]))),
+    ("q2s_block_64x64", QuantScheme.default().with_value(QuantValue.Q2S).with_level(QuantLevel.block([64, 64]))),
+]
+
+
+@pytest.mark.parametrize("name,scheme", BLOCKS_OF_ROWS, ids=[n for n, _ in BLOCKS_OF_ROWS])
+@pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
+def test_blocks_of_rows_on_short_rows(gpu, oracle, elem, name, scheme):
+    """Blocks of 8 - 64 rows on rows of at most 1 KiB: the fused abs-max + quantize runs as two launches (the
+    scales, then the streaming kernel lane by lane reading them back); given scales and dequantize take the
+    same lane-wise kernels."""
+    check_layouts(gpu, oracle, elem, name, scheme, ((2, 4, 64, 128), (192, 256), (3, 128, 64), (2, 64, 192)),
+                  ("contiguous", "pitched_aligned", "pitched_words", "every_other_row", "middle_swapped", "leading_swapped"))
+
+
 def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
     import torch
 
