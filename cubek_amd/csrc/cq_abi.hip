@@ -242,7 +242,8 @@ bool flat_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     if (!row_levels(floats, &lf) || !row_levels(values, &lv) || lf.rows != lv.rows) return false;
     const uint64_t rows_f = lf.rows;
     const uint64_t cols = p.shape[last];
-    const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+    // whole chunks and whole 32-bit words of codes (lanes that share a word store it together)
+    const uint64_t chunk_elems = per_chunk > 32u / p.bits ? per_chunk : 32u / p.bits;
     if (cols == 0 || cols % chunk_elems) return false;
     const uint64_t row_chunks = cols / per_chunk;
     // steps of 256 chunks, a row's last one with idle lanes where 256 does not divide the row.  Measured on
@@ -306,7 +307,8 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     if (!rows_contiguous(floats) || !aligned(floats->ptr, 4)) return false;
     if (values && (!rows_contiguous(values) || !aligned(values->ptr, 4))) return false;  // NULL: scales only
     const uint64_t cols = p.shape[last];
-    const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+    // whole chunks and whole 32-bit words of codes (lanes that share a word store it together)
+    const uint64_t chunk_elems = per_chunk > 32u / p.bits ? per_chunk : 32u / p.bits;
     if (cols == 0 || cols % chunk_elems) return false;
     const bool scales = !p.tensor_level;
     // blocks along the last dimension, or (where the scales are given) over the last two: the rows of a block
@@ -597,7 +599,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         a.scale_in_dtype = input_dtype;
         a.scale_out = out_scale->ptr;
         // whole chunks that also end on a stored-element boundary
-        uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+        uint64_t chunk_elems = per_chunk > 32u / p.bits ? per_chunk : 32u / p.bits;  // whole chunks and whole words of codes
         a.num_chunks = (p.n / chunk_elems) * chunk_elems / per_chunk;
         a.block = p.tensor_level ? 0 : p.block_last;
         a.param_dtype = pd;
@@ -674,7 +676,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         a.input = values->ptr;
         a.output = output->ptr;
         a.scale_in = params->ptr;
-        uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+        uint64_t chunk_elems = per_chunk > 32u / p.bits ? per_chunk : 32u / p.bits;  // whole chunks and whole words of codes
         a.num_chunks = (p.n / chunk_elems) * chunk_elems / per_chunk;
         a.block = p.tensor_level ? 0 : p.block_last;
         a.param_dtype = pd;
@@ -871,8 +873,10 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
     const bool native = scheme->store == CQ_STORE_NATIVE;
     const bool flat = flat_ok(p, input_dtype, input, output, out_scale, nullptr);
 
-    // fused single pass: abs-max, scale, quantize, pack in registers
-    if (flat && !p.tensor_level) {
+    // fused single pass: abs-max, scale, quantize, pack in registers (whole 32-bit words of codes: lanes that
+    // share a word store it together)
+    const uint64_t word_elems = per_chunk > 32u / p.bits ? per_chunk : 32u / p.bits;
+    if (flat && !p.tensor_level && p.n % word_elems == 0) {
         cq::FlatArgs a{};
         a.input = input->ptr;
         a.output = output->ptr;
@@ -941,7 +945,8 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
     }
 
     uint64_t flat_words = 0;
-    const uint64_t chunk_elems = per_chunk > p.nq ? per_chunk : p.nq;
+    // whole chunks and whole 32-bit words of codes (lanes that share a word store it together)
+    const uint64_t chunk_elems = per_chunk > 32u / p.bits ? per_chunk : 32u / p.bits;
     const uint64_t flat_chunks = flat ? (p.n / chunk_elems) * chunk_elems / per_chunk : 0;
     if (p.tensor_level && flat_chunks > 0) {
         // per tensor, two-pass grid reduction: pass 1 leaves one abs-max per workgroup in

@@ -170,6 +170,15 @@ def test_blocks_of_rows_on_short_rows(gpu, oracle, elem, name, scheme):
                   ("contiguous", "pitched_aligned", "pitched_words", "every_other_row", "middle_swapped", "leading_swapped"))
 
 
+def test_half_words_of_codes_per_row(gpu, oracle):
+    """f32 rows of 12 and 20 values as e2m1 bytes: a row ends in the middle of a 32-bit word of codes, so the
+    kernels whose lanes pair up to store a word must leave such rows (and a tensor of 3 x 4 values, whose
+    codes end half a word in) to the kernels that store bytes."""
+    scheme = QuantScheme.default().with_value(QuantValue.E2M1).with_store(QuantStore.Native).with_level(QuantLevel.block([4]))
+    check_layouts(gpu, oracle, ElemType.F32, "e2m1_native_block4", scheme, ((6, 12), (5, 3, 20), (3, 4), (1, 12)),
+                  ("contiguous", "pitched_aligned", "pitched_words", "every_other_row"))
+
+
 def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
     import torch
 
