@@ -218,7 +218,8 @@ __global__ __launch_bounds__(kT) void reduce_tile_kernel(const u32x4* __restrict
 
 // ---- strided inputs with a contiguous last dimension ------------------------------------
 // The dimensions that are not reduced, innermost first (`count` entries each, multiply-and-shift
-// divisions), with their input strides in 16-byte chunks; the outputs are contiguous.
+// divisions), with their input strides in 32-bit words (rows start on multiples of 4 bytes; the 16-byte
+// loads then sit off their natural alignment, which the hardware takes); the outputs are contiguous.
 struct ReduceLevels {
     uint32_t levels;
     uint32_t count[CQ_MAX_RANK], magic[CQ_MAX_RANK], shift[CQ_MAX_RANK];
@@ -241,6 +242,10 @@ __device__ __forceinline__ uint64_t level_offset(const ReduceLevels& r, uint32_t
     return off;
 }
 
+__device__ __forceinline__ const u32x4* words_at(const u32x4* base, uint64_t words) {
+    return reinterpret_cast<const u32x4*>(reinterpret_cast<const uint32_t*>(base) + words);
+}
+
 // reduce_rows_grouped_kernel with the rows (all dimensions but the last) found through `r`
 template <class F, int kGroup, int kUnroll>
 __global__ __launch_bounds__(kThreads) void reduce_rows_grouped_strided_kernel(const u32x4* __restrict__ in,
@@ -252,7 +257,7 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_grouped_strided_kernel(c
     for (int u = 0; u < kUnroll; u++) {
         uint64_t c = first + static_cast<uint64_t>(u) * kThreads;
         c = c < num_chunks ? c : num_chunks - 1;
-        raw[u] = stream_load(in + level_offset(r, static_cast<uint32_t>(c / kGroup)) + c % kGroup);
+        raw[u] = stream_load(words_at(in, level_offset(r, static_cast<uint32_t>(c / kGroup))) + c % kGroup);
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
@@ -277,7 +282,7 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_wave_strided_kernel(cons
     const uint64_t per_slice = (chunks_per_row + slices - 1) / slices;
     const uint64_t begin = slice * per_slice;
     const uint64_t end = begin + per_slice < chunks_per_row ? begin + per_slice : chunks_per_row;
-    const u32x4* p = in + level_offset(r, static_cast<uint32_t>(row));
+    const u32x4* p = words_at(in, level_offset(r, static_cast<uint32_t>(row)));
     float amax = 0.0f;
     for (uint64_t c0 = begin + lane; c0 < end; c0 += kWave * kUnroll) {
         u32x4 raw[kUnroll];
@@ -299,7 +304,7 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_wave_strided_kernel(cons
 }
 
 // reduce_cols_kernel with the output chunks (the last dimension in chunks, then the other kept
-// dimensions) found through `r`; the reduced axis steps `len_stride` chunks
+// dimensions) found through `r`; the reduced axis steps `len_stride` words
 template <class F, bool kPartial>
 __global__ __launch_bounds__(kThreads) void reduce_cols_strided_kernel(const u32x4* __restrict__ in, void* __restrict__ out,
                                                                        ReduceLevels r, uint64_t cols, uint64_t len,
@@ -313,7 +318,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols_strided_kernel(const u32
     const uint64_t per_slice = (len + slices - 1) / slices;
     const uint64_t begin = slice * per_slice;
     const uint64_t end = begin + per_slice < len ? begin + per_slice : len;
-    const u32x4* p = in + level_offset(r, static_cast<uint32_t>(col));
+    const u32x4* p = words_at(in, level_offset(r, static_cast<uint32_t>(col)));
     float amax[kN];
 #pragma unroll
     for (int i = 0; i < kN; i++) amax[i] = 0.0f;
@@ -322,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols_strided_kernel(const u32
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             const uint64_t l = l0 + u < end ? l0 + u : end - 1;
-            raw[u] = stream_load(p + l * len_stride);
+            raw[u] = stream_load(words_at(p, l * len_stride));
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
@@ -473,12 +478,13 @@ void launch_fold(hipStream_t s, const void* partials, void* out, uint64_t slices
     launch_tile<F32, F, kFoldThreads, kTileFinalChecked>(s, cw, tiles, partials, out, slices, chunks, tiles, 1u, 0, count);
 }
 
-// The levels of a strided input with a contiguous last dimension of whole chunks, aligned strides and
+// The levels of a strided input with a contiguous last dimension of whole chunks, strides of whole words and
 // fewer than 2^31 rows and output chunks; false: not such a tensor.
 template <class F>
 bool strided_levels(const ReduceArgs& a, ReduceLevels* r, uint64_t* len_stride) {
     constexpr uint64_t kN = F::kPerChunk;
-    if (a.rank < 2 || (reinterpret_cast<uintptr_t>(a.input) & 15u) != 0) return false;
+    constexpr uint64_t kWordElems = F::kBytes == 4 ? 1 : 2;  // elements per 32-bit word
+    if (a.rank < 2 || (reinterpret_cast<uintptr_t>(a.input) & 3u) != 0) return false;
     const uint32_t last = a.rank - 1;
     if (a.in_strides[last] != 1 || a.shape[last] % kN != 0) return false;
     *r = ReduceLevels{};
@@ -495,15 +501,15 @@ bool strided_levels(const ReduceArgs& a, ReduceLevels* r, uint64_t* len_stride) 
         }
         total *= count;
     };
-    if (a.axis != last) push(a.shape[last] / kN, 1);
+    if (a.axis != last) push(a.shape[last] / kN, 4);  // a chunk is four words
     for (int d = static_cast<int>(last) - 1; d >= 0; d--) {
-        if (a.in_strides[d] % kN != 0 && a.shape[d] > 1) return false;
+        if (a.in_strides[d] % kWordElems != 0 && a.shape[d] > 1) return false;
         if (static_cast<uint32_t>(d) == a.axis) {
-            *len_stride = a.in_strides[d] / kN;
+            *len_stride = a.in_strides[d] / kWordElems;
             continue;
         }
         if (a.shape[d] == 1) continue;
-        push(a.shape[d], a.in_strides[d] / kN);
+        push(a.shape[d], a.in_strides[d] / kWordElems);
     }
     if (r->levels == 0) push(1, 0);
     if (total >= (1ull << 31)) return false;

@@ -176,6 +176,8 @@ ROWWISE_STRIDED = [
     ((3, 5, 2048), (2048, 3 * 2048, 1)),                       # leading dimensions swapped
     ((4, 700, 256), (1024 * 320, 320, 1)),                     # a slice of a larger batch, pitched
     ((1, 9000, 8), (0, 16, 1)),                                # rows of one 16-byte chunk (two for f32) at a pitch
+    ((300, 1024), (1030, 1)),                                  # rows that start on multiples of 4 bytes only (bf16 / f16)
+    ((5, 64, 256), (64 * 258 + 2, 258, 1)),                    # the same behind a batch dimension
     ((256, 4096), (1, 256)),                                   # a transposed matrix: reduced in the order of its strides
     ((48, 40, 64), (1, 48, 48 * 40)),                          # all dimensions reversed in memory
     ((6, 512, 64), (512 * 64, 1, 512)),                        # last two dimensions swapped in memory
