@@ -20,7 +20,7 @@ EXPORTED_SYMBOLS = (
     "cq_value_size_bits", "cq_scheme_num_quants", "cq_value_range", "cq_quantize", "cq_dequantize",
     "cq_compute_scales", "cq_quantize_dynamic", "cq_workspace_bytes", "cq_strerror",
     "cq_last_hip_error", "cq_abi_version", "cq_reduce_max_abs", "cq_reduce_workspace_bytes",
-    "cq_into_contiguous_packed",
+    "cq_into_contiguous_packed", "cq_quantize_dynamic_static",
 )
 
 
@@ -46,7 +46,8 @@ class QuantError(RuntimeError):
 
 # status codes (mirrors enum cq_status)
 OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED_SCHEME, ERR_BLOCK_NOT_DIVISIBLE, ERR_SHAPE_MISMATCH, \
-    ERR_NON_CONTIGUOUS, ERR_WORKSPACE_TOO_SMALL, ERR_HIP, ERR_TOO_LARGE, ERR_INVALID_AXIS = range(10)
+    ERR_NON_CONTIGUOUS, ERR_WORKSPACE_TOO_SMALL, ERR_HIP, ERR_TOO_LARGE, ERR_INVALID_AXIS, \
+    ERR_SCRATCH_TOO_SMALL = range(11)
 
 _lib = None
 
@@ -84,6 +85,8 @@ def lib() -> ctypes.CDLL:
     L.cq_compute_scales.argtypes = [ctypes.c_void_p, tp, tp, sp, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
     L.cq_quantize_dynamic.restype = ctypes.c_int
     L.cq_quantize_dynamic.argtypes = [ctypes.c_void_p, tp, tp, tp, sp, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
+    L.cq_quantize_dynamic_static.restype = ctypes.c_int
+    L.cq_quantize_dynamic_static.argtypes = [ctypes.c_void_p, tp, tp, tp, sp, ctypes.c_int]
     L.cq_reduce_max_abs.restype = ctypes.c_int
     L.cq_reduce_max_abs.argtypes = [ctypes.c_void_p, tp, tp, ctypes.c_uint32, ctypes.c_int, ctypes.c_void_p,
                                     ctypes.c_size_t]

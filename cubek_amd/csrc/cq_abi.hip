@@ -5,6 +5,7 @@
 // precompiled gfx950 kernel launch on the caller's stream.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstring>
 #include <utility>
 
@@ -522,6 +523,32 @@ cq::GenericArgs generic_args(const Plan& p, const cq_scheme* s) {
     return g;
 }
 
+// Scratch of cq_quantize_dynamic_static: the abs-max partials of the per-tensor grid reduction.  Every GPU
+// holds its own copy of the array at its own address until the process ends.  In host code the array's name
+// is only a handle for hipGetSymbolAddress, never a device address: kernels get the resolved pointer.
+static __device__ __align__(256) unsigned char scratch[CQ_STATIC_SCRATCH_BYTES];
+static_assert(CQ_STATIC_SCRATCH_BYTES >= cq::kMaxPartials * sizeof(float), "the partials of one reduction must fit");
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device, resolved on the first call per device (threads that
+// race here resolve the same address).
+cq_status static_scratch(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_status(e);
+    if (dev < 0 || dev >= kMaxDevices) return CQ_ERR_INVALID_ARGUMENT;
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_status(e);
+        if (p == nullptr) return CQ_ERR_HIP;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *ptr = p;
+    return CQ_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -542,6 +569,7 @@ const char* cq_strerror(cq_status st) {
         case CQ_ERR_HIP: return "HIP runtime error";
         case CQ_ERR_TOO_LARGE: return "tensor too large";
         case CQ_ERR_INVALID_AXIS: return "the reduction axis must be smaller than the tensor rank";
+        case CQ_ERR_SCRATCH_TOO_SMALL: return "the call needs more scratch memory than the library's built-in array holds; use the entry point that takes a workspace";
         default: return "unknown status";
     }
 }
@@ -857,9 +885,9 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
     return produce_scales(stream, p, scheme, input, input_dtype, scales, input_dtype, workspace, workspace_bytes);
 }
 
-cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
-                              const cq_tensor* out_scale, const cq_scheme* scheme, cq_dtype input_dtype,
-                              void* workspace, size_t workspace_bytes) {
+static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                                  const cq_tensor* out_scale, const cq_scheme* scheme, cq_dtype input_dtype,
+                                  void* workspace, size_t workspace_bytes) {
     cq_status st = check_scheme(scheme);
     if (st != CQ_OK) return st;
     if (!out_scale) return CQ_ERR_INVALID_ARGUMENT;
@@ -1024,6 +1052,30 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
                                : cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
     }
     return st;
+}
+
+cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                              const cq_tensor* out_scale, const cq_scheme* scheme, cq_dtype input_dtype,
+                              void* workspace, size_t workspace_bytes) {
+    return quantize_dynamic(stream, input, output, out_scale, scheme, input_dtype, workspace, workspace_bytes);
+}
+
+cq_status cq_quantize_dynamic_static(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                                     const cq_tensor* out_scale, const cq_scheme* scheme, cq_dtype input_dtype) {
+    cq_status st = check_scheme(scheme);
+    if (st != CQ_OK) return st;
+    if (!tensor_ok(input)) return CQ_ERR_INVALID_ARGUMENT;
+    // what the call would ask of a caller's workspace must fit the array
+    uint64_t n = 1;
+    for (uint32_t d = 0; d < input->rank; d++) {
+        if (input->shape[d] != 0 && n > (1ull << 48) / input->shape[d]) return CQ_ERR_TOO_LARGE;
+        n *= input->shape[d];
+    }
+    if (cq_workspace_bytes(scheme, n) > CQ_STATIC_SCRATCH_BYTES) return CQ_ERR_SCRATCH_TOO_SMALL;
+    void* ws = nullptr;
+    st = static_scratch(&ws);
+    if (st != CQ_OK) return st;
+    return quantize_dynamic(stream, input, output, out_scale, scheme, input_dtype, ws, CQ_STATIC_SCRATCH_BYTES);
 }
 
 cq_status cq_into_contiguous_packed(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,

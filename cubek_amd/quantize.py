@@ -44,3 +44,13 @@ def launch_dynamic(client: ComputeClient, input: TensorHandleRef, output: Tensor
                                         scheme.to_c(), int(input_elem), workspace, workspace_bytes)
     if rc:
         _ffi.check(rc)
+
+
+def launch_dynamic_static(client: ComputeClient, input: TensorHandleRef, output: TensorHandleRef,
+                          out_scale: TensorHandleRef, scheme: QuantScheme, input_elem: ElemType) -> None:
+    """launch_dynamic for callers that cannot allocate a workspace: the scratch memory is an array
+    inside the library (one per GPU, shared by all calls on that GPU)."""
+    rc = _ffi.lib().cq_quantize_dynamic_static(client.stream, input.as_c(), output.as_c(), out_scale.as_c(),
+                                               scheme.to_c(), int(input_elem))
+    if rc:
+        _ffi.check(rc)

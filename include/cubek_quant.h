@@ -42,7 +42,8 @@ typedef enum cq_status {
     CQ_ERR_WORKSPACE_TOO_SMALL = 6,
     CQ_ERR_HIP = 7,                 /* a HIP runtime call failed; see cq_last_hip_error  */
     CQ_ERR_TOO_LARGE = 8,           /* more elements than an entry point accepts         */
-    CQ_ERR_INVALID_AXIS = 9         /* reduction axis >= rank (ReduceError::InvalidAxis) */
+    CQ_ERR_INVALID_AXIS = 9,        /* reduction axis >= rank (ReduceError::InvalidAxis) */
+    CQ_ERR_SCRATCH_TOO_SMALL = 10   /* cq_quantize_dynamic_static: the call needs more than CQ_STATIC_SCRATCH_BYTES */
 } cq_status;
 
 /* Float element types of value tensors and scale parameters
@@ -169,6 +170,23 @@ cq_status cq_quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const 
 
 /* Device bytes the two entry points above need for `num_elements` inputs. */
 size_t cq_workspace_bytes(const cq_scheme* scheme, uint64_t num_elements);
+
+/* cq_quantize_dynamic without a workspace argument.  No counterpart in the reference: it is for
+ * callers that cannot allocate device memory for a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  Same arguments otherwise, same codes and
+ * scales bit for bit.  The scratch memory (the abs-max partials of the per-tensor grid reduction)
+ * is an array of CQ_STATIC_SCRATCH_BYTES inside the library's device code; every GPU the library
+ * runs on holds its copy until the process ends.  The call allocates and frees nothing.
+ *   - a call whose scheme and size need more scratch than the array holds returns
+ *     CQ_ERR_SCRATCH_TOO_SMALL (cq_workspace_bytes() tells the need; today no scheme exceeds it);
+ *   - the device that is current when the call is made must be the stream's device; the first call
+ *     on a device looks the array's address up and must not run under stream capture;
+ *   - all calls on one GPU share that GPU's array: two calls that overlap in time on one GPU
+ *     (different streams, or threads) race on it.  Calls on one stream do not overlap. */
+#define CQ_STATIC_SCRATCH_BYTES 1024
+cq_status cq_quantize_dynamic_static(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
+                                     const cq_tensor* out_scale, const cq_scheme* scheme,
+                                     cq_dtype input_dtype);
 
 /* ---- abs-max along an axis (the step in front of the path) ---- */
 

@@ -205,6 +205,14 @@ inline void launch_dynamic(const ComputeClient& client, const TensorHandleRef& i
     detail::check(cq_quantize_dynamic(client.stream, &i, &o, &os, &c, static_cast<cq_dtype>(input_elem), workspace,
                                       workspace_size), scheme);
 }
+// the same without a workspace: the scratch memory is an array inside the library (one per GPU,
+// shared by all calls on that GPU), for callers that cannot allocate device memory
+inline void launch_dynamic_static(const ComputeClient& client, const TensorHandleRef& input, const TensorHandleRef& output,
+                                  const TensorHandleRef& out_scale, const scheme::QuantScheme& scheme, ElemType input_elem) {
+    cq_tensor i = input.as_c(), o = output.as_c(), os = out_scale.as_c();
+    cq_scheme c = scheme.to_c();
+    detail::check(cq_quantize_dynamic_static(client.stream, &i, &o, &os, &c, static_cast<cq_dtype>(input_elem)), scheme);
+}
 }  // namespace quantize
 
 namespace dequantize {

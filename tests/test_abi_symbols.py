@@ -50,8 +50,8 @@ def test_workspace_and_messages():
     per_block = QuantScheme.default().with_level(QuantLevel.block([32])).to_c()
     assert lib.cq_workspace_bytes(ctypes.byref(per_tensor), 1 << 20) == 1024
     assert lib.cq_workspace_bytes(ctypes.byref(per_block), 1 << 20) == 0
-    msgs = {lib.cq_strerror(i).decode() for i in range(10)}
-    assert len(msgs) == 10 and "success" in msgs
+    msgs = {lib.cq_strerror(i).decode() for i in range(11)}
+    assert len(msgs) == 11 and "success" in msgs
     assert ctypes.sizeof(_ffi.CTensor) == 32 and ctypes.sizeof(type(per_tensor)) == 12
 
 
