@@ -22,6 +22,11 @@ cq_status hip_status(hipError_t e) {
     return CQ_ERR_HIP;
 }
 
+// The launchers read hipGetLastError() after each launch.  An error left on the calling thread by earlier
+// HIP calls of the caller would be taken for a failed launch, so every entry point that launches kernels
+// clears it first (as any hipGetLastError() does).
+void drop_stale_hip_error() { (void)hipGetLastError(); }
+
 uint32_t dtype_size(int dtype) { return dtype == CQ_F32 ? 4u : 2u; }
 bool valid_dtype(int dtype) { return dtype == CQ_F32 || dtype == CQ_F16 || dtype == CQ_BF16; }
 int param_to_dtype(uint8_t p) { return p == CQ_PARAM_F32 ? CQ_F32 : (p == CQ_PARAM_F16 ? CQ_F16 : CQ_BF16); }
@@ -91,6 +96,7 @@ struct Plan {
     bool last_dim_blocks;   // block extents are 1 everywhere but the last dimension
     uint32_t block_last;
     uint64_t num_blocks;
+    bool block_splits_words;  // U32 store: the last block extent is not a multiple of the values per word
 };
 
 uint32_t stored_nq(const cq_scheme* s) {
@@ -98,20 +104,28 @@ uint32_t stored_nq(const cq_scheme* s) {
     return s->value == CQ_VALUE_E2M1 ? 2u : 1u;
 }
 
-// Line size the reference would pick for the native kernels: the widest of
-// 16 bytes / elem_size, halving until it divides the last dimension
-// (src/quantize.rs:235-240).  Only used for its block-size assertion.
-uint32_t native_line_size(uint32_t elem_size, uint64_t last_dim) {
-    uint32_t l = 16u / elem_size;
-    while (l > 1 && last_dim % l) l /= 2;
+// Line size the reference would pick for the native quantize kernel (src/quantize.rs:234-240,
+// cubecl's tensor_line_size_parallel over the line sizes of at most 16 bytes): 1 when the last
+// dimension is not contiguous, else the widest power of two up to 16 bytes / elem_size that divides
+// the last dimension and the smallest stride above 1.  Only used for its block-size assertion.
+uint32_t native_line_size(const cq_tensor* t) {
+    const uint32_t last = t->rank - 1;
+    if (t->strides[last] != 1) return 1;
+    uint64_t next_stride = 0;
+    for (uint32_t d = 0; d < t->rank; d++)
+        if (t->strides[d] > 1 && (next_stride == 0 || t->strides[d] < next_stride)) next_stride = t->strides[d];
+    uint32_t l = 16u / t->elem_size;
+    while (l > 1 && (t->shape[last] % l || next_stride % l)) l /= 2;
     return l;
 }
 
 // `values` is the stored tensor, `floats` the float tensor (input of quantize,
 // output of dequantize); they must agree in shape and may have any strides.
+// `quantizing`: the call is one the reference guards with check_block_size_compat (its quantize launchers
+// only: src/quantize.rs:260,305; dequantize_packed and dequantize_native do not call it).
 cq_status make_plan(const cq_scheme* s, const cq_tensor* floats, int dtype, const cq_tensor* values,
                     const cq_tensor* scale_a, uint32_t scale_a_size, const cq_tensor* scale_b,
-                    uint32_t scale_b_size, Plan* p) {
+                    uint32_t scale_b_size, bool quantizing, Plan* p) {
     if (!tensor_ok(floats) || !tensor_ok(values) || !tensor_ok(scale_a) || (scale_b && !tensor_ok(scale_b)))
         return CQ_ERR_INVALID_ARGUMENT;
     if (!valid_dtype(dtype)) return CQ_ERR_INVALID_ARGUMENT;
@@ -152,17 +166,22 @@ cq_status make_plan(const cq_scheme* s, const cq_tensor* floats, int dtype, cons
     p->last_dim_blocks = false;
     p->block_last = 0;
     p->num_blocks = 1;
+    p->block_splits_words = false;
     if (p->tensor_level) {
         if (numel(scale_a) < 1 || (scale_b && numel(scale_b) < 1)) return CQ_ERR_SHAPE_MISMATCH;
         return CQ_OK;
     }
     if (s->block_rank > p->rank) return CQ_ERR_SHAPE_MISMATCH;
-    // check_block_size_compat (src/lib.rs:20-33): the last block extent must be a
-    // multiple of num_quants (packed) or of the line size (native)
+    // check_block_size_compat (src/lib.rs:20-33): the last block extent must be a multiple of num_quants
+    // (packed) or of the line size (native), asserted where the reference quantizes.  Its dequantize
+    // launchers accept any block: the packed kernel then gives a whole word the scale of the word's first
+    // element (src/dequantize.rs:70-76), which the per-element kernel here reproduces; the native kernel gives
+    // every element the scale of its own block (the reference: of its line's first element, with a line
+    // size that differs between its runtimes; the two agree whenever the block is a multiple of the line).
     uint32_t last_block = s->block[s->block_rank - 1];
-    uint32_t div = s->store == CQ_STORE_U32 ? p->nq
-                                            : native_line_size(floats->elem_size, p->shape[p->rank - 1]);
-    if (last_block % div) return CQ_ERR_BLOCK_NOT_DIVISIBLE;
+    p->block_splits_words = s->store == CQ_STORE_U32 && last_block % p->nq != 0;
+    if (quantizing && last_block % (s->store == CQ_STORE_U32 ? p->nq : native_line_size(floats)) != 0)
+        return CQ_ERR_BLOCK_NOT_DIVISIBLE;
     if (scale_a->rank != p->rank || (scale_b && scale_b->rank != p->rank)) return CQ_ERR_SHAPE_MISMATCH;
     p->layout.rank = p->rank;
     p->last_dim_blocks = true;
@@ -606,12 +625,13 @@ size_t cq_workspace_bytes(const cq_scheme* s, uint64_t /*num_elements*/) {
 cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
                       const cq_tensor* scale, const cq_tensor* out_scale, const cq_scheme* scheme,
                       cq_dtype input_dtype) {
+    drop_stale_hip_error();
     cq_status st = check_scheme(scheme);
     if (st != CQ_OK) return st;
     Plan p;
     int pd = param_to_dtype(scheme->param);
     st = make_plan(scheme, input, input_dtype, output, scale, dtype_size(input_dtype), out_scale,
-                   dtype_size(pd), &p);
+                   dtype_size(pd), true, &p);
     if (st != CQ_OK) return st;
     if (!out_scale) return CQ_ERR_INVALID_ARGUMENT;
     if (p.n == 0) return CQ_OK;
@@ -688,18 +708,21 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
 
 cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_tensor* output,
                         const cq_tensor* params, const cq_scheme* scheme, cq_dtype output_dtype) {
+    drop_stale_hip_error();
     cq_status st = check_scheme(scheme);
     if (st != CQ_OK) return st;
     Plan p;
     int pd = param_to_dtype(scheme->param);
-    st = make_plan(scheme, output, output_dtype, values, params, dtype_size(pd), nullptr, 0, &p);
+    st = make_plan(scheme, output, output_dtype, values, params, dtype_size(pd), nullptr, 0, false, &p);
     if (st != CQ_OK) return st;
     if (p.n == 0) return CQ_OK;
 
     const bool native = scheme->store == CQ_STORE_NATIVE;
     const uint64_t per_chunk = 16 / dtype_size(output_dtype);
     uint64_t flat_words = 0;
-    if (flat_ok(p, output_dtype, output, values, params, nullptr)) {
+    // blocks that split a word: only the per-element kernel scales a whole word by its first element's block
+    const bool streaming = !p.block_splits_words;
+    if (streaming && flat_ok(p, output_dtype, output, values, params, nullptr)) {
         cq::FlatArgs a{};
         a.input = values->ptr;
         a.output = output->ptr;
@@ -715,7 +738,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
     cq::FlatArgs fr{};
-    if (flat_words == 0 && (flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr) ||
+    if (streaming && flat_words == 0 && (flat_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr) ||
                             lane_rows_ok(p, scheme, output_dtype, output, values, params, dtype_size(pd), nullptr, 0, true, &fr))) {
         fr.input = values->ptr;
         fr.output = output->ptr;
@@ -728,14 +751,14 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         return hip_status(cq::launch_dequantize_flat(stream, output_dtype, p.bits, fr));
     }
     cq::RowArgs r;
-    if (flat_words == 0 && rows_args(p, scheme, output_dtype, output, values, &r)) {
+    if (streaming && flat_words == 0 && rows_args(p, scheme, output_dtype, output, values, &r)) {
         r.input = values->ptr;
         r.output = output->ptr;
         r.scale_in = params->ptr;
         return hip_status(cq::launch_dequantize_rows(stream, output_dtype, static_cast<int>(p.bits), r));
     }
     cq::TransposedArgs tr;
-    if (flat_words == 0 && transposed_args(p, scheme, output_dtype, output, values, &tr)) {
+    if (streaming && flat_words == 0 && transposed_args(p, scheme, output_dtype, output, values, &tr)) {
         tr.input = values->ptr;
         tr.output = output->ptr;
         tr.scale_in = params->ptr;
@@ -814,6 +837,7 @@ static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_sche
 cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq_tensor* scales,
                             const cq_scheme* scheme, cq_dtype input_dtype, void* workspace,
                             size_t workspace_bytes) {
+    drop_stale_hip_error();
     cq_status st = check_scheme(scheme);
     if (st != CQ_OK) return st;
     if (!tensor_ok(input) || !tensor_ok(scales) || !valid_dtype(input_dtype)) return CQ_ERR_INVALID_ARGUMENT;
@@ -829,7 +853,7 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
     }
     cq_tensor values{input->ptr, vshape, vstrides, input->rank, scheme->store == CQ_STORE_U32 ? 4u : 1u};
     Plan p;
-    st = make_plan(scheme, input, input_dtype, &values, scales, dtype_size(input_dtype), nullptr, 0, &p);
+    st = make_plan(scheme, input, input_dtype, &values, scales, dtype_size(input_dtype), nullptr, 0, false, &p);
     if (st != CQ_OK) return st;
     if (p.n == 0) return CQ_OK;
 
@@ -888,12 +912,13 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
 static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
                                   const cq_tensor* out_scale, const cq_scheme* scheme, cq_dtype input_dtype,
                                   void* workspace, size_t workspace_bytes) {
+    drop_stale_hip_error();
     cq_status st = check_scheme(scheme);
     if (st != CQ_OK) return st;
     if (!out_scale) return CQ_ERR_INVALID_ARGUMENT;
     Plan p;
     int pd = param_to_dtype(scheme->param);
-    st = make_plan(scheme, input, input_dtype, output, out_scale, dtype_size(pd), nullptr, 0, &p);
+    st = make_plan(scheme, input, input_dtype, output, out_scale, dtype_size(pd), nullptr, 0, true, &p);
     if (st != CQ_OK) return st;
     if (p.n == 0) return CQ_OK;
 
@@ -1080,6 +1105,7 @@ cq_status cq_quantize_dynamic_static(cq_stream_t stream, const cq_tensor* input,
 
 cq_status cq_into_contiguous_packed(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
                                     const uint64_t* shape, uint32_t rank, uint32_t packing) {
+    drop_stale_hip_error();
     if (!tensor_ok(input) || !tensor_ok(output) || !shape) return CQ_ERR_INVALID_ARGUMENT;
     if (input->rank != rank || output->rank != rank) return CQ_ERR_SHAPE_MISMATCH;
     const uint32_t elem = input->elem_size;
@@ -1176,6 +1202,7 @@ size_t cq_reduce_workspace_bytes(const cq_tensor* input, uint32_t axis, cq_dtype
 
 cq_status cq_reduce_max_abs(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output, uint32_t axis,
                             cq_dtype dtype, void* workspace, size_t workspace_bytes) {
+    drop_stale_hip_error();
     if (!tensor_ok(input) || !tensor_ok(output) || !valid_dtype(dtype)) return CQ_ERR_INVALID_ARGUMENT;
     if (axis >= input->rank) return CQ_ERR_INVALID_AXIS;
     if (input->elem_size != dtype_size(dtype) || output->elem_size != dtype_size(dtype)) return CQ_ERR_SHAPE_MISMATCH;

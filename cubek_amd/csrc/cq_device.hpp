@@ -228,10 +228,13 @@ struct QuantParams {
 };
 
 // Divisors for which x * rcp(d) stays within 2^-21 relative error of x / d:
-// finite, normal and far from the ends of the exponent range (false for NaN).
+// positive, finite, normal and far from the ends of the exponent range (false for NaN).
+// Negative divisors (only a caller's own scales can be negative) take the IEEE division:
+// the residual steps of the f16 path add zeros of opposite sign, which loses the sign of
+// the zero quotient (-0) / d for d < 0.
 __device__ __forceinline__ bool divisor_is_tame(float d) {
-    // exponent field in [27, 227): 2^-100 <= |d| < 2^100
-    return ((f32_bits(d) & 0x7fffffffu) - 0x0d800000u) < (0x71800000u - 0x0d800000u);
+    // sign clear and exponent field in [27, 227): 2^-100 <= d < 2^100
+    return (f32_bits(d) - 0x0d800000u) < (0x71800000u - 0x0d800000u);
 }
 // abs-max values for which the scale 2*amax/width (width <= 2^17) and its
 // divisor are tame: 2^-80 <= amax < 2^80.

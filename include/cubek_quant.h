@@ -12,6 +12,12 @@
  *   - calls are asynchronous and ordered on the given HIP stream (NULL = the
  *     default stream); nothing here synchronises the device;
  *   - every function returns a cq_status (0 = success) and never aborts;
+ *   - an entry point that launches kernels first clears the calling thread's pending HIP error
+ *     (hipGetLastError), so that CQ_ERR_HIP always speaks of this call's own launches;
+ *   - special values follow IEEE arithmetic on the reference's formula with these choices, which the
+ *     reference leaves to its JIT backend and its tests do not observe: round() is round-half-to-even,
+ *     clamp() is max(lo, min(x, hi)) with minNum/maxNum, so a NaN quotient (NaN element, NaN scale, 0/0)
+ *     quantizes to q_max; abs-max ignores NaN elements; a zero result keeps the sign IEEE gives it;
  *   - calls are re-entrant and thread safe: the library keeps no state besides the
  *     per-thread code behind cq_last_hip_error().
  */

@@ -13,17 +13,28 @@
  * division and multiplication of 8- or 11-bit significands this equals the
  * correctly rounded F result because f32 carries >= 2p+2 bits.
  *
- * Behaviour the reference delegates to its JIT dependency (cubecl, not in the
- * reference tree) and that its own tests do not pin — PARITY UNPINNED, fixed
- * here by decision:
+ * How each function is pinned (tests/test_oracle_*.py; none of the pins retypes the formula):
+ *   float conversions          torch / numpy CPU conversions, nearest-value table search
+ *   cqo_scale_index, cqo_is_block_start   brute force over small N-D shapes
+ *   cqo_pack_word, cqo_unpack_word        exhaustive over fields and positions
+ *   cqo_quantize_packed, cqo_dequantize_packed   exact-rational fixtures (tests/golden/),
+ *                              hand-derived known answers, torch CPU bf16 arithmetic
+ *   cqo_quantize_native, cqo_dequantize_native   exact-rational fixtures of all five native
+ *                              value types (minifloats built from their bit fields), hand-written
+ *                              byte-level known answers (e2m1 nibbles, every i8 code), identities
+ *                              with the packed store, torch CPU float8 conversions
+ *   cqo_compute_scales, cqo_reduce_max_abs        numpy, exact rationals, permutation invariance
+ *
+ * Decisions.  The reference delegates these to its JIT dependency (cubecl, not in the
+ * reference tree) and its own tests do not observe them; no check can pin them, so they
+ * are fixed here by decision and stated as such wherever results are documented:
  *   - round()   = round-half-to-even (rint);
  *   - clamp()   = max(lo, min(x, hi)) with IEEE minNum/maxNum: NaN -> hi;
  *   - value ranges and num_quants as listed in cqo_value_range/cqo_num_quants;
+ *   - float -> e4m3 / e5m2 / e2m1 casts round to nearest, ties to the even code;
  *   - E2M1 native bytes hold element 2k in the low nibble, 2k+1 in the high;
  *   - abs-max ignores NaN elements (Rust f32::max in the reference's test).
- * Everything else (field order, two's-complement fields, scale indexing,
- * correctly rounded divide/multiply) is pinned by tests/test_oracle_*.py
- * against exact rational arithmetic, brute force and library float routines.
+ * Given these decisions, every function below is pinned as listed above.
  *
  * Build: gcc -O2 -fno-fast-math -ffp-contract=off (see Makefile).
  */

@@ -8,8 +8,14 @@ rounded quotient in F", "round half to even", "two's-complement field i at bits
 round-half-away, a transposed field order or a wrong scale index in the oracle
 shows up as a mismatch.  Pure Python, small inputs only, finite values only.
 
-Specification followed: crates/cubek-quant/src/quantize.rs:19-31,61-81,
-src/dequantize.rs:22-25,86-118, src/layout/scales.rs:144-160,179-194,
+The native store (one byte per value: i8, e4m3, e5m2; two e2m1 nibbles per byte)
+is stated the same way: the minifloat formats are built from their published bit
+fields (sign, exponent, mantissa, bias), "cast to Q" is "nearest value of the format,
+ties to the even code, saturating", and the sign of a zero result is the sign IEEE
+arithmetic gives it (sign(x) xor sign(scale)).
+
+Specification followed: crates/cubek-quant/src/quantize.rs:19-43,61-81,100-126,
+src/dequantize.rs:22-25,86-118,150-167, src/layout/scales.rs:144-160,179-194,
 tests/suite/symmetric.rs:35-38,156-179.
 """
 from __future__ import annotations
@@ -174,7 +180,10 @@ def dequantize_tensor(words: np.ndarray, fmt: str, shape: Sequence[int], scale_b
             si = sum(c * s for c, s in zip(bc, scale_strides))
         s = round_to_format(bits_to_fraction(int(scale_bits.reshape(-1)[si]), param_fmt), fmt)
         for i, c in enumerate(unpack(int(words[p]), bits)):
-            out[e0 + i] = fraction_to_bits(round_to_format(s * c, fmt), fmt)
+            # F(c) is +0 for the code 0, so the product's sign is the scale's when it is zero
+            y = round_to_format(s * c, fmt)
+            out[e0 + i] = (fraction_to_bits(abs(y), fmt) | (int((s < 0) != (c < 0)) << (31 if fmt == "f32" else 15))
+                           if y == 0 else fraction_to_bits(y, fmt))
     return out
 
 
@@ -203,3 +212,123 @@ def scales_from_absmax(x_bits: np.ndarray, fmt: str, shape: Sequence[int],
         s32 = round_to_format(two_a / (hi - lo), "f32")
         out[i] = fraction_to_bits(round_to_format(s32, fmt), fmt)
     return out.reshape(sshape)
+
+
+# ---------------------------------------------------------------- native store
+# name -> (exponent bits, mantissa bits, bias): OCP 8-bit floating point (E4M3 finite-only
+# with one NaN code, E5M2 IEEE-like) and OCP microscaling FP4 (E2M1, no NaN, no infinity)
+MINIFLOATS = {"E4M3": (4, 3, 7), "E5M2": (5, 2, 15), "E2M1": (2, 1, 1)}
+
+
+def minifloat_magnitudes(name: str) -> List[Fraction]:
+    """Finite magnitudes of the format by magnitude code 0, 1, 2, ... (sign bit excluded)."""
+    ebits, mbits, bias = MINIFLOATS[name]
+    out = []
+    for code in range(1 << (ebits + mbits)):
+        e, f = code >> mbits, code & ((1 << mbits) - 1)
+        if name == "E4M3" and code == 0x7F:
+            break  # S.1111.111 is NaN
+        if name == "E5M2" and e == (1 << ebits) - 1:
+            break  # infinities and NaNs
+        if e == 0:
+            out.append(Fraction(f, 1 << mbits) * Fraction(2) ** (1 - bias))
+        else:
+            out.append((1 + Fraction(f, 1 << mbits)) * Fraction(2) ** (e - bias))
+    return out
+
+
+def minifloat_encode(mag: Fraction, name: str) -> int:
+    """Magnitude code of the nearest finite value; a tie goes to the even code (the one whose
+    last mantissa bit is 0); magnitudes beyond the largest finite value saturate to it."""
+    table = minifloat_magnitudes(name)
+    assert mag >= 0
+    best = 0
+    for code, v in enumerate(table):
+        d, db = abs(v - mag), abs(table[best] - mag)
+        if d < db or (d == db and code % 2 == 0 and best % 2 == 1):
+            best = code
+    return best
+
+
+def sign_and_magnitude(bits: int, fmt: str) -> Tuple[bool, Fraction]:
+    width = 32 if fmt == "f32" else 16
+    neg = bool((bits >> (width - 1)) & 1)
+    return neg, abs(bits_to_fraction(bits, fmt))
+
+
+def signed_bits(neg: bool, mag: Fraction, fmt: str) -> int:
+    """Bit pattern of (-1)^neg * mag, mag representable in fmt; keeps the sign of zero."""
+    width = 32 if fmt == "f32" else 16
+    return fraction_to_bits(mag, fmt) | (int(neg) << (width - 1))
+
+
+def native_code(neg: bool, mag_q: Fraction, fmt: str, value: str) -> int:
+    """Stored byte (nibble for E2M1) of one element: ``mag_q`` = |x| / |divisor| exactly,
+    ``neg`` the sign of the quotient.  round to F, rint, clamp, cast to Q."""
+    lo, hi = RANGES[value]
+    k = rint_even(round_to_format(mag_q, fmt))  # |rint(t)|: both roundings are sign-symmetric
+    k = min(k, -lo) if neg else min(k, hi)
+    if value in ("Q8F", "Q8S"):
+        return (-k if neg else k) % 256          # i8 cast: two's complement byte, -0 -> 0
+    ebits, mbits, _ = MINIFLOATS[value]
+    return (int(neg) << (ebits + mbits)) | minifloat_encode(Fraction(k), value)
+
+
+def native_decode(code: int, value: str) -> Tuple[bool, Fraction]:
+    if value in ("Q8F", "Q8S"):
+        v = code - 256 if code >= 128 else code
+        return v < 0, Fraction(abs(v))
+    ebits, mbits, _ = MINIFLOATS[value]
+    return bool(code >> (ebits + mbits)), minifloat_magnitudes(value)[code & ((1 << (ebits + mbits)) - 1)]
+
+
+def _scale_lookup(e: int, shape, blk_vec, scale_strides):
+    if blk_vec is None:
+        return 0, e == 0
+    bc, start = block_of(e, shape, blk_vec)
+    return sum(c * s for c, s in zip(bc, scale_strides)), start
+
+
+def quantize_tensor_native(x_bits: np.ndarray, fmt: str, shape: Sequence[int], scale_bits: np.ndarray,
+                           scale_strides: Sequence[int], block: Sequence[int] | None, value: str,
+                           param_fmt: str):
+    """Native-store quantization of a contiguous tensor: one byte per element, or (E2M1) two
+    nibbles per byte with element 2k in the LOW nibble and element 2k+1 in the high one.
+    Returns (bytes uint8, out_scale bit patterns in param_fmt)."""
+    n = int(np.prod(shape))
+    per_byte = 2 if value == "E2M1" else 1
+    out = np.zeros(n // per_byte, dtype=np.uint8)
+    out_scale = np.zeros(scale_bits.size, dtype=np.uint32 if param_fmt == "f32" else np.uint16)
+    blk_vec = None if block is None else (1,) * (len(shape) - len(block)) + tuple(block)
+    flat = x_bits.reshape(-1)
+    for e in range(n):
+        si, start = _scale_lookup(e, shape, blk_vec, scale_strides)
+        s_neg, s_mag = sign_and_magnitude(int(scale_bits.reshape(-1)[si]), fmt)
+        s_fs = round_to_format(s_mag, param_fmt)
+        if start:
+            out_scale[si] = signed_bits(s_neg, s_fs, param_fmt)
+        d = round_to_format(s_fs, fmt)
+        x_neg, x_mag = sign_and_magnitude(int(flat[e]), fmt)
+        code = native_code(x_neg != s_neg, x_mag / d, fmt, value)
+        if per_byte == 2:
+            out[e // 2] |= code << (4 * (e % 2))
+        else:
+            out[e] = code
+    return out, out_scale
+
+
+def dequantize_tensor_native(codes: np.ndarray, fmt: str, shape: Sequence[int], scale_bits: np.ndarray,
+                             scale_strides: Sequence[int], block: Sequence[int] | None, value: str,
+                             param_fmt: str) -> np.ndarray:
+    """F(scale) * F(q), one rounding to F; a zero product keeps the sign IEEE gives it."""
+    n = int(np.prod(shape))
+    out = np.zeros(n, dtype=np.uint32 if fmt == "f32" else np.uint16)
+    blk_vec = None if block is None else (1,) * (len(shape) - len(block)) + tuple(block)
+    for e in range(n):
+        si, _ = _scale_lookup(e, shape, blk_vec, scale_strides)
+        s_neg, s_mag = sign_and_magnitude(int(scale_bits.reshape(-1)[si]), param_fmt)
+        s = round_to_format(s_mag, fmt)
+        code = int(codes[e // 2] >> (4 * (e % 2))) & 0xF if value == "E2M1" else int(codes[e])
+        q_neg, q_mag = native_decode(code, value)
+        out[e] = signed_bits(s_neg != q_neg, round_to_format(s * q_mag, fmt), fmt)
+    return out

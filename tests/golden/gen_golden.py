@@ -12,6 +12,11 @@ Cases
                   scales by the test's host rule.
   typed_small.npz f32/bf16/f16 inputs with many exact .5 quotients, other
                   param dtypes, N-D blocks, strided scales, E2M1/E4M3 ranges.
+  typed_native.npz the native store (crates/cubek-quant/src/quantize.rs:100-126,
+                  src/dequantize.rs:150-167): i8 / e4m3 / e5m2 bytes and e2m1 nibble
+                  pairs for f32/bf16/f16 inputs: every integer quotient of the value
+                  range and every half-integer in between, signed zeros, random data
+                  with abs-max scales per tensor and per block, f16/bf16 parameters.
 """
 from __future__ import annotations
 
@@ -40,15 +45,16 @@ def contiguous_strides(shape):
 
 
 def run_case(store, name, x_bits, fmt, shape, block, value, param_fmt, scale_bits=None,
-             scale_strides=None):
+             scale_strides=None, native=False):
     if scale_bits is None:
         scale_bits = em.scales_from_absmax(x_bits, fmt, shape, block, value)
     if scale_strides is None:
         scale_strides = (0,) * len(shape) if block is None else contiguous_strides(
             tuple(s // b for s, b in zip(shape, (1,) * (len(shape) - len(block)) + tuple(block))))
-    words, out_scale = em.quantize_tensor(x_bits, fmt, shape, scale_bits, scale_strides, block,
-                                          value, param_fmt)
-    deq = em.dequantize_tensor(words, fmt, shape, out_scale, scale_strides, block, value, param_fmt)
+    quantize, dequantize = ((em.quantize_tensor_native, em.dequantize_tensor_native) if native
+                            else (em.quantize_tensor, em.dequantize_tensor))
+    words, out_scale = quantize(x_bits, fmt, shape, scale_bits, scale_strides, block, value, param_fmt)
+    deq = dequantize(words, fmt, shape, out_scale, scale_strides, block, value, param_fmt)
     store[f"{name}/x"] = x_bits.reshape(-1)
     store[f"{name}/scale"] = scale_bits.reshape(-1)
     store[f"{name}/words"] = words
@@ -57,7 +63,7 @@ def run_case(store, name, x_bits, fmt, shape, block, value, param_fmt, scale_bit
     store[f"{name}/meta"] = np.array(
         [fmt, value, param_fmt, ",".join(map(str, shape)),
          "" if block is None else ",".join(map(str, block)),
-         ",".join(map(str, scale_strides))])
+         ",".join(map(str, scale_strides))] + (["native"] if native else []))
 
 
 def reference_ramps():
@@ -143,11 +149,77 @@ def typed_small():
             buf[r * 1 + c * 8] = sc_contig[r, c]
     run_case(store, "strided_bf16_Q8S", xb, "bf16", (8, 64), (32,), "Q8S", "f32", scale_bits=buf,
              scale_strides=(1, 8))
+    # negative scales (only a caller's own scales can be): the quotient changes sign, a zero code
+    # dequantizes to -0
+    for fmt in ("f32", "bf16", "f16"):
+        vals = [(Fraction(k) + h) * Fraction(-3, 8) for k in range(-9, 9) for h in (0, Fraction(1, 2))]
+        while len(vals) % 64:
+            vals.append(Fraction(0))
+        run_case(store, f"negscale_{fmt}_Q4S", to_fmt_bits(vals, fmt), fmt, (len(vals) // 64, 64), None, "Q4S", "f32",
+                 scale_bits=to_fmt_bits([Fraction(-3, 8)], fmt))
+        x = to_fmt_bits(gauss(2 * 64, 1.0), fmt)
+        neg = em.scales_from_absmax(x, fmt, (2, 64), (32,), "Q8S") | (1 << (31 if fmt == "f32" else 15))
+        run_case(store, f"negscale_{fmt}_Q8S_b32", x, fmt, (2, 64), (32,), "Q8S", "f32", scale_bits=neg)
     np.savez_compressed(os.path.join(HERE, "typed_small.npz"), **store)
+    return len(store) // 6
+
+
+def typed_native():
+    rng = np.random.default_rng(20250311)
+    store = {}
+
+    def gauss(n, sigma):
+        return [Fraction(float(v)) for v in rng.normal(0.0, sigma, n)]
+
+    def with_signed_zeros(bits, fmt, where):
+        """Turns the (zero) entries at ``where`` into -0."""
+        bits = bits.copy()
+        for i in where:
+            assert bits[i] == 0
+            bits[i] = 1 << (31 if fmt == "f32" else 15)
+        return bits
+
+    for fmt in ("f32", "bf16", "f16"):
+        for value in ("Q8S", "Q8F", "E4M3", "E5M2", "E2M1"):
+            lo, hi = em.RANGES[value]
+            if value == "E5M2":  # the range is too wide to walk: its ends, the small integers, powers of two
+                ks = list(range(-34, 35)) + [s * (2 ** p + o) for p in range(6, 16) for o in (-1, 0, 1) for s in (-1, 1)]
+                ks += list(range(57340, 57347)) + list(range(-57346, -57339))
+            else:
+                ks = list(range(lo - 2, hi + 3))
+            # integer and half-integer quotients under a power-of-two scale, +0 and -0, small negatives
+            vals = []
+            for k in ks:
+                vals += [Fraction(k), Fraction(k) + Fraction(1, 2)]
+            vals += [Fraction(-1, 4), Fraction(1, 4), Fraction(-3, 8), Fraction(-1, 2), Fraction(1, 2)]
+            zeros_at = list(range(len(vals), len(vals) + 4))
+            vals += [Fraction(0)] * 4
+            while len(vals) % 64:
+                vals.append(Fraction(0))
+            n = len(vals)
+            for tag, s in (("s0.25", Fraction(1, 4)), ("s-0.5", Fraction(-1, 2))):
+                x = with_signed_zeros(to_fmt_bits([v * s for v in vals], fmt), fmt, zeros_at[:2])
+                run_case(store, f"native_ties_{fmt}_{value}_{tag}", x, fmt, (n // 64, 64), None, value, "f32",
+                         scale_bits=to_fmt_bits([s], fmt), native=True)
+            # random data, scales from abs-max, per tensor and per block, other parameter types
+            x = to_fmt_bits(gauss(4 * 128, 0.02), fmt)
+            run_case(store, f"native_rand_{fmt}_{value}_tensor", x, fmt, (4, 128), None, value, "f32", native=True)
+            for param in ("f32", "f16", "bf16"):
+                if param != "f32" and value not in ("Q8S", "E4M3", "E2M1"):
+                    continue
+                x = to_fmt_bits(gauss(4 * 128, 0.02), fmt)
+                run_case(store, f"native_rand_{fmt}_{value}_b32_{param}", x, fmt, (4, 128), (32,), value, param,
+                         native=True)
+    # N-D blocks
+    x = to_fmt_bits(gauss(4 * 6 * 32, 0.5), "f32")
+    run_case(store, "native_nd_f32_E2M1_2x3x16", x, "f32", (4, 6, 32), (2, 3, 16), "E2M1", "f32", native=True)
+    run_case(store, "native_nd_f32_Q8S_3x8", x, "f32", (4, 6, 32), (3, 8), "Q8S", "f32", native=True)
+    np.savez_compressed(os.path.join(HERE, "typed_native.npz"), **store)
     return len(store) // 6
 
 
 if __name__ == "__main__":
     a = reference_ramps()
     b = typed_small()
-    print(f"wrote {a} reference ramp cases and {b} typed cases")
+    c = typed_native()
+    print(f"wrote {a} reference ramp cases, {b} typed cases and {c} native-store cases")

@@ -24,7 +24,7 @@ class GoldenCase:
     scale_strides: Tuple[int, ...]
     x: np.ndarray          # storage bits of the input (float32 view for f32)
     scale: np.ndarray      # scale buffer typed like the input
-    words: np.ndarray      # expected packed u32 words
+    words: np.ndarray      # expected packed u32 words (native store: bytes)
     out_scale: np.ndarray  # expected out_scale buffer (param dtype bits)
     deq: np.ndarray        # expected dequantized storage bits
 
@@ -40,17 +40,18 @@ def load(file: str):
     names = sorted({k.split("/")[0] for k in z.files})
     out = []
     for n in names:
-        fmt, value, param, shape, block, strides = [str(s) for s in z[f"{n}/meta"]]
+        fmt, value, param, shape, block, strides, *store = [str(s) for s in z[f"{n}/meta"]]
+        native = store == ["native"]
         shape = tuple(int(v) for v in shape.split(","))
         level = QuantLevel.Tensor if not block else QuantLevel.block([int(v) for v in block.split(",")])
         scheme = (QuantScheme.default().with_level(level).with_value(QuantValue[value])
-                  .with_store(QuantStore.U32).with_param(_PARAM[param]))
+                  .with_store(QuantStore.Native if native else QuantStore.U32).with_param(_PARAM[param]))
         elem = _ELEM[fmt]
         out.append(GoldenCase(
             name=n, elem=elem, scheme=scheme, shape=shape,
             scale_strides=tuple(int(v) for v in strides.split(",")),
             x=_as_storage(z[f"{n}/x"], elem), scale=_as_storage(z[f"{n}/scale"], elem),
-            words=z[f"{n}/words"].astype(np.uint32),
+            words=z[f"{n}/words"].astype(np.uint8 if native else np.uint32),
             out_scale=_as_storage(z[f"{n}/out_scale"], _ELEM[param]),
             deq=_as_storage(z[f"{n}/deq"], elem)))
     return out

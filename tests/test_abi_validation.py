@@ -81,6 +81,43 @@ def test_native_store_and_scheme_checks():
         == _ffi.ERR_INVALID_ARGUMENT
 
 
+def test_block_divisibility_is_asserted_where_the_reference_asserts_it():
+    """check_block_size_compat (src/lib.rs:20-33) guards the reference's quantize launchers only
+    (src/quantize.rs:260,305); its dequantize launchers take any block size.  Without a GPU an accepted
+    call goes on to its launch and fails there, with a HIP error."""
+    x, out = t((8, 64), 4), t((8, 16), 4)
+    b2 = Q8_B32.with_level(QuantLevel.block([2]))
+    sc = t((8, 32), 4)
+    assert status(lambda: qz.launch_ref(CLIENT, x, out, sc, sc, b2, ElemType.F32)) == _ffi.ERR_BLOCK_NOT_DIVISIBLE
+    assert status(lambda: qz.launch_dynamic(CLIENT, x, out, sc, b2, ElemType.F32)) == _ffi.ERR_BLOCK_NOT_DIVISIBLE
+    passed_validation = (_ffi.OK, _ffi.ERR_HIP)
+
+    def outcome(fn):
+        try:
+            fn()
+            return _ffi.OK
+        except _ffi.QuantError as e:
+            return e.status
+
+    assert outcome(lambda: dq.launch_ref(CLIENT, out, x, sc, b2, ElemType.F32)) in passed_validation
+    assert outcome(lambda: qz.compute_scales(CLIENT, x, sc, b2, ElemType.F32)) in passed_validation
+    # native store: the divisor is the line size the reference picks for the input tensor: at most 16 bytes,
+    # dividing the last dimension and the smallest stride above 1; 1 when the last dimension is strided
+    i8 = QuantScheme.default().with_value(QuantValue.Q8S).with_store(QuantStore.Native)
+    n2 = i8.with_level(QuantLevel.block([2]))
+    bytes_out = t((8, 64), 1)
+    assert status(lambda: qz.launch_ref(CLIENT, x, bytes_out, sc, sc, n2, ElemType.F32)) == _ffi.ERR_BLOCK_NOT_DIVISIBLE
+    x_odd_pitch = t((8, 64), 4, (66, 1))   # rows 66 elements apart: line size 2
+    assert outcome(lambda: qz.launch_ref(CLIENT, x_odd_pitch, bytes_out, sc, sc, n2, ElemType.F32)) in passed_validation
+    x_transposed = t((8, 64), 4, (1, 8))   # last dimension strided: line size 1
+    n1 = i8.with_level(QuantLevel.block([1]))
+    assert outcome(lambda: qz.launch_ref(CLIENT, x_transposed, bytes_out, t((8, 64), 4), t((8, 64), 4), n1,
+                                         ElemType.F32)) in passed_validation
+    assert status(lambda: qz.launch_ref(CLIENT, x, bytes_out, t((8, 64), 4), t((8, 64), 4), n1, ElemType.F32)) \
+        == _ffi.ERR_BLOCK_NOT_DIVISIBLE                                            # contiguous: line size 4
+    assert outcome(lambda: dq.launch_ref(CLIENT, bytes_out, x, sc, n2, ElemType.F32)) in passed_validation
+
+
 def test_per_tensor_dynamic_needs_its_workspace():
     scheme = QuantScheme.default().with_value(QuantValue.Q8S)
     x, out, one = t((8, 64), 4), t((8, 16), 4), t((1,), 4)

@@ -11,6 +11,7 @@ pytestmark = pytest.mark.gpu
 
 RAMPS = gc.load("ref_ramps.npz")
 TYPED = gc.load("typed_small.npz")
+NATIVE = gc.load("typed_native.npz")
 ALL_VALUES = list(QuantValue)
 INT_VALUES = [QuantValue.Q8F, QuantValue.Q8S, QuantValue.Q4F, QuantValue.Q4S, QuantValue.Q2F, QuantValue.Q2S]
 ELEMS = [ElemType.F32, ElemType.BF16, ElemType.F16]
@@ -49,7 +50,7 @@ def rand_input(rng, shape, elem, oracle, sigma=0.02, outliers=0.001):
 
 # ---------------------------------------------------------------- fixtures
 
-@pytest.mark.parametrize("case", RAMPS + TYPED, ids=lambda c: c.name)
+@pytest.mark.parametrize("case", RAMPS + TYPED + NATIVE, ids=lambda c: c.name)
 def test_golden_fixtures(gpu, case):
     sshape = (1,) if case.scheme.level.is_tensor else case.scheme.scales_shape(case.shape)
     strides = (1,) if case.scheme.level.is_tensor else case.scale_strides
@@ -321,6 +322,31 @@ def test_unaligned_base_pointers(gpu, oracle):
     torch.cuda.synchronize()
     assert np.array_equal(out_t.cpu().numpy().view(np.uint32), wt)
     assert os_t.cpu().numpy()[0] == ost.reshape(-1)[0] == sc_t.cpu().numpy()[0]
+
+
+@pytest.mark.parametrize("elem", ELEMS, ids=lambda e: e.name)
+def test_dequantize_blocks_that_split_a_word(gpu, oracle, elem):
+    """The reference's dequantize launchers take any block size (src/dequantize.rs:231-280 has no
+    check_block_size_compat).  A block smaller than a packed word then gives the whole word the scale of
+    the word's first element (src/dequantize.rs:70-76); native bytes take the scale of their own block."""
+    rng = np.random.default_rng(77 + int(elem))
+    shape = (6, 96)
+    for value, block, store in ((QuantValue.Q8S, [2], QuantStore.U32), (QuantValue.Q4S, [4], QuantStore.U32),
+                                (QuantValue.Q2F, [8], QuantStore.U32), (QuantValue.Q4F, [2, 12], QuantStore.U32),
+                                (QuantValue.Q8S, [3], QuantStore.Native), (QuantValue.E2M1, [1], QuantStore.Native),
+                                (QuantValue.E4M3, [2, 3], QuantStore.Native)):
+        scheme = QuantScheme.default().with_value(value).with_level(QuantLevel.block(block)).with_store(store)
+        n_stored = int(np.prod(scheme.packed_shape(shape)))
+        if store == QuantStore.U32:
+            stored = rng.integers(0, 2**32, n_stored, dtype=np.uint64).astype(np.uint32)
+        else:
+            stored = rng.integers(0, 256, n_stored, dtype=np.uint64).astype(np.uint8)
+            if value == QuantValue.E4M3:
+                stored[(stored & 0x7F) == 0x7F] = 0x3A  # no NaN codes
+        scales = rng.uniform(0.01, 2.0, scheme.scales_shape(shape)).astype(np.float32)
+        got = gpu.dequantize(stored, shape, scales, elem, scheme)
+        want = oracle.dequantize(stored, shape, scales, elem, scheme)
+        assert same_floats(got, want, elem), (value.name, block, store.name)
 
 
 # ---------------------------------------------------------------- native store

@@ -14,9 +14,10 @@ from cubek_amd.scheme import (ElemType, QuantLevel, QuantParam, QuantScheme, Qua
 
 RAMPS = gc.load("ref_ramps.npz")
 TYPED = gc.load("typed_small.npz")
+NATIVE = gc.load("typed_native.npz")
 
 
-@pytest.mark.parametrize("case", RAMPS + TYPED, ids=lambda c: c.name)
+@pytest.mark.parametrize("case", RAMPS + TYPED + NATIVE, ids=lambda c: c.name)
 def test_oracle_matches_exact_model(oracle, case):
     words, out_scale = oracle.quantize(case.x, case.elem, case.shape, case.scale, case.scheme,
                                        scale_strides=case.scale_strides)
@@ -233,3 +234,86 @@ def test_native_fp8_store_matches_torch_composition(oracle):
             y = oracle.dequantize(codes, shape, out_scale, ElemType.F32, scheme)
             y_want = (torch.from_numpy(want).view(tdt).to(torch.float32) * torch.from_numpy(s_full)).numpy()
             assert np.array_equal(y.reshape(shape), y_want), value.name
+
+
+# ---------------------------------------------------------------- native store pins
+
+def _native(value, block=None, param=QuantParam.F32):
+    level = QuantLevel.Tensor if block is None else QuantLevel.block(block)
+    return QuantScheme.default().with_value(value).with_store(QuantStore.Native).with_level(level).with_param(param)
+
+
+def test_native_e2m1_known_answer_bytes(oracle):
+    """Hand-written: scale 1, quotients are the inputs.  e2m1 codes by the OCP FP4 table
+    {0: 0, 0.5: 1, 1: 2, 1.5: 3, 2: 4, 3: 5, 4: 6, 6: 7}, sign in bit 3; the quantizer rounds to an
+    integer first (src/quantize.rs:26-30), so 0.5 -> 0 and 1.5 -> 2 (ties to even), 2.5 -> 2, 5 -> tie
+    between 4 and 6 -> the even code, 4; 7 clamps to 6.  Element 2k sits in the LOW nibble of byte k."""
+    x = np.array([0, 1, 2, 3, 4, 5, 6, 7,
+                  -1, -2, -3, -4, -5, -6, -7, 0.5,
+                  1.5, 2.5, 3.5, 4.5, 5.5, -0.5, -1.5, -0.25], np.float32).reshape(1, 24)
+    want_nibbles = [0x0, 0x2, 0x4, 0x5, 0x6, 0x6, 0x7, 0x7,
+                    0xA, 0xC, 0xD, 0xE, 0xE, 0xF, 0xF, 0x0,
+                    0x4, 0x4, 0x6, 0x6, 0x7, 0x8, 0xC, 0x8]   # 3.5 -> 4, 4.5 -> 4, 5.5 -> 6; -0.5, -0.25 -> -0
+    want_bytes = [lo | (hi << 4) for lo, hi in zip(want_nibbles[0::2], want_nibbles[1::2])]
+    codes, out_scale = oracle.quantize(x, ElemType.F32, (1, 24), np.array([1.0], np.float32), _native(QuantValue.E2M1))
+    assert codes.reshape(-1).tolist() == want_bytes
+    assert want_bytes[:4] == [0x20, 0x54, 0x66, 0x77]  # spelled out: element 0 low, element 1 high
+    y = oracle.dequantize(codes, (1, 24), np.array([0.5], np.float32), ElemType.F32, _native(QuantValue.E2M1))
+    mags = {0x0: 0.0, 0x2: 1.0, 0x4: 2.0, 0x5: 3.0, 0x6: 4.0, 0x7: 6.0}
+    want_y = [(-0.5 if n & 8 else 0.5) * mags[n & 7] for n in want_nibbles]
+    assert y.reshape(-1).tolist() == want_y
+    assert np.signbit(y.reshape(-1)).tolist() == [bool(n & 8) for n in want_nibbles]  # -0 survives
+
+
+def test_native_i8_known_answer_bytes(oracle):
+    """Every code of the i8 store: x = k * 0.5 with scale 0.5 gives quotient k; the stored byte is k in
+    two's complement (Q8S clamps -128 to -127, Q8F keeps it); dequantize returns scale * k."""
+    ks = np.arange(-130, 131)
+    x = np.zeros(264, np.float32)
+    x[:ks.size] = ks * 0.5
+    for value, lo in ((QuantValue.Q8S, -127), (QuantValue.Q8F, -128)):
+        codes, _ = oracle.quantize(x.reshape(1, -1), ElemType.F32, (1, 264), np.array([0.5], np.float32), _native(value))
+        want = np.clip(ks, lo, 127)
+        assert codes.reshape(-1)[:ks.size].tolist() == [int(k) & 0xFF for k in want]
+        assert not codes.reshape(-1)[ks.size:].any()
+        y = oracle.dequantize(codes, (1, 264), np.array([0.5], np.float32), ElemType.F32, _native(value))
+        assert y.reshape(-1)[:ks.size].tolist() == (want * 0.5).tolist()
+
+
+@pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
+def test_native_store_agrees_with_packed_store(oracle, elem):
+    """The two stores of one scheme hold the same codes in different containers, which ties the native
+    arms to the packed path that the exact-rational fixtures pin: native i8 byte e is field e % 4 of
+    packed word e / 4; a native e2m1 nibble decodes to the integer the packed E2M1 path stores, rounded
+    to the e2m1 grid (5 -> 4, the only integer of [-6, 6] off the grid); dequantized values agree wherever
+    the packed integer is on the grid."""
+    rng = np.random.default_rng(31)
+    shape = (8, 128)
+    x = rng.uniform(-0.1, 0.1, shape).astype(np.float32)  # quotients spread over the whole value range
+    xb = oracle.to_bits(x, elem)
+    for value in (QuantValue.Q8S, QuantValue.Q8F, QuantValue.E2M1):
+        for block in (None, [32], [2, 16]):
+            level = QuantLevel.Tensor if block is None else QuantLevel.block(block)
+            packed = QuantScheme.default().with_value(value).with_level(level)
+            s = oracle.compute_scales(xb, elem, shape, packed)
+            words, os_p = oracle.quantize(xb, elem, shape, s, packed)
+            codes, os_n = oracle.quantize(xb, elem, shape, s, _native(value, block))
+            assert gc.bits_equal(os_p, os_n)
+            bits = value.size_bits()
+            fields = (words.reshape(-1, 1) >> (bits * np.arange(32 // bits, dtype=np.uint32))) & ((1 << bits) - 1)
+            ints = fields.reshape(-1).astype(np.int64)
+            ints = np.where(ints >= 1 << (bits - 1), ints - (1 << bits), ints)
+            yp = oracle.from_bits(oracle.dequantize(words, shape, os_p, elem, packed), elem).reshape(-1)
+            yn = oracle.from_bits(oracle.dequantize(codes, shape, os_n, elem, _native(value, block)), elem).reshape(-1)
+            if bits == 8:
+                assert np.array_equal(codes.reshape(-1), fields.reshape(-1).astype(np.uint8))
+                assert np.array_equal(yp, yn)
+            else:
+                nib = np.stack([codes.reshape(-1) & 0xF, codes.reshape(-1) >> 4], axis=1).reshape(-1)
+                grid = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+                decoded = np.where(nib & 8, -1.0, 1.0) * grid[nib & 7]
+                want = np.where(np.abs(ints) == 5, np.sign(ints) * 4, ints)
+                assert np.array_equal(np.abs(decoded), np.abs(want)) and np.array_equal(decoded[want != 0], want[want != 0])
+                assert set(np.unique(np.abs(ints))) >= {0, 1, 2, 3, 4, 5, 6}  # the data reach every integer
+                on_grid = np.abs(ints) != 5
+                assert np.array_equal(yp[on_grid], yn[on_grid])
