@@ -6,8 +6,13 @@
 //   dequantize_symmetric                  crates/cubek-quant/src/dequantize.rs:20-25
 //   dequantize_symmetric_packed_value(s), dequantize_symmetric_packed_value_at   src/dequantize.rs:27-79
 //   unpack_q                              src/dequantize.rs:81-118
+//   the native-store line of dequantize_symmetric_native_kernel                  src/dequantize.rs:150-167
 //   ScalesLayout::{to_source_pos, is_block_start}, scales_layout   src/layout/scales.rs:15-247
-// Results are bit-identical to cq_dequantize for the same inputs.
+//   GlobalScaleLayout (scale of a (batch, row, col) coordinate)
+//                                         crates/cubek-matmul/src/components/global/memory/layout.rs:371-455
+// Like the reference's functions they are generic over the float type kF the arithmetic is
+// carried out in and over the storage type FS of the scales (float, _Float16, __bf16).
+// Results are bit-identical to cq_dequantize for the same inputs: y = kF(kF(scale) * kF(code)).
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -19,21 +24,68 @@ namespace device {
 // Float type the arithmetic is carried out in (the tensor's type in the reference).
 enum class Float { F32, F16, BF16 };
 
+// How the native store holds one value (QuantStore::Native; the U32 store always holds
+// two's-complement fields, whatever the value type).
+enum class Native { I8, E4M3, E5M2, E2M1x2 };
+
+// ---- scale parameters --------------------------------------------------------------------
+
+// A stored scale widened to f32 (exact for every storage type).
+__host__ __device__ inline float widen(float s) { return s; }
+__device__ __forceinline__ float widen(_Float16 s) { return static_cast<float>(s); }
+__device__ __forceinline__ float widen(__bf16 s) { return static_cast<float>(s); }
+
+// ---- division by launch-invariant divisors -------------------------------------------------
+
+// n / d and n % d for n < 2^31 as one 32 x 32 -> 64 bit multiplication and a shift (the
+// reference's FastDivmod, src/layout/scales.rs:112,153).  With s = ceil(log2 d) and
+// magic = floor(2^(31+s) / d) + 1 (which fits 32 bits): n / d == (n * magic) >> (31 + s).
+struct FastDivmod {
+    uint32_t divisor = 1, magic = 0x80000001u, shift = 31;  // default: division by 1
+    FastDivmod() = default;
+    __host__ __device__ explicit FastDivmod(uint32_t d) : divisor(d) {
+        uint32_t s = 0;
+        while ((1ull << s) < d) s++;
+        magic = static_cast<uint32_t>((1ull << (31 + s)) / d + 1);
+        shift = 31 + s;
+    }
+    __host__ __device__ uint32_t div(uint32_t n) const {
+        return static_cast<uint32_t>((static_cast<uint64_t>(n) * magic) >> shift);
+    }
+    __host__ __device__ void div_mod(uint32_t n, uint32_t* quotient, uint32_t* remainder) const {
+        *quotient = div(n);
+        *remainder = n - *quotient * divisor;
+    }
+};
+
+// ---- scale addressing ------------------------------------------------------------------
+
 // Element index -> scale index, per tensor (rank == 0) or N-D block scaled.
-// Plain data: fill it on the host, pass it by value to a kernel.
+// Plain data: build it on the host with scales_layout(), pass it by value to a kernel.
 struct ScalesLayout {
     uint32_t rank = 0;        // 0: one scale for the whole tensor
-    uint32_t shape[8] = {};   // unpacked (element) shape
-    uint32_t block[8] = {};   // block extents, left-padded with 1
+    FastDivmod shape[8];      // unpacked (element) shape
+    FastDivmod block[8];      // block extents, left-padded with 1
     uint64_t strides[8] = {}; // strides of the scales tensor, in elements
 
-    // ScalesLayout::to_source_pos
+    // ScalesLayout::to_source_pos.  Positions below 2^31 (the reference's positions are u32) take
+    // the multiply-and-shift divisions, larger ones plain 64-bit arithmetic.
     __host__ __device__ uint64_t to_source_pos(uint64_t pos) const {
-        uint64_t offs = pos, scale_offs = 0;
-        for (int d = static_cast<int>(rank) - 1; d >= 0; d--) {
-            const uint32_t local = static_cast<uint32_t>(offs % shape[d]);
-            offs /= shape[d];
-            scale_offs += static_cast<uint64_t>(local / block[d]) * strides[d];
+        uint64_t scale_offs = 0;
+        if (pos < (1ull << 31)) {
+            uint32_t offs = static_cast<uint32_t>(pos);
+            for (int d = static_cast<int>(rank) - 1; d >= 0; d--) {
+                uint32_t local;
+                shape[d].div_mod(offs, &offs, &local);
+                scale_offs += static_cast<uint64_t>(block[d].div(local)) * strides[d];
+            }
+        } else {
+            uint64_t offs = pos;
+            for (int d = static_cast<int>(rank) - 1; d >= 0; d--) {
+                const uint32_t local = static_cast<uint32_t>(offs % shape[d].divisor);
+                offs /= shape[d].divisor;
+                scale_offs += static_cast<uint64_t>(local / block[d].divisor) * strides[d];
+            }
         }
         return scale_offs;
     }
@@ -43,9 +95,9 @@ struct ScalesLayout {
         uint64_t offs = pos;
         bool start = true;
         for (int d = static_cast<int>(rank) - 1; d >= 0; d--) {
-            const uint32_t local = static_cast<uint32_t>(offs % shape[d]);
-            offs /= shape[d];
-            start = start && (local % block[d] == 0);
+            const uint32_t local = static_cast<uint32_t>(offs % shape[d].divisor);
+            offs /= shape[d].divisor;
+            start = start && (local % block[d].divisor == 0);
         }
         return start;
     }
@@ -64,12 +116,30 @@ inline ScalesLayout scales_layout(const uint64_t* values_shape, uint32_t rank, u
     if (block_rank == 0) return l;  // per tensor
     l.rank = rank;
     for (uint32_t d = 0; d < rank; d++) {
-        l.shape[d] = static_cast<uint32_t>(d + 1 == rank ? values_shape[d] * num_quants : values_shape[d]);
-        l.block[d] = d + block_rank < rank ? 1u : block[d + block_rank - rank];
+        l.shape[d] = FastDivmod(static_cast<uint32_t>(d + 1 == rank ? values_shape[d] * num_quants : values_shape[d]));
+        l.block[d] = FastDivmod(d + block_rank < rank ? 1u : block[d + block_rank - rank]);
         l.strides[d] = scales_strides[d];
     }
     return l;
 }
+
+// The scale of element (batch, row, col) of a quantized matrix operand: GlobalScaleLayout of the
+// reference's matmul, whose block size is a compile-time pair as well.  kBlockRows == 0: one scale
+// per tensor.  Dividing by the template constants compiles to shifts (powers of two) or a
+// multiplication: a kernel that walks rows and columns never divides.
+template <uint32_t kBlockRows, uint32_t kBlockCols>
+struct GlobalScaleLayout {
+    uint32_t stride_batch = 0, stride_row = 0, stride_col = 0;  // strides of the scales tensor, in elements
+    __host__ __device__ uint32_t to_source_pos(uint32_t batch, uint32_t row, uint32_t col) const {
+        if constexpr (kBlockRows == 0) {
+            return 0;
+        } else {
+            return batch * stride_batch + (row / kBlockRows) * stride_row + (col / kBlockCols) * stride_col;
+        }
+    }
+};
+
+// ---- rounding --------------------------------------------------------------------------
 
 // Round an f32 value to `kF` (round-to-nearest-even), widened back to f32.
 template <Float kF>
@@ -86,6 +156,23 @@ __device__ __forceinline__ float round_to(float v) {
     }
 }
 
+// Two values of a 16-bit kF as they sit in memory (the first in the low half).
+template <Float kF>
+__device__ __forceinline__ uint32_t pack_pair(float a, float b) {
+    static_assert(kF != Float::F32, "pairs are for the 16-bit types");
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    f32x2 v = {a, b};
+    if constexpr (kF == Float::BF16) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32
+    } else {
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));   // v_cvt_pk_f16_f32, keeps -0
+    }
+}
+
+// ---- packed (U32) store ----------------------------------------------------------------
+
 // unpack_q: the 32/kBits two's-complement fields of a word, element 0 in the low bits.
 template <int kBits>
 __device__ __forceinline__ void unpack_q(uint32_t word, float* out) {
@@ -98,39 +185,184 @@ __device__ __forceinline__ void unpack_q(uint32_t word, float* out) {
 }
 
 // dequantize_symmetric: x = F(scale) * x_q, computed in kF.
-template <Float kF>
-__device__ __forceinline__ float dequantize_symmetric(float value, float scale) {
-    return round_to<kF>(round_to<kF>(scale) * value);
+template <Float kF, class FS>
+__device__ __forceinline__ float dequantize_symmetric(float value, FS scale) {
+    return round_to<kF>(round_to<kF>(widen(scale)) * value);
 }
 
 // dequantize_symmetric_packed_value: one stored word -> 32/kBits values of type kF
 // (returned widened to f32; they are exactly representable in kF).
-template <Float kF, int kBits>
-__device__ __forceinline__ void dequantize_symmetric_packed_value(uint32_t word, float scale, float* out) {
+template <Float kF, int kBits, class FS>
+__device__ __forceinline__ void dequantize_symmetric_packed_value(uint32_t word, FS scale, float* out) {
     float q[32 / kBits];
     unpack_q<kBits>(word, q);
-    const float s = round_to<kF>(scale);
+    const float s = round_to<kF>(widen(scale));
 #pragma unroll
     for (int i = 0; i < 32 / kBits; i++) out[i] = round_to<kF>(s * q[i]);
 }
 
+// The same values, for a 16-bit kF, as 16/kBits packed pairs ready to be stored or fed to a
+// dot-product / matrix instruction: out[i] holds values 2i (low half) and 2i+1 (high half).
+// Bit-identical to dequantize_symmetric_packed_value, in about half the instructions:
+//   - the fields are biased to unsigned digits (one XOR per word) and separated by masks into
+//     the four bytes of a register, where v_cvt_f32_ubyteN turns each into a float;
+//   - one FMA per value removes the bias and applies the scale: digit * s - bias * s is the
+//     exact product s * code (at most 11 + 8 significant bits), so the single rounding of
+//     pack_pair is the reference's rounding of F(scale) * F(code);
+//   - f16 goes through packed f16 arithmetic instead: the digit is planted in the mantissa of
+//     1024 + digit, v_pk_add_f16 removes 1024 + bias exactly and v_pk_mul_f16 multiplies and
+//     rounds two values at a time.
+// Scales that are negative, NaN, zero, or outside [2^-100, 2^100) take the plain path: there
+// bias * s could overflow, and a zero code has to come out as s * (+0) with the scale's sign.
+template <Float kF, int kBits, class FS>
+__device__ __forceinline__ void dequantize_symmetric_packed_value_pairs(uint32_t word, FS scale, uint32_t* out) {
+    static_assert(kF != Float::F32, "pairs are for the 16-bit types");
+    static_assert(kBits == 2 || kBits == 4 || kBits == 8, "2, 4 or 8 bits per value");
+    constexpr int kN = 32 / kBits;
+    constexpr uint32_t kBias = 1u << (kBits - 1);
+    const float s = round_to<kF>(widen(scale));
+    // sign clear and exponent field in [27, 227)
+    const bool tame = (__builtin_bit_cast(uint32_t, s) - 0x0d800000u) < (0x71800000u - 0x0d800000u);
+    if (!tame) {
+        float v[kN];
+        dequantize_symmetric_packed_value<kF, kBits>(word, scale, v);
+#pragma unroll
+        for (int i = 0; i < kN / 2; i++) out[i] = pack_pair<kF>(v[2 * i], v[2 * i + 1]);
+        return;
+    }
+    constexpr uint32_t kBiasWord = kBits == 8 ? 0x80808080u : (kBits == 4 ? 0x88888888u : 0xAAAAAAAAu);
+    const uint32_t digits = word ^ kBiasWord;  // field + bias, unsigned
+    if constexpr (kF == Float::F16) {
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        const _Float16 sh = static_cast<_Float16>(s);
+        const f16x2 s2 = {sh, sh};
+        const _Float16 off = static_cast<_Float16>(-(1024.0f + static_cast<float>(kBias)));
+        const f16x2 off2 = {off, off};
+        constexpr uint32_t kDigit = (1u << kBits) - 1u;
+#pragma unroll
+        for (int i = 0; i < kN / 2; i++) {
+            // values 2i and 2i+1: their digits into the low mantissa bits of two halves holding 1024.0
+            const uint32_t lo = (digits >> (2 * i * kBits)) & kDigit;
+            const uint32_t hi = (digits >> ((2 * i + 1) * kBits)) & kDigit;
+            const uint32_t planted = 0x64006400u | lo | (hi << 16);
+            const f16x2 code = __builtin_bit_cast(f16x2, planted) + off2;  // exact
+            out[i] = __builtin_bit_cast(uint32_t, s2 * code);              // v_pk_mul_f16, one rounding
+        }
+    } else {
+        const float nbs = -static_cast<float>(kBias) * s;  // exact
+        if constexpr (kBits == 8) {
+            // bytes are digits already
+            const float v0 = __builtin_fmaf(static_cast<float>(digits & 0xffu), s, nbs);
+            const float v1 = __builtin_fmaf(static_cast<float>((digits >> 8) & 0xffu), s, nbs);
+            const float v2 = __builtin_fmaf(static_cast<float>((digits >> 16) & 0xffu), s, nbs);
+            const float v3 = __builtin_fmaf(static_cast<float>(digits >> 24), s, nbs);
+            out[0] = pack_pair<kF>(v0, v1);
+            out[1] = pack_pair<kF>(v2, v3);
+        } else if constexpr (kBits == 4) {
+            // even fields in the low nibble of each byte; odd fields stay in the high nibble: the byte
+            // reads 16 * digit, which s / 16 takes back (exact)
+            const uint32_t even = digits & 0x0f0f0f0fu, odd = digits & 0xf0f0f0f0u;
+            const float s16 = s * 0.0625f;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const float ve = __builtin_fmaf(static_cast<float>((even >> (8 * b)) & 0xffu), s, nbs);
+                const float vo = __builtin_fmaf(static_cast<float>((odd >> (8 * b)) & 0xffu), s16, nbs);
+                out[b] = pack_pair<kF>(ve, vo);
+            }
+        } else {
+            // field j of every byte, j = 0..3: byte b of (digits >> 2j) & 0x03030303 is value 4b + j
+            uint32_t plane[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) plane[j] = (digits >> (2 * j)) & 0x03030303u;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const float v0 = __builtin_fmaf(static_cast<float>((plane[0] >> (8 * b)) & 0xffu), s, nbs);
+                const float v1 = __builtin_fmaf(static_cast<float>((plane[1] >> (8 * b)) & 0xffu), s, nbs);
+                const float v2 = __builtin_fmaf(static_cast<float>((plane[2] >> (8 * b)) & 0xffu), s, nbs);
+                const float v3 = __builtin_fmaf(static_cast<float>((plane[3] >> (8 * b)) & 0xffu), s, nbs);
+                out[2 * b] = pack_pair<kF>(v0, v1);
+                out[2 * b + 1] = pack_pair<kF>(v2, v3);
+            }
+        }
+    }
+}
+
 // dequantize_symmetric_packed_value_at: a word the caller already holds (`position` is its
-// index in the packed tensor), its scale looked up through the layout (`scales` holds f32
-// parameters): the scale of the word's first element, as the reference indexes its scales view.
-template <Float kF, int kBits>
+// index in the packed tensor), its scale looked up through the layout: the scale of the word's
+// first element, as the reference indexes its scales view.
+template <Float kF, int kBits, class FS>
 __device__ __forceinline__ void dequantize_symmetric_packed_value_at(uint64_t position, uint32_t word,
-                                                                     const float* scales, const ScalesLayout& layout,
+                                                                     const FS* scales, const ScalesLayout& layout,
                                                                      float* out) {
     const uint64_t elem = position * (32 / kBits);
     dequantize_symmetric_packed_value<kF, kBits>(word, scales[layout.to_source_pos(elem)], out);
 }
 
 // dequantize_symmetric_packed_values: word `position` of a packed tensor.
-template <Float kF, int kBits>
+template <Float kF, int kBits, class FS>
 __device__ __forceinline__ void dequantize_symmetric_packed_values(uint64_t position, const uint32_t* values,
-                                                                   const float* scales, const ScalesLayout& layout,
+                                                                   const FS* scales, const ScalesLayout& layout,
                                                                    float* out) {
     dequantize_symmetric_packed_value_at<kF, kBits>(position, values[position], scales, layout, out);
+}
+
+// ---- native store ----------------------------------------------------------------------
+
+// Values per 32 bits of a native tensor.
+template <Native kNative>
+constexpr int native_values_per_word() {
+    return kNative == Native::E2M1x2 ? 8 : 4;
+}
+
+// The values held by 32 bits of a native tensor, element 0 in the low bits: four i8 / e4m3 /
+// e5m2 bytes, or eight e2m1 nibbles (element 2k in the low nibble of byte k).  The conversions
+// are gfx950 instructions; every stored value is exact in f32.
+template <Native kNative>
+__device__ __forceinline__ void decode_native(uint32_t word, float* out) {
+    if constexpr (kNative == Native::I8) {
+        unpack_q<8>(word, out);
+    } else if constexpr (kNative == Native::E4M3) {
+        out[0] = __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(word), 0);
+        out[1] = __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(word), 1);
+        out[2] = __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(word), 2);
+        out[3] = __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(word), 3);
+    } else if constexpr (kNative == Native::E5M2) {
+        out[0] = __builtin_amdgcn_cvt_f32_bf8(static_cast<int>(word), 0);
+        out[1] = __builtin_amdgcn_cvt_f32_bf8(static_cast<int>(word), 1);
+        out[2] = __builtin_amdgcn_cvt_f32_bf8(static_cast<int>(word), 2);
+        out[3] = __builtin_amdgcn_cvt_f32_bf8(static_cast<int>(word), 3);
+    } else {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        const f32x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0);
+        const f32x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1);
+        const f32x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2);
+        const f32x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3);
+        out[0] = p0[0], out[1] = p0[1], out[2] = p1[0], out[3] = p1[1];
+        out[4] = p2[0], out[5] = p2[1], out[6] = p3[0], out[7] = p3[1];
+    }
+}
+
+// One line of the native dequantize kernel (src/dequantize.rs:150-167): the values of 32 bits of
+// a native tensor times one scale, F(scale) * F(q).
+template <Float kF, Native kNative, class FS>
+__device__ __forceinline__ void dequantize_symmetric_native_value(uint32_t word, FS scale, float* out) {
+    constexpr int kN = native_values_per_word<kNative>();
+    float q[kN];
+    decode_native<kNative>(word, q);
+    const float s = round_to<kF>(widen(scale));
+#pragma unroll
+    for (int i = 0; i < kN; i++) out[i] = round_to<kF>(s * q[i]);  // F(q) is exact: every stored value fits kF
+}
+
+// 32 bits of a native tensor at `position` (in units of 32 bits), scaled by the scale of their first
+// element, as the reference's kernel scales a line (the last block extent must be a multiple of the
+// values per 32 bits).
+template <Float kF, Native kNative, class FS>
+__device__ __forceinline__ void dequantize_symmetric_native_values(uint64_t position, const uint32_t* values,
+                                                                   const FS* scales, const ScalesLayout& layout,
+                                                                   float* out) {
+    const uint64_t elem = position * native_values_per_word<kNative>();
+    dequantize_symmetric_native_value<kF, kNative>(values[position], scales[layout.to_source_pos(elem)], out);
 }
 
 }  // namespace device

@@ -17,13 +17,3 @@ def test_reference_suite_through_cpp_host_layer():
     lines = [l for l in proc.stdout.splitlines() if l.startswith(("PASS", "FAIL"))]
     assert proc.returncode == 0, proc.stdout
     assert len([l for l in lines if l.startswith("PASS")]) == 24 + 4 + 2 and not [l for l in lines if l.startswith("FAIL")]
-
-
-def test_device_header_consumer_kernels():
-    """Dequantize-on-read and a fused GEMV built on include/cubek_quant_device.hpp."""
-    binary = os.path.join(os.path.dirname(BINARY), "test_device_header")
-    assert os.path.exists(binary), "tests/cpp/test_device_header is not built (make -C cubek_amd/csrc)"
-    proc = subprocess.run([binary], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
-    print(proc.stdout)
-    assert proc.returncode == 0, proc.stdout
-    assert proc.stdout.count("PASS") == 10 and "FAIL" not in proc.stdout
