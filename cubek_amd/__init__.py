@@ -7,16 +7,17 @@ crate, rebuilt for MI355X (gfx950): hand-written HIP kernels behind a C ABI
     cubek_amd.dequantize  launch_ref
     cubek_amd.reduce      max_abs (abs-max along an axis, the step in front of quantize)
     cubek_amd.contiguous  into_contiguous_packed_ref (strided quantized tensor -> contiguous)
+    cubek_amd.matvec      launch_ref (y = dequantize(W) @ x straight from the packed weights)
 
 Importing the package does not load the native library; the first call does and
 raises if it has not been built.
 """
-from . import contiguous, dequantize, quantize, reduce, scheme  # noqa: F401
+from . import contiguous, dequantize, matvec, quantize, reduce, scheme  # noqa: F401
 from ._ffi import QuantError  # noqa: F401
 from .scheme import (BlockSize, ElemType, QuantLevel, QuantMode, QuantParam, QuantScheme,  # noqa: F401
                      QuantStore, QuantValue)
 from .tensor import ComputeClient, TensorHandleRef  # noqa: F401
 
-__all__ = ["quantize", "dequantize", "reduce", "contiguous", "scheme", "QuantError", "BlockSize", "ElemType", "QuantLevel",
+__all__ = ["quantize", "dequantize", "reduce", "contiguous", "matvec", "scheme", "QuantError", "BlockSize", "ElemType", "QuantLevel",
            "QuantMode", "QuantParam", "QuantScheme", "QuantStore", "QuantValue", "ComputeClient",
            "TensorHandleRef"]

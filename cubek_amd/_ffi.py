@@ -21,6 +21,7 @@ EXPORTED_SYMBOLS = (
     "cq_compute_scales", "cq_quantize_dynamic", "cq_workspace_bytes", "cq_strerror",
     "cq_last_hip_error", "cq_abi_version", "cq_reduce_max_abs", "cq_reduce_workspace_bytes",
     "cq_into_contiguous_packed", "cq_quantize_dynamic_static",
+    "cq_gemv_quantized",
 )
 
 
@@ -87,6 +88,8 @@ def lib() -> ctypes.CDLL:
     L.cq_quantize_dynamic.argtypes = [ctypes.c_void_p, tp, tp, tp, sp, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
     L.cq_quantize_dynamic_static.restype = ctypes.c_int
     L.cq_quantize_dynamic_static.argtypes = [ctypes.c_void_p, tp, tp, tp, sp, ctypes.c_int]
+    L.cq_gemv_quantized.restype = ctypes.c_int
+    L.cq_gemv_quantized.argtypes = [ctypes.c_void_p, tp, tp, sp, tp, tp, ctypes.c_int, ctypes.c_int]
     L.cq_reduce_max_abs.restype = ctypes.c_int
     L.cq_reduce_max_abs.argtypes = [ctypes.c_void_p, tp, tp, ctypes.c_uint32, ctypes.c_int, ctypes.c_void_p,
                                     ctypes.c_size_t]

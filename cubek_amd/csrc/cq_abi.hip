@@ -1140,6 +1140,57 @@ cq_status cq_into_contiguous_packed(cq_stream_t stream, const cq_tensor* input, 
     return hip_status(cq::launch_repack(stream, a));
 }
 
+cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const cq_tensor* params, const cq_scheme* scheme,
+                            const cq_tensor* x, const cq_tensor* y, cq_dtype dtype, cq_dtype y_dtype) {
+    drop_stale_hip_error();
+    cq_status st = check_scheme(scheme);
+    if (st != CQ_OK) return st;
+    if (scheme->store != CQ_STORE_U32) return CQ_ERR_UNSUPPORTED_SCHEME;
+    if (!tensor_ok(values) || !tensor_ok(params) || !tensor_ok(x) || !tensor_ok(y) || !valid_dtype(dtype) ||
+        !valid_dtype(y_dtype))
+        return CQ_ERR_INVALID_ARGUMENT;
+    const int pd = param_to_dtype(scheme->param);
+    if (values->rank != 2 || x->rank != 1 || y->rank != 1) return CQ_ERR_SHAPE_MISMATCH;
+    if (values->elem_size != 4 || x->elem_size != dtype_size(dtype) || y->elem_size != dtype_size(y_dtype) ||
+        params->elem_size != dtype_size(pd))
+        return CQ_ERR_SHAPE_MISMATCH;
+    const uint32_t bits = value_bits(scheme->value), nq = 32u / bits;
+    const uint64_t rows = values->shape[0], cols = values->shape[1] * nq;
+    if (rows > 0xffffffffull || cols > 0xffffffffull) return CQ_ERR_TOO_LARGE;
+    if (x->shape[0] != cols || y->shape[0] != rows) return CQ_ERR_SHAPE_MISMATCH;
+    if ((values->shape[1] != 1 && values->strides[1] != 1) || (cols != 1 && x->strides[0] != 1) ||
+        (rows != 1 && y->strides[0] != 1))
+        return CQ_ERR_NON_CONTIGUOUS;
+    cq::GemvArgs a{};
+    if (scheme->level == CQ_LEVEL_BLOCK) {
+        if (scheme->block_rank > 2 || params->rank != 2) return CQ_ERR_SHAPE_MISMATCH;
+        a.block_cols = scheme->block[scheme->block_rank - 1];
+        a.block_rows = scheme->block_rank == 2 ? scheme->block[0] : 1;
+        if (rows % a.block_rows || cols % a.block_cols || params->shape[0] != rows / a.block_rows ||
+            params->shape[1] != cols / a.block_cols)
+            return CQ_ERR_SHAPE_MISMATCH;
+        a.scale_stride_row = params->strides[0];
+        a.scale_stride_col = params->strides[1];
+    } else if (numel(params) < 1) {
+        return CQ_ERR_SHAPE_MISMATCH;
+    }
+    if (rows == 0) return CQ_OK;
+    a.words = values->ptr;
+    a.scales = params->ptr;
+    a.x = x->ptr;
+    a.y = y->ptr;
+    a.dtype = dtype;
+    a.y_dtype = y_dtype;
+    a.param_dtype = pd;
+    a.bits = bits;
+    a.rows = static_cast<uint32_t>(rows);
+    a.cols = static_cast<uint32_t>(cols);
+    a.word_pitch = values->strides[0];
+    a.x_aligned16 = aligned(x->ptr, 16);
+    a.words_aligned16 = aligned(values->ptr, 16);
+    return hip_status(cq::launch_gemv_quantized(stream, a));
+}
+
 static bool reduce_view(const cq_tensor* input, uint32_t axis, uint64_t* outer, uint64_t* len, uint64_t* inner) {
     *outer = *inner = 1;
     for (uint32_t d = 0; d < axis; d++) *outer *= input->shape[d];

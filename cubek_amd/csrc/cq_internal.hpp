@@ -204,4 +204,21 @@ struct RepackArgs {
 };
 hipError_t launch_repack(hipStream_t s, const RepackArgs& a);
 
+// y = dequantize(W) * x over a packed [rows, cols] weight matrix (cq_gemv_quantized).
+struct GemvArgs {
+    const void* words;   // u32 words, row r at words + r * word_pitch
+    const void* scales;  // typed param_dtype
+    const void* x;       // [cols], typed dtype
+    void* y;             // [rows], typed y_dtype
+    int dtype, y_dtype, param_dtype;
+    uint32_t bits;       // bits per value
+    uint32_t rows, cols;
+    uint64_t word_pitch;
+    uint32_t block_rows, block_cols;  // 0, 0: one scale per tensor
+    uint64_t scale_stride_row, scale_stride_col;
+    bool x_aligned16, words_aligned16;
+};
+bool gemv_streams(const GemvArgs& a);  // the launch takes the streaming kernel
+hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a);
+
 }  // namespace cq

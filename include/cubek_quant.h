@@ -225,6 +225,25 @@ size_t cq_reduce_workspace_bytes(const cq_tensor* input, uint32_t axis, cq_dtype
 cq_status cq_into_contiguous_packed(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
                                     const uint64_t* shape, uint32_t rank, uint32_t packing);
 
+/* ---- a consumer of the packed format (the weight-load path) ---- */
+
+/* y = dequantize(W) * x with W read once in its quantized form: stands where the reference's matmul
+ * takes a quantized operand and dequantizes it while loading (MatmulInputHandle::Quantized,
+ * crates/cubek-matmul/src/base.rs:309-317; scale lookup per (row, col),
+ * crates/cubek-matmul/src/components/global/memory/layout.rs:371-455), for the matrix-vector case.
+ * The kernels are written against include/cubek_quant_device.hpp only.
+ *   values : U32-store tensor [rows, cols / num_quants], rows may be pitched (stride 1 along the row)
+ *   params : scales typed scheme->param, shape [1] (per tensor) or [rows / block_rows, cols / block_cols]
+ *            for blocks over the last one or two dimensions, any strides
+ *   x      : [cols] of `dtype`, contiguous;  y : [rows] of `y_dtype`, contiguous
+ * Every weight enters as the value cq_dequantize would produce for `dtype`, F(F(scale) * F(code)); the
+ * products are accumulated in f32 (order unspecified) and the sum is rounded once to `y_dtype`.
+ * 4-bit codes with f32 scales on 1-D blocks of 32 and a 16-bit `dtype` stream at HBM rate; everything
+ * else takes a simple wave-per-row kernel. */
+cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const cq_tensor* params,
+                            const cq_scheme* scheme, const cq_tensor* x, const cq_tensor* y,
+                            cq_dtype dtype, cq_dtype y_dtype);
+
 /* ---- diagnostics ---- */
 const char* cq_strerror(cq_status status);
 /* hipError_t of the most recent failed HIP call on the calling thread (0 if none). */

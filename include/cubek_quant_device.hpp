@@ -205,31 +205,35 @@ __device__ __forceinline__ void dequantize_symmetric_packed_value(uint32_t word,
 // dot-product / matrix instruction: out[i] holds values 2i (low half) and 2i+1 (high half).
 // Bit-identical to dequantize_symmetric_packed_value, in about half the instructions:
 //   - the fields are biased to unsigned digits (one XOR per word) and separated by masks into
-//     the four bytes of a register, where v_cvt_f32_ubyteN turns each into a float;
+//     the four bytes of a register, where v_cvt_f32_ubyteN turns each into a float (4-bit fields:
+//     v_cvt_pk_f32_fp8 turns two at a time, reading a digit as a tiny e4m3 number);
 //   - one FMA per value removes the bias and applies the scale: digit * s - bias * s is the
 //     exact product s * code (at most 11 + 8 significant bits), so the single rounding of
 //     pack_pair is the reference's rounding of F(scale) * F(code);
 //   - f16 goes through packed f16 arithmetic instead: the digit is planted in the mantissa of
 //     1024 + digit, v_pk_add_f16 removes 1024 + bias exactly and v_pk_mul_f16 multiplies and
 //     rounds two values at a time.
-// Scales that are negative, NaN, zero, or outside [2^-100, 2^100) take the plain path: there
-// bias * s could overflow, and a zero code has to come out as s * (+0) with the scale's sign.
+// The short sequence needs a "tame" scale: positive, finite and in [2^-100, 2^100) after rounding
+// to kF.  For other scales (negative, zero, NaN, huge, tiny) bias * s could overflow, and a zero code
+// has to come out as s * (+0) with the scale's sign: they take the plain path.
+// dequantize_symmetric_packed_value_pairs() decides per call; a kernel that wants straight-line code
+// tests pairs_scale_is_tame() once for many words (say, with a wave-wide vote) and calls
+// dequantize_symmetric_packed_value_pairs_tame() directly.
+template <Float kF, class FS>
+__device__ __forceinline__ bool pairs_scale_is_tame(FS scale) {
+    const float s = round_to<kF>(widen(scale));
+    // sign clear and exponent field in [27, 227)
+    return (__builtin_bit_cast(uint32_t, s) - 0x0d800000u) < (0x71800000u - 0x0d800000u);
+}
+
+// Precondition: pairs_scale_is_tame<kF>(scale).
 template <Float kF, int kBits, class FS>
-__device__ __forceinline__ void dequantize_symmetric_packed_value_pairs(uint32_t word, FS scale, uint32_t* out) {
+__device__ __forceinline__ void dequantize_symmetric_packed_value_pairs_tame(uint32_t word, FS scale, uint32_t* out) {
     static_assert(kF != Float::F32, "pairs are for the 16-bit types");
     static_assert(kBits == 2 || kBits == 4 || kBits == 8, "2, 4 or 8 bits per value");
     constexpr int kN = 32 / kBits;
     constexpr uint32_t kBias = 1u << (kBits - 1);
     const float s = round_to<kF>(widen(scale));
-    // sign clear and exponent field in [27, 227)
-    const bool tame = (__builtin_bit_cast(uint32_t, s) - 0x0d800000u) < (0x71800000u - 0x0d800000u);
-    if (!tame) {
-        float v[kN];
-        dequantize_symmetric_packed_value<kF, kBits>(word, scale, v);
-#pragma unroll
-        for (int i = 0; i < kN / 2; i++) out[i] = pack_pair<kF>(v[2 * i], v[2 * i + 1]);
-        return;
-    }
     constexpr uint32_t kBiasWord = kBits == 8 ? 0x80808080u : (kBits == 4 ? 0x88888888u : 0xAAAAAAAAu);
     const uint32_t digits = word ^ kBiasWord;  // field + bias, unsigned
     if constexpr (kF == Float::F16) {
@@ -259,21 +263,28 @@ __device__ __forceinline__ void dequantize_symmetric_packed_value_pairs(uint32_t
             out[0] = pack_pair<kF>(v0, v1);
             out[1] = pack_pair<kF>(v2, v3);
         } else if constexpr (kBits == 4) {
-            // even fields in the low nibble of each byte; odd fields stay in the high nibble: the byte
-            // reads 16 * digit, which s / 16 takes back (exact)
-            const uint32_t even = digits & 0x0f0f0f0fu, odd = digits & 0xf0f0f0f0u;
-            const float s16 = s * 0.0625f;
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
-                const float ve = __builtin_fmaf(static_cast<float>((even >> (8 * b)) & 0xffu), s, nbs);
-                const float vo = __builtin_fmaf(static_cast<float>((odd >> (8 * b)) & 0xffu), s16, nbs);
-                out[b] = pack_pair<kF>(ve, vo);
-            }
+            // even and odd fields as the low nibbles of four bytes each.  A byte 0x0d read as an e4m3 number
+            // is d * 2^-9 for every d in 0..15 (denormals, then the first binade, in one linear run), so
+            // v_cvt_pk_f32_fp8 turns two digits into floats per instruction; s * 512 takes the 2^-9 back
+            typedef float f32x2 __attribute__((ext_vector_type(2)));
+            const uint32_t even = digits & 0x0f0f0f0fu, odd = (digits >> 4) & 0x0f0f0f0fu;
+            const f32x2 e01 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(even), false);
+            const f32x2 e23 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(even), true);
+            const f32x2 o01 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(odd), false);
+            const f32x2 o23 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(odd), true);
+            const float s512 = s * 512.0f;  // exact: s < 2^100
+            out[0] = pack_pair<kF>(__builtin_fmaf(e01[0], s512, nbs), __builtin_fmaf(o01[0], s512, nbs));
+            out[1] = pack_pair<kF>(__builtin_fmaf(e01[1], s512, nbs), __builtin_fmaf(o01[1], s512, nbs));
+            out[2] = pack_pair<kF>(__builtin_fmaf(e23[0], s512, nbs), __builtin_fmaf(o23[0], s512, nbs));
+            out[3] = pack_pair<kF>(__builtin_fmaf(e23[1], s512, nbs), __builtin_fmaf(o23[1], s512, nbs));
         } else {
             // field j of every byte, j = 0..3: byte b of (digits >> 2j) & 0x03030303 is value 4b + j
             uint32_t plane[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) plane[j] = (digits >> (2 * j)) & 0x03030303u;
+            for (int j = 0; j < 4; j++) {
+                plane[j] = (digits >> (2 * j)) & 0x03030303u;
+                asm("" : "+v"(plane[j]));  // as above: one conversion instruction per byte
+            }
 #pragma unroll
             for (int b = 0; b < 4; b++) {
                 const float v0 = __builtin_fmaf(static_cast<float>((plane[0] >> (8 * b)) & 0xffu), s, nbs);
@@ -284,6 +295,19 @@ __device__ __forceinline__ void dequantize_symmetric_packed_value_pairs(uint32_t
                 out[2 * b + 1] = pack_pair<kF>(v2, v3);
             }
         }
+    }
+}
+
+template <Float kF, int kBits, class FS>
+__device__ __forceinline__ void dequantize_symmetric_packed_value_pairs(uint32_t word, FS scale, uint32_t* out) {
+    constexpr int kN = 32 / kBits;
+    if (pairs_scale_is_tame<kF>(scale)) {
+        dequantize_symmetric_packed_value_pairs_tame<kF, kBits>(word, scale, out);
+    } else {
+        float v[kN];
+        dequantize_symmetric_packed_value<kF, kBits>(word, scale, v);
+#pragma unroll
+        for (int i = 0; i < kN / 2; i++) out[i] = pack_pair<kF>(v[2 * i], v[2 * i + 1]);
     }
 }
 

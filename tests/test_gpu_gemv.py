@@ -1,0 +1,139 @@
+"""cq_gemv_quantized (y = dequantize(W) @ x from the packed weights) against the GEMV over the ORACLE's
+dequantized weights, computed in float64.  Tolerance, stated once: the kernels accumulate in f32, at most
+~180 sequential additions per lane followed by a 6-step tree, each rounding 2^-24 relative, so
+|y - y_ref| <= 2e-5 * sum|w * x|; an output of a 16-bit type is the f32 sum rounded once (checked bit for
+bit against the f32 output)."""
+import numpy as np
+import pytest
+
+from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantParam, QuantScheme, QuantValue, TensorHandleRef,
+                       _ffi, matvec)
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # elem, value, block, param, rows, cols, word pitch (None: contiguous)     -- first five: the streaming kernel
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 1000, 4096, None),
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 77, 2048, None),
+    (ElemType.BF16, QuantValue.E2M1, [32], QuantParam.F32, 130, 11008, None),     # last strip partly idle
+    (ElemType.F16, QuantValue.Q4F, [32], QuantParam.F32, 333, 8192, None),
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 64, 4096, 520),         # pitched rows of words
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.BF16, 100, 1024, None),      # general kernel from here on
+    (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, 50, 512, None),
+    (ElemType.F32, QuantValue.Q2S, [64], QuantParam.F32, 96, 1024, None),
+    (ElemType.F32, QuantValue.Q8F, None, QuantParam.F32, 33, 260, None),          # per tensor
+    (ElemType.BF16, QuantValue.Q4S, [4, 16], QuantParam.F32, 64, 256, None),      # blocks over both dimensions
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 40, 1056, None),        # cols not a multiple of 64 blocks
+]
+
+
+def _id(c):
+    elem, value, block, param, rows, cols, pitch = c
+    return f"{elem.name}-{value.name}-{'x'.join(map(str, block)) if block else 'tensor'}-{param.name}-{rows}x{cols}" + \
+        ("-pitched" if pitch else "")
+
+
+@pytest.mark.parametrize("case", CASES, ids=_id)
+def test_gemv_matches_oracle_dequantized_weights(oracle, case):
+    import torch
+
+    elem, value, block, param, rows, cols, pitch = case
+    level = QuantLevel.Tensor if block is None else QuantLevel.block(block)
+    scheme = QuantScheme.default().with_value(value).with_level(level).with_param(param)
+    rng = np.random.default_rng(rows * 7 + cols)
+    w32 = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+    w32[rng.random((rows, cols)) < 0.002] *= 20
+    wb = oracle.to_bits(w32, elem)
+    scales = oracle.compute_scales(wb, elem, (rows, cols), scheme)
+    words, out_scale = oracle.quantize(wb, elem, (rows, cols), scales, scheme)
+    deq = oracle.from_bits(oracle.dequantize(words, (rows, cols), out_scale, elem, scheme), elem).astype(np.float64)
+    xb = oracle.to_bits(rng.normal(0, 1, cols).astype(np.float32), elem)
+    x64 = oracle.from_bits(xb, elem).astype(np.float64)
+    want = deq @ x64
+    mag = np.abs(deq) @ np.abs(x64)
+
+    nq = scheme.num_quants()
+    wpr = cols // nq
+    pitch = pitch or wpr
+    buf = np.zeros((rows, pitch), np.uint32)
+    buf[:, :wpr] = words.reshape(rows, wpr)
+    d_words = torch.from_numpy(buf.view(np.int32)).cuda()
+    to16 = lambda a: torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda() if a.dtype == np.uint16 \
+        else torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    d_scales, d_x = to16(out_scale), to16(xb)
+    sshape = (1,) if block is None else tuple(d_scales.shape)
+    h_words = TensorHandleRef(d_words.data_ptr(), (rows, wpr), (pitch, 1), 4)
+    h_scales = TensorHandleRef(d_scales.data_ptr(), sshape, tuple(d_scales.stride()) if block else (1,),
+                               d_scales.element_size())
+    client = ComputeClient.current()
+    y32 = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
+    matvec.launch_ref(client, h_words, h_scales, scheme, TensorHandleRef.from_torch(d_x), TensorHandleRef.from_torch(y32),
+                      elem, ElemType.F32)
+    torch.cuda.synchronize()
+    got = y32.cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), float(np.max(np.abs(got - want) / (mag + 1e-30)))
+    if elem != ElemType.F32:  # the same sums, rounded once to the 16-bit type
+        y16 = torch.zeros((rows,), dtype=torch.int16, device="cuda")
+        matvec.launch_ref(client, h_words, h_scales, scheme, TensorHandleRef.from_torch(d_x),
+                          TensorHandleRef.from_torch(y16), elem, elem)
+        torch.cuda.synchronize()
+        assert np.array_equal(y16.cpu().numpy().view(np.uint16), oracle.to_bits(y32.cpu().numpy(), elem))
+
+
+@pytest.mark.parametrize("elem", [ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
+def test_gemv_scales_of_every_kind(oracle, elem):
+    """Negative, zero, tiny and huge scales among ordinary ones (the streaming kernel sends their lanes down a
+    plain path): same tolerance against the oracle's dequantized weights."""
+    import torch
+
+    rows, cols = 96, 4096
+    scheme = QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([32]))
+    rng = np.random.default_rng(5)
+    words = rng.integers(0, 2**32, (rows, cols // 8), dtype=np.uint64).astype(np.uint32)
+    scales = rng.uniform(0.001, 0.02, (rows, cols // 32)).astype(np.float32)
+    odd = rng.random(scales.shape) < 0.05
+    scales[odd] = rng.choice(np.array([-0.01, 0.0, -0.0, 1e-36, -3.0, 2.0 ** -110, 3000.0, -1e-30], np.float32), int(odd.sum()))
+    deq = oracle.from_bits(oracle.dequantize(words, (rows, cols), scales, elem, scheme), elem).astype(np.float64)
+    xb = oracle.to_bits(rng.normal(0, 1, cols).astype(np.float32), elem)
+    x64 = oracle.from_bits(xb, elem).astype(np.float64)
+    assert np.all(np.isfinite(deq))
+    want, mag = deq @ x64, np.abs(deq) @ np.abs(x64)
+    d_words = torch.from_numpy(words.view(np.int32)).cuda()
+    d_scales = torch.from_numpy(scales).cuda()
+    d_x = torch.from_numpy(xb.view(np.int16)).cuda()
+    y = torch.zeros(rows, dtype=torch.float32, device="cuda")
+    h = TensorHandleRef.from_torch
+    matvec.launch_ref(ComputeClient.current(), h(d_words), h(d_scales), scheme, h(d_x), h(y), elem, ElemType.F32)
+    torch.cuda.synchronize()
+    got = y.cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), float(np.max(np.abs(got - want) / (mag + 1e-30)))
+
+
+def test_gemv_argument_checks():
+    import torch
+
+    scheme = QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([32]))
+    w = torch.zeros((8, 16), dtype=torch.int32, device="cuda")
+    s = torch.ones((8, 4), dtype=torch.float32, device="cuda")
+    x = torch.zeros(128, dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros(8, dtype=torch.float32, device="cuda")
+    h = TensorHandleRef.from_torch
+    client = ComputeClient.current()
+    matvec.launch_ref(client, h(w), h(s), scheme, h(x), h(y), ElemType.BF16, ElemType.F32)
+
+    def status(fn):
+        with pytest.raises(_ffi.QuantError) as e:
+            fn()
+        return e.value.status
+
+    assert status(lambda: matvec.launch_ref(client, h(w), h(s), scheme, h(x[:64]), h(y), ElemType.BF16, ElemType.F32)) \
+        == _ffi.ERR_SHAPE_MISMATCH
+    assert status(lambda: matvec.launch_ref(client, h(w), h(s[:, :3]), scheme, h(x), h(y), ElemType.BF16, ElemType.F32)) \
+        == _ffi.ERR_SHAPE_MISMATCH
+    assert status(lambda: matvec.launch_ref(client, h(w), h(s), scheme, h(x), h(y), ElemType.F32, ElemType.F32)) \
+        == _ffi.ERR_SHAPE_MISMATCH  # x is not f32
+    from cubek_amd import QuantStore
+    assert status(lambda: matvec.launch_ref(client, h(w), h(s), scheme.with_store(QuantStore.Native), h(x), h(y),
+                                            ElemType.BF16, ElemType.F32)) == _ffi.ERR_UNSUPPORTED_SCHEME
+    assert status(lambda: matvec.launch_ref(client, h(w.t()), h(s), scheme, h(x), h(y), ElemType.BF16, ElemType.F32)) \
+        in (_ffi.ERR_NON_CONTIGUOUS, _ffi.ERR_SHAPE_MISMATCH)
