@@ -492,7 +492,8 @@ def main():
             del ps, p, xi
             torch.cuda.empty_cache()
         result["per_config"] = table
-        result["adjacent_kernels"] = adjacent_kernels(torch)
+        if not os.environ.get("CQ_BENCH_SKIP_ADJACENT"):
+            result["adjacent_kernels"] = adjacent_kernels(torch)
 
     print(json.dumps(result))
 

@@ -393,6 +393,13 @@ void scale_in_to_out(cq::FlatArgs* a) {
     }
 }
 
+// E4M3 / E5M2 in the U32 store: the reference packs the rounded integer (up to +-448 / +-57344) into an 8-bit
+// field with `i32 & mask` (src/quantize.rs:75), so most codes wrap.  Faithfully reproduced, but only by the
+// per-element kernels: no streaming kernel is built for a combination nobody can use.
+bool wraps_its_field(const cq_scheme* s) {
+    return s->store == CQ_STORE_U32 && (s->value == CQ_VALUE_E4M3 || s->value == CQ_VALUE_E5M2);
+}
+
 // Stored encoding of the flat kernels (cq::Encoding) and the field width they see.
 int flat_encoding(const cq_scheme* s) {
     if (s->store == CQ_STORE_U32) return 0;
@@ -639,7 +646,8 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     const bool native = scheme->store == CQ_STORE_NATIVE;
     const uint64_t per_chunk = 16 / dtype_size(input_dtype);
     uint64_t flat_words = 0;
-    if (flat_ok(p, input_dtype, input, output, scale, out_scale)) {
+    const bool streaming = !wraps_its_field(scheme);
+    if (streaming && flat_ok(p, input_dtype, input, output, scale, out_scale)) {
         cq::FlatArgs a{};
         a.input = input->ptr;
         a.output = output->ptr;
@@ -658,7 +666,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
     cq::FlatArgs fr{};
-    if (flat_words == 0 && (flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
+    if (streaming && flat_words == 0 && (flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
                                          dtype_size(pd), true, &fr) ||
                             lane_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
                                          dtype_size(pd), true, &fr))) {
@@ -674,7 +682,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, fr));
     }
     cq::RowArgs r;
-    if (flat_words == 0 && rows_args(p, scheme, input_dtype, input, output, &r)) {
+    if (streaming && flat_words == 0 && rows_args(p, scheme, input_dtype, input, output, &r)) {
         r.input = input->ptr;
         r.output = output->ptr;
         r.scale_in = scale->ptr;
@@ -683,7 +691,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         return hip_status(cq::launch_quantize_rows(stream, input_dtype, static_cast<int>(p.bits), r));
     }
     cq::TransposedArgs tr;
-    if (flat_words == 0 && transposed_args(p, scheme, input_dtype, input, output, &tr)) {
+    if (streaming && flat_words == 0 && transposed_args(p, scheme, input_dtype, input, output, &tr)) {
         tr.input = input->ptr;
         tr.output = output->ptr;
         tr.scale_in = scale->ptr;
@@ -924,6 +932,20 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
 
     const uint64_t per_chunk = 16 / dtype_size(input_dtype);
     const bool native = scheme->store == CQ_STORE_NATIVE;
+    if (wraps_its_field(scheme)) {
+        // scales into out_scale, then the per-element quantize reading them back
+        st = produce_scales(stream, p, scheme, input, input_dtype, out_scale, pd, workspace, workspace_bytes);
+        if (st != CQ_OK) return st;
+        cq::GenericArgs g = generic_args(p, scheme);
+        g.input = input->ptr;
+        g.output = output->ptr;
+        g.scale_in = out_scale->ptr;
+        g.scale_in_dtype = pd;
+        g.scale_out = nullptr;
+        g.word_begin = 0;
+        g.word_end = p.n / p.nq;
+        return hip_status(cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
+    }
     const bool flat = flat_ok(p, input_dtype, input, output, out_scale, nullptr);
 
     // fused single pass: abs-max, scale, quantize, pack in registers (whole 32-bit words of codes: lanes that

@@ -161,14 +161,32 @@ struct F16 {
 
 // Round an f32 value to a runtime-selected dtype (scale parameters), widened back.
 __device__ __forceinline__ float round_to_dtype(int dtype, float v) {
-    if (dtype == CQ_F32) return v;
-    if (dtype == CQ_BF16) return BF16::round(v);
-    return F16::round(v);
+    // both roundings and a select: no branch in the middle of a kernel's arithmetic
+    const float as_bf16 = BF16::round(v), as_f16 = F16::round(v);
+    return dtype == CQ_F32 ? v : (dtype == CQ_BF16 ? as_bf16 : as_f16);
 }
 __device__ __forceinline__ float load_dtype(int dtype, const void* p, uint64_t i) {
     if (dtype == CQ_F32) return F32::load(p, i);
     if (dtype == CQ_BF16) return BF16::load(p, i);
     return F16::load(p, i);
+}
+// The same load in two steps, for kernels that issue all their loads before any arithmetic and learn the type
+// at run time.  Step one has no branch on the type (a branch around a load makes the compiler wait for the
+// load where the paths meet): two 16-bit loads, the halves of an f32 or twice the same 16-bit value, both
+// inside the tensor whatever the type.  Step two widens, behind all loads.
+struct RawScale {
+    uint32_t lo, hi;
+};
+__device__ __forceinline__ RawScale load_dtype_raw(int dtype, const void* p, uint64_t i) {
+    const bool wide = dtype == CQ_F32;
+    const uint16_t* lo = reinterpret_cast<const uint16_t*>(static_cast<const char*>(p) + (i << (wide ? 2 : 1)));
+    return RawScale{lo[0], lo[wide ? 1 : 0]};
+}
+__device__ __forceinline__ float widen_dtype_raw(int dtype, RawScale raw) {
+    const float from_f32 = bits_f32(raw.lo | (raw.hi << 16));
+    const float from_bf16 = bits_f32(raw.lo << 16);
+    const float from_f16 = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(raw.lo)));
+    return dtype == CQ_F32 ? from_f32 : (dtype == CQ_BF16 ? from_bf16 : from_f16);
 }
 __device__ __forceinline__ void store_dtype(int dtype, void* p, uint64_t i, float v) {
     if (dtype == CQ_F32)

@@ -209,6 +209,7 @@ struct LaneRows {
     uint32_t row_chunks, row_magic, row_shift;
     uint32_t total_chunks;  // < 2^31
     uint32_t levels;        // leading dimensions, 1 .. kMaxLaneLevels
+    uint32_t narrow;        // every byte offset the rows can reach in the four tensors is below 2^32
     // blocks of `scale_rows` entries of the innermost level (by a lane group of columns) share their scale
     // (given scales only); the scale strides of that level are per block of rows
     uint32_t scale_rows, scale_magic, scale_shift;
@@ -222,6 +223,7 @@ struct LanesGeo {
     void* out;
     const void* scale_in;
     void* scale_out;
+    uint32_t tile_begin;  // first tile of the launch (a launch may cover the end of a numbering only)
     LaneRows rows;
     template <int kUnroll, int kThreads, bool kChecked>
     using Steps = LaneSteps<kUnroll, kThreads>;  // always checked
@@ -237,15 +239,47 @@ struct LaneSteps {
     bool live_[kUnroll], first_[kUnroll], block_row_[kUnroll];
     __device__ __forceinline__ LaneSteps(const LanesGeo& g, uint32_t tile) {
         const LaneRows& r = g.rows;
+        // The shape of the launch is the same for every lane, so the cases below are scalar branches.
+        if (r.levels == 1 && r.count[0] == 1) {
+            // a single row (one contiguous run): chunk numbers are positions already
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                const uint32_t chunk = ((g.tile_begin + tile) * kUnroll + u) * kThreads + threadIdx.x;
+                live_[u] = chunk < r.total_chunks;
+                col_[u] = live_[u] ? chunk : r.total_chunks - 1;  // lanes past the end re-read the last chunk
+                first_[u] = true;
+                block_row_[u] = true;
+                in_[u] = static_cast<const char*>(g.in);
+                out_[u] = static_cast<char*>(g.out);
+                scale_in_[u] = static_cast<const char*>(g.scale_in);
+                scale_out_[u] = static_cast<char*>(g.scale_out);
+            }
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
-            const uint32_t chunk = (tile * kUnroll + u) * kThreads + threadIdx.x;
+            const uint32_t chunk = ((g.tile_begin + tile) * kUnroll + u) * kThreads + threadIdx.x;
             live_[u] = chunk < r.total_chunks;
             const uint32_t c = live_[u] ? chunk : r.total_chunks - 1;  // lanes past the end re-read the last chunk
             uint32_t row = magic_div(c, r.row_magic, r.row_shift);
             col_[u] = c - row * r.row_chunks;
             first_[u] = row == 0;
             block_row_[u] = true;
+            if (r.levels == 1 && r.narrow) {
+                // rows in one uniform run (pitched rows, a slice) whose offsets fit 32 bits: no walk over levels
+                uint32_t scale_row = row;
+                if (r.scale_rows > 1) {
+                    scale_row = magic_div(row, r.scale_magic, r.scale_shift);
+                    block_row_[u] = row == scale_row * r.scale_rows;
+                }
+                in_[u] = static_cast<const char*>(g.in) + row * static_cast<uint32_t>(r.in[0]);
+                out_[u] = static_cast<char*>(g.out) + row * static_cast<uint32_t>(r.out[0]);
+                scale_in_[u] = static_cast<const char*>(g.scale_in) + scale_row * static_cast<uint32_t>(r.scale_in[0]);
+                scale_out_[u] = g.scale_out == nullptr
+                                    ? nullptr
+                                    : static_cast<char*>(g.scale_out) + scale_row * static_cast<uint32_t>(r.scale_out[0]);
+                continue;
+            }
             uint64_t in = 0, out = 0, scale_in = 0, scale_out = 0;
 #pragma unroll
             for (int l = 0; l < kMaxLaneLevels; l++) {
@@ -316,14 +350,19 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
     // All kUnroll loads are issued back to back.
     u32x4 raw[kUnroll];
     float s_given[kUnroll];
+    RawScale s_stored[kUnroll];  // stored scales as loaded, widened behind the loads
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         const auto c = at.load_chunk(u);
         raw[u] = stream_load(static_cast<const u32x4*>(at.in(u)) + c);
         if constexpr (kScaleSrc == kScaleStored)
-            s_given[u] = F::round(load_dtype(param_dtype, at.scale_in(u), c / kDiv));
+            s_stored[u] = load_dtype_raw(param_dtype, at.scale_in(u), c / kDiv);
         else if constexpr (!kDynamic && kGroup != 0 && kScaleSrc != kScalePartials)
             s_given[u] = F::load(at.scale_in(u), c / kDiv);
+    }
+    if constexpr (kScaleSrc == kScaleStored) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) s_given[u] = F::round(widen_dtype_raw(param_dtype, s_stored[u]));
     }
     if constexpr (kScaleSrc == kScalePartials) {
         // second pass of the grid reduction: every workgroup reduces the (<= a few
@@ -403,38 +442,35 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
     }
 }
 
-template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
-          int kThreads, bool kChecked, int kEnc = kEncInt>
+// One contiguous run of whole tiles, f32 parameters: the hot launch.  Ragged ends, other parameter types and
+// rows that are not whole steps run lane by lane (quantize_flat_lanes_kernel), which keeps the number of
+// kernels in the library, and with it its size and load time, at a third.
+template <class F, int kBits, int kGroup, int kScaleSrc, bool kWide, int kUnroll, int kThreads, int kEnc = kEncInt>
 __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
-    void* __restrict__ scale_out, int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end,
-    QuantParams qp, uint32_t num_partials) {
+    void* __restrict__ scale_out, uint64_t chunk_begin, uint64_t chunk_end, QuantParams qp, uint32_t num_partials) {
     const RunGeo geo{in, out, scale_in, scale_out, chunk_begin, chunk_end};
-    quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParamF32, kWide, kUnroll, kThreads, kChecked, kEnc>(
-        geo, param_dtype_rt, qp, num_partials);
+    quantize_flat_body<F, kBits, kGroup, kScaleSrc, true, kWide, kUnroll, kThreads, false, kEnc>(geo, CQ_F32, qp, num_partials);
 }
 
-// Pitched rows, from step `step_begin` of the launch on.  A kernel of its own so that the launches
-// over one contiguous run carry none of the row arithmetic in their prologue.
-template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
-          int kThreads, bool kChecked, int kEnc = kEncInt>
+// Pitched rows of whole steps, from step `step_begin` of the launch on, f32 parameters.  A kernel of its own
+// so that the launches over one contiguous run carry none of the row arithmetic in their prologue.
+template <class F, int kBits, int kGroup, int kScaleSrc, bool kWide, int kUnroll, int kThreads, int kEnc = kEncInt>
 __global__ __launch_bounds__(kThreads) void quantize_flat_rows_kernel(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
-    void* __restrict__ scale_out, int param_dtype_rt, uint32_t step_begin, QuantParams qp, uint32_t num_partials,
-    FlatRows rows) {
-    const uint32_t out_scale_bytes = (kParamF32 || param_dtype_rt == CQ_F32) ? 4 : 2;
-    const RowsGeo<16, F::kPerChunk * kBits / 8, kGroup> geo{in, out, scale_in, scale_out, step_begin,
-                                                            F::kBytes, out_scale_bytes, rows};
-    quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParamF32, kWide, kUnroll, kThreads, kChecked, kEnc>(
-        geo, param_dtype_rt, qp, num_partials);
+    void* __restrict__ scale_out, uint32_t step_begin, QuantParams qp, uint32_t num_partials, FlatRows rows) {
+    const RowsGeo<16, F::kPerChunk * kBits / 8, kGroup> geo{in, out, scale_in, scale_out, step_begin, F::kBytes, 4, rows};
+    quantize_flat_body<F, kBits, kGroup, kScaleSrc, true, kWide, kUnroll, kThreads, false, kEnc>(geo, CQ_F32, qp, num_partials);
 }
 
-// Rows found lane by lane (LaneSteps); the scale type is read at run time.
+// Rows found lane by lane (LaneSteps), bounds-checked; the scale type is read at run time.  `tile_begin`:
+// the launch starts at that tile of the numbering (the ragged end behind a launch of whole tiles).
 template <class F, int kBits, int kGroup, int kScaleSrc, bool kWide, int kUnroll, int kThreads, int kEnc = kEncInt>
 __global__ __launch_bounds__(kThreads) void quantize_flat_lanes_kernel(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
-    void* __restrict__ scale_out, int param_dtype_rt, QuantParams qp, uint32_t num_partials, LaneRows rows) {
-    const LanesGeo geo{in, out, scale_in, scale_out, rows};
+    void* __restrict__ scale_out, int param_dtype_rt, QuantParams qp, uint32_t num_partials, uint32_t tile_begin,
+    LaneRows rows) {
+    const LanesGeo geo{in, out, scale_in, scale_out, tile_begin, rows};
     quantize_flat_body<F, kBits, kGroup, kScaleSrc, false, kWide, kUnroll, kThreads, true, kEnc>(geo, param_dtype_rt, qp,
                                                                                                num_partials);
 }
@@ -448,6 +484,7 @@ __device__ __forceinline__ void dequantize_flat_body(const Geo& geo, int param_d
     const typename Geo::template Steps<kUnroll, kThreads, kChecked> at(geo, blockIdx.x);
 
     uint32_t w0[kUnroll], w1[kUnroll];
+    RawScale sc_raw[kUnroll];  // scales as loaded: nothing in the loop below waits for a load
     float sc[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
@@ -466,9 +503,15 @@ __device__ __forceinline__ void dequantize_flat_body(const Geo& geo, int param_d
             w0[u] = w >> ((static_cast<uint32_t>(c) & (kLanesPerWord - 1)) * kChunkBits);
         }
         const auto si = kGroup == 0 ? 0 : c / (kGroup == 0 ? 1 : kGroup);
-        sc[u] = F::round(load_dtype(param_dtype, at.scale_in(u), si));  // Line::cast_from(scale)
+        if constexpr (kParamF32)
+            sc[u] = F32::load(at.scale_in(u), si);
+        else
+            sc_raw[u] = load_dtype_raw(param_dtype, at.scale_in(u), si);
     }
     __builtin_amdgcn_sched_barrier(0);  // keep every load ahead of the arithmetic
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++)  // Line::cast_from(scale)
+        sc[u] = F::round(kParamF32 ? sc[u] : widen_dtype_raw(param_dtype, sc_raw[u]));
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         float y[kN];
@@ -484,29 +527,28 @@ __device__ __forceinline__ void dequantize_flat_body(const Geo& geo, int param_d
     }
 }
 
-template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked,
-          int kEnc = kEncInt>
+// whole tiles of one contiguous run, f32 parameters (see quantize_flat_kernel)
+template <class F, int kBits, int kGroup, int kUnroll, int kThreads, int kEnc = kEncInt>
 __global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
-    const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params,
-    int param_dtype_rt, uint64_t chunk_begin, uint64_t chunk_end) {
+    const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params, uint64_t chunk_begin,
+    uint64_t chunk_end) {
     const RunGeo geo{in, out, params, nullptr, chunk_begin, chunk_end};
-    dequantize_flat_body<F, kBits, kGroup, kParamF32, kUnroll, kThreads, kChecked, kEnc>(geo, param_dtype_rt);
+    dequantize_flat_body<F, kBits, kGroup, true, kUnroll, kThreads, false, kEnc>(geo, CQ_F32);
 }
-template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked,
-          int kEnc = kEncInt>
+// pitched rows of whole steps, f32 parameters
+template <class F, int kBits, int kGroup, int kUnroll, int kThreads, int kEnc = kEncInt>
 __global__ __launch_bounds__(kThreads) void dequantize_flat_rows_kernel(
-    const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params,
-    int param_dtype_rt, uint32_t step_begin, FlatRows rows) {
-    const uint32_t param_bytes = (kParamF32 || param_dtype_rt == CQ_F32) ? 4 : 2;
-    const RowsGeo<F::kPerChunk * kBits / 8, 16, kGroup> geo{in, out, params, nullptr, step_begin, param_bytes, 0, rows};
-    dequantize_flat_body<F, kBits, kGroup, kParamF32, kUnroll, kThreads, kChecked, kEnc>(geo, param_dtype_rt);
+    const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params, uint32_t step_begin,
+    FlatRows rows) {
+    const RowsGeo<F::kPerChunk * kBits / 8, 16, kGroup> geo{in, out, params, nullptr, step_begin, 4, 0, rows};
+    dequantize_flat_body<F, kBits, kGroup, true, kUnroll, kThreads, false, kEnc>(geo, CQ_F32);
 }
-
+// lane by lane, bounds-checked, parameter type read at run time
 template <class F, int kBits, int kGroup, int kUnroll, int kThreads, int kEnc = kEncInt>
 __global__ __launch_bounds__(kThreads) void dequantize_flat_lanes_kernel(
     const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params, int param_dtype_rt,
-    LaneRows rows) {
-    const LanesGeo geo{in, out, params, nullptr, rows};
+    uint32_t tile_begin, LaneRows rows) {
+    const LanesGeo geo{in, out, params, nullptr, tile_begin, rows};
     dequantize_flat_body<F, kBits, kGroup, false, kUnroll, kThreads, true, kEnc>(geo, param_dtype_rt);
 }
 
@@ -554,7 +596,7 @@ template <class F, int kGroup, int kUnroll, int kThreads>
 __global__ __launch_bounds__(kThreads) void scales_flat_lanes_kernel(const u32x4* __restrict__ in,
                                                                      void* __restrict__ scales, QuantParams qp,
                                                                      LaneRows rows) {
-    const LanesGeo geo{in, nullptr, nullptr, scales, rows};
+    const LanesGeo geo{in, nullptr, nullptr, scales, 0, rows};
     scales_flat_body<F, kGroup, kUnroll, kThreads>(geo, qp);
 }
 

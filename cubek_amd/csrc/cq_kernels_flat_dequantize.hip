@@ -12,31 +12,31 @@ namespace {
 
 template <class F, int kBits, int kGroup, int kEnc>
 hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
-    auto in = static_cast<const uint32_t*>(a.input);
-    auto out = static_cast<u32x4*>(a.output);
-    const bool p32 = a.param_dtype == CQ_F32;
+    auto in = static_cast<const char*>(a.input);
+    auto out = static_cast<char*>(a.output);
     constexpr int kU = kUnrollD<F, kBits, kGroup>;
-    if (a.lanes.levels > 0) {
-        hipLaunchKernelGGL((dequantize_flat_lanes_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(lanes_grid(a, kU)),
-                           dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, lane_rows(a));
-        return hipGetLastError();
-    }
-    if (a.rows > 1)
-        return launch_row_steps(a, kU, [&](bool checked, uint32_t grid, uint32_t step_begin) {
-            auto kernel = checked ? (p32 ? dequantize_flat_rows_kernel<F, kBits, kGroup, true, kU, kThreads, true, kEnc>
-                                         : dequantize_flat_rows_kernel<F, kBits, kGroup, false, kU, kThreads, true, kEnc>)
-                                  : (p32 ? dequantize_flat_rows_kernel<F, kBits, kGroup, true, kU, kThreads, false, kEnc>
-                                         : dequantize_flat_rows_kernel<F, kBits, kGroup, false, kU, kThreads, false, kEnc>);
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, step_begin,
-                               flat_rows(a));
+    constexpr uint64_t kInChunk = F::kPerChunk * kBits / 8;  // stored bytes per chunk
+    constexpr uint64_t kDiv = kGroup == 0 ? 1 : kGroup;
+    const uint64_t param_bytes = kGroup == 0 ? 0 : (a.param_dtype == CQ_F32 ? 4 : 2);
+    return launch_flat(
+        a, kU,
+        [&](uint32_t grid, uint64_t) {
+            if (a.rows > 1)
+                hipLaunchKernelGGL((dequantize_flat_rows_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(grid), dim3(kThreads),
+                                   0, s, reinterpret_cast<const uint32_t*>(in), reinterpret_cast<u32x4*>(out), a.scale_in, 0u,
+                                   flat_rows(a));
+            else
+                hipLaunchKernelGGL((dequantize_flat_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(grid), dim3(kThreads), 0,
+                                   s, reinterpret_cast<const uint32_t*>(in), reinterpret_cast<u32x4*>(out), a.scale_in, 0ull,
+                                   static_cast<uint64_t>(grid) * kThreads * kU);
+        },
+        [&](const LaneRows& rows, uint32_t tile_begin, uint32_t grid, RunOffsets off) {
+            hipLaunchKernelGGL((dequantize_flat_lanes_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(grid), dim3(kThreads), 0,
+                               s, reinterpret_cast<const uint32_t*>(in + off.chunks * kInChunk),
+                               reinterpret_cast<u32x4*>(out + off.chunks * 16),
+                               static_cast<const char*>(a.scale_in) + off.chunks / kDiv * param_bytes, a.param_dtype, tile_begin,
+                               rows);
         });
-    return launch_tiles(a.num_chunks, kU, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
-        auto kernel = checked ? (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kU, kThreads, true, kEnc>
-                                     : dequantize_flat_kernel<F, kBits, kGroup, false, kU, kThreads, true, kEnc>)
-                              : (p32 ? dequantize_flat_kernel<F, kBits, kGroup, true, kU, kThreads, false, kEnc>
-                                     : dequantize_flat_kernel<F, kBits, kGroup, false, kU, kThreads, false, kEnc>);
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.param_dtype, begin, end);
-    });
 }
 
 template <class F, int kBits, int kGroup>

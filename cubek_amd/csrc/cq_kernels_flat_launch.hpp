@@ -81,6 +81,25 @@ FlatRows flat_rows(const FlatArgs& a) {
     return r;
 }
 
+// Whether every byte offset the rows of `r` can reach stays below 2^32 in each of the four tensors.
+void set_narrow(LaneRows* r) {
+    uint64_t reach[4] = {0, 0, 0, 0};
+    for (uint32_t l = 0; l < r->levels; l++) {
+        const uint64_t last = r->count[l] - 1;
+        const uint64_t steps[4] = {r->in[l], r->out[l], r->scale_in[l], r->scale_out[l]};
+        for (int t = 0; t < 4; t++) {
+            if (last != 0 && steps[t] > (1ull << 32) / last) {
+                r->narrow = 0;
+                return;
+            }
+            reach[t] += last * steps[t];
+        }
+    }
+    r->narrow = 1;
+    for (int t = 0; t < 4; t++)
+        if (reach[t] >= (1ull << 32)) r->narrow = 0;
+}
+
 // the same for the kernels that find each lane's row
 static_assert(kMaxLaneLevels == CQ_MAX_RANK - 1, "one level per leading dimension");
 LaneRows lane_rows(const FlatArgs& a) {
@@ -99,11 +118,48 @@ LaneRows lane_rows(const FlatArgs& a) {
         r.scale_in[l] = a.lanes.scale_in[l];
         r.scale_out[l] = a.lanes.scale_out[l];
     }
+    set_narrow(&r);
     return r;
 }
 inline uint32_t lanes_grid(const FlatArgs& a, int unroll) {
     const uint64_t per = static_cast<uint64_t>(kThreads) * unroll;
     return static_cast<uint32_t>((a.rows * a.num_chunks + per - 1) / per);
+}
+
+// One contiguous run of `chunks` chunks (< 2^31) as the lane-wise kernels see it: a single row.
+LaneRows lane_rows_of_run(uint64_t chunks) {
+    LaneRows r{};
+    r.row_chunks = static_cast<uint32_t>(chunks);
+    magic_of(r.row_chunks, &r.row_magic, &r.row_shift);
+    r.total_chunks = r.row_chunks;
+    r.levels = 1;
+    r.scale_rows = 1;
+    magic_of(1, &r.scale_magic, &r.scale_shift);
+    r.count[0] = 1;
+    magic_of(1, &r.magic[0], &r.shift[0]);
+    r.narrow = 1;
+    return r;
+}
+// Pitched rows (FlatArgs::rows > 1: groups of inner_rows rows) as the lane-wise kernels see them: one level for
+// the rows of a group, one for the groups.  rows * num_chunks < 2^31.
+LaneRows lane_rows_of_rows(const FlatArgs& a) {
+    LaneRows r{};
+    r.row_chunks = static_cast<uint32_t>(a.num_chunks);
+    magic_of(r.row_chunks, &r.row_magic, &r.row_shift);
+    r.total_chunks = static_cast<uint32_t>(a.rows * a.num_chunks);
+    r.scale_rows = a.scale_rows > 1 ? a.scale_rows : 1u;
+    magic_of(r.scale_rows, &r.scale_magic, &r.scale_shift);
+    const uint64_t inner = a.inner_rows == 0 ? a.rows : a.inner_rows;
+    r.levels = inner == a.rows ? 1 : 2;
+    r.count[0] = static_cast<uint32_t>(inner);
+    r.in[0] = a.in_pitch, r.out[0] = a.out_pitch, r.scale_in[0] = a.scale_in_pitch, r.scale_out[0] = a.scale_out_pitch;
+    if (r.levels == 2) {
+        r.count[1] = static_cast<uint32_t>(a.rows / inner);
+        r.in[1] = a.in_outer, r.out[1] = a.out_outer, r.scale_in[1] = a.scale_in_outer, r.scale_out[1] = a.scale_out_outer;
+    }
+    for (uint32_t l = 0; l < r.levels; l++) magic_of(r.count[l], &r.magic[l], &r.shift[l]);
+    set_narrow(&r);
+    return r;
 }
 
 QuantParams quant_params(const Range& r) {
@@ -115,44 +171,52 @@ QuantParams quant_params(const Range& r) {
     return p;
 }
 
-// Launches `kernel(false)` over the full tiles and `kernel(true)` (bounds-checked)
-// over the ragged rest; a tile is kThreads*unroll chunks.
-template <class LaunchFn>
-hipError_t launch_tiles(uint64_t num_chunks, int unroll, LaunchFn launch) {
+// How a flat launch is cut up.  The kernels over whole tiles (a contiguous run, or pitched rows of whole
+// steps) exist for f32 parameters only and check no bounds; everything else is the lane-wise kernel's:
+//   `whole(grid, begin)`                       tiles [begin, begin + grid) of the run / of the rows' steps
+//   `lanes(rows, tile_begin, grid, offsets)`   lane by lane; `offsets` = chunks / scales to advance the base
+//                                              pointers by (a contiguous run only)
+struct RunOffsets {
+    uint64_t chunks;  // 16-byte chunks of the float tensor
+};
+template <class WholeFn, class LanesFn>
+hipError_t launch_flat(const FlatArgs& a, int unroll, WholeFn whole, LanesFn lanes) {
     const uint64_t tile = static_cast<uint64_t>(kThreads) * unroll;
-    const uint64_t full = num_chunks / tile;
+    const bool p32 = a.param_dtype == CQ_F32;
+    hipError_t e = hipSuccess;
+    if (a.lanes.levels > 0) {
+        lanes(lane_rows(a), 0u, lanes_grid(a, unroll), RunOffsets{0});
+        return hipGetLastError();
+    }
+    if (a.rows > 1) {
+        const LaneRows lr = lane_rows_of_rows(a);
+        const uint32_t tiles = static_cast<uint32_t>((static_cast<uint64_t>(lr.total_chunks) + tile - 1) / tile);
+        // whole steps: a tile is `unroll` steps in both numberings, so the ragged last tile can go lane by lane
+        const uint32_t full = p32 && a.num_chunks % kThreads == 0 ? static_cast<uint32_t>(lr.total_chunks / tile) : 0u;
+        if (full > 0) {
+            whole(full, 0ull);
+            if ((e = hipGetLastError()) != hipSuccess) return e;
+        }
+        if (full < tiles) {
+            lanes(lr, full, tiles - full, RunOffsets{0});
+            e = hipGetLastError();
+        }
+        return e;
+    }
+    // one contiguous run
+    const uint64_t full = p32 ? a.num_chunks / tile : 0;
     if (full > 0) {
-        launch(false, static_cast<uint32_t>(full), 0, full * tile);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
+        whole(static_cast<uint32_t>(full), 0ull);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
     }
-    if (full * tile < num_chunks) {
-        launch(true, 1u, full * tile, num_chunks);
-        return hipGetLastError();
+    // the rest lane by lane, in pieces the 32-bit chunk numbers of those kernels can hold
+    const uint64_t piece = (1ull << 30);  // a multiple of every tile and every block
+    for (uint64_t begin = full * tile; begin < a.num_chunks; begin += piece) {
+        const uint64_t n = a.num_chunks - begin < piece ? a.num_chunks - begin : piece;
+        lanes(lane_rows_of_run(n), 0u, static_cast<uint32_t>((n + tile - 1) / tile), RunOffsets{begin});
+        if ((e = hipGetLastError()) != hipSuccess) return e;
     }
-    return hipSuccess;
-}
-
-// The same over pitched rows: `launch(checked, grid, step_begin)`.  Rows of whole steps run
-// unchecked but for the workgroup that holds the launch's last steps; other rows run checked throughout.
-template <class LaunchFn>
-hipError_t launch_row_steps(const FlatArgs& a, int unroll, LaunchFn launch) {
-    const uint32_t total = flat_rows(a).total_steps;
-    if (a.num_chunks % kThreads != 0) {
-        launch(true, (total + unroll - 1) / unroll, 0u);
-        return hipGetLastError();
-    }
-    const uint32_t full = total / unroll;
-    if (full > 0) {
-        launch(false, full, 0u);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
-    if (full * unroll < total) {
-        launch(true, 1u, full * unroll);
-        return hipGetLastError();
-    }
-    return hipSuccess;
+    return e;
 }
 
 template <class F, int kBits, int kGroup, int kSrc, bool kWide, int kEnc>
@@ -161,44 +225,42 @@ hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
     // input-typed tensor; per-tensor launches read it or finish the grid reduction
     if constexpr ((kGroup == 0 && (kSrc == kScaleDynamic || kSrc == kScaleStored)) || (kGroup != 0 && kSrc == kScalePartials)) {
         return hipErrorInvalidValue;
-    } else if constexpr (kSrc == kScaleStored) {
-        // read back by the second pass of a two-launch dynamic quantize, which runs lane by lane only
-        if (a.lanes.levels == 0) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((quantize_flat_lanes_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
-                           dim3(lanes_grid(a, kUnrollQ)), dim3(kThreads), 0, s, static_cast<const u32x4*>(a.input),
-                           static_cast<uint32_t*>(a.output), a.scale_in, a.scale_out, a.param_dtype, quant_params(a.range),
-                           a.num_partials, lane_rows(a));
-        return hipGetLastError();
     } else {
-        auto in = static_cast<const u32x4*>(a.input);
-        auto out = static_cast<uint32_t*>(a.output);
+        // stored scales are read back by the second pass of a two-launch dynamic quantize, which runs lane by lane only
+        if (kSrc == kScaleStored && a.lanes.levels == 0) return hipErrorInvalidValue;
+        auto in = static_cast<const char*>(a.input);
+        auto out = static_cast<char*>(a.output);
         const QuantParams qp = quant_params(a.range);
-        const bool p32 = a.param_dtype == CQ_F32;
-        if (a.lanes.levels > 0) {
-            hipLaunchKernelGGL((quantize_flat_lanes_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
-                               dim3(lanes_grid(a, kUnrollQ)), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
-                               a.param_dtype, qp, a.num_partials, lane_rows(a));
-            return hipGetLastError();
-        }
-        if (a.rows > 1)
-            return launch_row_steps(a, kUnrollQ, [&](bool checked, uint32_t grid, uint32_t step_begin) {
-                auto kernel =
-                    checked ? (p32 ? quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, true, kEnc>
-                                   : quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, true, kEnc>)
-                            : (p32 ? quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false, kEnc>
-                                   : quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false, kEnc>);
-                hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out, a.param_dtype,
-                                   step_begin, qp, a.num_partials, flat_rows(a));
+        constexpr uint64_t kOutChunk = F::kPerChunk * kBits / 8;  // stored bytes per chunk
+        // bytes per scale of the two scale tensors (per-tensor launches and the partials never move their pointers)
+        const uint64_t scale_in_bytes = kGroup == 0 ? 0 : (kSrc == kScaleStored ? (a.param_dtype == CQ_F32 ? 4 : 2) : F::kBytes);
+        const uint64_t scale_out_bytes = kGroup == 0 ? 0 : (a.param_dtype == CQ_F32 ? 4 : 2);
+        constexpr uint64_t kDiv = kGroup == 0 ? 1 : kGroup;
+        return launch_flat(
+            a, kUnrollQ,
+            [&](uint32_t grid, uint64_t) {
+                if constexpr (kSrc != kScaleStored) {
+                    if (a.rows > 1)
+                        hipLaunchKernelGGL((quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
+                                           dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
+                                           reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0u, qp, a.num_partials,
+                                           flat_rows(a));
+                    else
+                        hipLaunchKernelGGL((quantize_flat_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
+                                           dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
+                                           reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0ull,
+                                           static_cast<uint64_t>(grid) * kThreads * kUnrollQ, qp, a.num_partials);
+                }
+            },
+            [&](const LaneRows& rows, uint32_t tile_begin, uint32_t grid, RunOffsets off) {
+                const uint64_t scales = off.chunks / kDiv;
+                const void* scale_in = a.scale_in == nullptr ? nullptr : static_cast<const char*>(a.scale_in) + scales * scale_in_bytes;
+                void* scale_out = a.scale_out == nullptr ? nullptr : static_cast<char*>(a.scale_out) + scales * scale_out_bytes;
+                hipLaunchKernelGGL((quantize_flat_lanes_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
+                                   dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in + off.chunks * 16),
+                                   reinterpret_cast<uint32_t*>(out + off.chunks * kOutChunk), scale_in, scale_out,
+                                   a.param_dtype, qp, a.num_partials, tile_begin, rows);
             });
-        return launch_tiles(a.num_chunks, kUnrollQ, [&](bool checked, uint32_t grid, uint64_t begin, uint64_t end) {
-            auto kernel =
-                checked ? (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, true, kEnc>
-                               : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, true, kEnc>)
-                        : (p32 ? quantize_flat_kernel<F, kBits, kGroup, kSrc, true, kWide, kUnrollQ, kThreads, false, kEnc>
-                               : quantize_flat_kernel<F, kBits, kGroup, kSrc, false, kWide, kUnrollQ, kThreads, false, kEnc>);
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, s, in, out, a.scale_in, a.scale_out,
-                               a.param_dtype, begin, end, qp, a.num_partials);
-        });
     }
 }
 
@@ -220,13 +282,10 @@ hipError_t quantize_launch_enc(hipStream_t s, ScaleSource src, const FlatArgs& a
 template <class F, int kBits, int kGroup, bool kGiven>
 hipError_t quantize_launch(hipStream_t s, ScaleSource src, const FlatArgs& a) {
     switch (a.encoding) {
-        case kEncInt: {
-            // only 8-bit fields can be narrower than their value range (E4M3, E5M2)
-            const bool wide = kBits == 8 && (a.range.hi > 127.0f || a.range.lo < -128.0f);
-            if constexpr (kBits == 8)
-                if (wide) return quantize_launch_enc<F, kBits, kGroup, true, kEncInt, kGiven>(s, src, a);
+        case kEncInt:
+            // value ranges wider than their field (E4M3 / E5M2 in the U32 store) never come here
+            if (kBits == 8 && (a.range.hi > 127.0f || a.range.lo < -128.0f)) return hipErrorInvalidValue;
             return quantize_launch_enc<F, kBits, kGroup, false, kEncInt, kGiven>(s, src, a);
-        }
         case kEncE4M3:
             if constexpr (kBits == 8) return quantize_launch_enc<F, 8, kGroup, false, kEncE4M3, kGiven>(s, src, a);
             break;

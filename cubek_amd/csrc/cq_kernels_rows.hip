@@ -472,7 +472,7 @@ hipError_t quantize_rows(hipStream_t s, int bits, RowArgs a) {
         case kEncInt:
             if (bits == 2) CQ_LAUNCH(2, false, kEncInt)
             if (bits == 4) CQ_LAUNCH(4, false, kEncInt)
-            if (bits == 8 && wide) CQ_LAUNCH(8, true, kEncInt)
+            if (bits == 8 && wide) break;  // ranges wider than their field take the per-element kernels
             if (bits == 8) CQ_LAUNCH(8, false, kEncInt)
             break;
         case kEncE4M3: if (bits == 8) CQ_LAUNCH(8, false, kEncE4M3) break;
@@ -599,7 +599,7 @@ hipError_t quantize_blocks(hipStream_t s, int bits, const RowArgs& a) {
         case kEncInt:
             if (bits == 2) return quantize_blocks_rows<F, 2, false, kEncInt>(s, a, g, qp);
             if (bits == 4) return quantize_blocks_rows<F, 4, false, kEncInt>(s, a, g, qp);
-            if (bits == 8 && wide) return quantize_blocks_rows<F, 8, true, kEncInt>(s, a, g, qp);
+            if (bits == 8 && wide) break;  // ranges wider than their field take the per-element kernels
             if (bits == 8) return quantize_blocks_rows<F, 8, false, kEncInt>(s, a, g, qp);
             break;
         case kEncE4M3: if (bits == 8) return quantize_blocks_rows<F, 8, false, kEncE4M3>(s, a, g, qp); break;

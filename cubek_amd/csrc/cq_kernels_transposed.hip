@@ -603,7 +603,7 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
         case kEncInt:
             if (bits == 2) CQ_LAUNCH(2, false, kEncInt)
             if (bits == 4) CQ_LAUNCH(4, false, kEncInt)
-            if (bits == 8 && wide) CQ_LAUNCH(8, true, kEncInt)
+            if (bits == 8 && wide) break;  // ranges wider than their field take the per-element kernels
             if (bits == 8) CQ_LAUNCH(8, false, kEncInt)
             break;
         case kEncE4M3: if (bits == 8) CQ_LAUNCH(8, false, kEncE4M3) break;
