@@ -21,7 +21,7 @@ EXPORTED_SYMBOLS = (
     "cq_compute_scales", "cq_quantize_dynamic", "cq_workspace_bytes", "cq_strerror",
     "cq_last_hip_error", "cq_abi_version", "cq_reduce_max_abs", "cq_reduce_workspace_bytes",
     "cq_into_contiguous_packed", "cq_quantize_dynamic_static",
-    "cq_gemv_quantized",
+    "cq_gemv_quantized", "cq_plan_kind",
 )
 
 
@@ -88,6 +88,8 @@ def lib() -> ctypes.CDLL:
     L.cq_quantize_dynamic.argtypes = [ctypes.c_void_p, tp, tp, tp, sp, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
     L.cq_quantize_dynamic_static.restype = ctypes.c_int
     L.cq_quantize_dynamic_static.argtypes = [ctypes.c_void_p, tp, tp, tp, sp, ctypes.c_int]
+    L.cq_plan_kind.restype = ctypes.c_int
+    L.cq_plan_kind.argtypes = [ctypes.c_int, tp, tp, tp, tp, sp, ctypes.c_int, ctypes.POINTER(ctypes.c_uint32)]
     L.cq_gemv_quantized.restype = ctypes.c_int
     L.cq_gemv_quantized.argtypes = [ctypes.c_void_p, tp, tp, sp, tp, tp, ctypes.c_int, ctypes.c_int]
     L.cq_reduce_max_abs.restype = ctypes.c_int
@@ -117,3 +119,21 @@ def make_tensor(ptr: int, shape: Sequence[int], strides: Sequence[int], elem_siz
     strd = (ctypes.c_uint64 * rank)(*[int(s) for s in strides])
     t = CTensor(ctypes.c_void_p(ptr), shp, strd, rank, elem_size)
     return t, (shp, strd)
+
+
+#: enum cq_kernel_family
+FAMILY_NONE, FAMILY_FLAT, FAMILY_FLAT_ROWS, FAMILY_FLAT_LANES, FAMILY_ROWS, FAMILY_BLOCKS, FAMILY_TRANSPOSED, \
+    FAMILY_PER_ELEMENT = range(8)
+FAMILY_NAMES = ("none", "flat", "flat_rows", "flat_lanes", "rows", "blocks", "transposed", "per_element")
+#: enum cq_op
+OP_QUANTIZE, OP_QUANTIZE_DYNAMIC, OP_DEQUANTIZE, OP_COMPUTE_SCALES = range(4)
+
+
+def plan_kind(op: int, floats, values, scale, out_scale, scheme, elem) -> str:
+    """Name of the kernel family a call would run on (``cq_plan_kind``); tensors are ``TensorHandleRef`` or None."""
+    fam = ctypes.c_uint32(0)
+    c = lambda t: t.as_c() if t is not None else None
+    rc = lib().cq_plan_kind(op, c(floats), c(values), c(scale), c(out_scale), scheme.to_c(), int(elem), ctypes.byref(fam))
+    if rc:
+        check(rc)
+    return FAMILY_NAMES[fam.value]

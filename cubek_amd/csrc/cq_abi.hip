@@ -16,6 +16,28 @@ namespace {
 
 thread_local int g_last_hip_error = 0;
 
+// cq_plan_kind() runs an entry point's planning with launches switched off and notes which kernel family
+// each launch would have used: the family that moves the value tensors, or, for calls that only produce
+// scales, the family that reads the floats.
+struct PlanProbe {
+    bool on = false;
+    uint32_t main = CQ_FAMILY_NONE, aux = CQ_FAMILY_NONE;
+};
+thread_local PlanProbe g_probe;
+// true: probing, the launch is to be skipped
+bool probing(uint32_t family, bool aux) {
+    if (!g_probe.on) return false;
+    uint32_t& slot = aux ? g_probe.aux : g_probe.main;
+    if (slot == CQ_FAMILY_NONE) slot = family;
+    return true;
+}
+#define CQ_RUN(family, call) (probing(family, false) ? CQ_OK : hip_status(call))
+#define CQ_RUN_AUX(family, call) (probing(family, true) ? CQ_OK : hip_status(call))
+
+void drop_stale_hip_error() {
+    if (!g_probe.on) (void)hipGetLastError();
+}
+
 cq_status hip_status(hipError_t e) {
     if (e == hipSuccess) return CQ_OK;
     g_last_hip_error = static_cast<int>(e);
@@ -25,7 +47,7 @@ cq_status hip_status(hipError_t e) {
 // The launchers read hipGetLastError() after each launch.  An error left on the calling thread by earlier
 // HIP calls of the caller would be taken for a failed launch, so every entry point that launches kernels
 // clears it first (as any hipGetLastError() does).
-void drop_stale_hip_error() { (void)hipGetLastError(); }
+void drop_stale_hip_error();
 
 uint32_t dtype_size(int dtype) { return dtype == CQ_F32 ? 4u : 2u; }
 bool valid_dtype(int dtype) { return dtype == CQ_F32 || dtype == CQ_F16 || dtype == CQ_BF16; }
@@ -661,7 +683,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
         a.range = p.range;
-        st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, a));
+        st = CQ_RUN(cq::flat_family(a), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, a));
         if (st != CQ_OK) return st;
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
@@ -679,7 +701,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
-        return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, fr));
+        return CQ_RUN(cq::flat_family(fr), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, fr));
     }
     cq::RowArgs r;
     if (streaming && flat_words == 0 && rows_args(p, scheme, input_dtype, input, output, &r)) {
@@ -688,7 +710,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         r.scale_in = scale->ptr;
         r.scale_in_dtype = input_dtype;
         r.scale_out = out_scale->ptr;
-        return hip_status(cq::launch_quantize_rows(stream, input_dtype, static_cast<int>(p.bits), r));
+        return CQ_RUN(CQ_FAMILY_ROWS, cq::launch_quantize_rows(stream, input_dtype, static_cast<int>(p.bits), r));
     }
     cq::TransposedArgs tr;
     if (streaming && flat_words == 0 && transposed_args(p, scheme, input_dtype, input, output, &tr)) {
@@ -697,7 +719,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         tr.scale_in = scale->ptr;
         tr.scale_in_dtype = input_dtype;
         tr.scale_out = out_scale->ptr;
-        return hip_status(cq::launch_quantize_transposed(stream, input_dtype, static_cast<int>(p.bits), false, tr));
+        return CQ_RUN(CQ_FAMILY_TRANSPOSED, cq::launch_quantize_transposed(stream, input_dtype, static_cast<int>(p.bits), false, tr));
     }
     if (flat_words < p.n / p.nq) {
         cq::GenericArgs g = generic_args(p, scheme);
@@ -708,7 +730,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         g.scale_out = out_scale->ptr;
         g.word_begin = flat_words;
         g.word_end = p.n / p.nq;
-        st = hip_status(native ? cq::launch_quantize_native(stream, input_dtype, g)
+        st = CQ_RUN(CQ_FAMILY_PER_ELEMENT, native ? cq::launch_quantize_native(stream, input_dtype, g)
                                : cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
     }
     return st;
@@ -741,7 +763,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
         a.range = p.range;
-        st = hip_status(cq::launch_dequantize_flat(stream, output_dtype, p.bits, a));
+        st = CQ_RUN(cq::flat_family(a), cq::launch_dequantize_flat(stream, output_dtype, p.bits, a));
         if (st != CQ_OK) return st;
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
@@ -756,21 +778,21 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
-        return hip_status(cq::launch_dequantize_flat(stream, output_dtype, p.bits, fr));
+        return CQ_RUN(cq::flat_family(fr), cq::launch_dequantize_flat(stream, output_dtype, p.bits, fr));
     }
     cq::RowArgs r;
     if (streaming && flat_words == 0 && rows_args(p, scheme, output_dtype, output, values, &r)) {
         r.input = values->ptr;
         r.output = output->ptr;
         r.scale_in = params->ptr;
-        return hip_status(cq::launch_dequantize_rows(stream, output_dtype, static_cast<int>(p.bits), r));
+        return CQ_RUN(CQ_FAMILY_ROWS, cq::launch_dequantize_rows(stream, output_dtype, static_cast<int>(p.bits), r));
     }
     cq::TransposedArgs tr;
     if (streaming && flat_words == 0 && transposed_args(p, scheme, output_dtype, output, values, &tr)) {
         tr.input = values->ptr;
         tr.output = output->ptr;
         tr.scale_in = params->ptr;
-        return hip_status(cq::launch_dequantize_transposed(stream, output_dtype, static_cast<int>(p.bits), tr));
+        return CQ_RUN(CQ_FAMILY_TRANSPOSED, cq::launch_dequantize_transposed(stream, output_dtype, static_cast<int>(p.bits), tr));
     }
     if (flat_words < p.n / p.nq) {
         cq::GenericArgs g = generic_args(p, scheme);
@@ -779,7 +801,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         g.scale_in = params->ptr;
         g.word_begin = flat_words;
         g.word_end = p.n / p.nq;
-        st = hip_status(native ? cq::launch_dequantize_native(stream, output_dtype, g)
+        st = CQ_RUN(CQ_FAMILY_PER_ELEMENT, native ? cq::launch_dequantize_native(stream, output_dtype, g)
                                : cq::launch_dequantize_generic(stream, output_dtype, p.bits, g));
     }
     return st;
@@ -796,20 +818,20 @@ static cq_status absmax_partials(cq_stream_t stream, const Plan& p, const cq_sch
     cq::RowArgs r;
     if (p.vs.on && is_dense_permutation(input)) {
         // the order does not matter for a maximum: read the buffer front to back
-        return hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n, static_cast<float*>(workspace),
+        return CQ_RUN_AUX(CQ_FAMILY_FLAT, cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n, static_cast<float*>(workspace),
                                                      num_partials));
     }
     if (p.vs.on && rows_args(p, scheme, input_dtype, input, nullptr, &r)) {
         r.input = input->ptr;
-        return hip_status(cq::launch_absmax_partials_rows(stream, input_dtype, r, static_cast<float*>(workspace), num_partials));
+        return CQ_RUN_AUX(CQ_FAMILY_ROWS, cq::launch_absmax_partials_rows(stream, input_dtype, r, static_cast<float*>(workspace), num_partials));
     }
     if (p.vs.on) {
         cq::GenericArgs g = generic_args(p, scheme);
         g.input = input->ptr;
-        return hip_status(cq::launch_absmax_partials_strided(stream, input_dtype, g, p.n, static_cast<float*>(workspace),
+        return CQ_RUN_AUX(CQ_FAMILY_PER_ELEMENT, cq::launch_absmax_partials_strided(stream, input_dtype, g, p.n, static_cast<float*>(workspace),
                                                              num_partials));
     }
-    return hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n, static_cast<float*>(workspace),
+    return CQ_RUN_AUX(CQ_FAMILY_FLAT, cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n, static_cast<float*>(workspace),
                                                  num_partials));
 }
 
@@ -820,7 +842,7 @@ static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_sche
         uint32_t num_partials = 0;
         const cq_status st = absmax_partials(stream, p, scheme, input, input_dtype, workspace, workspace_bytes, &num_partials);
         if (st != CQ_OK) return st;
-        return hip_status(cq::launch_tensor_scale(stream, input_dtype, out_dtype,
+        return CQ_RUN_AUX(CQ_FAMILY_FLAT, cq::launch_tensor_scale(stream, input_dtype, out_dtype,
                                                   static_cast<const float*>(workspace), num_partials,
                                                   p.range, scales->ptr));
     }
@@ -828,18 +850,18 @@ static cq_status produce_scales(cq_stream_t stream, const Plan& p, const cq_sche
     if (scales_rows_ok(p) && rows_args(p, scheme, input_dtype, input, nullptr, &r)) {
         r.input = input->ptr;
         r.scale_out = scales->ptr;
-        return hip_status(cq::launch_scales_rows(stream, input_dtype, out_dtype, r));
+        return CQ_RUN_AUX(CQ_FAMILY_ROWS, cq::launch_scales_rows(stream, input_dtype, out_dtype, r));
     }
     cq::TransposedArgs tr;
     if (transposed_args(p, scheme, input_dtype, input, nullptr, &tr)) {
         tr.input = input->ptr;
         tr.scale_out = scales->ptr;
-        return hip_status(cq::launch_scales_transposed(stream, input_dtype, out_dtype, tr));
+        return CQ_RUN_AUX(CQ_FAMILY_TRANSPOSED, cq::launch_scales_transposed(stream, input_dtype, out_dtype, tr));
     }
     cq::GenericArgs g = generic_args(p, scheme);
     g.input = input->ptr;
     g.scale_out = scales->ptr;
-    return hip_status(cq::launch_scales_generic(stream, input_dtype, out_dtype, g, p.num_blocks));
+    return CQ_RUN_AUX(CQ_FAMILY_PER_ELEMENT, cq::launch_scales_generic(stream, input_dtype, out_dtype, g, p.num_blocks));
 }
 
 cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq_tensor* scales,
@@ -873,7 +895,7 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
         a.num_chunks = p.n / (16 / dtype_size(input_dtype));
         a.block = p.block_last;
         a.range = p.range;
-        return hip_status(cq::launch_scales_flat(stream, input_dtype, a));
+        return CQ_RUN_AUX(cq::flat_family(a), cq::launch_scales_flat(stream, input_dtype, a));
     }
     // pitched rows of at least a step of 256 chunks, 1-D blocks: the same kernel over the rows' steps
     // (rows in one uniform run or in groups with a pitch of their own, as in flat_rows_ok())
@@ -901,7 +923,7 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
             a.scale_out_outer = outer_of(ls) * elem;
             a.block = p.block_last;
             a.range = p.range;
-            return hip_status(cq::launch_scales_flat(stream, input_dtype, a));
+            return CQ_RUN_AUX(cq::flat_family(a), cq::launch_scales_flat(stream, input_dtype, a));
         }
     }
     // short rows, rows behind several levels of strides: every lane finds its row
@@ -912,7 +934,7 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
         fl.scale_out = scales->ptr;
         fl.block = p.block_last;
         fl.range = p.range;
-        return hip_status(cq::launch_scales_flat(stream, input_dtype, fl));
+        return CQ_RUN_AUX(cq::flat_family(fl), cq::launch_scales_flat(stream, input_dtype, fl));
     }
     return produce_scales(stream, p, scheme, input, input_dtype, scales, input_dtype, workspace, workspace_bytes);
 }
@@ -944,7 +966,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         g.scale_out = nullptr;
         g.word_begin = 0;
         g.word_end = p.n / p.nq;
-        return hip_status(cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
+        return CQ_RUN(CQ_FAMILY_PER_ELEMENT, cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
     }
     const bool flat = flat_ok(p, input_dtype, input, output, out_scale, nullptr);
 
@@ -961,7 +983,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
         a.range = p.range;
-        return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
+        return CQ_RUN(cq::flat_family(a), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
     }
 
     // pitched rows with 1-D blocks: the same fused kernel over the rows' steps
@@ -976,7 +998,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
-        return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, fr));
+        return CQ_RUN(cq::flat_family(fr), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, fr));
     }
 
     // blocks over the last two dimensions (or 1-D blocks on layouts the flat kernel refuses): one
@@ -997,7 +1019,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
             f2.param_dtype = pd;
             f2.encoding = flat_encoding(scheme);
             f2.range = p.range;
-            return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Stored, f2));
+            return CQ_RUN(cq::flat_family(f2), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Stored, f2));
         }
     }
 
@@ -1007,7 +1029,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         rb.input = input->ptr;
         rb.output = output->ptr;
         rb.scale_out = out_scale->ptr;
-        return hip_status(cq::launch_quantize_blocks_dynamic(stream, input_dtype, static_cast<int>(p.bits), rb));
+        return CQ_RUN(CQ_FAMILY_BLOCKS, cq::launch_quantize_blocks_dynamic(stream, input_dtype, static_cast<int>(p.bits), rb));
     }
 
     cq::TransposedArgs tr;
@@ -1016,7 +1038,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         tr.input = input->ptr;
         tr.output = output->ptr;
         tr.scale_out = out_scale->ptr;
-        return hip_status(cq::launch_quantize_transposed(stream, input_dtype, static_cast<int>(p.bits), true, tr));
+        return CQ_RUN(CQ_FAMILY_TRANSPOSED, cq::launch_quantize_transposed(stream, input_dtype, static_cast<int>(p.bits), true, tr));
     }
 
     uint64_t flat_words = 0;
@@ -1030,7 +1052,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         if (!workspace || workspace_bytes < cq::kMaxPartials * sizeof(float)) return CQ_ERR_WORKSPACE_TOO_SMALL;
         if (!aligned(workspace, 4)) return CQ_ERR_INVALID_ARGUMENT;
         uint32_t num_partials = 0;
-        st = hip_status(cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n,
+        st = CQ_RUN_AUX(CQ_FAMILY_FLAT, cq::launch_absmax_partials(stream, input_dtype, input->ptr, p.n,
                                                    static_cast<float*>(workspace), &num_partials));
         if (st != CQ_OK) return st;
         cq::FlatArgs a{};
@@ -1044,7 +1066,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
         a.range = p.range;
-        st = hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, a));
+        st = CQ_RUN(cq::flat_family(a), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, a));
         if (st != CQ_OK) return st;
         flat_words = flat_chunks * per_chunk / p.nq;
     } else if (p.tensor_level && (flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) ||
@@ -1062,7 +1084,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
-        return hip_status(cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, fr));
+        return CQ_RUN(cq::flat_family(fr), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, fr));
     } else {
         // scales as FS(F(scale)) into out_scale first, then quantize reading them back
         // (the divisor F(FS(scale)) is the same either way)
@@ -1076,7 +1098,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         r.scale_in = out_scale->ptr;
         r.scale_in_dtype = pd;
         r.scale_out = nullptr;
-        return hip_status(cq::launch_quantize_rows(stream, input_dtype, static_cast<int>(p.bits), r));
+        return CQ_RUN(CQ_FAMILY_ROWS, cq::launch_quantize_rows(stream, input_dtype, static_cast<int>(p.bits), r));
     }
     if (flat_words == 0 && transposed) {
         tr.input = input->ptr;
@@ -1084,7 +1106,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         tr.scale_in = out_scale->ptr;
         tr.scale_in_dtype = pd;
         tr.scale_out = nullptr;
-        return hip_status(cq::launch_quantize_transposed(stream, input_dtype, static_cast<int>(p.bits), false, tr));
+        return CQ_RUN(CQ_FAMILY_TRANSPOSED, cq::launch_quantize_transposed(stream, input_dtype, static_cast<int>(p.bits), false, tr));
     }
     if (flat_words < p.n / p.nq) {
         cq::GenericArgs g = generic_args(p, scheme);
@@ -1095,7 +1117,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         g.scale_out = nullptr;
         g.word_begin = flat_words;
         g.word_end = p.n / p.nq;
-        st = hip_status(native ? cq::launch_quantize_native(stream, input_dtype, g)
+        st = CQ_RUN(CQ_FAMILY_PER_ELEMENT, native ? cq::launch_quantize_native(stream, input_dtype, g)
                                : cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
     }
     return st;
@@ -1211,6 +1233,30 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
     a.x_aligned16 = aligned(x->ptr, 16);
     a.words_aligned16 = aligned(values->ptr, 16);
     return hip_status(cq::launch_gemv_quantized(stream, a));
+}
+
+cq_status cq_plan_kind(cq_op op, const cq_tensor* floats, const cq_tensor* values, const cq_tensor* scale,
+                       const cq_tensor* out_scale, const cq_scheme* scheme, cq_dtype dtype, uint32_t* family) {
+    if (!family) return CQ_ERR_INVALID_ARGUMENT;
+    *family = CQ_FAMILY_NONE;
+    // a workspace that satisfies every check; with the launches switched off nothing touches it
+    alignas(256) static char workspace[CQ_STATIC_SCRATCH_BYTES];
+    g_probe = PlanProbe{};
+    g_probe.on = true;
+    cq_status st = CQ_ERR_INVALID_ARGUMENT;
+    switch (op) {
+        case CQ_OP_QUANTIZE: st = cq_quantize(nullptr, floats, values, scale, out_scale, scheme, dtype); break;
+        case CQ_OP_QUANTIZE_DYNAMIC:
+            st = quantize_dynamic(nullptr, floats, values, out_scale, scheme, dtype, workspace, sizeof(workspace));
+            break;
+        case CQ_OP_DEQUANTIZE: st = cq_dequantize(nullptr, values, floats, scale, scheme, dtype); break;
+        case CQ_OP_COMPUTE_SCALES:
+            st = cq_compute_scales(nullptr, floats, scale, scheme, dtype, workspace, sizeof(workspace));
+            break;
+    }
+    *family = g_probe.main != CQ_FAMILY_NONE ? g_probe.main : g_probe.aux;
+    g_probe = PlanProbe{};
+    return st;
 }
 
 static bool reduce_view(const cq_tensor* input, uint32_t axis, uint64_t* outer, uint64_t* len, uint64_t* inner) {

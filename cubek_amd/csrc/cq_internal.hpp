@@ -62,6 +62,9 @@ hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource 
 hipError_t launch_dequantize_flat(hipStream_t s, int dtype, int bits, const FlatArgs& a);
 hipError_t launch_scales_flat(hipStream_t s, int dtype, const FlatArgs& a);  // block abs-max -> scales typed like input
 bool flat_block_supported(int dtype, uint32_t block);
+// the cq_kernel_family a flat launch with these arguments runs on (whole tiles of a run, whole steps of
+// pitched rows, or lane by lane)
+uint32_t flat_family(const FlatArgs& a);
 
 // Per-tensor abs-max, pass 1: writes `*num_partials` f32 partial maxima.
 constexpr uint32_t kMaxPartials = 256;

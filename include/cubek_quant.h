@@ -244,6 +244,40 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
                             const cq_scheme* scheme, const cq_tensor* x, const cq_tensor* y,
                             cq_dtype dtype, cq_dtype y_dtype);
 
+/* ---- which kernels a call would run on ---- */
+
+/* No counterpart in the reference (its one kernel per entry point takes every layout at the same, low,
+ * speed).  Here the layout of the tensors decides between kernel families whose throughput differs by more
+ * than a factor of ten; this query tells a caller which one a call would take, without launching anything,
+ * so that a slow path does not go unnoticed. */
+typedef enum cq_kernel_family {
+    CQ_FAMILY_NONE = 0,        /* nothing to launch (empty tensor)                                            */
+    CQ_FAMILY_FLAT = 1,        /* contiguous tensors, whole 16 KiB tiles: the streaming kernels (HBM rate)     */
+    CQ_FAMILY_FLAT_ROWS = 2,   /* the same kernels over pitched rows of whole 4 KiB steps                      */
+    CQ_FAMILY_FLAT_LANES = 3,  /* the same arithmetic, every lane finding its own row: short, ragged or
+                                  permuted rows, f16 / bf16 parameters, small tensors (55 - 80 % of HBM rate)  */
+    CQ_FAMILY_ROWS = 4,        /* contiguous last dimension, any blocks and strides (35 - 70 %)                */
+    CQ_FAMILY_BLOCKS = 5,      /* fused abs-max + quantize for blocks over the last two dimensions (55 - 70 %) */
+    CQ_FAMILY_TRANSPOSED = 6,  /* float tensor whose contiguous dimension is the second to last (45 - 70 %)    */
+    CQ_FAMILY_PER_ELEMENT = 7  /* everything else, one thread per stored element (3 - 30 %)                    */
+} cq_kernel_family;
+
+typedef enum cq_op {
+    CQ_OP_QUANTIZE = 0,          /* cq_quantize: scale and out_scale given                    */
+    CQ_OP_QUANTIZE_DYNAMIC = 1,  /* cq_quantize_dynamic: `scale` ignored (may be NULL)        */
+    CQ_OP_DEQUANTIZE = 2,        /* cq_dequantize: `scale` = params, `out_scale` ignored      */
+    CQ_OP_COMPUTE_SCALES = 3     /* cq_compute_scales: `values` and `out_scale` ignored       */
+} cq_op;
+
+/* The family of the kernel that would move the value tensors of the call (for CQ_OP_COMPUTE_SCALES: that
+ * would read the floats).  Same argument checks and status codes as the entry point itself; only the
+ * layouts are looked at, no pointer is dereferenced.
+ *   floats : the float tensor (input of quantize, output of dequantize), typed `dtype`
+ *   values : the quantized tensor */
+cq_status cq_plan_kind(cq_op op, const cq_tensor* floats, const cq_tensor* values, const cq_tensor* scale,
+                       const cq_tensor* out_scale, const cq_scheme* scheme, cq_dtype dtype,
+                       uint32_t* family);
+
 /* ---- diagnostics ---- */
 const char* cq_strerror(cq_status status);
 /* hipError_t of the most recent failed HIP call on the calling thread (0 if none). */

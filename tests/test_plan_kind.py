@@ -1,0 +1,116 @@
+"""cq_plan_kind: which kernel family a call would run on.  Nothing is launched and no pointer is
+dereferenced, so this runs without a GPU.  Every BASELINE configuration must land on the streaming kernels,
+and every layout the design names must land on the family the design claims for it."""
+import pytest
+
+from cubek_amd import ElemType, QuantLevel, QuantParam, QuantScheme, QuantStore, QuantValue, TensorHandleRef, _ffi
+
+BASE = 0x7F0000000000  # 4 KiB aligned fake device addresses, far apart
+F32, BF16 = ElemType.F32, ElemType.BF16
+
+
+def t(shape, elem_size, strides=None, offset=0, slot=0):
+    if strides is None:
+        strides, acc = [], 1
+        for n in reversed(shape):
+            strides.append(acc)
+            acc *= n
+        strides = tuple(reversed(strides))
+    return TensorHandleRef(BASE + slot * (1 << 36) + offset, tuple(shape), tuple(strides), elem_size)
+
+
+def kinds(scheme, elem, shape, f_strides=None, v_strides=None, s_strides=None, f_offset=0, ops=None):
+    esz = 4 if elem == F32 else 2
+    floats = t(shape, esz, f_strides, f_offset, 0)
+    values = t(scheme.packed_shape(shape), 4 if scheme.store == QuantStore.U32 else 1, v_strides, 0, 1)
+    sshape = scheme.scales_shape(shape)
+    psz = 4 if scheme.param == QuantParam.F32 else 2
+    scale_in = t(sshape, esz, s_strides, 0, 2)        # typed like the input
+    params = t(sshape, psz, s_strides, 0, 3)          # typed scheme.param
+    out = {}
+    for name, op, sc, osc in (("quantize", _ffi.OP_QUANTIZE, scale_in, params),
+                              ("dynamic", _ffi.OP_QUANTIZE_DYNAMIC, None, params),
+                              ("dequantize", _ffi.OP_DEQUANTIZE, params, None),
+                              ("scales", _ffi.OP_COMPUTE_SCALES, scale_in, None)):
+        if ops is None or name in ops:
+            out[name] = _ffi.plan_kind(op, floats, values, sc, osc, scheme, elem)
+    return out
+
+
+def scheme_of(value, block=None, store=QuantStore.U32, param=QuantParam.F32):
+    level = QuantLevel.Tensor if block is None else QuantLevel.block(block)
+    return QuantScheme.default().with_value(value).with_level(level).with_store(store).with_param(param)
+
+
+@pytest.mark.parametrize("name,elem,value,block,shape", [
+    ("cfg1", F32, QuantValue.Q8S, None, (1024, 1024)),
+    ("cfg2", BF16, QuantValue.Q8S, [32], (4096, 4096)),
+    ("cfg3", BF16, QuantValue.Q4S, [32], (14336, 4096)),
+    ("cfg4", F32, QuantValue.Q2S, [64], (8192, 8192)),
+    ("cfg5", BF16, QuantValue.E2M1, [32], (28672, 8192)),
+])
+def test_baseline_configurations_take_the_streaming_kernels(name, elem, value, block, shape):
+    got = kinds(scheme_of(value, block), elem, shape)
+    assert got == {"quantize": "flat", "dynamic": "flat", "dequantize": "flat", "scales": "flat"}, name
+
+
+def test_layouts_land_on_the_family_the_design_claims():
+    e2m1 = scheme_of(QuantValue.E2M1, [32])
+    rows, cols = 28672, 8192
+    # pitched rows of whole 4 KiB steps: the flat kernels over row steps
+    got = kinds(e2m1, BF16, (rows, cols), f_strides=(cols + 64, 1))
+    assert got == {"quantize": "flat_rows", "dynamic": "flat_rows", "dequantize": "flat_rows", "scales": "flat_rows"}
+    # ragged pitched rows (576 chunks = 2.25 steps), short rows: lane by lane
+    assert set(kinds(e2m1, BF16, (32768, 4608), f_strides=(4672, 1)).values()) == {"flat_lanes"}
+    assert set(kinds(e2m1, BF16, (262144, 256), f_strides=(320, 1)).values()) == {"flat_lanes"}
+    # f16 / bf16 parameters: lane by lane (scale production has no stored parameters and stays on whole tiles)
+    got = kinds(scheme_of(QuantValue.E2M1, [32], param=QuantParam.BF16), BF16, (rows, cols))
+    assert got == {"quantize": "flat_lanes", "dynamic": "flat_lanes", "dequantize": "flat_lanes", "scales": "flat"}
+    # attention layout: [batch, heads, positions, head dimension] view of a [batch, positions, heads, head dimension] buffer
+    nb, nh, ns, nd = 8, 32, 4096, 128
+    got = kinds(e2m1, BF16, (nb, nh, ns, nd), f_strides=(ns * nh * nd, nd, nh * nd, 1))
+    assert set(got.values()) == {"flat_lanes"}
+    # a tensor too small for a whole tile
+    assert kinds(e2m1, BF16, (4, 64), ops=("dynamic",)) == {"dynamic": "flat_lanes"}
+    # 128 x 128 weight blocks, e4m3 bytes: fused block kernel; given scales: the flat kernels over row steps
+    blocks = scheme_of(QuantValue.E4M3, [128, 128], store=QuantStore.Native)
+    got = kinds(blocks, BF16, (rows, cols))
+    assert got == {"quantize": "flat_rows", "dynamic": "blocks", "dequantize": "flat_rows", "scales": "rows"}
+    # transposed float tensor
+    got = kinds(e2m1, BF16, (rows, cols), f_strides=(1, rows))
+    assert got == {"quantize": "transposed", "dynamic": "transposed", "dequantize": "transposed", "scales": "transposed"}
+    # blocks that are not a power-of-two number of lanes: row kernels (fused block kernel for dynamic)
+    got = kinds(scheme_of(QuantValue.Q4S, [24]), BF16, (8192, 8184))
+    assert got == {"quantize": "rows", "dynamic": "blocks", "dequantize": "rows", "scales": "rows"}
+    # scales stored column-major: row kernels
+    got = kinds(e2m1, BF16, (8192, 8192), s_strides=(1, 8192), ops=("quantize", "dequantize"))
+    assert got == {"quantize": "rows", "dequantize": "rows"}
+
+
+def test_slow_paths_are_reported():
+    e2m1 = scheme_of(QuantValue.E2M1, [32])
+    # rows that start on odd multiples of 2 bytes
+    got = kinds(e2m1, BF16, (8192, 8192), f_strides=(8193, 1), ops=("quantize", "dynamic", "dequantize"))
+    assert set(got.values()) == {"per_element"}
+    # a quantized tensor whose last dimension is not the contiguous one
+    got = kinds(e2m1, BF16, (4096, 4096), v_strides=(1, 4096), ops=("quantize", "dequantize"))
+    assert set(got.values()) == {"per_element"}
+    # E4M3 in the u32 store (codes wrap their field): per-element quantize, streaming dequantize
+    got = kinds(scheme_of(QuantValue.E4M3, [32]), BF16, (4096, 4096), ops=("quantize", "dynamic", "dequantize"))
+    assert got == {"quantize": "per_element", "dynamic": "per_element", "dequantize": "flat"}
+    # blocks smaller than a packed word on dequantize
+    got = kinds(scheme_of(QuantValue.Q8S, [2]), BF16, (4096, 4096), ops=("dequantize",))
+    assert got == {"dequantize": "per_element"}
+
+
+def test_plan_kind_validates_like_the_entry_points():
+    s = scheme_of(QuantValue.Q8S, [32])
+    with pytest.raises(_ffi.QuantError) as e:
+        _ffi.plan_kind(_ffi.OP_QUANTIZE, t((8, 64), 4), t((8, 15), 4), t((8, 2), 4), t((8, 2), 4), s, F32)
+    assert e.value.status == _ffi.ERR_SHAPE_MISMATCH
+    bad = scheme_of(QuantValue.Q8S, [2])
+    with pytest.raises(_ffi.QuantError) as e:
+        _ffi.plan_kind(_ffi.OP_QUANTIZE, t((8, 64), 4), t((8, 16), 4), t((8, 32), 4), t((8, 32), 4), bad, F32)
+    assert e.value.status == _ffi.ERR_BLOCK_NOT_DIVISIBLE
+    # an empty tensor launches nothing
+    assert _ffi.plan_kind(_ffi.OP_DEQUANTIZE, t((0, 64), 4), t((0, 16), 4), t((0, 2), 4), None, s, F32) == "none"
