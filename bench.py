@@ -17,7 +17,9 @@ roofline   = the quantize kernel alone: algorithmic bytes / its average launch d
              over a region of K back-to-back launches between two HIP events on the
              launch stream, against the 8 TB/s HBM peak
 cpu_baseline = the CPU oracle (oracle/cq_oracle.c, the scalar restatement of the
-             reference algorithm) on a bounded row sample of the same tensor
+             reference algorithm) on a bounded row sample of the same tensor, best of three
+             runs on every hardware thread the job may use
+inputs     = generated on the host with numpy's PCG64 (make_input), uploaded, rounded to the tensor's type
 
 Prints ONE JSON line on stdout.
 """
@@ -48,13 +50,14 @@ WORKLOADS = {
                  desc="per-block(32) e2m1 (4-bit fields), bf16 [28672,8192] ~N(0,0.02) + 1% Student-t(3)"),
 }
 
-# HBM bytes per launch of the quantize kernel measured with rocprofv3 --pmc
-# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); filled from
-# the summaries under profiles/.  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/quantize_dequantize_flat_bf16_e2m1_b32_cfg5.md: (229432.5*2.0 + 143360.0) KiB
-    "cfg5": 616678400,
-}
+def measured_traffic():
+    """HBM bytes per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a copy of known size) of the
+    three kernels of every configuration, as recorded in profiles/traffic.json; {} when the file is absent."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return {}
+    with open(path) as f:
+        return json.load(f).get("hbm_bytes_per_launch", {})
 
 
 def algorithmic_bytes(w) -> int:
@@ -66,38 +69,52 @@ def algorithmic_bytes(w) -> int:
     return n * elem_bytes + n * bits // 8 + scales * 4
 
 
+GEN_CHUNK_ELEMS = 1 << 24  # the host generator draws whole rows, this many elements at a time
+
+
 def make_input(torch, w):
-    """Seeded synthetic tensor generated on the device, chunked to bound memory."""
+    """The seeded synthetic tensor of a configuration, generated on the HOST and uploaded, so that the bytes do
+    not depend on the GPU or on the torch version.
+
+    Generator: numpy.random.Generator(numpy.random.PCG64(seed)), seed = the configuration's number.  The
+    tensor is produced in chunks of max(1, 2^24 // cols) whole rows, first row first; per chunk, in this
+    order of draws (n = elements of the chunk, all float32):
+      normal1          z = standard_normal(n)                                   x = z
+      normal           z = standard_normal(n)                                   x = 0.02 z
+      normal_outliers  z = standard_normal(n); u = random(n)                    x = 0.02 z * (50 if u < 0.001 else 1)
+      laplace          u = random(n) - 0.5                                      x = -0.01 sign(u) log1p(-2 min(|u|, 0.4999999))
+      normal_t3        z = standard_normal(n); u = random(n);
+                       t = standard_t(3, size = number of u < 0.01)             x = 0.02 t where u < 0.01, else 0.02 z
+    The float32 chunk is copied to the device and rounded there to the tensor's type (round to nearest even)."""
+    import numpy as np
+
     rows, cols = w["shape"]
-    g = torch.Generator(device="cuda")
-    g.manual_seed(w["seed"])
+    rng = np.random.Generator(np.random.PCG64(w["seed"]))
     dt = torch.float32 if w["elem"] == "F32" else torch.bfloat16
     out = torch.empty((rows, cols), dtype=dt, device="cuda")
-    step = max(1, (64 << 20) // (cols * 4))
+    step = max(1, GEN_CHUNK_ELEMS // cols)
+    dist = w["dist"]
     for r0 in range(0, rows, step):
         r1 = min(rows, r0 + step)
-        shp = (r1 - r0, cols)
-        dist = w["dist"]
+        n = (r1 - r0) * cols
         if dist == "normal1":
-            x = torch.randn(shp, generator=g, device="cuda")
+            x = rng.standard_normal(n, dtype=np.float32)
         elif dist == "normal":
-            x = torch.randn(shp, generator=g, device="cuda") * 0.02
+            x = rng.standard_normal(n, dtype=np.float32) * np.float32(0.02)
         elif dist == "normal_outliers":
-            x = torch.randn(shp, generator=g, device="cuda") * 0.02
-            m = torch.rand(shp, generator=g, device="cuda") < 0.001
-            x = torch.where(m, x * 50.0, x)
+            x = rng.standard_normal(n, dtype=np.float32) * np.float32(0.02)
+            u = rng.random(n, dtype=np.float32)
+            x[u < np.float32(0.001)] *= np.float32(50.0)
         elif dist == "laplace":
-            u = torch.rand(shp, generator=g, device="cuda") - 0.5
-            x = -0.01 * torch.sign(u) * torch.log1p(-2.0 * u.abs().clamp(max=0.4999999))
+            u = rng.random(n, dtype=np.float32) - np.float32(0.5)
+            x = np.float32(-0.01) * np.sign(u) * np.log1p(np.float32(-2.0) * np.minimum(np.abs(u), np.float32(0.4999999)))
         elif dist == "normal_t3":
-            x = torch.randn(shp, generator=g, device="cuda") * 0.02
-            m = torch.rand(shp, generator=g, device="cuda") < 0.01
-            z = torch.randn(shp, generator=g, device="cuda")
-            chi = (torch.randn((3,) + shp, generator=g, device="cuda") ** 2).sum(0) / 3.0
-            x = torch.where(m, 0.02 * z / chi.sqrt(), x)
+            x = rng.standard_normal(n, dtype=np.float32) * np.float32(0.02)
+            m = rng.random(n, dtype=np.float32) < np.float32(0.01)
+            x[m] = np.float32(0.02) * rng.standard_t(3, int(m.sum())).astype(np.float32)
         else:
             raise ValueError(dist)
-        out[r0:r1] = x.to(dt)
+        out[r0:r1] = torch.from_numpy(x.astype(np.float32, copy=False).reshape(r1 - r0, cols)).to("cuda").to(dt)
     return out
 
 
@@ -172,14 +189,22 @@ def replicas(torch, w, x, min_footprint=1 << 30, max_sets=8):
     return paths
 
 
+def cpu_threads() -> int:
+    """Worker threads for the CPU baseline: every hardware thread this process may use, and never more than the
+    16 a one-GPU box of this pool gives a job (its CPU share, whatever the core count of the host shows)."""
+    return min(16, len(os.sched_getaffinity(0)))
+
+
 def cpu_baseline(torch, w, path, budget_s=12.0):
-    """The CPU oracle on a bounded sample of rows: quantize (given scales) + dequantize."""
+    """CPU restatement of the reference algorithm (the oracle, oracle/cq_oracle.c: scalar C, -O2, one pthread per
+    slice of words) on a bounded sample of rows of the same tensor: quantize with given scales + dequantize, the
+    reference's two launches.  Best of three runs on all threads, and one thread on a shorter sample."""
     import numpy as np
 
     from oracle import oracle
 
     rows, cols = w["shape"]
-    threads = min(16, len(os.sched_getaffinity(0)))
+    threads = cpu_threads()
     elem = path.elem
 
     def host_rows(nrows):
@@ -198,23 +223,58 @@ def cpu_baseline(torch, w, path, budget_s=12.0):
         return time.perf_counter() - t0
 
     probe_rows = max(threads, min(rows, (1 << 21) // cols))
+    run(probe_rows)  # first touch: page in the library, start the threads
     t_probe = run(probe_rows)
-    nrows = int(min(rows, max(probe_rows, probe_rows * budget_s / max(t_probe, 1e-3))))
+    # three runs of the sample inside the budget
+    nrows = int(min(rows, max(probe_rows, probe_rows * (budget_s / 3.0) / max(t_probe, 1e-3))))
     nrows = max(threads, nrows // threads * threads)
-    t = min(run(nrows) for _ in range(3 if nrows == rows else 1))
+    times = sorted(run(nrows) for _ in range(3))
+    t = times[0]
     sample_bytes = 2 * algorithmic_bytes(dict(w, shape=(nrows, cols)))
     # the same on one thread, on a sample an eighth as long
     rows1 = max(1, nrows // 8)
-    t1 = run(rows1, 1)
+    t1 = min(run(rows1, 1) for _ in range(2))
     bytes1 = 2 * algorithmic_bytes(dict(w, shape=(rows1, cols)))
     return {
         "value": sample_bytes / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+        "what": "CPU restatement of the reference algorithm (this repository's oracle), not the reference's own "
+                "CPU runtime, which cannot be built here",
         "sample": f"first {nrows} of {rows} rows of the headline tensor ({nrows * cols} elements), "
-                  f"quantize with given scales + dequantize, {t:.2f} s on {threads} threads",
+                  f"quantize with given scales + dequantize, best of 3 runs: {t:.2f} s on {threads} threads "
+                  f"(all three: {', '.join(f'{v:.2f}' for v in times)} s)",
         "elements_per_s": nrows * cols / t,
         "one_thread": {"value": round(bytes1 / t1 / 1e9, 3), "unit": "GB/s", "cores": 1,
-                       "sample": f"first {rows1} rows, {t1:.2f} s"},
+                       "sample": f"first {rows1} rows, best of 2 runs: {t1:.2f} s"},
     }
+
+
+def packed_gemv(torch):
+    """The consumer side of the packed format: cq_gemv_quantized over 4-bit weights with f32 scales on blocks of
+    32 (configuration 3's weight-load path and two larger weights), weights rotated through enough sets that
+    no launch finds them in the Infinity Cache.  HBM roofline on the packed bytes."""
+    from cubek_amd import ComputeClient, ElemType, QuantLevel, QuantScheme, QuantValue, TensorHandleRef, matvec
+
+    client = ComputeClient.current()
+    h = TensorHandleRef.from_torch
+    scheme = QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([32]))
+    out = []
+    for rows, cols in ((14336, 4096), (4096, 14336), (28672, 8192)):
+        b = rows * cols // 2 + rows * cols // 32 * 4 + cols * 2 + rows * 2
+        sets = max(2, min(16, -(-(1 << 30) // b)))
+        ws = [torch.randint(-2**31, 2**31 - 1, (rows, cols // 8), dtype=torch.int32, device="cuda") for _ in range(sets)]
+        ss = [torch.rand((rows, cols // 32), dtype=torch.float32, device="cuda") * 0.01 + 0.001 for _ in range(sets)]
+        x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+        y = torch.zeros(rows, device="cuda", dtype=torch.bfloat16)
+        hw, hs, hx, hy = [h(t) for t in ws], [h(t) for t in ss], h(x), h(y)
+        fn = lambda i: matvec.launch_ref(client, hw[i % sets], hs[i % sets], scheme, hx, hy, ElemType.BF16, ElemType.BF16)
+        ms = sorted(timed_region(torch, fn, 48)[0] for _ in range(3))[1]
+        out.append({"kernel": f"gemv_quantized, q4 blocks of 32, f32 scales, bf16 x and y, weights [{rows}, {cols}]",
+                    "algorithmic_bytes": b, "buffer_sets_rotated": sets, "ms": round(ms, 4),
+                    "GBps": round(b / (ms * 1e-3) / 1e9, 1), "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                    "weights_per_s": round(rows * cols / (ms * 1e-3))})
+        del ws, ss, hw, hs
+        torch.cuda.empty_cache()
+    return out
 
 
 def adjacent_kernels(torch):
@@ -394,6 +454,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--adjacent-only", action="store_true",
                     help="run only the abs-max / re-pack kernels on the headline tensor (for profiling)")
+    ap.add_argument("--gemv-only", action="store_true",
+                    help="run only the matrix-vector product over packed weights (for profiling)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run 3 plain device copies of the input (known bytes) to calibrate rocprof counters")
     args = ap.parse_args()
@@ -410,7 +472,10 @@ def main():
     torch.cuda.set_device(0)
 
     if args.adjacent_only:
-        print(json.dumps({"adjacent_kernels": adjacent_kernels(torch)}))
+        print(json.dumps({"adjacent_kernels": adjacent_kernels(torch) + packed_gemv(torch)}))
+        return
+    if args.gemv_only:
+        print(json.dumps({"adjacent_kernels": packed_gemv(torch)}))
         return
 
     w = WORKLOADS[args.workload]
@@ -441,7 +506,8 @@ def main():
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     q_gbps = q_bytes / (q_ms * 1e-3) / 1e9
     d_gbps = q_bytes / (d_ms * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES.get(args.workload)
+    traffic_table = measured_traffic()
+    traffic = traffic_table.get(args.workload, {}).get("quantize_dynamic")
 
     result = {
         "metric": "quant/dequant GB/s (bytes read+written) and % of MI355X HBM peak, 1 GPU",
@@ -487,13 +553,13 @@ def main():
                 fn = lambda i, m=meth: getattr(ps[i % len(ps)], m)()
                 med_ms = sorted(timed_region(torch, fn, 32)[0] for _ in range(3))[1]
                 row[label] = {"ms": round(med_ms, 4), "GBps": round(b / (med_ms * 1e-3) / 1e9, 1),
-                              "frac_hbm_peak": round(b / (med_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+                              "frac_hbm_peak": round(b / (med_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                              "traffic": traffic_table.get(name, {}).get(label)}
             table.append(row)
             del ps, p, xi
             torch.cuda.empty_cache()
         result["per_config"] = table
-        if not os.environ.get("CQ_BENCH_SKIP_ADJACENT"):
-            result["adjacent_kernels"] = adjacent_kernels(torch)
+        result["adjacent_kernels"] = adjacent_kernels(torch) + packed_gemv(torch)
 
     print(json.dumps(result))
 
