@@ -278,11 +278,14 @@ template <dev::Float kF>
 hipError_t launch_stream(hipStream_t s, const GemvArgs& a) {
     const uint32_t blocks_per_row = a.cols / 32;
     const uint32_t strips = (blocks_per_row + 63) / 64;
-    // four waves per SIMD (256 compute units x 4 SIMDs), all resident at once and all with the same number
-    // of rows: one round of workgroups without a tail
-    const uint64_t want_waves = 4096;
-    uint32_t rows_per_group = static_cast<uint32_t>((static_cast<uint64_t>(a.rows) * strips + want_waves - 1) / want_waves);
+    // Seven rows per wave, fewer where that would leave fewer than four waves per SIMD (256 compute units x 4
+    // SIMDs).  Measured on MI355X with 4096 / 8192 / 16384 / 32768 waves per launch: weights [14336, 4096]
+    // 11.5 / 11.7 / 13.4 / 19.4 us, [28672, 8192] 34.5 / 31.7 / 30.0 / 31.5 us: about seven rows per wave in
+    // both, enough rows to pay for a wave's 64 bytes of x per lane and enough waves to even out their ends.
+    const uint64_t row_strips = static_cast<uint64_t>(a.rows) * strips;
+    uint32_t rows_per_group = static_cast<uint32_t>((row_strips + 4095) / 4096);
     if (rows_per_group < 1) rows_per_group = 1;
+    if (rows_per_group > 7) rows_per_group = 7;
     const dim3 grid((a.rows + rows_per_group - 1) / rows_per_group), block(64 * strips);
     dev::GlobalScaleLayout<1, 32> scale_at;
     scale_at.stride_row = static_cast<uint32_t>(a.scale_stride_row);

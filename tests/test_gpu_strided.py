@@ -256,16 +256,45 @@ def check_layouts(gpu, oracle, elem, name, scheme, shapes, only):
             assert np.all(got[mask] == fill), tag + ("dequantize wrote outside the view",)
 
 
+LARGE_TRANSPOSED_SCHEMES = {
+    "q4s_block32": QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([32])),
+    "q8s_tensor": QuantScheme.default().with_value(QuantValue.Q8S),
+    "e4m3_native_block32": (QuantScheme.default().with_value(QuantValue.E4M3).with_store(QuantStore.Native)
+                            .with_level(QuantLevel.block([32]))),
+    "e2m1_block32": QuantScheme.default().with_value(QuantValue.E2M1).with_level(QuantLevel.block([32])),
+    "q2s_block32": QuantScheme.default().with_value(QuantValue.Q2S).with_level(QuantLevel.block([32])),
+    "q8s_block32": QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([32])),
+    "q4s_block64": QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([64])),
+    "e5m2_native_tensor": QuantScheme.default().with_value(QuantValue.E5M2).with_store(QuantStore.Native),
+}
+
+
 @pytest.mark.parametrize("elem,rows,cols", [(ElemType.BF16, 12288, 8192), (ElemType.F32, 6144, 8192)],
                          ids=["bf16", "f32"])
 def test_large_transposed_floats_match_the_contiguous_path(gpu, elem, rows, cols):
     """A transposed float tensor of 192 MiB (grids of thousands of workgroups, offsets beyond
     32 bits in bytes): codes, scales and dequantized values must equal what the contiguous
     kernels, checked against the oracle elsewhere, give for the same logical tensor."""
+    transposed_against_contiguous(gpu, elem, rows, cols, ("q4s_block32", "q8s_tensor", "e4m3_native_block32"))
+
+
+@pytest.mark.parametrize("elem,rows,cols,names", [
+    (ElemType.BF16, 4104, 32864, ("q4s_block32", "e2m1_block32", "q2s_block32", "e5m2_native_tensor")),
+    (ElemType.F16, 2056, 32832, ("q8s_block32", "q4s_block64", "e4m3_native_block32")),
+    (ElemType.F32, 2052, 16416, ("q4s_block32", "q8s_block32")),
+    (ElemType.BF16, 4096, 65536, ("q2s_block32",)),
+], ids=["bf16", "f16", "f32", "bf16_2bit"])
+def test_transposed_tiles_with_ragged_edges_match_the_contiguous_path(gpu, elem, rows, cols, names):
+    """Transposed float tensors of thousands of 64 x 256-byte tiles whose last tiles are cut short along both
+    axes (the sizes at which whole tiles go through shared memory), against the contiguous kernels."""
+    transposed_against_contiguous(gpu, elem, rows, cols, names)
+
+
+def transposed_against_contiguous(gpu, elem, rows, cols, names):
     import torch
 
     client = ComputeClient.current()
-    tdt = torch.float32 if elem == ElemType.F32 else torch.bfloat16
+    tdt = {ElemType.F32: torch.float32, ElemType.BF16: torch.bfloat16, ElemType.F16: torch.float16}[elem]
     eb = 4 if elem == ElemType.F32 else 2
     g = torch.Generator(device="cuda")
     g.manual_seed(rows + int(elem))
@@ -275,11 +304,9 @@ def test_large_transposed_floats_match_the_contiguous_path(gpu, elem, rows, cols
     h = TensorHandleRef.from_torch
     h_x = h(x)
     h_xt = TensorHandleRef(h(xt).handle, (rows, cols), (1, rows), eb)
-    for name, scheme in (("q4s_block32", QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([32]))),
-                         ("q8s_tensor", QuantScheme.default().with_value(QuantValue.Q8S)),
-                         ("e4m3_native_block32", QuantScheme.default().with_value(QuantValue.E4M3)
-                          .with_store(QuantStore.Native).with_level(QuantLevel.block([32])))):
-        print(name, elem.name, flush=True)
+    for name in names:
+        scheme = LARGE_TRANSPOSED_SCHEMES[name]
+        print(name, elem.name, rows, cols, flush=True)
         native = scheme.store == QuantStore.Native
         pshape = scheme.packed_shape((rows, cols)) if not native else (rows, cols)
         sshape = scheme.scales_shape((rows, cols))
