@@ -128,11 +128,19 @@ class Path:
 
         self.torch, self.qz, self.dq = torch, qz, dq
         self.elem = ElemType[w["elem"]]
+        from cubek_amd import QuantStore
+
         level = QuantLevel.Tensor if w["block"] is None else QuantLevel.block([w["block"]])
-        self.scheme = QuantScheme.default().with_value(QuantValue[w["value"]]).with_level(level)
+        native = w.get("store", "U32") == "Native"
+        self.scheme = (QuantScheme.default().with_value(QuantValue[w["value"]]).with_level(level)
+                       .with_store(QuantStore.Native if native else QuantStore.U32))
         shape = tuple(x.shape)
         self.x = x
-        self.codes = torch.empty(self.scheme.packed_shape(shape), dtype=torch.int32, device="cuda")
+        if native:  # one byte per value, or two 4-bit values per byte
+            per_byte = 2 if w["value"] == "E2M1" else 1
+            self.codes = torch.empty(shape[:-1] + (shape[-1] // per_byte,), dtype=torch.uint8, device="cuda")
+        else:
+            self.codes = torch.empty(self.scheme.packed_shape(shape), dtype=torch.int32, device="cuda")
         self.scales = torch.empty(self.scheme.scales_shape(shape), dtype=torch.float32, device="cuda")
         self.in_scales = torch.empty(self.scheme.scales_shape(shape), dtype=x.dtype, device="cuda")
         self.y = torch.empty_like(x)
@@ -273,6 +281,51 @@ def packed_gemv(torch):
                     "GBps": round(b / (ms * 1e-3) / 1e9, 1), "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                     "weights_per_s": round(rows * cols / (ms * 1e-3))})
         del ws, ss, hw, hs
+        torch.cuda.empty_cache()
+    return out
+
+
+def copy_yardstick(torch, x, launches=24):
+    """A plain device-to-device copy of the input tensor (torch.Tensor.copy_, the runtime's copy kernel), timed like
+    the kernels of the path on rotated buffers: what this GPU gives a kernel that reads and writes the same
+    number of bytes and computes nothing."""
+    sets = max(2, min(8, -(-(1 << 30) // (2 * x.numel() * x.element_size()))))
+    src = [x] + [x.clone() for _ in range(sets - 1)]
+    dst = [torch.empty_like(x) for _ in range(sets)]
+    ms = sorted(timed_region(torch, lambda i: dst[i % sets].copy_(src[i % sets]), launches)[0] for _ in range(3))[1]
+    b = 2 * x.numel() * x.element_size()
+    return {"what": "torch.Tensor.copy_ of the input tensor, device to device, rotated buffer sets",
+            "bytes_read_plus_written": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+            "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+
+
+def scheme_matrix(torch):
+    """Every float type x value x store on the headline shape, blocks of 32, f32 parameters: the three launches of
+    the path, reported only (`--matrix`).  Inputs ~N(0, 0.02) from torch's generator, three rotated buffer sets."""
+    rows, cols = WORKLOADS["cfg5"]["shape"]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    base = torch.randn((rows, cols), generator=g, device="cuda", dtype=torch.float32).mul_(0.02)
+    out = []
+    for elem, tdt in (("BF16", torch.bfloat16), ("F16", torch.float16), ("F32", torch.float32)):
+        x = base.to(tdt)
+        for value, store, bits in (("Q8S", "U32", 8), ("Q4S", "U32", 4), ("Q2S", "U32", 2), ("E2M1", "U32", 4),
+                                   ("Q8S", "Native", 8), ("E4M3", "Native", 8),
+                                   ("E5M2", "Native", 8), ("E2M1", "Native", 4)):
+            w = dict(shape=(rows, cols), elem=elem, value=value, block=32, store=store)
+            ps = [Path(torch, w, x if i == 0 else x.clone()) for i in range(3)]
+            b = rows * cols * x.element_size() + rows * cols * bits // 8 + rows * cols // 32 * 4
+            for p in ps:
+                p.compute_scales()
+            row = {"elem": elem, "value": value, "store": store, "algorithmic_bytes": b}
+            for label, meth in (("quantize_dynamic", "quantize_dynamic"), ("quantize_given_scales", "quantize_given"),
+                                ("dequantize", "dequantize")):
+                fn = lambda i, m=meth: getattr(ps[i % len(ps)], m)()
+                ms = sorted(timed_region(torch, fn, 16)[0] for _ in range(3))[1]
+                row[label] = {"ms": round(ms, 4), "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+            out.append(row)
+            del ps, p
+        del x
         torch.cuda.empty_cache()
     return out
 
@@ -456,6 +509,8 @@ def main():
                     help="run only the abs-max / re-pack kernels on the headline tensor (for profiling)")
     ap.add_argument("--gemv-only", action="store_true",
                     help="run only the matrix-vector product over packed weights (for profiling)")
+    ap.add_argument("--matrix", action="store_true",
+                    help="run only the float type x value x store matrix on the headline shape (reported only)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run 3 plain device copies of the input (known bytes) to calibrate rocprof counters")
     args = ap.parse_args()
@@ -476,6 +531,9 @@ def main():
         return
     if args.gemv_only:
         print(json.dumps({"adjacent_kernels": packed_gemv(torch)}))
+        return
+    if args.matrix:
+        print(json.dumps({"scheme_matrix": scheme_matrix(torch)}))
         return
 
     w = WORKLOADS[args.workload]
@@ -498,6 +556,7 @@ def main():
     q_ms, _ = timed_region(torch, lambda i: paths[i % len(paths)].quantize_dynamic(), args.steps)
     d_ms, _ = timed_region(torch, lambda i: paths[i % len(paths)].dequantize(), args.steps)
 
+    yardstick = copy_yardstick(torch, x)
     if args.copy_probe:
         for _ in range(3):
             path.y.copy_(path.x)  # same size as the input tensor
@@ -528,6 +587,7 @@ def main():
                                 "algorithmic_bytes_per_launch": q_bytes, "avg_launch_ms": round(d_ms, 4)},
     }
 
+    result["copy_yardstick"] = yardstick
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, w, path)
         result["cpu_baseline"]["value"] = round(result["cpu_baseline"]["value"], 3)

@@ -205,11 +205,16 @@ struct RowSteps {
 // that row in the four tensors.  Blocks lie along the row, or (given scales) over rows of the innermost
 // level as well, or there is one scale per tensor.
 constexpr int kMaxLaneLevels = 7;
+constexpr int kNearLaneLevels = 4;  // levels the lanes' short cut from their tile's first row walks (LaneRows::near)
 struct LaneRows {
     uint32_t row_chunks, row_magic, row_shift;
     uint32_t total_chunks;  // < 2^31
     uint32_t levels;        // leading dimensions, 1 .. kMaxLaneLevels
     uint32_t narrow;        // every byte offset the rows can reach in the four tensors is below 2^32
+    // narrow, no blocks over rows, and the innermost level is longer than the rows one tile can span, its
+    // strides below 2^24 bytes: a tile's lanes find their rows from the tile's first row by one step of at most
+    // one carry
+    uint32_t near;
     // blocks of `scale_rows` entries of the innermost level (by a lane group of columns) share their scale
     // (given scales only); the scale strides of that level are per block of rows
     uint32_t scale_rows, scale_magic, scale_shift;
@@ -253,6 +258,64 @@ struct LaneSteps {
                 out_[u] = static_cast<char*>(g.out);
                 scale_in_[u] = static_cast<const char*>(g.scale_in);
                 scale_out_[u] = static_cast<char*>(g.scale_out);
+            }
+            return;
+        }
+        if (r.near) {
+            // The tile's first row is the same for every lane: its digits and offsets come from the scalar unit.
+            // A lane's row lies `drow` rows further on; when that runs over the end of the innermost level, the
+            // carry walks up the levels that sit on their last entry, which the tile's first row decides too.
+            const uint32_t c0 = (g.tile_begin + tile) * (kUnroll * kThreads);  // < total_chunks
+            const uint32_t row0 = magic_div(c0, r.row_magic, r.row_shift);
+            const uint32_t col0 = c0 - row0 * r.row_chunks;
+            uint32_t base[4] = {0, 0, 0, 0}, carried[4] = {0, 0, 0, 0};
+            uint32_t rest = row0, digit0 = 0;
+            bool carry = true;
+#pragma unroll
+            for (int l = 0; l < kNearLaneLevels; l++) {  // unrolled: the loads of every level's entries go out together
+                if (l < static_cast<int>(r.levels)) {
+                    const bool last = l + 1 == static_cast<int>(r.levels);
+                    uint32_t digit = rest;
+                    if (!last) {
+                        const uint32_t q = magic_div(rest, r.magic[l], r.shift[l]);
+                        digit = rest - q * r.count[l];
+                        rest = q;
+                    }
+                    const uint32_t step[4] = {static_cast<uint32_t>(r.in[l]), static_cast<uint32_t>(r.out[l]),
+                                              static_cast<uint32_t>(r.scale_in[l]), static_cast<uint32_t>(r.scale_out[l])};
+                    const bool stays = last || digit + 1 < r.count[l];  // a carry into this level ends here
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        base[t] += digit * step[t];
+                        if (l == 0)
+                            carried[t] -= r.count[0] * step[t];
+                        else if (carry)
+                            carried[t] += stays ? step[t] : 0u - (r.count[l] - 1) * step[t];
+                    }
+                    if (l == 0) digit0 = digit;
+                    if (l > 0 && stays) carry = false;
+                }
+            }
+            const uint32_t step0[4] = {static_cast<uint32_t>(r.in[0]), static_cast<uint32_t>(r.out[0]),
+                                       static_cast<uint32_t>(r.scale_in[0]), static_cast<uint32_t>(r.scale_out[0])};
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                const uint32_t chunk = c0 + u * kThreads + threadIdx.x;
+                live_[u] = chunk < r.total_chunks;
+                const uint32_t c = live_[u] ? chunk : r.total_chunks - 1;  // lanes past the end re-read the last chunk
+                const uint32_t k = col0 + (c - c0);
+                const uint32_t drow = magic_div(k, r.row_magic, r.row_shift);
+                col_[u] = k - __umul24(drow, r.row_chunks);
+                first_[u] = row0 + drow == 0;
+                block_row_[u] = true;
+                const bool wraps = digit0 + drow >= r.count[0];
+                uint32_t off[4];
+#pragma unroll
+                for (int t = 0; t < 4; t++) off[t] = base[t] + __umul24(drow, step0[t]) + (wraps ? carried[t] : 0u);
+                in_[u] = static_cast<const char*>(g.in) + off[0];
+                out_[u] = static_cast<char*>(g.out) + off[1];
+                scale_in_[u] = static_cast<const char*>(g.scale_in) + off[2];
+                scale_out_[u] = g.scale_out == nullptr ? nullptr : static_cast<char*>(g.scale_out) + off[3];
             }
             return;
         }

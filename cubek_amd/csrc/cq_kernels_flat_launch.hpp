@@ -81,6 +81,8 @@ FlatRows flat_rows(const FlatArgs& a) {
     return r;
 }
 
+// the most chunks a tile of the lane-wise kernels holds (threads x the deepest unroll in use)
+constexpr uint32_t kLaneTileChunks = kThreads * 8;
 // Whether every byte offset the rows of `r` can reach stays below 2^32 in each of the four tensors.
 void set_narrow(LaneRows* r) {
     uint64_t reach[4] = {0, 0, 0, 0};
@@ -98,6 +100,10 @@ void set_narrow(LaneRows* r) {
     r->narrow = 1;
     for (int t = 0; t < 4; t++)
         if (reach[t] >= (1ull << 32)) r->narrow = 0;
+    // rows of one tile (at most kLaneTileChunks chunks) within one step of the tile's first row
+    const uint64_t span = kLaneTileChunks / r->row_chunks + 2;
+    r->near = r->narrow && r->levels >= 2 && r->levels <= static_cast<uint32_t>(kNearLaneLevels) && r->scale_rows == 1 && r->row_chunks < (1u << 24) && r->count[0] >= span &&
+              r->in[0] < (1u << 24) && r->out[0] < (1u << 24) && r->scale_in[0] < (1u << 24) && r->scale_out[0] < (1u << 24);
 }
 
 // the same for the kernels that find each lane's row

@@ -151,6 +151,16 @@ def test_short_rows_behind_permuted_dimensions(gpu, oracle, elem, name, scheme):
                   ("middle_swapped", "middle_swapped_floats", "pitched_aligned", "pitched_words", "every_other_row", "leading_swapped"))
 
 
+@pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
+@pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
+def test_short_rows_behind_a_long_innermost_dimension(gpu, oracle, elem, name, scheme):
+    """Attention-shaped views whose position axis is longer than the rows one workgroup spans: the lanes step
+    from their workgroup's first row, with a carry through one, two and three outer dimensions, and the last
+    workgroup runs past the end."""
+    check_layouts(gpu, oracle, elem, name, scheme, ((2, 3, 1100, 128), (1, 2, 2102, 64), (2, 2, 3, 302, 64)),
+                  ("middle_swapped", "middle_swapped_floats", "leading_swapped"))
+
+
 BLOCKS_OF_ROWS = [
     ("q8s_block_16x32", QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([16, 32]))),
     ("q4s_block_8x64", QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([8, 64]))),
