@@ -320,9 +320,12 @@ __device__ __forceinline__ float scale_from_absmax_tame(float amax, const QuantP
 //   not decided by the clamp, and turns an infinite t (infinite x) into a finite
 //   one so that the residual is +-inf (clamped like the IEEE quotient), not NaN.
 // Negation commutes with every step (multiply, RNE rounding, rint).
-template <class F, int kN>
+// kNegated = false gives the codes themselves: the last rounding takes its operand negated (a source
+// modifier), which the conversions to fp8 / fp4 cannot do for theirs.
+template <class F, int kN, bool kNegated = true>
 __device__ __forceinline__ void quantize_values_neg(const float* x, float d, bool d_tame, float lo,
                                                     float hi, float* qn) {
+    constexpr float kSign = kNegated ? 1.0f : -1.0f;
     if constexpr (F::kDtype == CQ_BF16) {
         if (d_tame) {
             const float nr = -__builtin_amdgcn_rcpf(d);
@@ -332,8 +335,8 @@ __device__ __forceinline__ void quantize_values_neg(const float* x, float d, boo
                 const float a = neg_clamp_of_neg(x[i] * nr, nhi, nlo);
                 const float b = neg_clamp_of_neg(x[i + 1] * nr, nhi, nlo);
                 const uint32_t p = BF16::pack2(a, b);
-                qn[i] = __builtin_rintf(bits_f32(p << 16));
-                qn[i + 1] = __builtin_rintf(bits_f32(p & 0xffff0000u));
+                qn[i] = __builtin_rintf(kSign * bits_f32(p << 16));
+                qn[i + 1] = __builtin_rintf(kSign * bits_f32(p & 0xffff0000u));
             }
             return;
         }
@@ -346,7 +349,7 @@ __device__ __forceinline__ void quantize_values_neg(const float* x, float d, boo
                 const float tn = neg_clamp_of_neg(x[i] * nr, nhi_t, nlo_t);  // -t
                 const float e = __builtin_fmaf(tn, d, x[i]);                 // x - t*d
                 const float qn1 = __builtin_fmaf(e, nr, tn);                 // -(t + e*r)
-                qn[i] = __builtin_rintf(F16::round(neg_clamp_of_neg(qn1, nhi, nlo)));
+                qn[i] = __builtin_rintf(kSign * F16::round(neg_clamp_of_neg(qn1, nhi, nlo)));
             }
             return;
         }
@@ -359,16 +362,16 @@ __device__ __forceinline__ void quantize_values_neg(const float* x, float d, boo
             for (int i = 0; i < kN; i += 2) {
                 const float t0 = neg_clamp_of_neg(x[i] * nr, nhi_q, nlo_q);
                 const float t1 = neg_clamp_of_neg(x[i + 1] * nr, nhi_q, nlo_q);
-                qn[i] = __builtin_rintf(t0);
-                qn[i + 1] = __builtin_rintf(t1);
-                worst = fmaxf(worst, fmaxf(fabsf(t0 - qn[i]), fabsf(t1 - qn[i + 1])));
+                qn[i] = __builtin_rintf(kSign * t0);
+                qn[i + 1] = __builtin_rintf(kSign * t1);
+                worst = fmaxf(worst, fmaxf(fabsf(t0 - kSign * qn[i]), fabsf(t1 - kSign * qn[i + 1])));
             }
             const float window = (fmaxf(fabsf(lo), fabsf(hi)) + 1.0f) * 0x1p-21f;
             if (worst < 0.5f - window) return;
         }
     }
 #pragma unroll
-    for (int i = 0; i < kN; i++) qn[i] = -quantize_exact<F>(x[i], d, lo, hi);
+    for (int i = 0; i < kN; i++) qn[i] = -kSign * quantize_exact<F>(x[i], d, lo, hi);
 }
 
 // ---- bit packing -----------------------------------------------------------
@@ -460,14 +463,15 @@ constexpr int encoding_bits(int int_bits) {
     return kEnc == kEncInt ? int_bits : (kEnc == kEncE2M1 ? 4 : 8);
 }
 
-// kN negated integer-valued floats -> kN stored values, same word layout as pack_chunk_neg.
+// kN integer-valued floats (the codes themselves, not negated) -> kN stored values, same word layout as
+// pack_chunk_neg.
 template <int kEnc, int kN>
-__device__ __forceinline__ void encode_chunk_neg(const float* qn, uint32_t* w) {
+__device__ __forceinline__ void encode_chunk(const float* q, uint32_t* w) {
     if constexpr (kEnc == kEncE2M1) {
         uint32_t r = 0;
         static_for<0, kN / 2>([&](auto byte) {
             constexpr int b = decltype(byte)::value;
-            r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, -qn[2 * b], -qn[2 * b + 1], 1.0f, b);
+            r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, q[2 * b], q[2 * b + 1], 1.0f, b);
         });
         w[0] = r;
     } else {
@@ -475,11 +479,11 @@ __device__ __forceinline__ void encode_chunk_neg(const float* qn, uint32_t* w) {
         for (int j = 0; j < kN / 4; j++) {
             int r = 0;
             if constexpr (kEnc == kEncE4M3) {
-                r = __builtin_amdgcn_cvt_pk_fp8_f32(-qn[4 * j], -qn[4 * j + 1], r, false);
-                r = __builtin_amdgcn_cvt_pk_fp8_f32(-qn[4 * j + 2], -qn[4 * j + 3], r, true);
+                r = __builtin_amdgcn_cvt_pk_fp8_f32(q[4 * j], q[4 * j + 1], r, false);
+                r = __builtin_amdgcn_cvt_pk_fp8_f32(q[4 * j + 2], q[4 * j + 3], r, true);
             } else {
-                r = __builtin_amdgcn_cvt_pk_bf8_f32(-qn[4 * j], -qn[4 * j + 1], r, false);
-                r = __builtin_amdgcn_cvt_pk_bf8_f32(-qn[4 * j + 2], -qn[4 * j + 3], r, true);
+                r = __builtin_amdgcn_cvt_pk_bf8_f32(q[4 * j], q[4 * j + 1], r, false);
+                r = __builtin_amdgcn_cvt_pk_bf8_f32(q[4 * j + 2], q[4 * j + 3], r, true);
             }
             w[j] = static_cast<uint32_t>(r);
         }

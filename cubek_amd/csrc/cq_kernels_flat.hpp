@@ -485,12 +485,12 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         if constexpr (!(kDynamic && kParamF32 && F::kDtype != CQ_F16)) tame = divisor_is_tame(d);
 
         float qn[kN];  // negated codes
-        quantize_values_neg<F, kN>(v, d, tame, qp.lo, qp.hi, qn);
+        quantize_values_neg<F, kN, kEnc == kEncInt>(v, d, tame, qp.lo, qp.hi, qn);
         uint32_t w[2];
         if constexpr (kEnc == kEncInt)
             pack_chunk_neg<kBits, kN, kWide>(qn, w);
         else
-            encode_chunk_neg<kEnc, kN>(qn, w);
+            encode_chunk<kEnc, kN>(qn, w);
 
         if constexpr (kChunkBits == 64) {
             if (live) stream_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(out) + c);

@@ -118,12 +118,12 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(RowArgs a) {
         for (int i = 0; i < U::kChunks; i++) {
             float v[kN], qn[kN];
             F::unpack(raw[u][i], v);
-            quantize_values_neg<F, kN>(v, d, tame, a.range.lo, a.range.hi, qn);
+            quantize_values_neg<F, kN, kEnc == kEncInt>(v, d, tame, a.range.lo, a.range.hi, qn);
             uint32_t cw[2] = {0, 0};
             if constexpr (kEnc == kEncInt)
                 pack_chunk_neg<kBits, kN, kWide>(qn, cw);
             else
-                encode_chunk_neg<kEnc, kN>(qn, cw);
+                encode_chunk<kEnc, kN>(qn, cw);
             if constexpr (U::kChunks == 1) {
                 w[0] = cw[0];
                 w[1] = cw[1];
@@ -289,16 +289,19 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
         return p;
     };
     auto load = [&](const Pos& p, u32x4 (&raw)[kCols][kRows]) {
-        const u32x4* src = static_cast<const u32x4*>(a.input) + p.f;
+        // this thread's rows lie ph_per_block rows apart: one 64-bit product, then steps of a tile-wide constant
+        const u32x4* src = static_cast<const u32x4*>(a.input) + p.f + pin * pitch_f;
+        const uint64_t row_step = g.ph_per_block * pitch_f;
 #pragma unroll
         for (int c = 0; c < kCols; c++) {
             const uint32_t jc = p.jc0 + c * g.tj_eff;
+            const u32x4* at = src + jc;
 #pragma unroll
             for (int k = 0; k < kRows; k++) {
                 const uint32_t rr = pin + k * g.ph_per_block;
                 raw[c][k] = u32x4{0, 0, 0, 0};
-                if (p.rows_live && jl < g.tj_eff && jc < chunks_per_row && rr < br)
-                    raw[c][k] = stream_load(src + rr * pitch_f + jc);
+                if (p.rows_live && jl < g.tj_eff && jc < chunks_per_row && rr < br) raw[c][k] = stream_load(at);
+                at += row_step;
             }
         }
     };
@@ -345,20 +348,20 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
             const float d = F::round(s_fs);
             const bool tame = divisor_is_tame(d);
             if (!live) continue;
-            uint32_t* out = static_cast<uint32_t*>(a.output) + pos.v;
+            uint32_t* dst = static_cast<uint32_t*>(a.output) + pos.v + pin * pitch_v;
+            const uint64_t out_step = g.ph_per_block * pitch_v;
 #pragma unroll
-            for (int k = 0; k < kRows; k++) {
+            for (int k = 0; k < kRows; k++, dst += out_step) {
                 const uint32_t rr = pin + k * g.ph_per_block;
                 const bool row_live = rr < br;  // the same for every lane of a word
                 float v[kN], qn[kN];
                 F::unpack(raw[c][k], v);
-                quantize_values_neg<F, kN>(v, d, tame, qp.lo, qp.hi, qn);
+                quantize_values_neg<F, kN, kEnc == kEncInt>(v, d, tame, qp.lo, qp.hi, qn);
                 uint32_t w[2] = {0, 0};
                 if constexpr (kEnc == kEncInt)
                     pack_chunk_neg<kBits, kN, kWide>(qn, w);
                 else
-                    encode_chunk_neg<kEnc, kN>(qn, w);
-                uint32_t* dst = out + rr * pitch_v;
+                    encode_chunk<kEnc, kN>(qn, w);
                 if constexpr (kChunkBits == 64) {
                     if (row_live) {
                         stream_store(w[0], dst + 2 * static_cast<uint64_t>(jc));

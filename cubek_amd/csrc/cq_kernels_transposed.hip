@@ -163,12 +163,12 @@ __device__ __forceinline__ void quantize_piece_words(const float* v, float d, bo
 #pragma unroll
         for (int i = 0; i < U::kChunks; i++) {
             float qn[kN];
-            quantize_values_neg<F, kN>(v + u * U::kV + i * kN, d, tame, qp.lo, qp.hi, qn);
+            quantize_values_neg<F, kN, kEnc == kEncInt>(v + u * U::kV + i * kN, d, tame, qp.lo, qp.hi, qn);
             uint32_t cw[2] = {0, 0};
             if constexpr (kEnc == kEncInt)
                 pack_chunk_neg<kBits, kN, kWide>(qn, cw);
             else
-                encode_chunk_neg<kEnc, kN>(qn, cw);
+                encode_chunk<kEnc, kN>(qn, cw);
             if constexpr (U::kChunks == 1) {
                 w[0] = cw[0];
                 w[1] = cw[1];
