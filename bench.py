@@ -544,6 +544,15 @@ def main():
 
     paths = replicas(torch, w, x)
     path = paths[0]
+    # the process's first launches: what the runtime takes to load the library's code objects is in here
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    path.quantize_dynamic()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    path.dequantize()
+    torch.cuda.synchronize()
+    first_ms = [(t1 - t0) * 1e3, (time.perf_counter() - t1) * 1e3]
 
     def step(i):
         p = paths[i % len(paths)]
@@ -588,6 +597,8 @@ def main():
     }
 
     result["copy_yardstick"] = yardstick
+    result["first_call_ms"] = {"quantize_dynamic": round(first_ms[0], 2), "dequantize": round(first_ms[1], 2),
+                               "library_bytes": os.path.getsize(_ffi.LIB_PATH)}
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, w, path)
         result["cpu_baseline"]["value"] = round(result["cpu_baseline"]["value"], 3)

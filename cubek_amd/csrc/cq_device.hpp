@@ -229,6 +229,18 @@ __device__ __forceinline__ float group_max(float v) {
     return bits_f32(b);
 }
 
+// The same with the group size (2^log2 lanes, log2 <= 6) known at run time only; `log2` is the same for every lane.
+__device__ __forceinline__ float group_max_rt(float v, uint32_t log2) {
+    uint32_t b = f32_bits(v);
+    if (log2 >= 1) b = max(b, dpp<kDppXor1>(b));
+    if (log2 >= 2) b = max(b, dpp<kDppXor2>(b));
+    if (log2 >= 3) b = max(b, dpp<kDppHalfMirror>(b));
+    if (log2 >= 4) b = max(b, dpp<kDppMirror>(b));
+    if (log2 >= 5) b = max(b, static_cast<uint32_t>(__shfl_xor(static_cast<int>(b), 16, kWave)));
+    if (log2 >= 6) b = max(b, static_cast<uint32_t>(__shfl_xor(static_cast<int>(b), 32, kWave)));
+    return bits_f32(b);
+}
+
 // OR over aligned groups of 2 or 4 lanes (bit-field assembly across lanes).
 template <int kGroup>
 __device__ __forceinline__ uint32_t group_or(uint32_t v) {

@@ -10,8 +10,8 @@ template <class F, int kGroup>
 hipError_t scales_launch(hipStream_t s, const FlatArgs& a) {
     dim3 grid(grid_for(a.num_chunks, kUnrollQ)), block(kThreads);
     if (a.lanes.levels > 0) {
-        hipLaunchKernelGGL((scales_flat_lanes_kernel<F, kGroup, kUnrollQ, kThreads>), dim3(lanes_grid(a, kUnrollQ)), block, 0, s,
-                           static_cast<const u32x4*>(a.input), a.scale_out, quant_params(a.range), lane_rows(a));
+        hipLaunchKernelGGL((scales_flat_lanes_kernel<F, kGroupRt, kUnrollQ, kThreads>), dim3(lanes_grid(a, kUnrollQ)), block, 0, s,
+                           static_cast<const u32x4*>(a.input), a.scale_out, quant_params(a.range), with_group(lane_rows(a), kGroup));
     } else if (a.rows > 1) {
         const FlatRows rows = flat_rows(a);
         hipLaunchKernelGGL((scales_flat_rows_kernel<F, kGroup, kUnrollQ, kThreads>), dim3((rows.total_steps + kUnrollQ - 1) / kUnrollQ),

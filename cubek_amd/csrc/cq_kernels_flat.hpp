@@ -204,6 +204,9 @@ struct RowSteps {
 // dimension (innermost first, `count` entries each, multiply-and-shift divisions), the byte offsets of
 // that row in the four tensors.  Blocks lie along the row, or (given scales) over rows of the innermost
 // level as well, or there is one scale per tensor.
+// kGroup of the lane-wise kernels that serve every block size: the lanes per block come with the launch
+// (LaneRows::group_log2), one instantiation instead of one per block size.  Per tensor stays kGroup = 0.
+constexpr int kGroupRt = -1;
 constexpr int kMaxLaneLevels = 7;
 constexpr int kNearLaneLevels = 4;  // levels the lanes' short cut from their tile's first row walks (LaneRows::near)
 struct LaneRows {
@@ -211,10 +214,11 @@ struct LaneRows {
     uint32_t total_chunks;  // < 2^31
     uint32_t levels;        // leading dimensions, 1 .. kMaxLaneLevels
     uint32_t narrow;        // every byte offset the rows can reach in the four tensors is below 2^32
-    // narrow, no blocks over rows, and the innermost level is longer than the rows one tile can span, its
-    // strides below 2^24 bytes: a tile's lanes find their rows from the tile's first row by one step of at most
-    // one carry
+    // narrow, no blocks over rows, at most kNearLaneLevels levels, and the innermost level is longer than the rows
+    // one tile can span, its strides below 2^24 bytes: a tile's lanes find their rows from the tile's first row by
+    // one step of at most one carry
     uint32_t near;
+    uint32_t group_log2;    // lanes per block as a power of two, for the kernels that take it at run time (kGroupRt)
     // blocks of `scale_rows` entries of the innermost level (by a lane group of columns) share their scale
     // (given scales only); the scale strides of that level are per block of rows
     uint32_t scale_rows, scale_magic, scale_shift;
@@ -264,54 +268,72 @@ struct LaneSteps {
         if (r.near) {
             // The tile's first row is the same for every lane: its digits and offsets come from the scalar unit.
             // A lane's row lies `drow` rows further on; when that runs over the end of the innermost level, the
-            // carry walks up the levels that sit on their last entry, which the tile's first row decides too.
+            // carry walks up the levels that sit on their last entry, which the tile's first row decides too
+            // (worked out only in the few tiles that hold such a lane).
             const uint32_t c0 = (g.tile_begin + tile) * (kUnroll * kThreads);  // < total_chunks
             const uint32_t row0 = magic_div(c0, r.row_magic, r.row_shift);
             const uint32_t col0 = c0 - row0 * r.row_chunks;
-            uint32_t base[4] = {0, 0, 0, 0}, carried[4] = {0, 0, 0, 0};
-            uint32_t rest = row0, digit0 = 0;
-            bool carry = true;
+            uint32_t base[4] = {0, 0, 0, 0};  // narrow: every offset stays below 2^32
+            uint32_t digits[kNearLaneLevels];
+            uint32_t rest = row0;
 #pragma unroll
             for (int l = 0; l < kNearLaneLevels; l++) {  // unrolled: the loads of every level's entries go out together
+                digits[l] = 0;
                 if (l < static_cast<int>(r.levels)) {
-                    const bool last = l + 1 == static_cast<int>(r.levels);
-                    uint32_t digit = rest;
-                    if (!last) {
+                    digits[l] = rest;
+                    if (l + 1 < static_cast<int>(r.levels)) {
                         const uint32_t q = magic_div(rest, r.magic[l], r.shift[l]);
-                        digit = rest - q * r.count[l];
+                        digits[l] = rest - q * r.count[l];
                         rest = q;
                     }
                     const uint32_t step[4] = {static_cast<uint32_t>(r.in[l]), static_cast<uint32_t>(r.out[l]),
                                               static_cast<uint32_t>(r.scale_in[l]), static_cast<uint32_t>(r.scale_out[l])};
-                    const bool stays = last || digit + 1 < r.count[l];  // a carry into this level ends here
 #pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        base[t] += digit * step[t];
-                        if (l == 0)
-                            carried[t] -= r.count[0] * step[t];
-                        else if (carry)
-                            carried[t] += stays ? step[t] : 0u - (r.count[l] - 1) * step[t];
-                    }
-                    if (l == 0) digit0 = digit;
-                    if (l > 0 && stays) carry = false;
+                    for (int t = 0; t < 4; t++) base[t] += digits[l] * step[t];
                 }
             }
             const uint32_t step0[4] = {static_cast<uint32_t>(r.in[0]), static_cast<uint32_t>(r.out[0]),
                                        static_cast<uint32_t>(r.scale_in[0]), static_cast<uint32_t>(r.scale_out[0])};
+            uint32_t drow[kUnroll];
+            bool wraps[kUnroll], any_wraps = false;
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
                 const uint32_t chunk = c0 + u * kThreads + threadIdx.x;
                 live_[u] = chunk < r.total_chunks;
                 const uint32_t c = live_[u] ? chunk : r.total_chunks - 1;  // lanes past the end re-read the last chunk
                 const uint32_t k = col0 + (c - c0);
-                const uint32_t drow = magic_div(k, r.row_magic, r.row_shift);
-                col_[u] = k - __umul24(drow, r.row_chunks);
-                first_[u] = row0 + drow == 0;
+                drow[u] = magic_div(k, r.row_magic, r.row_shift);
+                col_[u] = k - __umul24(drow[u], r.row_chunks);
+                first_[u] = row0 + drow[u] == 0;
                 block_row_[u] = true;
-                const bool wraps = digit0 + drow >= r.count[0];
+                wraps[u] = digits[0] + drow[u] >= r.count[0];
+                any_wraps = any_wraps || wraps[u];
+            }
+            uint32_t carried[4] = {0, 0, 0, 0};  // modulo 2^32: the sums it enters are exact
+            if (__any(any_wraps)) {
+                bool carry = true;
+#pragma unroll
+                for (int l = 0; l < kNearLaneLevels; l++) {
+                    if (l < static_cast<int>(r.levels)) {
+                        const uint32_t step[4] = {static_cast<uint32_t>(r.in[l]), static_cast<uint32_t>(r.out[l]),
+                                              static_cast<uint32_t>(r.scale_in[l]), static_cast<uint32_t>(r.scale_out[l])};
+                        const bool stays = l + 1 == static_cast<int>(r.levels) || digits[l] + 1 < r.count[l];  // a carry into this level ends here
+#pragma unroll
+                        for (int t = 0; t < 4; t++) {
+                            if (l == 0)
+                                carried[t] -= r.count[0] * step[t];
+                            else if (carry)
+                                carried[t] += stays ? step[t] : 0u - (r.count[l] - 1) * step[t];
+                        }
+                        if (l > 0 && stays) carry = false;
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
                 uint32_t off[4];
 #pragma unroll
-                for (int t = 0; t < 4; t++) off[t] = base[t] + __umul24(drow, step0[t]) + (wraps ? carried[t] : 0u);
+                for (int t = 0; t < 4; t++) off[t] = base[t] + __umul24(drow[u], step0[t]) + (wraps[u] ? carried[t] : 0u);
                 in_[u] = static_cast<const char*>(g.in) + off[0];
                 out_[u] = static_cast<char*>(g.out) + off[1];
                 scale_in_[u] = static_cast<const char*>(g.scale_in) + off[2];
@@ -344,7 +366,7 @@ struct LaneSteps {
                 continue;
             }
             uint64_t in = 0, out = 0, scale_in = 0, scale_out = 0;
-#pragma unroll
+#pragma unroll  // a loop over l would index the launch's arguments at run time, which sends all of them through scratch memory
             for (int l = 0; l < kMaxLaneLevels; l++) {
                 if (l < static_cast<int>(r.levels)) {
                     uint32_t index = row;
@@ -395,7 +417,13 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
     constexpr bool kDynamic = kScaleSrc == kScaleDynamic;
     static_assert(kScaleSrc != kScalePartials || kGroup == 0, "partials feed the per-tensor scale only");
     static_assert(kScaleSrc != kScaleStored || kGroup != 0, "stored scales are read back per block only");
-    constexpr int kDiv = kGroup == 0 ? 1 : kGroup;
+    constexpr int kDiv = kGroup <= 0 ? 1 : kGroup;
+    constexpr bool kRtGroup = kGroup == kGroupRt;
+    uint32_t group_log2 = 0;
+    if constexpr (kRtGroup) group_log2 = geo.rows.group_log2;
+    // chunk -> its block, and whether it starts one
+    const auto block_of = [&](auto c) { return kRtGroup ? c >> group_log2 : c / kDiv; };
+    const auto starts_block = [&](auto c) { return kRtGroup ? (c & ((1u << group_log2) - 1u)) == 0 : (c % kDiv) == 0; };
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;  // 64, 32, 16 or 8
     const int param_dtype = kParamF32 ? static_cast<int>(CQ_F32) : param_dtype_rt;
@@ -419,9 +447,9 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         const auto c = at.load_chunk(u);
         raw[u] = stream_load(static_cast<const u32x4*>(at.in(u)) + c);
         if constexpr (kScaleSrc == kScaleStored)
-            s_stored[u] = load_dtype_raw(param_dtype, at.scale_in(u), c / kDiv);
+            s_stored[u] = load_dtype_raw(param_dtype, at.scale_in(u), block_of(c));
         else if constexpr (!kDynamic && kGroup != 0 && kScaleSrc != kScalePartials)
-            s_given[u] = F::load(at.scale_in(u), c / kDiv);
+            s_given[u] = F::load(at.scale_in(u), block_of(c));
     }
     if constexpr (kScaleSrc == kScaleStored) {
 #pragma unroll
@@ -465,7 +493,10 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
             float amax = 0.0f;
 #pragma unroll
             for (int i = 0; i < kN; i++) amax = fmaxf(amax, fabsf(v[i]));  // NaN elements drop out
-            amax = group_max<kGroup>(amax);
+            if constexpr (kRtGroup)
+                amax = group_max_rt(amax, group_log2);
+            else
+                amax = group_max<kGroup>(amax);
             tame = absmax_is_tame(amax);
             const float s32 = tame ? scale_from_absmax_tame(amax, qp) : scale_from_absmax(amax, qp.width);
             s_f = F::round(s32);
@@ -474,8 +505,8 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         }
         // write_scale (src/quantize.rs:83-98): FS(scale), stored by the block's first lane
         const float s_fs = round_to_dtype(param_dtype, s_f);
-        const auto si = kGroup == 0 ? 0 : c / kDiv;
-        const bool block_start = kGroup == 0 ? at.tensor_start(u) : (at.first_row(u) && (c % kDiv) == 0);
+        const auto si = kGroup == 0 ? 0 : block_of(c);
+        const bool block_start = kGroup == 0 ? at.tensor_start(u) : (at.first_row(u) && starts_block(c));
         if constexpr (kScaleSrc != kScaleStored)
             if (scale_out != nullptr && live && block_start) store_dtype(param_dtype, scale_out, si, s_fs);
         // divisor F(FS(scale)); s_f is an F value, so f32 params leave it unchanged
@@ -565,7 +596,8 @@ __device__ __forceinline__ void dequantize_flat_body(const Geo& geo, int param_d
             uint32_t w = in[c / kLanesPerWord];  // neighbouring lanes share the word
             w0[u] = w >> ((static_cast<uint32_t>(c) & (kLanesPerWord - 1)) * kChunkBits);
         }
-        const auto si = kGroup == 0 ? 0 : c / (kGroup == 0 ? 1 : kGroup);
+        auto si = kGroup == 0 ? 0 : c / (kGroup <= 0 ? 1 : kGroup);
+        if constexpr (kGroup == kGroupRt) si = c >> geo.rows.group_log2;
         if constexpr (kParamF32)
             sc[u] = F32::load(at.scale_in(u), si);
         else
@@ -632,10 +664,21 @@ __device__ __forceinline__ void scales_flat_body(const Geo& geo, const QuantPara
         float amax = 0.0f;
 #pragma unroll
         for (int i = 0; i < kN; i++) amax = fmaxf(amax, fabsf(v[i]));
-        amax = group_max<kGroup>(amax);
+        bool starts;
+        auto block = c;
+        if constexpr (kGroup == kGroupRt) {
+            const uint32_t log2 = geo.rows.group_log2;
+            amax = group_max_rt(amax, log2);
+            starts = (c & ((1u << log2) - 1u)) == 0;
+            block = c >> log2;
+        } else {
+            amax = group_max<kGroup>(amax);
+            starts = (c % kGroup) == 0;
+            block = c / kGroup;
+        }
         const float s32 = absmax_is_tame(amax) ? scale_from_absmax_tame(amax, qp)
                                                : scale_from_absmax(amax, qp.width);
-        if (at.live(u) && (c % kGroup) == 0) F::store(at.scale_out(u), c / kGroup, s32);
+        if (at.live(u) && starts) F::store(at.scale_out(u), block, s32);
     }
 }
 

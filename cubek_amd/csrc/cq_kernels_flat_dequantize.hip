@@ -31,11 +31,11 @@ hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
                                    static_cast<uint64_t>(grid) * kThreads * kU);
         },
         [&](const LaneRows& rows, uint32_t tile_begin, uint32_t grid, RunOffsets off) {
-            hipLaunchKernelGGL((dequantize_flat_lanes_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(grid), dim3(kThreads), 0,
+            hipLaunchKernelGGL((dequantize_flat_lanes_kernel<F, kBits, lanes_group(kGroup), kU, kThreads, kEnc>), dim3(grid), dim3(kThreads), 0,
                                s, reinterpret_cast<const uint32_t*>(in + off.chunks * kInChunk),
                                reinterpret_cast<u32x4*>(out + off.chunks * 16),
                                static_cast<const char*>(a.scale_in) + off.chunks / kDiv * param_bytes, a.param_dtype, tile_begin,
-                               rows);
+                               with_group(rows, kGroup));
         });
 }
 

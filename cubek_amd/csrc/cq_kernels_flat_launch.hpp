@@ -81,6 +81,14 @@ FlatRows flat_rows(const FlatArgs& a) {
     return r;
 }
 
+// The lane-wise kernels take the lanes per block at run time (one instantiation for every block size); one scale
+// per tensor (kGroup 0) stays a kernel of its own.
+constexpr int lanes_group(int group) { return group == 0 ? 0 : kGroupRt; }
+inline LaneRows with_group(LaneRows r, int group) {
+    r.group_log2 = 0;
+    while ((1 << r.group_log2) < group) r.group_log2++;
+    return r;
+}
 // the most chunks a tile of the lane-wise kernels holds (threads x the deepest unroll in use)
 constexpr uint32_t kLaneTileChunks = kThreads * 8;
 // Whether every byte offset the rows of `r` can reach stays below 2^32 in each of the four tensors.
@@ -100,10 +108,14 @@ void set_narrow(LaneRows* r) {
     r->narrow = 1;
     for (int t = 0; t < 4; t++)
         if (reach[t] >= (1ull << 32)) r->narrow = 0;
-    // rows of one tile (at most kLaneTileChunks chunks) within one step of the tile's first row
+}
+// Whether the lanes of a tile can find their rows from the tile's first row (LaneRows::near): the rows one tile
+// spans (at most kLaneTileChunks chunks) run over the end of the innermost level once at most.
+void set_near(LaneRows* r) {
     const uint64_t span = kLaneTileChunks / r->row_chunks + 2;
-    r->near = r->narrow && r->levels >= 2 && r->levels <= static_cast<uint32_t>(kNearLaneLevels) && r->scale_rows == 1 && r->row_chunks < (1u << 24) && r->count[0] >= span &&
-              r->in[0] < (1u << 24) && r->out[0] < (1u << 24) && r->scale_in[0] < (1u << 24) && r->scale_out[0] < (1u << 24);
+    r->near = r->narrow && r->levels >= 2 && r->levels <= static_cast<uint32_t>(kNearLaneLevels) && r->scale_rows == 1 &&
+              r->row_chunks < (1u << 24) && r->count[0] >= span && r->in[0] < (1u << 24) && r->out[0] < (1u << 24) &&
+              r->scale_in[0] < (1u << 24) && r->scale_out[0] < (1u << 24);
 }
 
 // the same for the kernels that find each lane's row
@@ -125,6 +137,7 @@ LaneRows lane_rows(const FlatArgs& a) {
         r.scale_out[l] = a.lanes.scale_out[l];
     }
     set_narrow(&r);
+    set_near(&r);
     return r;
 }
 inline uint32_t lanes_grid(const FlatArgs& a, int unroll) {
@@ -165,6 +178,7 @@ LaneRows lane_rows_of_rows(const FlatArgs& a) {
     }
     for (uint32_t l = 0; l < r.levels; l++) magic_of(r.count[l], &r.magic[l], &r.shift[l]);
     set_narrow(&r);
+    set_near(&r);
     return r;
 }
 
@@ -262,10 +276,10 @@ hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
                 const uint64_t scales = off.chunks / kDiv;
                 const void* scale_in = a.scale_in == nullptr ? nullptr : static_cast<const char*>(a.scale_in) + scales * scale_in_bytes;
                 void* scale_out = a.scale_out == nullptr ? nullptr : static_cast<char*>(a.scale_out) + scales * scale_out_bytes;
-                hipLaunchKernelGGL((quantize_flat_lanes_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
+                hipLaunchKernelGGL((quantize_flat_lanes_kernel<F, kBits, lanes_group(kGroup), kSrc, kWide, kUnrollQ, kThreads, kEnc>),
                                    dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in + off.chunks * 16),
                                    reinterpret_cast<uint32_t*>(out + off.chunks * kOutChunk), scale_in, scale_out,
-                                   a.param_dtype, qp, a.num_partials, tile_begin, rows);
+                                   a.param_dtype, qp, a.num_partials, tile_begin, with_group(rows, kGroup));
             });
     }
 }
