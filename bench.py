@@ -414,26 +414,35 @@ def adjacent_kernels(torch):
     torch.cuda.empty_cache()
     # the headline scheme on pitched rows: [rows, cols] views of [rows, cols + 64] buffers, at the headline
     # row length and with the same elements in rows a quarter as long
-    pad = 64
-    for pr, pc in ((rows, cols), (rows * 4, cols // 4)):
+    # ... with rows whose last step of 256 chunks is cut short (576 chunks a row), and with bf16 parameters on the
+    # contiguous tensor: the layouts that the lane-wise streaming kernels take whole
+    from cubek_amd import QuantParam
+
+    f32_scheme = scheme
+    for pr, pc, pad, param in ((rows, cols, 64, "F32"), (rows * 4, cols // 4, 64, "F32"), (32768, 4608, 64, "F32"),
+                               (rows, cols, 0, "BF16")):
+        scheme = f32_scheme.with_param(QuantParam[param])
         xp = [torch.randn((pr, pc + pad), device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
         yp = [torch.empty((pr, pc + pad), device="cuda", dtype=torch.bfloat16) for _ in range(2)]
         words = [torch.empty((pr, pc // 8), dtype=torch.int32, device="cuda") for _ in range(2)]
-        bscales = [torch.empty((pr, pc // 32), dtype=torch.float32, device="cuda") for _ in range(2)]
+        bscales = [torch.empty((pr, pc // 32), dtype=torch.float32 if param == "F32" else torch.bfloat16, device="cuda")
+                   for _ in range(2)]
         pitched = lambda t: TensorHandleRef(h(t).handle, (pr, pc), (pc + pad, 1), 2)
         hxp, hyp = [pitched(t) for t in xp], [pitched(t) for t in yp]
         hw, hb = [h(t) for t in words], [h(t) for t in bscales]
-        b = pr * pc * 2 + pr * pc // 2 + bscales[0].numel() * 4
+        b = pr * pc * 2 + pr * pc // 2 + bscales[0].numel() * bscales[0].element_size()
+        what = (f"pitched bf16 rows: [{pr}, {pc}] view of a [{pr}, {pc + pad}] buffer" if pad else
+                f"contiguous bf16 [{pr}, {pc}]") + ("" if param == "F32" else f", {param.lower()} parameters")
         for label, fn in (
                 ("quantize_dynamic", lambda i: cq_quantize.launch_dynamic(client, hxp[i % sets], hw[i % 2], hb[i % 2], scheme,
                                                                            ElemType.BF16)),
                 ("dequantize", lambda i: cq_dequantize.launch_ref(client, hw[i % 2], hyp[i % 2], hb[i % 2], scheme,
                                                                   ElemType.BF16))):
             ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
-            out.append({"kernel": f"{label}, e2m1 blocks of 32, pitched bf16 rows: [{pr}, {pc}] view of a [{pr}, {pc + pad}] buffer",
+            out.append({"kernel": f"{label}, e2m1 blocks of 32, {what}",
                         "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                         "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
-        if pc == cols:  # abs-max along both axes of the same pitched rows
+        if pc == cols and pad:  # abs-max along both axes of the same pitched rows
             for axis in (1, 0):
                 o = torch.zeros((pr, 1) if axis == 1 else (1, pc), device="cuda", dtype=torch.bfloat16)
                 nbytes = cq_reduce.workspace_bytes(hxp[0], axis, ElemType.BF16)
@@ -448,6 +457,7 @@ def adjacent_kernels(torch):
                             "frac_hbm_peak": round(pr * pc * 2 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
         del xp, yp, words, bscales, hxp, hyp, hw, hb
         torch.cuda.empty_cache()
+    scheme = f32_scheme
     # the headline scheme on an attention layout: the [batch, heads, positions, head dimension] view of a
     # [batch, positions, heads, head dimension] buffer (rows of 128 elements behind permuted dimensions)
     nb, nh, ns, nd = 8, 32, 4096, 128
