@@ -503,17 +503,21 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         } else {
             s_f = s_given[u];
         }
-        // write_scale (src/quantize.rs:83-98): FS(scale), stored by the block's first lane
-        const float s_fs = round_to_dtype(param_dtype, s_f);
+        // write_scale (src/quantize.rs:83-98): FS(scale), stored by the block's first lane.  s_f is an F value, so
+        // FS rounds it only where FS is a 16-bit type other than F (the same for the whole launch: a scalar branch)
+        const bool fs_rounds = !kParamF32 && param_dtype != CQ_F32 && param_dtype != F::kDtype;
+        float s_fs = s_f;
+        if (fs_rounds) s_fs = round_to_dtype(param_dtype, s_f);
         const auto si = kGroup == 0 ? 0 : block_of(c);
         const bool block_start = kGroup == 0 ? at.tensor_start(u) : (at.first_row(u) && starts_block(c));
         if constexpr (kScaleSrc != kScaleStored)
             if (scale_out != nullptr && live && block_start) store_dtype(param_dtype, scale_out, si, s_fs);
-        // divisor F(FS(scale)); s_f is an F value, so f32 params leave it unchanged
-        float d = s_fs;
-        if constexpr (!kParamF32) d = F::round(s_fs);
+        // divisor F(FS(scale)): s_f itself unless FS rounded it
+        float d = s_f;
+        if (fs_rounds) d = F::round(s_fs);
         if constexpr (kScaleSrc == kScaleStored) d = s_f;  // F(stored) as loaded
-        if constexpr (!(kDynamic && kParamF32 && F::kDtype != CQ_F16)) tame = divisor_is_tame(d);
+        // a tame abs-max gives a tame scale; every other divisor is looked at itself
+        if (!(kDynamic && F::kDtype != CQ_F16) || fs_rounds) tame = divisor_is_tame(d);
 
         float qn[kN];  // negated codes
         quantize_values_neg<F, kN, kEnc == kEncInt>(v, d, tame, qp.lo, qp.hi, qn);
