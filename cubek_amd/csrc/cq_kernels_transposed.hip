@@ -686,35 +686,42 @@ __global__ __launch_bounds__(kThreads) void dequantize_transposed_wide_kernel(Tr
 }
 
 // The same tile the other way round: a workgroup takes 256 bytes of codes of each of its 64 * kRp rows into LDS in one
-// go (16 lanes x 16 bytes per row), then walks the tile 128 columns at a time: thread (rp, part) decodes 32 columns
-// of kRp rows and leaves them in LDS as [column][word of rows], and every column leaves as 16-byte pieces, 256 bytes
-// per column and step.  Blocks of any multiple of 32 columns, or per tensor.
+// go (16 lanes x 16 bytes per row), then walks the tile 64 columns at a time: thread (row pair, 16 columns)
+// decodes its columns of kRp rows and leaves them in LDS as [column][word of rows], and every column leaves as
+// 16-byte pieces, 256 bytes per column and step.  Sixteen columns per thread keep the step's floats at 16 KiB, so
+// that three workgroups fit a compute unit; the words of a column are stored rotated by its group of sixteen
+// columns, which spreads the four column groups of a wave over the banks.  Blocks of any multiple of 32
+// columns, or per tensor.
+constexpr uint32_t kDeqStepCols = 64, kDeqPart = 16;
 template <class F, int kBits, int kEnc>
 __global__ __launch_bounds__(kThreads) void dequantize_transposed_tile_kernel(TransposedArgs a) {
     using U = Unit<F, kBits>;
     constexpr uint32_t kRp = kTileRowsPerThread<F>;
     constexpr uint32_t kTileRows = 64 * kRp;
-    constexpr uint32_t kSteps = 16 / kBits;
-    constexpr uint32_t kPartWords = kTilePart / U::kNq;
-    constexpr uint32_t kStepWords = kTileStepCols / U::kNq;
-    constexpr uint32_t kRowWords = kSteps * kStepWords;              // 64
+    constexpr uint32_t kRowWords = 64;                                // 256 bytes of codes per row and tile
+    constexpr uint32_t kTileCols = kRowWords * U::kNq;
+    constexpr uint32_t kSteps = kTileCols / kDeqStepCols;             // 8 (4-bit), 4 (8-bit), 16 (2-bit)
+    constexpr uint32_t kPartWords = kDeqPart / U::kNq;                // words of a thread per row and step
+    static_assert(kPartWords >= 1, "a thread's sixteen columns are whole words");
+    constexpr uint32_t kStepWords = kDeqStepCols / U::kNq;
     constexpr uint32_t kPieceRows = 16 / F::kBytes;                  // rows of one 16-byte piece
     constexpr uint32_t kRowPitch = kRowWords + 4;                    // rows start four banks apart
     constexpr uint32_t kHeld = kTileRows * (kRowWords / 4) / kThreads;
+    constexpr uint32_t kStorePieces = kDeqStepCols * 16 / kThreads;  // 16-byte pieces a thread stores per step
     __shared__ __attribute__((aligned(16))) uint32_t lds_words[kTileRows * kRowPitch];
-    __shared__ __attribute__((aligned(16))) uint32_t lds_floats[kTileStepCols * 64];  // [column][word of rows]
+    __shared__ __attribute__((aligned(16))) uint32_t lds_floats[kDeqStepCols * 64];  // [column][word of rows, rotated]
 
     const uint32_t t = threadIdx.x;
     const uint32_t tile_r0 = blockIdx.x * kTileRows;
-    const uint32_t tile_c0 = blockIdx.y * (kSteps * kTileStepCols);
+    const uint32_t tile_c0 = blockIdx.y * kTileCols;
     const uint32_t cols = a.segments * a.segment;
     const BatchPos b = batch_pos(a, blockIdx.z);
-    const uint32_t steps_left = (cols - tile_c0 + kTileStepCols - 1) / kTileStepCols;
+    const uint32_t steps_left = (cols - tile_c0 + kDeqStepCols - 1) / kDeqStepCols;
     const uint32_t total = steps_left < kSteps ? steps_left : kSteps;
     const uint32_t rows_here = a.rows - tile_r0 < kTileRows ? a.rows - tile_r0 : kTileRows;
     const uint32_t words_here = (cols - tile_c0) / U::kNq < kRowWords ? (cols - tile_c0) / U::kNq : kRowWords;
 
-    // every load of the workgroup goes out first: its codes, then the scales of this thread's rows and parts
+    // every load of the workgroup's codes goes out first
     const uint32_t* tile_in = static_cast<const uint32_t*>(a.input) + b.v + static_cast<uint64_t>(tile_r0) * a.vrow + tile_c0 / U::kNq;
     u32x4 held[kHeld];
 #pragma unroll
@@ -724,19 +731,11 @@ __global__ __launch_bounds__(kThreads) void dequantize_transposed_tile_kernel(Tr
         held[k] = live ? stream_load(reinterpret_cast<const u32x4*>(tile_in + static_cast<uint64_t>(live ? row : 0) * a.vrow + (live ? q * 4 : 0)))
                        : u32x4{0u, 0u, 0u, 0u};
     }
-    const uint32_t rp = t & 63u, part = t >> 6;
+    // thread (rp, part): rows rp * kRp ..., columns part * 16 ... of every step
+    const uint32_t part = t & 3u, rp = t >> 2;
     const uint32_t row0 = tile_r0 + rp * kRp;
-    RawScale raw_scale[kSteps][kRp];
-#pragma unroll
-    for (uint32_t step = 0; step < kSteps; step++) {
-        const uint32_t c0 = tile_c0 + step * kTileStepCols + part * kTilePart;
-        const bool live = row0 < a.rows && c0 < cols && !a.tensor_level;  // rows is a multiple of kRp
-#pragma unroll
-        for (uint32_t j = 0; j < kRp; j++) {
-            const uint64_t si = live ? b.sa + static_cast<uint64_t>(row0 + j) * a.sa_row + static_cast<uint64_t>(c0 / a.segment) * a.sa_col : 0;
-            raw_scale[step][j] = load_dtype_raw(a.param_dtype, a.scale_in, si);
-        }
-    }
+    const bool row_live = row0 < a.rows;  // rows is a multiple of kRp
+    const char* const scale0 = static_cast<const char*>(a.scale_in);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (uint32_t k = 0; k < kHeld; k++) {
@@ -748,9 +747,16 @@ __global__ __launch_bounds__(kThreads) void dequantize_transposed_tile_kernel(Tr
     const uint32_t piece = t & 15u, col_sub = t >> 4;
     const bool rows_live = tile_r0 + piece * kPieceRows < a.rows;    // rows is a multiple of kPieceRows
     char* const out0 = static_cast<char*>(a.output) + (b.f + tile_r0 + static_cast<uint64_t>(piece) * kPieceRows) * F::kBytes;
+    for (uint32_t step = 0; step < total; step++) {
+        // the scales of this thread's rows for the step (the words are on their way or there already)
+        const uint32_t c0 = tile_c0 + step * kDeqStepCols + part * kDeqPart;
+        const bool live = row_live && c0 < cols && !a.tensor_level;
+        RawScale raw_scale[kRp];
 #pragma unroll
-    for (uint32_t step = 0; step < kSteps; step++) {
-        if (step >= total) break;  // the same for the whole workgroup
+        for (uint32_t j = 0; j < kRp; j++) {
+            const uint64_t si = live ? b.sa + static_cast<uint64_t>(row0 + j) * a.sa_row + static_cast<uint64_t>(c0 / a.segment) * a.sa_col : 0;
+            raw_scale[j] = load_dtype_raw(a.param_dtype, scale0, si);
+        }
         __syncthreads();  // the words are in LDS (first step); the previous step's columns have left the floats
         uint32_t w[kRp][kPartWords];
 #pragma unroll
@@ -758,7 +764,8 @@ __global__ __launch_bounds__(kThreads) void dequantize_transposed_tile_kernel(Tr
             load_words<kPartWords>(&lds_words[(rp * kRp + j) * kRowPitch + step * kStepWords + part * kPartWords], w[j], kPartWords);
         float sc[kRp];
 #pragma unroll
-        for (uint32_t j = 0; j < kRp; j++) sc[j] = F::round(widen_dtype_raw(a.param_dtype, raw_scale[step][j]));  // Line::cast_from(scale)
+        for (uint32_t j = 0; j < kRp; j++) sc[j] = F::round(widen_dtype_raw(a.param_dtype, raw_scale[j]));  // Line::cast_from(scale)
+        const uint32_t word_of_rows = rp ^ (part << 4);  // this thread's place in every column of its group
 #pragma unroll
         for (uint32_t k = 0; k < kPartWords; k++) {
             float y[kRp][U::kNq];
@@ -770,19 +777,20 @@ __global__ __launch_bounds__(kThreads) void dequantize_transposed_tile_kernel(Tr
                 if constexpr (F::kBytes == 4) {
                     word = f32_bits(sc[0] * y[0][i]);
                 } else if constexpr (F::kDtype == CQ_BF16) {
-                    word = BF16::pack2(sc[0] * y[0][i], sc[1] * y[1][i]);
+                    word = BF16::pack2(sc[0] * y[0][i], sc[kRp - 1] * y[kRp - 1][i]);
                 } else {
-                    word = element_bits<F>(sc[0] * y[0][i]) | element_bits<F>(sc[1] * y[1][i]) << 16;
+                    word = element_bits<F>(sc[0] * y[0][i]) | element_bits<F>(sc[kRp - 1] * y[kRp - 1][i]) << 16;
                 }
-                lds_floats[(part * kTilePart + k * U::kNq + i) * 64 + rp] = word;
+                lds_floats[(part * kDeqPart + k * U::kNq + i) * 64 + word_of_rows] = word;
             }
         }
         __syncthreads();
 #pragma unroll
-        for (uint32_t i = 0; i < 8; i++) {
-            const uint32_t c = tile_c0 + step * kTileStepCols + i * 16 + col_sub;
+        for (uint32_t i = 0; i < kStorePieces; i++) {
+            const uint32_t lc = i * 16 + col_sub;  // column of the step; its group of sixteen is i
+            const uint32_t c = tile_c0 + step * kDeqStepCols + lc;
             if (rows_live && c < cols)
-                stream_store(*reinterpret_cast<const u32x4*>(&lds_floats[(i * 16 + col_sub) * 64 + piece * 4]),
+                stream_store(*reinterpret_cast<const u32x4*>(&lds_floats[lc * 64 + ((piece * 4) ^ (i << 4))]),
                              reinterpret_cast<u32x4*>(out0 + static_cast<uint64_t>(c) * a.pitch_f * F::kBytes));
         }
     }
