@@ -443,6 +443,20 @@ template <class F>
 constexpr uint32_t kTileRowsPerThread = 4 / F::kBytes;
 constexpr uint32_t kTileStepCols = 128, kTilePart = 32;
 
+// Which tile a workgroup of the tile kernels takes.  Workgroup i of a launch runs on XCD i % 8, each with an L2 of
+// its own: XCD x takes the x-th eighth of the tiles, in order, rows fastest, so that the 256-byte runs which
+// neighbouring row tiles read or write in the same columns pass through one L2 at about the same time.
+// The grid is (8 * ceil(tiles / 8), 1, batches); workgroups beyond the last tile leave at once.
+struct TilePlace {
+    uint32_t row_tile, col_tile;
+    bool live;
+};
+__device__ __forceinline__ TilePlace tile_place(uint32_t row_tiles, uint32_t col_tiles) {
+    const uint32_t total = row_tiles * col_tiles, per_xcd = gridDim.x / 8;
+    const uint32_t tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    return TilePlace{tile % row_tiles, tile / row_tiles, tile < total};
+}
+
 template <class F, int kBits, int kEnc, int kScale>
 __global__ __launch_bounds__(kThreads) void quantize_transposed_tile_kernel(TransposedArgs a, QuantParams qp) {
     using U = Unit<F, kBits>;
@@ -460,9 +474,12 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_tile_kernel(Tran
     __shared__ uint32_t lds_scales[kTileRows * kRowParts];
 
     const uint32_t t = threadIdx.x;
-    const uint32_t tile_r0 = blockIdx.x * kTileRows;
-    const uint32_t tile_c0 = blockIdx.y * (kSteps * kTileStepCols);
     const uint32_t cols = a.segments * a.segment;
+    const TilePlace place = tile_place((a.rows + kTileRows - 1) / kTileRows,
+                                       (cols + kSteps * kTileStepCols - 1) / (kSteps * kTileStepCols));
+    if (!place.live) return;  // the whole workgroup
+    const uint32_t tile_r0 = place.row_tile * kTileRows;
+    const uint32_t tile_c0 = place.col_tile * (kSteps * kTileStepCols);
     const uint32_t parts_per_block = a.segment / kTilePart;
     const BatchPos b = batch_pos(a, blockIdx.z);
     const uint32_t steps_left = (cols - tile_c0 + kTileStepCols - 1) / kTileStepCols;
@@ -712,9 +729,11 @@ __global__ __launch_bounds__(kThreads) void dequantize_transposed_tile_kernel(Tr
     __shared__ __attribute__((aligned(16))) uint32_t lds_floats[kDeqStepCols * 64];  // [column][word of rows, rotated]
 
     const uint32_t t = threadIdx.x;
-    const uint32_t tile_r0 = blockIdx.x * kTileRows;
-    const uint32_t tile_c0 = blockIdx.y * kTileCols;
     const uint32_t cols = a.segments * a.segment;
+    const TilePlace place = tile_place((a.rows + kTileRows - 1) / kTileRows, (cols + kTileCols - 1) / kTileCols);
+    if (!place.live) return;  // the whole workgroup
+    const uint32_t tile_r0 = place.row_tile * kTileRows;
+    const uint32_t tile_c0 = place.col_tile * kTileCols;
     const BatchPos b = batch_pos(a, blockIdx.z);
     const uint32_t steps_left = (cols - tile_c0 + kDeqStepCols - 1) / kDeqStepCols;
     const uint32_t total = steps_left < kSteps ? steps_left : kSteps;
@@ -860,11 +879,12 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
                  (cols / (32u / static_cast<uint32_t>(bits))) % 4 == 0 && a.batches <= 65535;
     for (uint32_t k = 0; k < a.num_batch_dims; k++) tiles = tiles && a.batch_v[k] % 4 == 0;
     const uint32_t tile_cols = 16u / static_cast<uint32_t>(bits) * kTileStepCols;
-    const dim3 tile_grid((a.rows + 64 * kTileRowsPerThread<F> - 1) / (64 * kTileRowsPerThread<F>), (cols + tile_cols - 1) / tile_cols,
-                         a.batches);
+    const uint64_t tile_count = static_cast<uint64_t>((a.rows + 64 * kTileRowsPerThread<F> - 1) / (64 * kTileRowsPerThread<F>)) *
+                                ((cols + tile_cols - 1) / tile_cols);
+    const dim3 tile_grid(static_cast<uint32_t>((tile_count + 7) / 8 * 8), 1, a.batches);  // see tile_place()
     // two rounds of resident workgroups and more; below that the quads kernel's many small workgroups win
     // (bf16 [4096, 4096], 4-bit: 14.3 us against 16.0 us; [8192, 8192], 2-bit: 43.6 us against 51.1 us)
-    if (tile_grid.y > 65535 || static_cast<uint64_t>(tile_grid.x) * tile_grid.y * tile_grid.z < 1024) tiles = false;
+    if (tile_count >= (1u << 31) || tile_count * a.batches < 1024) tiles = false;
 #define CQ_LAUNCH(B, W, E)                                                                                        \
     {                                                                                                             \
         if (tiles && !W)                                                                                          \
@@ -906,12 +926,13 @@ hipError_t dequantize_transposed(hipStream_t s, int bits, const TransposedArgs& 
                  a.vrow % 4 == 0 && (cols / (32u / static_cast<uint32_t>(bits))) % 4 == 0 && a.batches <= 65535;
     for (uint32_t k = 0; k < a.num_batch_dims; k++) tiles = tiles && a.batch_v[k] % 4 == 0;
     const uint32_t tile_cols = 16u / static_cast<uint32_t>(bits) * kTileStepCols;
-    const dim3 tile_grid((a.rows + 64 * kTileRowsPerThread<F> - 1) / (64 * kTileRowsPerThread<F>), (cols + tile_cols - 1) / tile_cols,
-                         a.batches);
+    const uint64_t tile_count = static_cast<uint64_t>((a.rows + 64 * kTileRowsPerThread<F> - 1) / (64 * kTileRowsPerThread<F>)) *
+                                ((cols + tile_cols - 1) / tile_cols);
+    const dim3 tile_grid(static_cast<uint32_t>((tile_count + 7) / 8 * 8), 1, a.batches);  // see tile_place()
     // 16-bit floats in four rounds of resident workgroups and more: bf16 [28672, 8192], 4-bit, 125 us against 134 us,
     // [8192, 28672] 115 us against 134 us; [8192, 8192] 37 us against 31 us and f32 [8192, 8192] 61 us against 47 us
     // stay with the lane-per-row kernel
-    if (F::kBytes != 2 || tile_grid.y > 65535 || static_cast<uint64_t>(tile_grid.x) * tile_grid.y * tile_grid.z < 2048) tiles = false;
+    if (F::kBytes != 2 || tile_count >= (1u << 31) || tile_count * a.batches < 2048) tiles = false;
 #define CQ_LAUNCH(B, E)                                                                                       \
     {                                                                                                         \
         if constexpr (F::kBytes == 2) {                                                                       \
