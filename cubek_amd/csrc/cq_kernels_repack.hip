@@ -134,6 +134,8 @@ struct TileArgs {
     const uint32_t* in;
     uint32_t* out;
     uint32_t wp, wl;        // input words along p, output words along l
+    uint32_t tiles_p, tiles_l;  // tiles along p and along l
+    uint32_t by_xcd;            // tiles numbered XCD by XCD (launches of 2048 tiles and more)
     uint64_t in_l_stride;   // input stride of the last dimension, in words
     uint64_t out_p_stride;  // output stride of the packed dimension, in words
     uint32_t num_batch_dims;
@@ -172,7 +174,17 @@ __global__ __launch_bounds__(kTileWords / 4 * kTileCols) void repack_tile_kernel
     constexpr int kRot = 64 / kQuads >= 4 ? 64 / kQuads : 4;
     __shared__ uint32_t lds[kTileRows * kTileCols];
     const uint32_t pq = threadIdx.x % kQuads, lw = threadIdx.x / kQuads;
-    const uint32_t pw0 = blockIdx.x * kTileWords, lw0 = blockIdx.y * kTileCols;
+    // Workgroup i of a launch runs on XCD i % 8, each with an L2 of its own.  In launches of many tiles XCD x takes
+    // the x-th eighth of the tiles, in order (along the packed dimension first, for 8-bit fields along the last
+    // one), so that neighbouring tiles pass through one L2: transposed 4-bit codes [8192, 28672] 47.5 -> 45.9 us,
+    // with a row pitch of 8320 words' worth 54.2 -> 48.3 us; 8-bit fields 96.6 -> 88.9 us.  The grid is
+    // (8 * ceil(tiles / 8), 1, batches).
+    const uint32_t per_xcd = gridDim.x / 8;
+    const uint32_t tile = a.by_xcd ? (blockIdx.x % 8) * per_xcd + blockIdx.x / 8 : blockIdx.x;
+    if (tile >= a.tiles_p * a.tiles_l) return;  // the whole workgroup
+    const bool p_first = kP != 4 || !a.by_xcd;
+    const uint32_t pw0 = (p_first ? tile % a.tiles_p : tile / a.tiles_l) * kTileWords;
+    const uint32_t lw0 = (p_first ? tile / a.tiles_p : tile % a.tiles_l) * kTileCols;
     uint64_t in_base = 0, out_base = 0;
     {
         uint32_t rem = blockIdx.z;
@@ -251,8 +263,11 @@ bool plan_tiles(const RepackArgs& a, TileArgs* t, dim3* grid, uint32_t tile_word
     }
     const uint64_t tiles_p = (t->wp + tile_words - 1) / tile_words;
     const uint64_t tiles_l = (t->wl + tile_cols - 1) / tile_cols;
-    if (batches > 65535 || tiles_l > 65535 || tiles_p > 0x7fffffffull) return false;
-    *grid = dim3(static_cast<uint32_t>(tiles_p), static_cast<uint32_t>(tiles_l), static_cast<uint32_t>(batches));
+    if (batches > 65535 || tiles_p * tiles_l > 0x7ffffff0ull) return false;
+    t->tiles_p = static_cast<uint32_t>(tiles_p);
+    t->tiles_l = static_cast<uint32_t>(tiles_l);
+    t->by_xcd = tiles_p * tiles_l >= 2048;
+    *grid = dim3(static_cast<uint32_t>((tiles_p * tiles_l + 7) / 8 * 8), 1, static_cast<uint32_t>(batches));
     return true;
 }
 
