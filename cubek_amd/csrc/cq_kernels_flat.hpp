@@ -219,6 +219,11 @@ struct LaneRows {
     // one step of at most one carry
     uint32_t near;
     uint32_t group_log2;    // lanes per block as a power of two, for the kernels that take it at run time (kGroupRt)
+    // Tile order (0 = as numbered).  Where whole tiles fit the innermost level and the next level lies closer in
+    // memory in the tensor that is read (heads next to each other behind positions, rows of 512 bytes and more),
+    // workgroups that run together take the same tile of neighbouring entries of that level: slabs of order_inner x order_outer tiles are walked
+    // outer entry first, and what the strided tensor sees are runs side by side instead of one run per workgroup.
+    uint32_t order_inner, order_outer, order_outer_magic, order_outer_shift, order_slab_magic, order_slab_shift;
     // blocks of `scale_rows` entries of the innermost level (by a lane group of columns) share their scale
     // (given scales only); the scale strides of that level are per block of rows
     uint32_t scale_rows, scale_magic, scale_shift;
@@ -246,8 +251,17 @@ struct LaneSteps {
     char* scale_out_[kUnroll];
     uint32_t col_[kUnroll];  // the lane's chunk within its row
     bool live_[kUnroll], first_[kUnroll], block_row_[kUnroll];
-    __device__ __forceinline__ LaneSteps(const LanesGeo& g, uint32_t tile) {
+    __device__ __forceinline__ LaneSteps(const LanesGeo& g, uint32_t tile_as_launched) {
         const LaneRows& r = g.rows;
+        uint32_t tile = tile_as_launched;
+        if (r.order_inner != 0) {  // only launches that start at tile 0 carry an order
+            const uint32_t slab_tiles = r.order_inner * r.order_outer;
+            const uint32_t slab = magic_div(tile, r.order_slab_magic, r.order_slab_shift);
+            const uint32_t within = tile - slab * slab_tiles;
+            const uint32_t inner = magic_div(within, r.order_outer_magic, r.order_outer_shift);
+            const uint32_t outer = within - inner * r.order_outer;
+            tile = slab * slab_tiles + outer * r.order_inner + inner;
+        }
         // The shape of the launch is the same for every lane, so the cases below are scalar branches.
         if (r.levels == 1 && r.count[0] == 1) {
             // a single row (one contiguous run): chunk numbers are positions already
