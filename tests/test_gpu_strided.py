@@ -161,6 +161,16 @@ def test_short_rows_behind_a_long_innermost_dimension(gpu, oracle, elem, name, s
                   ("middle_swapped", "middle_swapped_floats", "leading_swapped"))
 
 
+@pytest.mark.parametrize("name,scheme", SCHEMES, ids=[n for n, _ in SCHEMES])
+@pytest.mark.parametrize("elem", [ElemType.F32, ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
+def test_long_rows_behind_permuted_dimensions_in_whole_tiles(gpu, oracle, elem, name, scheme):
+    """Attention-shaped views with rows of 512 bytes and more whose position axis is a whole number of workgroup
+    tiles: the launch reads them head by head (its workgroups take their tiles in another order than they are
+    numbered in)."""
+    check_layouts(gpu, oracle, elem, name, scheme, ((2, 3, 1024, 256), (1, 5, 512, 512), (2, 2, 3, 256, 256)),
+                  ("middle_swapped", "middle_swapped_floats"))
+
+
 BLOCKS_OF_ROWS = [
     ("q8s_block_16x32", QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([16, 32]))),
     ("q4s_block_8x64", QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([8, 64]))),
