@@ -378,6 +378,7 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
             l.count[k - 1] * n < (1ull << 31)) {
             l.count[k - 1] *= static_cast<uint32_t>(n);
         } else {
+            if (k == static_cast<uint32_t>(cq::kMaxLaneLevels)) return false;  // too many levels: the row kernels' layout
             l.count[k] = static_cast<uint32_t>(n);
             l.in[k] = in;
             l.out[k] = out;

@@ -24,10 +24,14 @@ struct Range {
 
 // Rows that each lane finds for itself (short rows, leading dimensions with strides of their own):
 // the leading dimensions innermost first, `count` entries each, and the bytes per entry in the four tensors.
+// The lane-wise kernels walk at most this many levels of leading dimensions (after neighbours that every tensor
+// steps through uniformly are merged): rank 5 without any merging.  Their launch arguments live in scalar
+// registers, and seven levels spilled a third of them.  Deeper layouts take the row kernels.
+constexpr int kMaxLaneLevels = 4;
 struct LaneLevels {
     uint32_t levels;  // 0: not used
-    uint32_t count[CQ_MAX_RANK - 1];
-    uint64_t in[CQ_MAX_RANK - 1], out[CQ_MAX_RANK - 1], scale_in[CQ_MAX_RANK - 1], scale_out[CQ_MAX_RANK - 1];
+    uint32_t count[kMaxLaneLevels];
+    uint64_t in[kMaxLaneLevels], out[kMaxLaneLevels], scale_in[kMaxLaneLevels], scale_out[kMaxLaneLevels];
 };
 
 // Flat fast path: contiguous tensors, scales contiguous, blocks are runs of

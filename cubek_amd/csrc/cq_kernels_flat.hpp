@@ -207,8 +207,7 @@ struct RowSteps {
 // kGroup of the lane-wise kernels that serve every block size: the lanes per block come with the launch
 // (LaneRows::group_log2), one instantiation instead of one per block size.  Per tensor stays kGroup = 0.
 constexpr int kGroupRt = -1;
-constexpr int kMaxLaneLevels = 7;
-constexpr int kNearLaneLevels = 4;  // levels the lanes' short cut from their tile's first row walks (LaneRows::near)
+constexpr int kNearLaneLevels = kMaxLaneLevels;  // levels the lanes' short cut from their tile's first row walks (LaneRows::near)
 struct LaneRows {
     uint32_t row_chunks, row_magic, row_shift;
     uint32_t total_chunks;  // < 2^31

@@ -119,7 +119,6 @@ void set_near(LaneRows* r) {
 }
 
 // the same for the kernels that find each lane's row
-static_assert(kMaxLaneLevels == CQ_MAX_RANK - 1, "one level per leading dimension");
 // `unroll` > 0: the launch covers the whole tensor from tile 0 with tiles of kThreads * unroll chunks, so its
 // workgroups may take the tiles in another order (LaneRows::order_*).
 LaneRows lane_rows(const FlatArgs& a, int unroll = 0) {
