@@ -151,12 +151,12 @@ __device__ __forceinline__ void load_words(const uint32_t* src, uint32_t* w, uin
     for (int k = 0; k < kCount; k++) w[k] = static_cast<uint32_t>(k) < valid ? src[k] : 0u;
 }
 
-// 32 values of one row -> codes -> the piece's stored words
-template <class F, int kBits, bool kWide, int kEnc>
+// kPiece (32 or 16) values of one row -> codes -> the piece's stored words
+template <class F, int kBits, bool kWide, int kEnc, uint32_t kPiece = 32>
 __device__ __forceinline__ void quantize_piece_words(const float* v, float d, bool tame, const QuantParams& qp, uint32_t* pw) {
     using U = Unit<F, kBits>;
     constexpr int kN = U::kN;
-    constexpr uint32_t kPiece = 32;
+    static_assert(kPiece % U::kV == 0, "a piece is whole units");
 #pragma unroll
     for (uint32_t u = 0; u < kPiece / U::kV; u++) {
         uint32_t w[2] = {0, 0};
@@ -433,15 +433,15 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_quads_kernel(Tra
 // Tiles through LDS, for runs of 16 bytes along r: the float side and the stored side both move whole runs.
 // The kernels above keep a block's floats in registers (64 - 128 of them per lane, two waves per SIMD, loads
 // and arithmetic of a wave taking turns); here the registers hold only what is in flight.  A workgroup owns
-// kTileRows = 128 (16-bit types) or 64 (f32) rows by 16 / kBits * 128 columns and walks the columns 128 at a
-// time.  Per step: every thread loads eight 16-byte pieces (a wave: four columns by 256 bytes) into registers,
-// which go to LDS behind a barrier while the next step's loads are already on their way; then a thread takes
-// 32 columns of one LDS word of rows (two rows of a 16-bit type: 32 conflict-free ds_read_b32), quantizes
-// them as the other kernels do, and leaves words and scales in LDS.  After the last step the tile's words leave
-// as runs of 256 bytes per row, its scales as runs of up to 64.
+// kTileRows = 128 (16-bit types) or 64 (f32) rows and walks its columns 64 at a time.  Per step: every thread
+// loads four 16-byte pieces (a wave: four columns by 256 bytes) into registers, which go to LDS behind a
+// barrier while the next step's loads are already on their way; then a thread takes 16 columns of one LDS
+// word of rows (two rows of a 16-bit type: 16 conflict-free ds_read_b32), quantizes them as the other kernels
+// do, and leaves words and scales in LDS.  After the last step the tile's words leave as runs of 128 bytes
+// per row, its scales as runs of up to 32.
 template <class F>
 constexpr uint32_t kTileRowsPerThread = 4 / F::kBytes;
-constexpr uint32_t kTileStepCols = 128, kTilePart = 32;
+constexpr uint32_t kTilePart = 32;  // columns of the smallest block the tile kernels take
 
 // Which tile a workgroup of the tile kernels takes.  Workgroup i of a launch runs on XCD i % 8, each with an L2 of
 // its own: XCD x takes the x-th eighth of the tiles, in order, rows fastest, so that the 256-byte runs which
@@ -457,75 +457,83 @@ __device__ __forceinline__ TilePlace tile_place(uint32_t row_tiles, uint32_t col
     return TilePlace{tile % row_tiles, tile / row_tiles, tile < total};
 }
 
+// The quantize tile kernel in steps of 64 columns: thread (row pair, 16 columns), two neighbouring lanes share a
+// block of 32 columns (their maxima meet by DPP), 128 bytes of codes per row and tile.  16 KiB of floats, 18 KiB of
+// words and 4 KiB of scales per workgroup: four workgroups fit a compute unit instead of two.
+constexpr uint32_t kQStepCols = 64, kQPart = 16;
 template <class F, int kBits, int kEnc, int kScale>
 __global__ __launch_bounds__(kThreads) void quantize_transposed_tile_kernel(TransposedArgs a, QuantParams qp) {
     using U = Unit<F, kBits>;
     constexpr uint32_t kRp = kTileRowsPerThread<F>;
     constexpr uint32_t kTileRows = 64 * kRp;
-    constexpr uint32_t kSteps = 16 / kBits;                          // steps per tile: 256 bytes of codes per row
-    constexpr uint32_t kPartWords = kTilePart / U::kNq;
-    constexpr uint32_t kStepWords = kTileStepCols / U::kNq;
-    constexpr uint32_t kRowWords = kSteps * kStepWords;              // 64
-    constexpr uint32_t kRowParts = kSteps * (kTileStepCols / kTilePart);
+    constexpr uint32_t kRowWords = 32;                                // 128 bytes of codes per row and tile
+    constexpr uint32_t kTileCols = kRowWords * U::kNq;
+    constexpr uint32_t kSteps = kTileCols / kQStepCols;
+    constexpr uint32_t kPartWords = kQPart / U::kNq;
+    static_assert(kPartWords >= 1, "a thread's sixteen columns are whole words");
+    constexpr uint32_t kStepWords = kQStepCols / U::kNq;
+    constexpr uint32_t kRowParts = kTileCols / kTilePart;            // blocks of 32 columns per row and tile
     constexpr uint32_t kPieceRows = 16 / F::kBytes;                  // rows of one 16-byte piece
     constexpr uint32_t kRowPitch = kRowWords + 4;                    // rows start four banks apart
-    __shared__ __attribute__((aligned(16))) uint32_t lds_floats[kTileStepCols * 64];  // [column][word of rows]
+    constexpr uint32_t kHeld = kQStepCols * 16 / kThreads;           // 16-byte pieces a thread loads per step
+    __shared__ __attribute__((aligned(16))) uint32_t lds_floats[kQStepCols * 64];  // [column][word of rows, rotated]
     __shared__ __attribute__((aligned(16))) uint32_t lds_words[kTileRows * kRowPitch];
     __shared__ uint32_t lds_scales[kTileRows * kRowParts];
 
     const uint32_t t = threadIdx.x;
     const uint32_t cols = a.segments * a.segment;
-    const TilePlace place = tile_place((a.rows + kTileRows - 1) / kTileRows,
-                                       (cols + kSteps * kTileStepCols - 1) / (kSteps * kTileStepCols));
+    const TilePlace place = tile_place((a.rows + kTileRows - 1) / kTileRows, (cols + kTileCols - 1) / kTileCols);
     if (!place.live) return;  // the whole workgroup
     const uint32_t tile_r0 = place.row_tile * kTileRows;
-    const uint32_t tile_c0 = place.col_tile * (kSteps * kTileStepCols);
+    const uint32_t tile_c0 = place.col_tile * kTileCols;
     const uint32_t parts_per_block = a.segment / kTilePart;
     const BatchPos b = batch_pos(a, blockIdx.z);
-    const uint32_t steps_left = (cols - tile_c0 + kTileStepCols - 1) / kTileStepCols;
-    const uint32_t total = steps_left < kSteps ? steps_left : kSteps;  // steps of this workgroup
+    const uint32_t steps_left = (cols - tile_c0 + kQStepCols - 1) / kQStepCols;
+    const uint32_t total = steps_left < kSteps ? steps_left : kSteps;
     const uint32_t rows_here = a.rows - tile_r0 < kTileRows ? a.rows - tile_r0 : kTileRows;
 
-    // loads: piece k (16 bytes of rows) of column i * 16 + t / 16 of the step
+    // loads: piece `piece` (16 bytes of rows) of column i * 16 + t / 16 of the step
     const uint32_t piece = t & 15u, col_sub = t >> 4;
     const bool rows_live = tile_r0 + piece * kPieceRows < a.rows;    // rows is a multiple of kPieceRows
     const char* const in0 = static_cast<const char*>(a.input) +
                             (b.f + tile_r0 + static_cast<uint64_t>(piece) * kPieceRows) * F::kBytes;
-    const auto load_step = [&](u32x4* held, uint32_t step) {
+    u32x4 held[kHeld];
+    const auto load_step = [&](uint32_t step) {
 #pragma unroll
-        for (uint32_t i = 0; i < 8; i++) {
-            const uint32_t c = tile_c0 + step * kTileStepCols + i * 16 + col_sub;
+        for (uint32_t i = 0; i < kHeld; i++) {
+            const uint32_t c = tile_c0 + step * kQStepCols + i * 16 + col_sub;
             const bool live = rows_live && c < cols;
             const uint64_t off = static_cast<uint64_t>(live ? c : 0) * a.pitch_f * F::kBytes;
             held[i] = live ? stream_load(reinterpret_cast<const u32x4*>(in0 + off)) : u32x4{0u, 0u, 0u, 0u};
         }
         __builtin_amdgcn_sched_barrier(0);  // the loads go out here, a step ahead of their use
     };
-    // arithmetic: rows rp * kRp ... of part `part` (32 columns) of the step
-    const uint32_t rp = t & 63u, part = t >> 6;
+    // arithmetic: rows rp * kRp ..., columns part * 16 ... of the step; lanes 2k and 2k + 1 share a block of 32
+    const uint32_t part = t & 3u, rp = t >> 2;
     const uint32_t row0 = tile_r0 + rp * kRp;
+    const uint32_t word_of_rows = rp ^ (part << 4);  // this thread's place in every column of its group
 
-    // one step: the held pieces into LDS, the loads of the next step, then 32 columns per thread
-    const auto do_step = [&](u32x4* held, uint32_t step) {
+    load_step(0);
+    for (uint32_t step = 0; step < total; step++) {
         __syncthreads();  // the previous step's readers are done with the floats
 #pragma unroll
-        for (uint32_t i = 0; i < 8; i++)
-            *reinterpret_cast<u32x4*>(&lds_floats[(i * 16 + col_sub) * 64 + piece * 4]) = held[i];
+        for (uint32_t i = 0; i < kHeld; i++)
+            *reinterpret_cast<u32x4*>(&lds_floats[(i * 16 + col_sub) * 64 + ((piece * 4) ^ (i << 4))]) = held[i];
         __syncthreads();
-        if (step + 1 < total) load_step(held, step + 1);
+        if (step + 1 < total) load_step(step + 1);
 
-        const uint32_t c0 = tile_c0 + step * kTileStepCols + part * kTilePart;
+        const uint32_t c0 = tile_c0 + step * kQStepCols + part * kQPart;
         const bool live = row0 < a.rows && c0 < cols;  // rows is a multiple of kRp
-        uint32_t raw[kTilePart];
+        uint32_t raw[kQPart];
 #pragma unroll
-        for (uint32_t i = 0; i < kTilePart; i++) raw[i] = lds_floats[(part * kTilePart + i) * 64 + rp];
+        for (uint32_t i = 0; i < kQPart; i++) raw[i] = lds_floats[(part * kQPart + i) * 64 + word_of_rows];
         const uint32_t seg = c0 / a.segment;
         const bool first_part = (c0 % a.segment) == 0;
 #pragma unroll
         for (uint32_t j = 0; j < kRp; j++) {
-            float v[kTilePart];
+            float v[kQPart];
 #pragma unroll
-            for (uint32_t i = 0; i < kTilePart; i++) {
+            for (uint32_t i = 0; i < kQPart; i++) {
                 if constexpr (F::kBytes == 4) {
                     v[i] = bits_f32(raw[i]);
                 } else if constexpr (F::kDtype == CQ_BF16) {
@@ -536,10 +544,11 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_tile_kernel(Tran
                 }
             }
             float s_f;
-            if constexpr (kScale == 0) {  // blocks of 32 columns: the abs-max never leaves the thread
+            if constexpr (kScale == 0) {  // blocks of 32 columns: two lanes
                 float amax = 0.0f;
 #pragma unroll
-                for (uint32_t i = 0; i < kTilePart; i++) amax = fmaxf(amax, fabsf(v[i]));  // NaN elements drop out
+                for (uint32_t i = 0; i < kQPart; i++) amax = fmaxf(amax, fabsf(v[i]));  // NaN elements drop out
+                amax = group_max<2>(amax);
                 const float s32 = absmax_is_tame(amax) ? scale_from_absmax_tame(amax, qp) : scale_from_absmax(amax, qp.width);
                 s_f = F::round(s32);
             } else {
@@ -551,20 +560,16 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_tile_kernel(Tran
             if (a.tensor_level) {
                 if (a.scale_out != nullptr && b.first && row0 + j == 0 && c0 == 0) store_dtype(a.param_dtype, a.scale_out, 0, s_fs);
             } else if (first_part) {
-                lds_scales[(rp * kRp + j) * kRowParts + (step * kTileStepCols + part * kTilePart) / a.segment] = f32_bits(s_fs);
+                lds_scales[(rp * kRp + j) * kRowParts + (step * kQStepCols + part * kQPart) / a.segment] = f32_bits(s_fs);
             }
             const float d = F::round(s_fs);
             uint32_t pw[kPartWords];
-            quantize_piece_words<F, kBits, false, kEnc>(v, d, divisor_is_tame(d), qp, pw);
+            quantize_piece_words<F, kBits, false, kEnc, kQPart>(v, d, divisor_is_tame(d), qp, pw);
             store_words<kPartWords>(&lds_words[(rp * kRp + j) * kRowPitch + step * kStepWords + part * kPartWords], pw, kPartWords);
         }
-    };
-
-    u32x4 held[8];
-    load_step(held, 0);
-    for (uint32_t step = 0; step < total; step++) do_step(held, step);
+    }
     __syncthreads();
-    // the tile's words and scales out of LDS: 16 lanes x 16 bytes per row, then the scales of every row
+    // the tile's words and scales out of LDS: 8 lanes x 16 bytes per row, then the scales of every row
     const uint32_t words_here = (cols - tile_c0) / U::kNq < kRowWords ? (cols - tile_c0) / U::kNq : kRowWords;
     uint32_t* tile_out = static_cast<uint32_t*>(a.output) + b.v + static_cast<uint64_t>(tile_r0) * a.vrow + tile_c0 / U::kNq;
 #pragma unroll
@@ -878,7 +883,7 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
                  (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0 && a.vrow % 4 == 0 &&
                  (cols / (32u / static_cast<uint32_t>(bits))) % 4 == 0 && a.batches <= 65535;
     for (uint32_t k = 0; k < a.num_batch_dims; k++) tiles = tiles && a.batch_v[k] % 4 == 0;
-    const uint32_t tile_cols = 16u / static_cast<uint32_t>(bits) * kTileStepCols;
+    const uint32_t tile_cols = 32u * (32u / static_cast<uint32_t>(bits));  // 128 bytes of codes per row
     const uint64_t tile_count = static_cast<uint64_t>((a.rows + 64 * kTileRowsPerThread<F> - 1) / (64 * kTileRowsPerThread<F>)) *
                                 ((cols + tile_cols - 1) / tile_cols);
     const dim3 tile_grid(static_cast<uint32_t>((tile_count + 7) / 8 * 8), 1, a.batches);  // see tile_place()
@@ -925,7 +930,7 @@ hipError_t dequantize_transposed(hipStream_t s, int bits, const TransposedArgs& 
     bool tiles = a.segment % kTilePart == 0 && runs_of_16_bytes<F>(a, a.output) && (reinterpret_cast<uintptr_t>(a.input) & 15u) == 0 &&
                  a.vrow % 4 == 0 && (cols / (32u / static_cast<uint32_t>(bits))) % 4 == 0 && a.batches <= 65535;
     for (uint32_t k = 0; k < a.num_batch_dims; k++) tiles = tiles && a.batch_v[k] % 4 == 0;
-    const uint32_t tile_cols = 16u / static_cast<uint32_t>(bits) * kTileStepCols;
+    const uint32_t tile_cols = 64u * (32u / static_cast<uint32_t>(bits));  // 256 bytes of codes per row
     const uint64_t tile_count = static_cast<uint64_t>((a.rows + 64 * kTileRowsPerThread<F> - 1) / (64 * kTileRowsPerThread<F>)) *
                                 ((cols + tile_cols - 1) / tile_cols);
     const dim3 tile_grid(static_cast<uint32_t>((tile_count + 7) / 8 * 8), 1, a.batches);  // see tile_place()
