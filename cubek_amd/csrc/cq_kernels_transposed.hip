@@ -17,6 +17,7 @@
 // dequantize_transposed_kernel.
 #include "cq_device.hpp"
 #include "cq_internal.hpp"
+#include "cq_magic_div.hpp"
 
 namespace cq {
 namespace {
@@ -462,7 +463,9 @@ __device__ __forceinline__ TilePlace tile_place(uint32_t row_tiles, uint32_t col
 // words and 4 KiB of scales per workgroup: four workgroups fit a compute unit instead of two.
 constexpr uint32_t kQStepCols = 64, kQPart = 16;
 template <class F, int kBits, int kEnc, int kScale>
-__global__ __launch_bounds__(kThreads) void quantize_transposed_tile_kernel(TransposedArgs a, QuantParams qp) {
+// seg_magic / seg_shift: column / a.segment as a multiplication and a shift (cq_magic_div.hpp; columns below 2^31)
+__global__ __launch_bounds__(kThreads) void quantize_transposed_tile_kernel(TransposedArgs a, QuantParams qp, uint32_t seg_magic,
+                                                                            uint32_t seg_shift) {
     using U = Unit<F, kBits>;
     constexpr uint32_t kRp = kTileRowsPerThread<F>;
     constexpr uint32_t kTileRows = 64 * kRp;
@@ -527,8 +530,11 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_tile_kernel(Tran
         uint32_t raw[kQPart];
 #pragma unroll
         for (uint32_t i = 0; i < kQPart; i++) raw[i] = lds_floats[(part * kQPart + i) * 64 + word_of_rows];
-        const uint32_t seg = c0 / a.segment;
-        const bool first_part = (c0 % a.segment) == 0;
+        // the fused abs-max is launched for blocks of 32 columns only; other block sizes divide by multiplication
+        const uint32_t seg = kScale == 0 ? c0 / kTilePart : magic_div(c0, seg_magic, seg_shift);
+        const uint32_t segment = kScale == 0 ? kTilePart : a.segment;
+        const bool first_part = c0 == seg * segment;
+        const uint32_t scale_slot = seg - (kScale == 0 ? tile_c0 / kTilePart : magic_div(tile_c0, seg_magic, seg_shift));
 #pragma unroll
         for (uint32_t j = 0; j < kRp; j++) {
             float v[kQPart];
@@ -560,7 +566,7 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_tile_kernel(Tran
             if (a.tensor_level) {
                 if (a.scale_out != nullptr && b.first && row0 + j == 0 && c0 == 0) store_dtype(a.param_dtype, a.scale_out, 0, s_fs);
             } else if (first_part) {
-                lds_scales[(rp * kRp + j) * kRowParts + (step * kQStepCols + part * kQPart) / a.segment] = f32_bits(s_fs);
+                lds_scales[(rp * kRp + j) * kRowParts + scale_slot] = f32_bits(s_fs);
             }
             const float d = F::round(s_fs);
             uint32_t pw[kPartWords];
@@ -716,7 +722,8 @@ __global__ __launch_bounds__(kThreads) void dequantize_transposed_wide_kernel(Tr
 // columns, or per tensor.
 constexpr uint32_t kDeqStepCols = 64, kDeqPart = 16;
 template <class F, int kBits, int kEnc>
-__global__ __launch_bounds__(kThreads) void dequantize_transposed_tile_kernel(TransposedArgs a) {
+__global__ __launch_bounds__(kThreads) void dequantize_transposed_tile_kernel(TransposedArgs a, uint32_t seg_magic,
+                                                                              uint32_t seg_shift) {
     using U = Unit<F, kBits>;
     constexpr uint32_t kRp = kTileRowsPerThread<F>;
     constexpr uint32_t kTileRows = 64 * kRp;
@@ -778,7 +785,9 @@ __global__ __launch_bounds__(kThreads) void dequantize_transposed_tile_kernel(Tr
         RawScale raw_scale[kRp];
 #pragma unroll
         for (uint32_t j = 0; j < kRp; j++) {
-            const uint64_t si = live ? b.sa + static_cast<uint64_t>(row0 + j) * a.sa_row + static_cast<uint64_t>(c0 / a.segment) * a.sa_col : 0;
+            const uint64_t si = live ? b.sa + static_cast<uint64_t>(row0 + j) * a.sa_row +
+                                           static_cast<uint64_t>(magic_div(c0, seg_magic, seg_shift)) * a.sa_col
+                                     : 0;
             raw_scale[j] = load_dtype_raw(a.param_dtype, scale0, si);
         }
         __syncthreads();  // the words are in LDS (first step); the previous step's columns have left the floats
@@ -879,7 +888,9 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
     // abs-max, any multiple of 32 for given scales): 4-bit codes of a transposed bf16 view [28672, 8192],
     // rotated buffers, against the quads kernel.
     const uint32_t cols = a.segments * a.segment;
-    bool tiles = runs_of_16_bytes<F>(a, a.input) && a.segment % kTilePart == 0 && (kScale == 1 || a.segment == kTilePart) &&
+    uint32_t seg_magic = 0, seg_shift = 0;
+    magic_of(a.segment, &seg_magic, &seg_shift);
+    bool tiles = cols < (1u << 31) && runs_of_16_bytes<F>(a, a.input) && a.segment % kTilePart == 0 && (kScale == 1 || a.segment == kTilePart) &&
                  (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0 && a.vrow % 4 == 0 &&
                  (cols / (32u / static_cast<uint32_t>(bits))) % 4 == 0 && a.batches <= 65535;
     for (uint32_t k = 0; k < a.num_batch_dims; k++) tiles = tiles && a.batch_v[k] % 4 == 0;
@@ -893,7 +904,8 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
 #define CQ_LAUNCH(B, W, E)                                                                                        \
     {                                                                                                             \
         if (tiles && !W)                                                                                          \
-            hipLaunchKernelGGL((quantize_transposed_tile_kernel<F, B, E, kScale>), tile_grid, dim3(kThreads), 0, s, a, qp); \
+            hipLaunchKernelGGL((quantize_transposed_tile_kernel<F, B, E, kScale>), tile_grid, dim3(kThreads), 0, s, a, qp, \
+                               seg_magic, seg_shift);                                                             \
         else if (quads)                                                                                           \
             hipLaunchKernelGGL((quantize_transposed_quads_kernel<F, B, W, E, kScale>), grid, dim3(kThreads), 0, s, q, qp); \
         else                                                                                                      \
@@ -927,7 +939,9 @@ hipError_t dequantize_transposed(hipStream_t s, int bits, const TransposedArgs& 
                     a.batches);
     // Tiles through LDS wherever both sides allow 16-byte accesses
     const uint32_t cols = a.segments * a.segment;
-    bool tiles = a.segment % kTilePart == 0 && runs_of_16_bytes<F>(a, a.output) && (reinterpret_cast<uintptr_t>(a.input) & 15u) == 0 &&
+    uint32_t seg_magic = 0, seg_shift = 0;
+    magic_of(a.segment, &seg_magic, &seg_shift);
+    bool tiles = cols < (1u << 31) && a.segment % kTilePart == 0 && runs_of_16_bytes<F>(a, a.output) && (reinterpret_cast<uintptr_t>(a.input) & 15u) == 0 &&
                  a.vrow % 4 == 0 && (cols / (32u / static_cast<uint32_t>(bits))) % 4 == 0 && a.batches <= 65535;
     for (uint32_t k = 0; k < a.num_batch_dims; k++) tiles = tiles && a.batch_v[k] % 4 == 0;
     const uint32_t tile_cols = 64u * (32u / static_cast<uint32_t>(bits));  // 256 bytes of codes per row
@@ -942,7 +956,8 @@ hipError_t dequantize_transposed(hipStream_t s, int bits, const TransposedArgs& 
     {                                                                                                         \
         if constexpr (F::kBytes == 2) {                                                                       \
             if (tiles) {                                                                                      \
-                hipLaunchKernelGGL((dequantize_transposed_tile_kernel<F, B, E>), tile_grid, dim3(kThreads), 0, s, a); \
+                hipLaunchKernelGGL((dequantize_transposed_tile_kernel<F, B, E>), tile_grid, dim3(kThreads), 0, s, a, \
+                                   seg_magic, seg_shift);                                                     \
                 return hipGetLastError();                                                                     \
             }                                                                                                 \
         }                                                                                                     \
