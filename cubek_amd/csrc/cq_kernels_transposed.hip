@@ -495,19 +495,24 @@ __global__ __launch_bounds__(kThreads) void quantize_transposed_tile_kernel(Tran
     const uint32_t total = steps_left < kSteps ? steps_left : kSteps;
     const uint32_t rows_here = a.rows - tile_r0 < kTileRows ? a.rows - tile_r0 : kTileRows;
 
-    // loads: piece `piece` (16 bytes of rows) of column i * 16 + t / 16 of the step
+    // loads: piece `piece` (16 bytes of rows) of column i * 16 + t / 16 of the step.  A step's address is a base
+    // that is the same for the whole workgroup plus 32 bits per thread (the launcher checked that 64 columns
+    // span less than 4 GiB); threads past the tensor's edge re-read the step's first piece, which nobody stores.
     const uint32_t piece = t & 15u, col_sub = t >> 4;
     const bool rows_live = tile_r0 + piece * kPieceRows < a.rows;    // rows is a multiple of kPieceRows
-    const char* const in0 = static_cast<const char*>(a.input) +
-                            (b.f + tile_r0 + static_cast<uint64_t>(piece) * kPieceRows) * F::kBytes;
+    const char* const in_tile = static_cast<const char*>(a.input) + (b.f + tile_r0) * F::kBytes;
+    const uint64_t col_bytes = a.pitch_f * F::kBytes;
+    const uint32_t off0 = col_sub * static_cast<uint32_t>(col_bytes) + piece * 16u;
     u32x4 held[kHeld];
     const auto load_step = [&](uint32_t step) {
+        const uint32_t step_c0 = tile_c0 + step * kQStepCols;
+        const char* const base = in_tile + step_c0 * col_bytes;
+        const uint32_t cols_left = cols - step_c0;
 #pragma unroll
         for (uint32_t i = 0; i < kHeld; i++) {
-            const uint32_t c = tile_c0 + step * kQStepCols + i * 16 + col_sub;
-            const bool live = rows_live && c < cols;
-            const uint64_t off = static_cast<uint64_t>(live ? c : 0) * a.pitch_f * F::kBytes;
-            held[i] = live ? stream_load(reinterpret_cast<const u32x4*>(in0 + off)) : u32x4{0u, 0u, 0u, 0u};
+            const bool live = rows_live && i * 16 + col_sub < cols_left;
+            const uint32_t off = off0 + i * 16u * static_cast<uint32_t>(col_bytes);
+            held[i] = stream_load(reinterpret_cast<const u32x4*>(base + (live ? off : 0u)));
         }
         __builtin_amdgcn_sched_barrier(0);  // the loads go out here, a step ahead of their use
     };
@@ -890,7 +895,7 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
     const uint32_t cols = a.segments * a.segment;
     uint32_t seg_magic = 0, seg_shift = 0;
     magic_of(a.segment, &seg_magic, &seg_shift);
-    bool tiles = cols < (1u << 31) && runs_of_16_bytes<F>(a, a.input) && a.segment % kTilePart == 0 && (kScale == 1 || a.segment == kTilePart) &&
+    bool tiles = cols < (1u << 31) && a.pitch_f * F::kBytes < (1u << 25) && runs_of_16_bytes<F>(a, a.input) && a.segment % kTilePart == 0 && (kScale == 1 || a.segment == kTilePart) &&
                  (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0 && a.vrow % 4 == 0 &&
                  (cols / (32u / static_cast<uint32_t>(bits))) % 4 == 0 && a.batches <= 65535;
     for (uint32_t k = 0; k < a.num_batch_dims; k++) tiles = tiles && a.batch_v[k] % 4 == 0;
