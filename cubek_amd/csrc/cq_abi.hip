@@ -684,7 +684,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
         a.range = p.range;
-        st = CQ_RUN(cq::flat_family(a), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, a));
+        st = CQ_RUN(cq::flat_family(a, input_dtype), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, a));
         if (st != CQ_OK) return st;
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
@@ -702,7 +702,7 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
-        return CQ_RUN(cq::flat_family(fr), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, fr));
+        return CQ_RUN(cq::flat_family(fr, input_dtype), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, fr));
     }
     cq::RowArgs r;
     if (streaming && flat_words == 0 && rows_args(p, scheme, input_dtype, input, output, &r)) {
@@ -764,7 +764,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
         a.range = p.range;
-        st = CQ_RUN(cq::flat_family(a), cq::launch_dequantize_flat(stream, output_dtype, p.bits, a));
+        st = CQ_RUN(cq::flat_family(a, output_dtype), cq::launch_dequantize_flat(stream, output_dtype, p.bits, a));
         if (st != CQ_OK) return st;
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
@@ -779,7 +779,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
-        return CQ_RUN(cq::flat_family(fr), cq::launch_dequantize_flat(stream, output_dtype, p.bits, fr));
+        return CQ_RUN(cq::flat_family(fr, output_dtype), cq::launch_dequantize_flat(stream, output_dtype, p.bits, fr));
     }
     cq::RowArgs r;
     if (streaming && flat_words == 0 && rows_args(p, scheme, output_dtype, output, values, &r)) {
@@ -896,7 +896,7 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
         a.num_chunks = p.n / (16 / dtype_size(input_dtype));
         a.block = p.block_last;
         a.range = p.range;
-        return CQ_RUN_AUX(cq::flat_family(a), cq::launch_scales_flat(stream, input_dtype, a));
+        return CQ_RUN_AUX(cq::flat_family(a, input_dtype), cq::launch_scales_flat(stream, input_dtype, a));
     }
     // pitched rows of at least a step of 256 chunks, 1-D blocks: the same kernel over the rows' steps
     // (rows in one uniform run or in groups with a pitch of their own, as in flat_rows_ok())
@@ -924,7 +924,7 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
             a.scale_out_outer = outer_of(ls) * elem;
             a.block = p.block_last;
             a.range = p.range;
-            return CQ_RUN_AUX(cq::flat_family(a), cq::launch_scales_flat(stream, input_dtype, a));
+            return CQ_RUN_AUX(cq::flat_family(a, input_dtype), cq::launch_scales_flat(stream, input_dtype, a));
         }
     }
     // short rows, rows behind several levels of strides: every lane finds its row
@@ -935,7 +935,7 @@ cq_status cq_compute_scales(cq_stream_t stream, const cq_tensor* input, const cq
         fl.scale_out = scales->ptr;
         fl.block = p.block_last;
         fl.range = p.range;
-        return CQ_RUN_AUX(cq::flat_family(fl), cq::launch_scales_flat(stream, input_dtype, fl));
+        return CQ_RUN_AUX(cq::flat_family(fl, input_dtype), cq::launch_scales_flat(stream, input_dtype, fl));
     }
     return produce_scales(stream, p, scheme, input, input_dtype, scales, input_dtype, workspace, workspace_bytes);
 }
@@ -984,7 +984,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
         a.range = p.range;
-        return CQ_RUN(cq::flat_family(a), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
+        return CQ_RUN(cq::flat_family(a, input_dtype), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
     }
 
     // pitched rows with 1-D blocks: the same fused kernel over the rows' steps
@@ -999,7 +999,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
-        return CQ_RUN(cq::flat_family(fr), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, fr));
+        return CQ_RUN(cq::flat_family(fr, input_dtype), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, fr));
     }
 
     // blocks over the last two dimensions (or 1-D blocks on layouts the flat kernel refuses): one
@@ -1020,7 +1020,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
             f2.param_dtype = pd;
             f2.encoding = flat_encoding(scheme);
             f2.range = p.range;
-            return CQ_RUN(cq::flat_family(f2), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Stored, f2));
+            return CQ_RUN(cq::flat_family(f2, input_dtype), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Stored, f2));
         }
     }
 
@@ -1067,7 +1067,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
         a.range = p.range;
-        st = CQ_RUN(cq::flat_family(a), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, a));
+        st = CQ_RUN(cq::flat_family(a, input_dtype), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, a));
         if (st != CQ_OK) return st;
         flat_words = flat_chunks * per_chunk / p.nq;
     } else if (p.tensor_level && (flat_rows_ok(p, scheme, input_dtype, input, output, out_scale, dtype_size(pd), nullptr, 0, false, &fr) ||
@@ -1085,7 +1085,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
-        return CQ_RUN(cq::flat_family(fr), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, fr));
+        return CQ_RUN(cq::flat_family(fr, input_dtype), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Partials, fr));
     } else {
         // scales as FS(F(scale)) into out_scale first, then quantize reading them back
         // (the divisor F(FS(scale)) is the same either way)

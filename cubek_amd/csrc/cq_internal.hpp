@@ -57,6 +57,7 @@ struct FlatArgs {
     int param_dtype;      // cq_dtype of the stored scales
     int encoding;         // 0 two's-complement fields (U32 store, native i8); 1 e4m3, 2 e5m2 bytes; 3 e2m1 nibbles
     Range range;
+    uint32_t whole_grid = 0;  // set between the launchers' objects only: whole tiles of the run to launch
 };
 
 enum class ScaleSource { Given, Dynamic, Partials, Stored };  // Stored: lane-wise launches only (FlatArgs::lanes)
@@ -68,7 +69,7 @@ hipError_t launch_scales_flat(hipStream_t s, int dtype, const FlatArgs& a);  // 
 bool flat_block_supported(int dtype, uint32_t block);
 // the cq_kernel_family a flat launch with these arguments runs on (whole tiles of a run, whole steps of
 // pitched rows, or lane by lane)
-uint32_t flat_family(const FlatArgs& a);
+uint32_t flat_family(const FlatArgs& a, int f_dtype);
 
 // Per-tensor abs-max, pass 1: writes `*num_partials` f32 partial maxima.
 constexpr uint32_t kMaxPartials = 256;

@@ -207,6 +207,7 @@ struct RowSteps {
 // kGroup of the lane-wise kernels that serve every block size: the lanes per block come with the launch
 // (LaneRows::group_log2), one instantiation instead of one per block size.  Per tensor stays kGroup = 0.
 constexpr int kGroupRt = -1;
+constexpr int kParamRt = -1;  // the type of the stored scales is a launch argument
 constexpr int kNearLaneLevels = kMaxLaneLevels;  // levels the lanes' short cut from their tile's first row walks (LaneRows::near)
 struct LaneRows {
     uint32_t row_chunks, row_magic, row_shift;
@@ -416,14 +417,14 @@ struct LaneSteps {
     __device__ __forceinline__ void* scale_out(int u) const { return scale_out_[u]; }
 };
 
-// kParamF32: the stored scales are f32 (the common case, resolved at compile
-//            time); otherwise `param_dtype_rt` selects f16 / bf16 at run time.
+// kParam   : the type of the stored scales where the kernel is compiled for one (f32, or the float type of the
+//            tensor itself); kParamRt: `param_dtype_rt` selects it at run time.
 // kWide    : the value range does not fit its field (E4M3 / E5M2 in 8 bits).
 // kChecked : the launch may run past `chunk_end` (ragged last tile): addresses
 //            are clamped and stores masked.  Full tiles use the unchecked variant.
 // kEnc     : stored encoding (kEncInt for the U32 store and native i8; e4m3 / e5m2 /
 //            e2m1 for the native float stores, where kBits is the stored width).
-template <class F, int kBits, int kGroup, int kScaleSrc, bool kParamF32, bool kWide, int kUnroll,
+template <class F, int kBits, int kGroup, int kScaleSrc, int kParam, bool kWide, int kUnroll,
           int kThreads, bool kChecked, int kEnc, class Geo>
 __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dtype_rt, const QuantParams& qp,
                                                    uint32_t num_partials) {
@@ -439,7 +440,7 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
     const auto starts_block = [&](auto c) { return kRtGroup ? (c & ((1u << group_log2) - 1u)) == 0 : (c % kDiv) == 0; };
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;  // 64, 32, 16 or 8
-    const int param_dtype = kParamF32 ? static_cast<int>(CQ_F32) : param_dtype_rt;
+    const int param_dtype = kParam != kParamRt ? kParam : param_dtype_rt;
     // Pass 2 of the per-tensor reduction walks the tiles last to first: pass 1 has just read the
     // tensor first to last, so what it read last is what the L2 caches still hold.  Groups of
     // eight consecutive tiles keep their places, because workgroup i runs on XCD i % 8 and tile
@@ -518,7 +519,7 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         }
         // write_scale (src/quantize.rs:83-98): FS(scale), stored by the block's first lane.  s_f is an F value, so
         // FS rounds it only where FS is a 16-bit type other than F (the same for the whole launch: a scalar branch)
-        const bool fs_rounds = !kParamF32 && param_dtype != CQ_F32 && param_dtype != F::kDtype;
+        const bool fs_rounds = param_dtype != CQ_F32 && param_dtype != F::kDtype;
         float s_fs = s_f;
         if (fs_rounds) s_fs = round_to_dtype(param_dtype, s_f);
         const auto si = kGroup == 0 ? 0 : block_of(c);
@@ -553,25 +554,28 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
     }
 }
 
-// One contiguous run of whole tiles, f32 parameters: the hot launch.  Ragged ends, other parameter types and
-// rows that are not whole steps run lane by lane (quantize_flat_lanes_kernel), which keeps the number of
-// kernels in the library, and with it its size and load time, at a third.
-template <class F, int kBits, int kGroup, int kScaleSrc, bool kWide, int kUnroll, int kThreads, int kEnc = kEncInt>
+// One contiguous run of whole tiles, parameters typed f32 or like the tensor (kParam): the hot launch.  Ragged
+// ends, other parameter types and rows that are not whole steps run lane by lane (quantize_flat_lanes_kernel),
+// which keeps the number of kernels in the library, and with it its size and load time, down.
+template <class F, int kBits, int kGroup, int kScaleSrc, bool kWide, int kUnroll, int kThreads, int kEnc = kEncInt,
+          int kParam = CQ_F32>
 __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
     void* __restrict__ scale_out, uint64_t chunk_begin, uint64_t chunk_end, QuantParams qp, uint32_t num_partials) {
     const RunGeo geo{in, out, scale_in, scale_out, chunk_begin, chunk_end};
-    quantize_flat_body<F, kBits, kGroup, kScaleSrc, true, kWide, kUnroll, kThreads, false, kEnc>(geo, CQ_F32, qp, num_partials);
+    quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParam, kWide, kUnroll, kThreads, false, kEnc>(geo, kParam, qp, num_partials);
 }
 
-// Pitched rows of whole steps, from step `step_begin` of the launch on, f32 parameters.  A kernel of its own
+// Pitched rows of whole steps, from step `step_begin` of the launch on, parameters as in quantize_flat_kernel.  A kernel of its own
 // so that the launches over one contiguous run carry none of the row arithmetic in their prologue.
-template <class F, int kBits, int kGroup, int kScaleSrc, bool kWide, int kUnroll, int kThreads, int kEnc = kEncInt>
+template <class F, int kBits, int kGroup, int kScaleSrc, bool kWide, int kUnroll, int kThreads, int kEnc = kEncInt,
+          int kParam = CQ_F32>
 __global__ __launch_bounds__(kThreads) void quantize_flat_rows_kernel(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
     void* __restrict__ scale_out, uint32_t step_begin, QuantParams qp, uint32_t num_partials, FlatRows rows) {
-    const RowsGeo<16, F::kPerChunk * kBits / 8, kGroup> geo{in, out, scale_in, scale_out, step_begin, F::kBytes, 4, rows};
-    quantize_flat_body<F, kBits, kGroup, kScaleSrc, true, kWide, kUnroll, kThreads, false, kEnc>(geo, CQ_F32, qp, num_partials);
+    const RowsGeo<16, F::kPerChunk * kBits / 8, kGroup> geo{in, out, scale_in, scale_out, step_begin, F::kBytes,
+                                                            kParam == CQ_F32 ? 4 : 2, rows};
+    quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParam, kWide, kUnroll, kThreads, false, kEnc>(geo, kParam, qp, num_partials);
 }
 
 // Rows found lane by lane (LaneSteps), bounds-checked; the scale type is read at run time.  `tile_begin`:
@@ -582,14 +586,14 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_lanes_kernel(
     void* __restrict__ scale_out, int param_dtype_rt, QuantParams qp, uint32_t num_partials, uint32_t tile_begin,
     LaneRows rows) {
     const LanesGeo geo{in, out, scale_in, scale_out, tile_begin, rows};
-    quantize_flat_body<F, kBits, kGroup, kScaleSrc, false, kWide, kUnroll, kThreads, true, kEnc>(geo, param_dtype_rt, qp,
+    quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParamRt, kWide, kUnroll, kThreads, true, kEnc>(geo, param_dtype_rt, qp,
                                                                                                num_partials);
 }
 
 // `scale_in` of the geometry holds the stored scales
-template <class F, int kBits, int kGroup, bool kParamF32, int kUnroll, int kThreads, bool kChecked, int kEnc, class Geo>
+template <class F, int kBits, int kGroup, int kParam, int kUnroll, int kThreads, bool kChecked, int kEnc, class Geo>
 __device__ __forceinline__ void dequantize_flat_body(const Geo& geo, int param_dtype_rt) {
-    const int param_dtype = kParamF32 ? static_cast<int>(CQ_F32) : param_dtype_rt;
+    const int param_dtype = kParam != kParamRt ? kParam : param_dtype_rt;
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;
     const typename Geo::template Steps<kUnroll, kThreads, kChecked> at(geo, blockIdx.x);
@@ -615,7 +619,7 @@ __device__ __forceinline__ void dequantize_flat_body(const Geo& geo, int param_d
         }
         auto si = kGroup == 0 ? 0 : c / (kGroup <= 0 ? 1 : kGroup);
         if constexpr (kGroup == kGroupRt) si = c >> geo.rows.group_log2;
-        if constexpr (kParamF32)
+        if constexpr (kParam == CQ_F32)
             sc[u] = F32::load(at.scale_in(u), si);
         else
             sc_raw[u] = load_dtype_raw(param_dtype, at.scale_in(u), si);
@@ -623,7 +627,7 @@ __device__ __forceinline__ void dequantize_flat_body(const Geo& geo, int param_d
     __builtin_amdgcn_sched_barrier(0);  // keep every load ahead of the arithmetic
 #pragma unroll
     for (int u = 0; u < kUnroll; u++)  // Line::cast_from(scale)
-        sc[u] = F::round(kParamF32 ? sc[u] : widen_dtype_raw(param_dtype, sc_raw[u]));
+        sc[u] = F::round(kParam == CQ_F32 ? sc[u] : widen_dtype_raw(param_dtype, sc_raw[u]));
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         float y[kN];
@@ -639,21 +643,21 @@ __device__ __forceinline__ void dequantize_flat_body(const Geo& geo, int param_d
     }
 }
 
-// whole tiles of one contiguous run, f32 parameters (see quantize_flat_kernel)
-template <class F, int kBits, int kGroup, int kUnroll, int kThreads, int kEnc = kEncInt>
+// whole tiles of one contiguous run, parameters typed f32 or like the tensor (see quantize_flat_kernel)
+template <class F, int kBits, int kGroup, int kUnroll, int kThreads, int kEnc = kEncInt, int kParam = CQ_F32>
 __global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
     const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params, uint64_t chunk_begin,
     uint64_t chunk_end) {
     const RunGeo geo{in, out, params, nullptr, chunk_begin, chunk_end};
-    dequantize_flat_body<F, kBits, kGroup, true, kUnroll, kThreads, false, kEnc>(geo, CQ_F32);
+    dequantize_flat_body<F, kBits, kGroup, kParam, kUnroll, kThreads, false, kEnc>(geo, kParam);
 }
-// pitched rows of whole steps, f32 parameters
-template <class F, int kBits, int kGroup, int kUnroll, int kThreads, int kEnc = kEncInt>
+// pitched rows of whole steps
+template <class F, int kBits, int kGroup, int kUnroll, int kThreads, int kEnc = kEncInt, int kParam = CQ_F32>
 __global__ __launch_bounds__(kThreads) void dequantize_flat_rows_kernel(
     const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params, uint32_t step_begin,
     FlatRows rows) {
-    const RowsGeo<F::kPerChunk * kBits / 8, 16, kGroup> geo{in, out, params, nullptr, step_begin, 4, 0, rows};
-    dequantize_flat_body<F, kBits, kGroup, true, kUnroll, kThreads, false, kEnc>(geo, CQ_F32);
+    const RowsGeo<F::kPerChunk * kBits / 8, 16, kGroup> geo{in, out, params, nullptr, step_begin, kParam == CQ_F32 ? 4 : 2, 0, rows};
+    dequantize_flat_body<F, kBits, kGroup, kParam, kUnroll, kThreads, false, kEnc>(geo, kParam);
 }
 // lane by lane, bounds-checked, parameter type read at run time
 template <class F, int kBits, int kGroup, int kUnroll, int kThreads, int kEnc = kEncInt>
@@ -661,7 +665,7 @@ __global__ __launch_bounds__(kThreads) void dequantize_flat_lanes_kernel(
     const uint32_t* __restrict__ in, u32x4* __restrict__ out, const void* __restrict__ params, int param_dtype_rt,
     uint32_t tile_begin, LaneRows rows) {
     const LanesGeo geo{in, out, params, nullptr, tile_begin, rows};
-    dequantize_flat_body<F, kBits, kGroup, false, kUnroll, kThreads, true, kEnc>(geo, param_dtype_rt);
+    dequantize_flat_body<F, kBits, kGroup, kParamRt, kUnroll, kThreads, true, kEnc>(geo, param_dtype_rt);
 }
 
 // Block abs-max -> scale typed like the input (what quantize takes as `scale`).

@@ -15,20 +15,37 @@ hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
     auto in = static_cast<const char*>(a.input);
     auto out = static_cast<char*>(a.output);
     constexpr int kU = kUnrollD<F, kBits, kGroup>;
-    constexpr uint64_t kInChunk = F::kPerChunk * kBits / 8;  // stored bytes per chunk
-    constexpr uint64_t kDiv = kGroup == 0 ? 1 : kGroup;
-    const uint64_t param_bytes = kGroup == 0 ? 0 : (a.param_dtype == CQ_F32 ? 4 : 2);
-    return launch_flat(
-        a, kU,
+    [[maybe_unused]] constexpr uint64_t kInChunk = F::kPerChunk * kBits / 8;  // stored bytes per chunk
+    [[maybe_unused]] constexpr uint64_t kDiv = kGroup == 0 ? 1 : kGroup;
+    [[maybe_unused]] const uint64_t param_bytes = kGroup == 0 ? 0 : (a.param_dtype == CQ_F32 ? 4 : 2);
+#if CQ_TU_SAME
+    // this object: the whole tiles of a contiguous run, parameters typed like the tensor
+    if constexpr (F::kBytes == 2) {
+        hipLaunchKernelGGL((dequantize_flat_kernel<F, kBits, kGroup, kU, kThreads, kEnc, F::kDtype>), dim3(a.whole_grid),
+                           dim3(kThreads), 0, s, reinterpret_cast<const uint32_t*>(in), reinterpret_cast<u32x4*>(out), a.scale_in,
+                           0ull, static_cast<uint64_t>(a.whole_grid) * kThreads * kU);
+        return hipGetLastError();
+    } else {
+        return hipErrorInvalidValue;
+    }
+#else
+    hipError_t same = hipSuccess;
+    const hipError_t e = launch_flat(
+        a, F::kDtype, kU,
         [&](uint32_t grid, uint64_t) {
-            if (a.rows > 1)
+            if (a.param_dtype != CQ_F32) {  // a contiguous run, parameters typed like the tensor
+                FlatArgs b = a;
+                b.whole_grid = grid;
+                same = dequantize_flat_same<F>(s, kBits, b);
+            } else if (a.rows > 1) {
                 hipLaunchKernelGGL((dequantize_flat_rows_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(grid), dim3(kThreads),
                                    0, s, reinterpret_cast<const uint32_t*>(in), reinterpret_cast<u32x4*>(out), a.scale_in, 0u,
                                    flat_rows(a));
-            else
+            } else {
                 hipLaunchKernelGGL((dequantize_flat_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(grid), dim3(kThreads), 0,
                                    s, reinterpret_cast<const uint32_t*>(in), reinterpret_cast<u32x4*>(out), a.scale_in, 0ull,
                                    static_cast<uint64_t>(grid) * kThreads * kU);
+            }
         },
         [&](const LaneRows& rows, uint32_t tile_begin, uint32_t grid, RunOffsets off) {
             hipLaunchKernelGGL((dequantize_flat_lanes_kernel<F, kBits, lanes_group(kGroup), kU, kThreads, kEnc>), dim3(grid), dim3(kThreads), 0,
@@ -37,6 +54,8 @@ hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
                                static_cast<const char*>(a.scale_in) + off.chunks / kDiv * param_bytes, a.param_dtype, tile_begin,
                                with_group(rows, kGroup));
         });
+    return e != hipSuccess ? e : same;
+#endif
 }
 
 template <class F, int kBits, int kGroup>
@@ -58,7 +77,11 @@ hipError_t dequantize_launch(hipStream_t s, const FlatArgs& a) {
 
 }  // namespace
 
+#if CQ_TU_SAME
+hipError_t CQ_DEQUANTIZE_FLAT_SAME_TU(CQ_TU_FLOAT)(hipStream_t s, int bits, const FlatArgs& a) {
+#else
 hipError_t CQ_DEQUANTIZE_FLAT_TU(CQ_TU_FLOAT)(hipStream_t s, int bits, const FlatArgs& a) {
+#endif
     int g = group_of(CQ_TU_FLOAT::kDtype, a.block);
     CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (dequantize_launch<CQ_TU_FLOAT, kB, kG>(s, a))))
 }

@@ -3,6 +3,7 @@
 // instantiates for its own scale sources.
 #pragma once
 
+#include <type_traits>
 #include "cq_internal.hpp"
 #include "cq_kernels_flat.hpp"
 
@@ -19,6 +20,41 @@ hipError_t CQ_QUANTIZE_FLAT_TU(BF16, 1)(hipStream_t s, int bits, ScaleSource src
 hipError_t CQ_QUANTIZE_FLAT_TU(F16, 0)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
 hipError_t CQ_QUANTIZE_FLAT_TU(F16, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
 // the dequantize launchers, one per float type, each compiled from cq_kernels_flat_dequantize.hip
+// The whole-tile kernels of a contiguous run for parameters typed like the float tensor (bf16 scales of a bf16
+// tensor, f16 of f16) live in objects of their own (-DCQ_TU_SAME=1): the runtime loads an object's code on its
+// first launch, so launches with f32 parameters do not pay for them.  FlatArgs::whole_grid tiles, nothing else.
+#ifndef CQ_TU_SAME
+#define CQ_TU_SAME 0
+#endif
+#define CQ_QUANTIZE_FLAT_SAME_TU_(f, g) launch_quantize_flat_same_##f##_##g
+#define CQ_QUANTIZE_FLAT_SAME_TU(f, g) CQ_QUANTIZE_FLAT_SAME_TU_(f, g)
+hipError_t CQ_QUANTIZE_FLAT_SAME_TU(BF16, 0)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
+hipError_t CQ_QUANTIZE_FLAT_SAME_TU(BF16, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
+hipError_t CQ_QUANTIZE_FLAT_SAME_TU(F16, 0)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
+hipError_t CQ_QUANTIZE_FLAT_SAME_TU(F16, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
+#define CQ_DEQUANTIZE_FLAT_SAME_TU_(f) launch_dequantize_flat_same_##f
+#define CQ_DEQUANTIZE_FLAT_SAME_TU(f) CQ_DEQUANTIZE_FLAT_SAME_TU_(f)
+hipError_t CQ_DEQUANTIZE_FLAT_SAME_TU(BF16)(hipStream_t s, int bits, const FlatArgs& a);
+hipError_t CQ_DEQUANTIZE_FLAT_SAME_TU(F16)(hipStream_t s, int bits, const FlatArgs& a);
+template <class F>
+hipError_t quantize_flat_same(bool given, hipStream_t s, int bits, ScaleSource src, const FlatArgs& a) {
+    if constexpr (std::is_same_v<F, BF16>)
+        return given ? CQ_QUANTIZE_FLAT_SAME_TU(BF16, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_SAME_TU(BF16, 0)(s, bits, src, a);
+    else if constexpr (std::is_same_v<F, F16>)
+        return given ? CQ_QUANTIZE_FLAT_SAME_TU(F16, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_SAME_TU(F16, 0)(s, bits, src, a);
+    else
+        return hipErrorInvalidValue;
+}
+template <class F>
+hipError_t dequantize_flat_same(hipStream_t s, int bits, const FlatArgs& a) {
+    if constexpr (std::is_same_v<F, BF16>)
+        return CQ_DEQUANTIZE_FLAT_SAME_TU(BF16)(s, bits, a);
+    else if constexpr (std::is_same_v<F, F16>)
+        return CQ_DEQUANTIZE_FLAT_SAME_TU(F16)(s, bits, a);
+    else
+        return hipErrorInvalidValue;
+}
+
 #define CQ_DEQUANTIZE_FLAT_TU_(f) launch_dequantize_flat_##f
 #define CQ_DEQUANTIZE_FLAT_TU(f) CQ_DEQUANTIZE_FLAT_TU_(f)
 hipError_t CQ_DEQUANTIZE_FLAT_TU(F32)(hipStream_t s, int bits, const FlatArgs& a);
@@ -203,8 +239,9 @@ QuantParams quant_params(const Range& r) {
     return p;
 }
 
-// How a flat launch is cut up.  The kernels over whole tiles (a contiguous run, or pitched rows of whole
-// steps) exist for f32 parameters only and check no bounds; everything else is the lane-wise kernel's:
+// How a flat launch is cut up.  The kernels over whole tiles check no bounds and exist for f32 parameters (a
+// contiguous run, or pitched rows of whole steps) and for parameters typed like the float tensor, `f_dtype` (a
+// contiguous run); everything else is the lane-wise kernel's:
 //   `whole(grid, begin)`                       tiles [begin, begin + grid) of the run / of the rows' steps
 //   `lanes(rows, tile_begin, grid, offsets)`   lane by lane; `offsets` = chunks / scales to advance the base
 //                                              pointers by (a contiguous run only)
@@ -212,7 +249,7 @@ struct RunOffsets {
     uint64_t chunks;  // 16-byte chunks of the float tensor
 };
 template <class WholeFn, class LanesFn>
-hipError_t launch_flat(const FlatArgs& a, int unroll, WholeFn whole, LanesFn lanes) {
+hipError_t launch_flat(const FlatArgs& a, int f_dtype, int unroll, WholeFn whole, LanesFn lanes) {
     const uint64_t tile = static_cast<uint64_t>(kThreads) * unroll;
     const bool p32 = a.param_dtype == CQ_F32;
     hipError_t e = hipSuccess;
@@ -236,7 +273,7 @@ hipError_t launch_flat(const FlatArgs& a, int unroll, WholeFn whole, LanesFn lan
         return e;
     }
     // one contiguous run
-    const uint64_t full = p32 ? a.num_chunks / tile : 0;
+    const uint64_t full = p32 || a.param_dtype == f_dtype ? a.num_chunks / tile : 0;
     if (full > 0) {
         whole(static_cast<uint32_t>(full), 0ull);
         if ((e = hipGetLastError()) != hipSuccess) return e;
@@ -252,7 +289,7 @@ hipError_t launch_flat(const FlatArgs& a, int unroll, WholeFn whole, LanesFn lan
 }
 
 template <class F, int kBits, int kGroup, int kSrc, bool kWide, int kEnc>
-hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
+hipError_t quantize_launch_src(hipStream_t s, ScaleSource src, const FlatArgs& a) {
     // scale sources that exist: per-block launches compute the scale or read the
     // input-typed tensor; per-tensor launches read it or finish the grid reduction
     if constexpr ((kGroup == 0 && (kSrc == kScaleDynamic || kSrc == kScaleStored)) || (kGroup != 0 && kSrc == kScalePartials)) {
@@ -263,25 +300,43 @@ hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
         auto in = static_cast<const char*>(a.input);
         auto out = static_cast<char*>(a.output);
         const QuantParams qp = quant_params(a.range);
-        constexpr uint64_t kOutChunk = F::kPerChunk * kBits / 8;  // stored bytes per chunk
+        [[maybe_unused]] constexpr uint64_t kOutChunk = F::kPerChunk * kBits / 8;  // stored bytes per chunk
         // bytes per scale of the two scale tensors (per-tensor launches and the partials never move their pointers)
-        const uint64_t scale_in_bytes = kGroup == 0 ? 0 : (kSrc == kScaleStored ? (a.param_dtype == CQ_F32 ? 4 : 2) : F::kBytes);
-        const uint64_t scale_out_bytes = kGroup == 0 ? 0 : (a.param_dtype == CQ_F32 ? 4 : 2);
-        constexpr uint64_t kDiv = kGroup == 0 ? 1 : kGroup;
-        return launch_flat(
-            a, kUnrollQ,
+        [[maybe_unused]] const uint64_t scale_in_bytes = kGroup == 0 ? 0 : (kSrc == kScaleStored ? (a.param_dtype == CQ_F32 ? 4 : 2) : F::kBytes);
+        [[maybe_unused]] const uint64_t scale_out_bytes = kGroup == 0 ? 0 : (a.param_dtype == CQ_F32 ? 4 : 2);
+        [[maybe_unused]] constexpr uint64_t kDiv = kGroup == 0 ? 1 : kGroup;
+#if CQ_TU_SAME
+        // this object: the whole tiles of a contiguous run, parameters typed like the tensor
+        if constexpr (kSrc != kScaleStored && F::kBytes == 2) {
+            hipLaunchKernelGGL((quantize_flat_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc, F::kDtype>),
+                               dim3(a.whole_grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
+                               reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0ull,
+                               static_cast<uint64_t>(a.whole_grid) * kThreads * kUnrollQ, qp, a.num_partials);
+            return hipGetLastError();
+        } else {
+            return hipErrorInvalidValue;
+        }
+#else
+        hipError_t same = hipSuccess;
+        const hipError_t e = launch_flat(
+            a, F::kDtype, kUnrollQ,
             [&](uint32_t grid, uint64_t) {
                 if constexpr (kSrc != kScaleStored) {
-                    if (a.rows > 1)
+                    if (a.param_dtype != CQ_F32) {  // a contiguous run, parameters typed like the tensor
+                        FlatArgs b = a;
+                        b.whole_grid = grid;
+                        same = quantize_flat_same<F>(kSrc == kScaleGivenF, s, kBits, src, b);
+                    } else if (a.rows > 1) {
                         hipLaunchKernelGGL((quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
                                            dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
                                            reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0u, qp, a.num_partials,
                                            flat_rows(a));
-                    else
+                    } else {
                         hipLaunchKernelGGL((quantize_flat_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
                                            dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
                                            reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0ull,
                                            static_cast<uint64_t>(grid) * kThreads * kUnrollQ, qp, a.num_partials);
+                    }
                 }
             },
             [&](const LaneRows& rows, uint32_t tile_begin, uint32_t grid, RunOffsets off) {
@@ -293,6 +348,8 @@ hipError_t quantize_launch_src(hipStream_t s, const FlatArgs& a) {
                                    reinterpret_cast<uint32_t*>(out + off.chunks * kOutChunk), scale_in, scale_out,
                                    a.param_dtype, qp, a.num_partials, tile_begin, with_group(rows, kGroup));
             });
+        return e != hipSuccess ? e : same;
+#endif
     }
 }
 
@@ -302,11 +359,11 @@ template <class F, int kBits, int kGroup, bool kWide, int kEnc, bool kGiven>
 hipError_t quantize_launch_enc(hipStream_t s, ScaleSource src, const FlatArgs& a) {
     if constexpr (kGiven) {
         if (src == ScaleSource::Given && a.scale_in_dtype == F::kDtype)  // given scales are typed like the input
-            return quantize_launch_src<F, kBits, kGroup, kScaleGivenF, kWide, kEnc>(s, a);
-        if (src == ScaleSource::Stored) return quantize_launch_src<F, kBits, kGroup, kScaleStored, kWide, kEnc>(s, a);
+            return quantize_launch_src<F, kBits, kGroup, kScaleGivenF, kWide, kEnc>(s, src, a);
+        if (src == ScaleSource::Stored) return quantize_launch_src<F, kBits, kGroup, kScaleStored, kWide, kEnc>(s, src, a);
     } else {
-        if (src == ScaleSource::Dynamic) return quantize_launch_src<F, kBits, kGroup, kScaleDynamic, kWide, kEnc>(s, a);
-        if (src == ScaleSource::Partials) return quantize_launch_src<F, kBits, kGroup, kScalePartials, kWide, kEnc>(s, a);
+        if (src == ScaleSource::Dynamic) return quantize_launch_src<F, kBits, kGroup, kScaleDynamic, kWide, kEnc>(s, src, a);
+        if (src == ScaleSource::Partials) return quantize_launch_src<F, kBits, kGroup, kScalePartials, kWide, kEnc>(s, src, a);
     }
     return hipErrorInvalidValue;
 }

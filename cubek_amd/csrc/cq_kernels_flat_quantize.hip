@@ -1,7 +1,8 @@
 // Launchers of the flat quantize kernels of one float type and one family of scale sources.  The
 // Makefile compiles this file six times (-DCQ_TU_FLOAT=F32|BF16|F16, -DCQ_TU_GIVEN=0|1: scales produced
 // in the launch, or given), each into an object of its own, so that the build runs in parallel: in
-// one translation unit the instantiations take minutes.
+// one translation unit the instantiations take minutes.  Four more objects (-DCQ_TU_SAME=1, BF16 and F16) hold the
+// whole-tile kernels for parameters typed like the tensor.
 #include "cq_kernels_flat_launch.hpp"
 
 #ifndef CQ_TU_FLOAT
@@ -13,7 +14,11 @@
 
 namespace cq {
 
+#if CQ_TU_SAME
+hipError_t CQ_QUANTIZE_FLAT_SAME_TU(CQ_TU_FLOAT, CQ_TU_GIVEN)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a) {
+#else
 hipError_t CQ_QUANTIZE_FLAT_TU(CQ_TU_FLOAT, CQ_TU_GIVEN)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a) {
+#endif
     int g = group_of(CQ_TU_FLOAT::kDtype, a.block);
     CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (quantize_launch<CQ_TU_FLOAT, kB, kG, CQ_TU_GIVEN != 0>(s, src, a))))
 }

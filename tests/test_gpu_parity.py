@@ -128,6 +128,36 @@ def test_param_dtypes(gpu, oracle, elem, param):
                            oracle.dequantize(w_ref, shape, os_ref, elem, scheme), elem)
 
 
+@pytest.mark.parametrize("elem", [ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
+def test_params_typed_like_the_tensor_on_whole_tiles(gpu, oracle, elem):
+    """bf16 scales of a bf16 tensor, f16 of f16: a contiguous tensor runs kernels compiled for that parameter
+    type over its whole tiles (four of them here) and the lane-wise kernels over the ragged rest."""
+    param = QuantParam.BF16 if elem == ElemType.BF16 else QuantParam.F16
+    rng = np.random.default_rng(4100 + int(elem))
+    shape = (33, 1024)
+    x = rand_input(rng, shape, elem, oracle, sigma=2.0)
+    for value, level, store in ((QuantValue.Q8S, QuantLevel.block([32]), QuantStore.U32),
+                                (QuantValue.Q4S, QuantLevel.block([16]), QuantStore.U32),
+                                (QuantValue.Q2S, QuantLevel.block([64]), QuantStore.U32),
+                                (QuantValue.E2M1, QuantLevel.block([32]), QuantStore.U32),
+                                (QuantValue.Q4F, QuantLevel.block([128]), QuantStore.U32),
+                                (QuantValue.Q8F, QuantLevel.Tensor, QuantStore.U32),
+                                (QuantValue.E4M3, QuantLevel.block([32]), QuantStore.Native),
+                                (QuantValue.E5M2, QuantLevel.block([128]), QuantStore.Native),
+                                (QuantValue.E2M1, QuantLevel.block([32]), QuantStore.Native),
+                                (QuantValue.Q8S, QuantLevel.block([8]), QuantStore.Native)):
+        scheme = QuantScheme.default().with_value(value).with_level(level).with_store(store).with_param(param)
+        pe = gpu.param_elem(scheme)
+        s_ref = oracle.compute_scales(x, elem, shape, scheme)
+        w_ref, os_ref = oracle.quantize(x, elem, shape, s_ref, scheme)
+        w_gpu, os_gpu = gpu.quantize(x, elem, shape, s_ref, scheme)
+        assert np.array_equal(w_gpu, w_ref) and same_floats(os_gpu, os_ref, pe), (value, level)
+        w_dyn, os_dyn = gpu.quantize_dynamic(x, elem, shape, scheme)
+        assert np.array_equal(w_dyn, w_ref) and same_floats(os_dyn, os_ref, pe), (value, level)
+        assert same_floats(gpu.dequantize(w_ref, shape, os_ref, elem, scheme),
+                           oracle.dequantize(w_ref, shape, os_ref, elem, scheme), elem), (value, level)
+
+
 # ---------------------------------------------------------------- adversarial arithmetic
 
 def test_bf16_all_significand_pairs(gpu, oracle):

@@ -63,9 +63,14 @@ def test_layouts_land_on_the_family_the_design_claims():
     # ragged pitched rows (576 chunks = 2.25 steps), short rows: lane by lane
     assert set(kinds(e2m1, BF16, (32768, 4608), f_strides=(4672, 1)).values()) == {"flat_lanes"}
     assert set(kinds(e2m1, BF16, (262144, 256), f_strides=(320, 1)).values()) == {"flat_lanes"}
-    # f16 / bf16 parameters: lane by lane (scale production has no stored parameters and stays on whole tiles)
+    # parameters typed like the tensor (bf16 scales of a bf16 tensor): whole tiles on a contiguous run; any other
+    # 16-bit parameter type, and pitched rows, lane by lane (scale production has no stored parameters)
     got = kinds(scheme_of(QuantValue.E2M1, [32], param=QuantParam.BF16), BF16, (rows, cols))
+    assert got == {"quantize": "flat", "dynamic": "flat", "dequantize": "flat", "scales": "flat"}
+    got = kinds(scheme_of(QuantValue.E2M1, [32], param=QuantParam.F16), BF16, (rows, cols))
     assert got == {"quantize": "flat_lanes", "dynamic": "flat_lanes", "dequantize": "flat_lanes", "scales": "flat"}
+    got = kinds(scheme_of(QuantValue.E2M1, [32], param=QuantParam.BF16), BF16, (rows, cols), f_strides=(cols + 64, 1))
+    assert got == {"quantize": "flat_lanes", "dynamic": "flat_lanes", "dequantize": "flat_lanes", "scales": "flat_rows"}
     # attention layout: [batch, heads, positions, head dimension] view of a [batch, positions, heads, head dimension] buffer
     nb, nh, ns, nd = 8, 32, 4096, 128
     got = kinds(e2m1, BF16, (nb, nh, ns, nd), f_strides=(ns * nh * nd, nd, nh * nd, 1))
