@@ -9,7 +9,9 @@ followed by dequantize of the result.  Launches rotate through independent buffe
 sets (>= 1 GiB in total) so that no launch finds its operands in the 256 MB
 Infinity Cache from an earlier launch.  The headline workload is the largest
 configuration (cfg5: e2m1 block 32, bf16 [28672, 8192]); the other four
-configurations are measured in short loops and reported under "per_config".
+configurations are measured in short loops and reported under "per_config"
+(launches shorter than 16 us also as a replayed HIP graph, "graph_replay_ms":
+the host's share of an eager call bounds them).
 
 value      = algorithmic bytes of one step / wall time per step  (GB/s, 1e9)
              algorithmic bytes = input once + codes once + scales once, per direction
@@ -183,6 +185,42 @@ def timed_region(torch, fn, launches, warmup=3):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     return a.elapsed_time(b) / launches, wall * 1e3 / launches
+
+
+def graph_region(torch, paths, method, launches=32, replays=5):
+    """The launches of timed_region captured once into a HIP graph and replayed: the GPU's time
+    per launch without the host's share (a call costs the host ~4 us through the Python mirror,
+    which bounds eager launches of a few microseconds).  Median over `replays` replays."""
+    from cubek_amd import ComputeClient
+
+    def run(n):
+        client = ComputeClient.current()  # the stream being captured
+        for i in range(n):
+            p = paths[i % len(paths)]
+            saved, p.client = p.client, client
+            getattr(p, method)()
+            p.client = saved
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(len(paths))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(launches)
+    graph.replay()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(replays):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        graph.replay()
+        b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b) / launches)
+    return sorted(times)[len(times) // 2]
 
 
 def replicas(torch, w, x, min_footprint=1 << 30, max_sets=8):
@@ -636,6 +674,8 @@ def main():
                 row[label] = {"ms": round(med_ms, 4), "GBps": round(b / (med_ms * 1e-3) / 1e9, 1),
                               "frac_hbm_peak": round(b / (med_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                               "traffic": traffic_table.get(name, {}).get(label)}
+                if med_ms < 0.016:  # within four host enqueue times: also as a replayed HIP graph
+                    row[label]["graph_replay_ms"] = round(graph_region(torch, ps, meth), 4)
             table.append(row)
             del ps, p, xi
             torch.cuda.empty_cache()
