@@ -748,7 +748,10 @@ __global__ __launch_bounds__(kThreads) void absmax_partials_kernel(const void* _
 #pragma unroll
                 for (int u = 0; u < kUnroll; u++) {
                     const uint64_t c = c0 + static_cast<uint64_t>(u) * total;
-                    raw[u] = stream_load(in + (c < num_chunks ? c : num_chunks - 1));
+                    // a plain load, not a streaming one: pass 2 reads the tensor again, and what stays in the L2
+                    // and the Infinity Cache from here it does not fetch from HBM (tensors of 32 MiB: 16.4 -> 13.0 us
+                    // for both passes, 128 MiB: 54.6 -> 50.5 us, 448 MiB: 181 -> 177 us)
+                    raw[u] = in[c < num_chunks ? c : num_chunks - 1];
                 }
 #pragma unroll
                 for (int u = 0; u < kUnroll; u++) {
