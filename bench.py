@@ -448,7 +448,25 @@ def adjacent_kernels(torch):
         out.append({"kernel": f"{label}, e2m1 blocks of 32, transposed bf16 view [{rows}, {cols}] of a [{cols}, {rows}] buffer",
                     "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
-    del xs, codes, scales, ys, hx, hc, hs, hy, words, bscales, hxt, hyt, hw, hb
+    # one scale per tensor: two launches, the tensor read twice (pass 1 leaves what it can in the caches for pass 2)
+    tensor_scheme = QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.Tensor)
+    ws_bytes = cq_quantize.workspace_bytes(tensor_scheme, rows * cols)
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device="cuda")
+    for pr, pc in ((rows, cols), (8192, 8192), (4096, 4096)):
+        n_sets = sets if (pr, pc) == (rows, cols) else 8
+        xq = xs if (pr, pc) == (rows, cols) else [torch.randn((pr, pc), device="cuda", dtype=torch.bfloat16) for _ in range(n_sets)]
+        words = [torch.empty((pr, pc // 4), dtype=torch.int32, device="cuda") for _ in range(2)]
+        one = [torch.empty((1,), dtype=torch.float32, device="cuda") for _ in range(2)]
+        hxq, hw, ho = [h(t) for t in xq], [h(t) for t in words], [h(t) for t in one]
+        fn = lambda i: cq_quantize.launch_dynamic(client, hxq[i % n_sets], hw[i % 2], ho[i % 2], tensor_scheme, ElemType.BF16,
+                                                  ws.data_ptr(), ws_bytes)
+        ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
+        b = pr * pc * 3 + 4
+        out.append({"kernel": f"quantize_dynamic, q8 per tensor (two passes), bf16 [{pr}, {pc}]", "algorithmic_bytes": b,
+                    "buffer_sets_rotated": n_sets, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                    "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+        del xq, words, one, hxq, hw, ho
+    del xs, codes, scales, ys, hx, hc, hs, hy, bscales, hxt, hyt, hb
     torch.cuda.empty_cache()
     # the headline scheme on pitched rows: [rows, cols] views of [rows, cols + 64] buffers, at the headline
     # row length and with the same elements in rows a quarter as long
