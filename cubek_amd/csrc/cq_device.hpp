@@ -255,7 +255,28 @@ __device__ __forceinline__ uint32_t group_or(uint32_t v) {
 struct QuantParams {
     float lo, hi;         // q_min, q_max
     float width, rwidth;  // q_max - q_min and its correctly rounded reciprocal
+    uint32_t keep = 0;    // the flat quantize kernels: codes leave through output_store(keep = true): they stay in the
+                          // Infinity Cache for the kernel that reads them next
 };
+// A store that streams past the caches, or one that is written through the L2 at system scope (sc0 sc1): it leaves
+// no dirty line behind in the L2, as a plain store would (which costs the launch 4 - 8 %), but unlike the streaming
+// store it leaves the data in the memory-side Infinity Cache.  `keep` is the same for the whole launch: a scalar
+// branch.  A relaxed atomic store of 4 or 8 bytes is how the compiler is told the scope; nothing here is atomic
+// in any other sense.
+template <class T>
+__device__ __forceinline__ void output_store(bool keep, T v, T* p) {
+    static_assert(sizeof(T) == 4 || sizeof(T) == 8, "codes leave as one or two words per lane");
+    if (keep) {
+        if constexpr (sizeof(T) == 8)
+            __scoped_atomic_store_n(reinterpret_cast<uint64_t*>(p), __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
+                                    __MEMORY_SCOPE_SYSTEM);
+        else
+            __scoped_atomic_store_n(reinterpret_cast<uint32_t*>(p), __builtin_bit_cast(uint32_t, v), __ATOMIC_RELAXED,
+                                    __MEMORY_SCOPE_SYSTEM);
+    } else {
+        stream_store(v, p);
+    }
+}
 
 // Divisors for which x * rcp(d) stays within 2^-21 relative error of x / d:
 // positive, finite, normal and far from the ends of the exponent range (false for NaN).

@@ -541,15 +541,16 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         else
             encode_chunk<kEnc, kN>(qn, w);
 
+        const bool keep = qp.keep != 0;
         if constexpr (kChunkBits == 64) {
-            if (live) stream_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(out) + c);
+            if (live) output_store(keep, u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(out) + c);
         } else if constexpr (kChunkBits == 32) {
-            if (live) stream_store(w[0], out + c);
+            if (live) output_store(keep, w[0], out + c);
         } else {
             constexpr int kLanesPerWord = 32 / kChunkBits;  // 2 or 4
             const uint32_t sub = static_cast<uint32_t>(c) & (kLanesPerWord - 1);
             const uint32_t word = group_or<kLanesPerWord>(w[0] << (sub * kChunkBits));
-            if (live && sub == 0) stream_store(word, out + c / kLanesPerWord);
+            if (live && sub == 0) output_store(keep, word, out + c / kLanesPerWord);
         }
     }
 }
