@@ -304,7 +304,7 @@ hipError_t quantize_launch_src(hipStream_t s, ScaleSource src, const FlatArgs& a
         [[maybe_unused]] constexpr uint64_t kOutChunk = F::kPerChunk * kBits / 8;  // stored bytes per chunk
         // Codes that fit the 256 MB Infinity Cache with room to spare are stored to stay there for whoever reads
         // them next: on 147 MB of codes and scales (bf16 [28672, 8192], 4-bit, blocks of 32) a dequantize right
-        // behind this launch takes 83 us instead of 98 us, the launch itself 1 - 2 % longer.  Larger outputs stream
+        // behind this launch takes 84 us instead of 98 us, the launch itself 2 - 5 % longer.  Larger outputs stream
         // past the caches.
         {
             const uint64_t chunks = a.num_chunks * (a.rows > 1 ? a.rows : 1);
