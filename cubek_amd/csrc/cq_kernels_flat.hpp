@@ -524,6 +524,7 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         if (fs_rounds) s_fs = round_to_dtype(param_dtype, s_f);
         const auto si = kGroup == 0 ? 0 : block_of(c);
         const bool block_start = kGroup == 0 ? at.tensor_start(u) : (at.first_row(u) && starts_block(c));
+        // (the scales leave through plain stores either way: written through like the codes below they cost 1 - 2 %)
         if constexpr (kScaleSrc != kScaleStored)
             if (scale_out != nullptr && live && block_start) store_dtype(param_dtype, scale_out, si, s_fs);
         // divisor F(FS(scale)): s_f itself unless FS rounded it
