@@ -652,6 +652,10 @@ def main():
                    "shape": list(w["shape"]), "block": w["block"], "value": w["value"], "store": "U32",
                    "param": "F32", "algorithmic_bytes_per_step": step_bytes},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 1),
+        "value_note": "algorithmic bytes of the step (each direction: floats + codes + scales once) per second; the "
+                      "dequantize of a step reads the codes and scales its quantize has just left in the 256 MB Infinity "
+                      "Cache, so fewer bytes than these cross the HBM interface; `roofline` and `roofline_dequantize` time "
+                      "each kernel alone on operands from HBM",
         "elements_per_s": round(2 * n / (ms_per_step * 1e-3)),
         "roofline": {"bound": "hbm", "kernel": "quantize_flat_kernel (fused abs-max+scale+quantize+pack)",
                      "achieved": round(q_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
