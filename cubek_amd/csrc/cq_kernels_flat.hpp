@@ -218,6 +218,11 @@ struct LaneRows {
     // one tile can span, its strides below 2^24 bytes: a tile's lanes find their rows from the tile's first row by
     // one step of at most one carry
     uint32_t near;
+    // near, and rows of a power of two of chunks (1 + its log2 here; 0 = not so) that a step of the workgroup holds
+    // whole, in a launch of whole tiles none of which runs over the end of the innermost level: a lane keeps its
+    // column and its place among a step's rows for all of its chunks, and the step from chunk to chunk is the same
+    // for every lane
+    uint32_t whole_rows;
     uint32_t group_log2;    // lanes per block as a power of two, for the kernels that take it at run time (kGroupRt)
     // Tile order (0 = as numbered).  Where whole tiles fit the innermost level and the next level lies closer in
     // memory in the tensor that is read (heads next to each other behind positions, rows of 512 bytes and more),
@@ -308,6 +313,27 @@ struct LaneSteps {
             }
             const uint32_t step0[4] = {static_cast<uint32_t>(r.in[0]), static_cast<uint32_t>(r.out[0]),
                                        static_cast<uint32_t>(r.scale_in[0]), static_cast<uint32_t>(r.scale_out[0])};
+            if (r.whole_rows != 0) {
+                const uint32_t log2 = r.whole_rows - 1;
+                const uint32_t lane_row = threadIdx.x >> log2, col = threadIdx.x & (r.row_chunks - 1u);
+                const uint32_t rows_per_step = kThreads >> log2;
+                uint32_t off[4];
+#pragma unroll
+                for (int t = 0; t < 4; t++) off[t] = base[t] + __umul24(lane_row, step0[t]);
+#pragma unroll
+                for (int u = 0; u < kUnroll; u++) {
+                    live_[u] = true;
+                    col_[u] = col;
+                    first_[u] = u == 0 && row0 == 0 && lane_row == 0;
+                    block_row_[u] = true;
+                    const uint32_t rows = u * rows_per_step;  // the same for every lane
+                    in_[u] = static_cast<const char*>(g.in) + (off[0] + rows * step0[0]);
+                    out_[u] = static_cast<char*>(g.out) + (off[1] + rows * step0[1]);
+                    scale_in_[u] = static_cast<const char*>(g.scale_in) + (off[2] + rows * step0[2]);
+                    scale_out_[u] = g.scale_out == nullptr ? nullptr : static_cast<char*>(g.scale_out) + (off[3] + rows * step0[3]);
+                }
+                return;
+            }
             uint32_t drow[kUnroll];
             bool wraps[kUnroll], any_wraps = false;
 #pragma unroll

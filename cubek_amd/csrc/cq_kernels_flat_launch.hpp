@@ -179,6 +179,12 @@ LaneRows lane_rows(const FlatArgs& a, int unroll = 0) {
     const uint64_t run_chunks = static_cast<uint64_t>(r.count[0]) * r.row_chunks;  // chunks of one innermost run
     // measured on attention-shaped views (quantize / dequantize, us): reads of 512-byte rows gain (f32 rows of 128:
     // 143 -> 120, bf16 rows of 256: 86 -> 67), reads of 256-byte rows stay where they are, writes lose (68 -> 76)
+    if (unroll > 0 && r.near && (r.row_chunks & (r.row_chunks - 1)) == 0 && r.row_chunks <= kThreads &&
+        r.total_chunks % tile_chunks == 0 && r.count[0] % (tile_chunks / r.row_chunks) == 0) {
+        uint32_t log2 = 0;
+        while ((1u << log2) < r.row_chunks) log2++;
+        r.whole_rows = 1 + log2;
+    }
     const bool closer = r.levels >= 2 && r.in[1] < r.in[0] && r.row_chunks >= 32;
     if (unroll > 0 && r.near && closer && run_chunks % tile_chunks == 0 && r.count[1] > 1) {
         r.order_inner = static_cast<uint32_t>(run_chunks / tile_chunks);
