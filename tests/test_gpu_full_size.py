@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at their full sizes.
+"""The five BASELINE configurations at their full sizes, and two tensors whose codes exceed the Infinity Cache.
 
 The CPU oracle checks a band of rows of each tensor bit for bit; the whole tensor
 is checked through properties that do not depend on size:
@@ -24,6 +24,10 @@ CONFIGS = [
     ("cfg3", (14336, 4096), ElemType.BF16, QuantValue.Q4S, 32, "normal", 3),
     ("cfg4", (8192, 8192), ElemType.F32, QuantValue.Q2S, 64, "laplace", 4),
     ("cfg5", (28672, 8192), ElemType.BF16, QuantValue.E2M1, 32, "normal_t3", 5),
+    # codes + scales above 192 MiB: the quantize kernels stream such outputs past the caches, where the five
+    # configurations above (and every small test) write theirs through to the Infinity Cache
+    ("large_output_block32", (16384, 12800), ElemType.BF16, QuantValue.Q8S, 32, "normal", 6),
+    ("large_output_per_tensor", (16384, 12800), ElemType.BF16, QuantValue.Q8S, None, "normal1", 7),
 ]
 
 
@@ -92,7 +96,7 @@ def test_full_size_config(oracle, name, shape, elem, value, block, dist, seed):
             assert np.array_equal(codes[r0:r0 + band].cpu().numpy().view(np.uint32), w_ref)
             assert np.array_equal(scales[r0:r0 + band].cpu().numpy().reshape(-1), os_ref.reshape(-1))
     else:
-        x_np = x.cpu().numpy()
+        x_np = x.cpu().numpy() if elem == ElemType.F32 else x.view(torch.int16).cpu().numpy().view(np.uint16)
         s_ref = oracle.compute_scales(x_np, elem, shape, scheme)
         w_ref, os_ref = oracle.quantize(x_np, elem, shape, s_ref, scheme, threads=8)
         assert np.array_equal(codes.cpu().numpy().view(np.uint32), w_ref)
