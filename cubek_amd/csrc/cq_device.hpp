@@ -68,6 +68,10 @@ struct F32 {
     __device__ static __forceinline__ float load(const void* p, uint64_t i) {
         return static_cast<const float*>(p)[i];
     }
+    // an element that is read once (see stream_load)
+    __device__ static __forceinline__ float load_once(const void* p, uint64_t i) {
+        return stream_load(static_cast<const float*>(p) + i);
+    }
     __device__ static __forceinline__ void store(void* p, uint64_t i, float v) {
         static_cast<float*>(p)[i] = v;
     }
@@ -97,6 +101,9 @@ struct BF16 {
     }
     __device__ static __forceinline__ float load(const void* p, uint64_t i) {
         return bits_f32(static_cast<uint32_t>(static_cast<const uint16_t*>(p)[i]) << 16);
+    }
+    __device__ static __forceinline__ float load_once(const void* p, uint64_t i) {
+        return bits_f32(static_cast<uint32_t>(stream_load(static_cast<const uint16_t*>(p) + i)) << 16);
     }
     __device__ static __forceinline__ void store(void* p, uint64_t i, float v) {
         static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(pack2(v, 0.0f) & 0xffffu);
@@ -132,6 +139,9 @@ struct F16 {
     __device__ static __forceinline__ float round(float v) { return static_cast<float>(static_cast<_Float16>(v)); }
     __device__ static __forceinline__ float load(const void* p, uint64_t i) {
         return static_cast<float>(static_cast<const _Float16*>(p)[i]);
+    }
+    __device__ static __forceinline__ float load_once(const void* p, uint64_t i) {
+        return static_cast<float>(stream_load(static_cast<const _Float16*>(p) + i));
     }
     __device__ static __forceinline__ void store(void* p, uint64_t i, float v) {
         static_cast<_Float16*>(p)[i] = narrow(v);
