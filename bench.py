@@ -698,6 +698,15 @@ def main():
                               "traffic": traffic_table.get(name, {}).get(label)}
                 if med_ms < 0.016:  # within four host enqueue times: also as a replayed HIP graph
                     row[label]["graph_replay_ms"] = round(graph_region(torch, ps, meth), 4)
+            # the two kernels back to back on one buffer set, as in the headline step: the dequantize reads what
+            # its quantize has just written
+            def both(i, ps=ps):
+                ps[i % len(ps)].quantize_dynamic()
+                ps[i % len(ps)].dequantize()
+            step_ms = sorted(timed_region(torch, both, 32)[0] for _ in range(3))[1]
+            row["step_quantize_dynamic_then_dequantize"] = {
+                "ms": round(step_ms, 4), "GBps": round(2 * b / (step_ms * 1e-3) / 1e9, 1),
+                "sum_of_the_two_alone_ms": round(row["quantize_dynamic"]["ms"] + row["dequantize"]["ms"], 4)}
             table.append(row)
             del ps, p, xi
             torch.cuda.empty_cache()
