@@ -310,8 +310,8 @@ hipError_t quantize_launch_src(hipStream_t s, ScaleSource src, const FlatArgs& a
         [[maybe_unused]] constexpr uint64_t kOutChunk = F::kPerChunk * kBits / 8;  // stored bytes per chunk
         // Codes that fit the 256 MB Infinity Cache with room to spare are stored to stay there for whoever reads
         // them next: on 147 MB of codes and scales (bf16 [28672, 8192], 4-bit, blocks of 32) a dequantize right
-        // behind this launch takes 84 us instead of 98 us, the launch itself 2 - 5 % longer.  Larger outputs stream
-        // past the caches.
+        // behind this launch takes 79 us instead of 96 us, the launch itself 0 - 3 % longer (up to 6 % on smaller
+        // tensors).  Larger outputs stream past the caches.
         {
             const uint64_t chunks = a.num_chunks * (a.rows > 1 ? a.rows : 1);
             const uint64_t scales = kGroup == 0 ? 0 : chunks / kGroup * (a.param_dtype == CQ_F32 ? 4 : 2);
