@@ -45,7 +45,7 @@ enum ScaleSrc : int {
 // base pointer belongs to chunks [i * kDiv, (i + 1) * kDiv).
 
 // One contiguous run of chunks [chunk_begin, chunk_end): the same pointers for every step.
-template <int kUnroll, int kThreads, bool kChecked>
+template <int kUnroll, int kThreads, bool kChecked, bool kWaveRuns = false>
 struct RunSteps;
 struct RunGeo {
     const void* in;
@@ -53,17 +53,30 @@ struct RunGeo {
     const void* scale_in;
     void* scale_out;
     uint64_t chunk_begin, chunk_end;
+    static constexpr bool kWaveRuns = false;
     template <int kUnroll, int kThreads, bool kChecked>
     using Steps = RunSteps<kUnroll, kThreads, kChecked>;
 };
-template <int kUnroll, int kThreads, bool kChecked>
+// The same run with the tile's chunks dealt out wave by wave: a wave takes kUnroll * 64 consecutive chunks, step u
+// of it the u-th 64 of them (RunGeo: step u of the workgroup is the u-th kThreads chunks of the tile).  Every load
+// still covers 1 KiB; what changes is that the codes of a wave's steps lie next to each other, so that chunks of
+// 8 or 16 bits of codes leave as one run of 256 or 512 bytes per wave instead of 64-byte pieces.
+struct RunGeoWaves : RunGeo {
+    static constexpr bool kWaveRuns = true;
+    template <int kUnroll, int kThreads, bool kChecked>
+    using Steps = RunSteps<kUnroll, kThreads, kChecked, true>;
+};
+template <int kUnroll, int kThreads, bool kChecked, bool kWaveRuns>
 struct RunSteps {
     using Index = uint64_t;
+    static constexpr int kStep = kWaveRuns ? kWave : kThreads;  // chunks from one step of a lane to its next
     const RunGeo& g;
     const uint64_t first;
     __device__ __forceinline__ RunSteps(const RunGeo& geo, uint32_t tile)
-        : g(geo), first(geo.chunk_begin + static_cast<uint64_t>(tile) * (kThreads * kUnroll) + threadIdx.x) {}
-    __device__ __forceinline__ Index chunk(int u) const { return first + static_cast<uint64_t>(u) * kThreads; }
+        : g(geo),
+          first(geo.chunk_begin + static_cast<uint64_t>(tile) * (kThreads * kUnroll) +
+                (kWaveRuns ? (threadIdx.x / kWave) * (kWave * kUnroll) + (threadIdx.x & (kWave - 1)) : threadIdx.x)) {}
+    __device__ __forceinline__ Index chunk(int u) const { return first + static_cast<uint64_t>(u) * kStep; }
     // checked launches let out-of-range lanes re-read the last chunk instead of branching
     __device__ __forceinline__ Index load_chunk(int u) const {
         const Index c = chunk(u);
@@ -100,6 +113,7 @@ struct RowSteps;
 // kInBytes / kOutBytes: bytes of a chunk in `in` / `out`; kDiv: chunks per scale, 0 = one scale per tensor
 template <int kInBytes, int kOutBytes, int kDiv>
 struct RowsGeo {
+    static constexpr bool kWaveRuns = false;
     const void* in;
     void* out;
     const void* scale_in;
@@ -238,6 +252,7 @@ struct LaneRows {
 template <int kUnroll, int kThreads>
 struct LaneSteps;
 struct LanesGeo {
+    static constexpr bool kWaveRuns = false;
     const void* in;
     void* out;
     const void* scale_in;
@@ -466,6 +481,10 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
     const auto starts_block = [&](auto c) { return kRtGroup ? (c & ((1u << group_log2) - 1u)) == 0 : (c % kDiv) == 0; };
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;  // 64, 32, 16 or 8
+    // chunks of less than a word of codes in a launch of whole tiles dealt out wave by wave: the words are stored
+    // after the last step, one per lane
+    constexpr bool kWordsLater = Geo::kWaveRuns && !kChecked && kChunkBits < 32 && kUnroll % (32 / (kChunkBits < 32 ? kChunkBits : 32)) == 0;
+    [[maybe_unused]] uint32_t words[kUnroll];
     const int param_dtype = kParam != kParamRt ? kParam : param_dtype_rt;
     // Pass 2 of the per-tensor reduction walks the tiles last to first: pass 1 has just read the
     // tensor first to last, so what it read last is what the L2 caches still hold.  Groups of
@@ -579,7 +598,25 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
             constexpr int kLanesPerWord = 32 / kChunkBits;  // 2 or 4
             const uint32_t sub = static_cast<uint32_t>(c) & (kLanesPerWord - 1);
             const uint32_t word = group_or<kLanesPerWord>(w[0] << (sub * kChunkBits));
-            if (live && sub == 0) output_store(keep, word, out + c / kLanesPerWord);
+            if constexpr (kWordsLater)
+                words[u] = word;  // every lane of the word holds it: stored below
+            else if (live && sub == 0)
+                output_store(keep, word, out + c / kLanesPerWord);
+        }
+    }
+    if constexpr (kWordsLater) {
+        // A wave's steps are neighbours in memory (RunGeoWaves): lane `sub` of a word's lanes stores the word of
+        // step g * kLanesPerWord + sub, so every lane stores and a wave's store covers kLanesPerWord * 64 bytes in a row.
+        constexpr int kLanesPerWord = 32 / kChunkBits;
+        const bool keep = qp.keep != 0;
+        const uint32_t sub = threadIdx.x & (kLanesPerWord - 1);
+#pragma unroll
+        for (int g = 0; g < kUnroll / kLanesPerWord; g++) {
+            uint32_t mine = words[g * kLanesPerWord];
+#pragma unroll
+            for (int j = 1; j < kLanesPerWord; j++) mine = sub == static_cast<uint32_t>(j) ? words[g * kLanesPerWord + j] : mine;
+            const auto c = at.chunk(g * kLanesPerWord) + sub * (kWave);
+            output_store(keep, mine, static_cast<uint32_t*>(at.out(0)) + c / kLanesPerWord);
         }
     }
 }
@@ -593,7 +630,12 @@ __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
     const u32x4* __restrict__ in, uint32_t* __restrict__ out, const void* __restrict__ scale_in,
     void* __restrict__ scale_out, uint64_t chunk_begin, uint64_t chunk_end, QuantParams qp, uint32_t num_partials) {
     const RunGeo geo{in, out, scale_in, scale_out, chunk_begin, chunk_end};
-    quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParam, kWide, kUnroll, kThreads, false, kEnc>(geo, kParam, qp, num_partials);
+    if constexpr (F::kPerChunk * kBits < 32) {  // less than a word of codes per chunk
+        const RunGeoWaves waves{geo};
+        quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParam, kWide, kUnroll, kThreads, false, kEnc>(waves, kParam, qp, num_partials);
+    } else {
+        quantize_flat_body<F, kBits, kGroup, kScaleSrc, kParam, kWide, kUnroll, kThreads, false, kEnc>(geo, kParam, qp, num_partials);
+    }
 }
 
 // Pitched rows of whole steps, from step `step_begin` of the launch on, parameters as in quantize_flat_kernel.  A kernel of its own
