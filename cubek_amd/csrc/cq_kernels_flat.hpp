@@ -509,7 +509,9 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
             s_stored[u] = load_dtype_raw(param_dtype, at.scale_in(u), block_of(c));
         else if constexpr (!kDynamic && kGroup != 0 && kScaleSrc != kScalePartials)
             // read once, like the floats: with a plain load the launch takes 4 % longer where its codes are written
-            // through the L2 (cfg5: 100.3 against 96.2 us)
+            // through the L2 (cfg5: 100.3 against 96.2 us).  Where the codes stream (outputs above 192 MiB) it is
+            // the other way round by 3 % (8-bit codes of the same tensor: 115 against 112 us); choosing per launch
+            // puts a branch among the loads, which costs the common case 1 - 5 %.
             s_given[u] = F::load_once(at.scale_in(u), block_of(c));
     }
     if constexpr (kScaleSrc == kScaleStored) {
