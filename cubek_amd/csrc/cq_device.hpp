@@ -485,6 +485,54 @@ __device__ __forceinline__ void pack_chunk_neg(const float* c, uint32_t* w) {
     }
 }
 
+// f16, two's-complement fields that hold the whole value range, a tame divisor: quotient, rounding, clamp and
+// packing of one chunk (eight values) with the tail in packed f16 arithmetic.  The quotient is the one of
+// quantize_values_neg (x * rcp(d), one residual step: within 2^-22 of x / d, which rounds to f16 as x / d does);
+// then, two values per instruction: rounded to f16 (v_cvt_pk_f16_f32), clamped to [lo, hi] (integers, so clamp and
+// rint commute), and added to 1536 + bias, where f16 numbers are one apart: the sum is rint(q) + bias + 1536 with
+// the tie going to the even code (1536 and the bias are even), and its low bits are the biased field, since
+// 1536 = 0x6600 has none of them set.  The two values of a pair are taken kBits * (pairs per half word) fields
+// apart, so that masks and shifts on whole registers put every field in its place.
+// Word layout as pack_chunk_neg<kBits, 8, false>.
+template <int kBits>
+__device__ __forceinline__ void quantize_pack_f16_tame(const float* x, float d, float lo, float hi, uint32_t* w) {
+    static_assert(kBits == 2 || kBits == 4 || kBits == 8, "2, 4 or 8 bits per value");
+    const float nr = -__builtin_amdgcn_rcpf(d);
+    const float nhi_t = -(hi + 1.0f), nlo_t = -(lo - 1.0f);
+    float q[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const float tn = neg_clamp_of_neg(x[i] * nr, nhi_t, nlo_t);  // -t
+        const float e = __builtin_fmaf(tn, d, x[i]);                 // x - t*d
+        q[i] = -__builtin_fmaf(e, nr, tn);                           // t + e*r (the negation folds into the conversion)
+    }
+    constexpr float kMagic = 1536.0f + static_cast<float>(1 << (kBits - 1));
+    const _Float16 lo_h = static_cast<_Float16>(lo), hi_h = static_cast<_Float16>(hi), magic_h = static_cast<_Float16>(kMagic);
+    const f16x2 lo2 = {lo_h, lo_h}, hi2 = {hi_h, hi_h}, magic2 = {magic_h, magic_h};
+    // fields of the pair (a, b): biased, in the low bits of the two halves
+    const auto fields = [&](int a, int b) {
+        f16x2 h = {static_cast<_Float16>(q[a]), static_cast<_Float16>(q[b])};
+        h = __builtin_elementwise_max(lo2, __builtin_elementwise_min(h, hi2));  // NaN -> hi, as the other paths
+        return __builtin_bit_cast(uint32_t, h + magic2);
+    };
+    constexpr uint32_t kMask = ((1u << kBits) - 1u) * 0x00010001u;
+    if constexpr (kBits == 8) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const uint32_t a = fields(4 * j, 4 * j + 2) & kMask, b = fields(4 * j + 1, 4 * j + 3) & kMask;
+            w[j] = (a | (b << 8)) ^ field_bias<8>(32);
+        }
+    } else {
+        uint32_t v = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) v |= (fields(k, k + 4) & kMask) << (k * kBits);
+        if constexpr (kBits == 4)
+            w[0] = v ^ field_bias<4>(32);
+        else
+            w[0] = ((v | (v >> 8)) & 0xffffu) ^ field_bias<2>(16);
+    }
+}
+
 // Sign-extended field i of a word (v_bfe_i32).
 template <int kBits>
 __device__ __forceinline__ float unpack_field(uint32_t w, int i) {

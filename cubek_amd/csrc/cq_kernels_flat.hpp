@@ -583,13 +583,23 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         // a tame abs-max gives a tame scale; every other divisor is looked at itself
         if (!(kDynamic && F::kDtype != CQ_F16) || fs_rounds) tame = divisor_is_tame(d);
 
-        float qn[kN];  // negated codes
-        quantize_values_neg<F, kN, kEnc == kEncInt>(v, d, tame, qp.lo, qp.hi, qn);
         uint32_t w[2];
-        if constexpr (kEnc == kEncInt)
-            pack_chunk_neg<kBits, kN, kWide>(qn, w);
-        else
-            encode_chunk<kEnc, kN>(qn, w);
+        const auto by_value = [&](bool d_tame) {
+            float qn[kN];  // negated codes
+            quantize_values_neg<F, kN, kEnc == kEncInt>(v, d, d_tame, qp.lo, qp.hi, qn);
+            if constexpr (kEnc == kEncInt)
+                pack_chunk_neg<kBits, kN, kWide>(qn, w);
+            else
+                encode_chunk<kEnc, kN>(qn, w);
+        };
+        if constexpr (F::kDtype == CQ_F16 && kEnc == kEncInt && !kWide) {
+            if (tame)
+                quantize_pack_f16_tame<kBits>(v, d, qp.lo, qp.hi, w);
+            else
+                by_value(false);
+        } else {
+            by_value(tame);
+        }
 
         const bool keep = qp.keep != 0;
         if constexpr (kChunkBits == 64) {

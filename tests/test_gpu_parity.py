@@ -504,11 +504,12 @@ def test_scale_division_all_significands(gpu):
                     (value, exp_field, k)
 
 
-@pytest.mark.parametrize("value", [QuantValue.E5M2, QuantValue.Q2S], ids=lambda v: v.name)
+@pytest.mark.parametrize("value", [QuantValue.E5M2, QuantValue.Q2S, QuantValue.Q4S, QuantValue.Q8F], ids=lambda v: v.name)
 def test_f16_every_input_every_divisor(gpu, oracle, value):
-    """The f16 kernels replace the division by a reciprocal and one residual step.  All
+    """The f16 kernels replace the division by a reciprocal and one residual step, and for fields
+    that hold the whole range (Q2 / Q4 / Q8) round, clamp and pack in packed f16 arithmetic.  All
     65536 x 65536 (element, divisor) bit patterns, NaN, infinities, zeros and subnormals
-    included, against the oracle's IEEE division; a wide and a narrow clamp range."""
+    included, against the oracle's IEEE division; a wide clamp range and the three field widths."""
     import torch
     from cubek_amd import ComputeClient
     from cubek_amd import quantize as qz
