@@ -79,65 +79,65 @@ __device__ __forceinline__ void store_y(int dtype, void* y, uint64_t i, float v)
 }
 
 // ---- streaming kernel: 16-bit float types, 1-D blocks of 32 values, 4-bit codes ---------------------
-// A lane owns one block per row: four words (one 16-byte load) and one scale.  A wave covers a strip of
-// 64 blocks = 2048 columns; the waves of a workgroup are the strips of a row, so the 32 values of x a lane
-// needs never change: they stay in 16 registers as packed pairs while the workgroup walks its rows in
-// passes of up to kRows * kChunks rows.  Inside a pass the loads of chunk c + 1 (kRows rows) are issued
-// before chunk c is worked on, so memory and arithmetic overlap inside every wave; the per-lane sums of
-// a pass stay in registers and meet once, at its end: six DPP additions per row, then one LDS exchange
-// across the strips.  Per value: one byte-to-float conversion and one FMA
-// (dequantize_symmetric_packed_value_pairs), half a v_cvt_pk, half a v_dot2.
-// kRows rows of one lane: the four words of its block and the block's scale, per row
-template <class FS, int kRows>
-struct RowChunk {
-    u32x4 w[kRows];
-    FS s[kRows];
-};
+// A wave owns kRows rows and walks along them, strip by strip (64 blocks = 2048 columns, a lane per block: four
+// words, one 16-byte load, and one scale per row), so every wave of a launch does the same work whatever the
+// number of strips, and the row sums never leave the wave: six DPP additions per row at its end, no exchange
+// between waves, no barrier after the first.  (With a wave per strip and the strips of a row in one workgroup,
+// 5 to 8 strips all took the time of 8: the waves of a workgroup go round the four SIMDs from the first one, and
+// the arithmetic, which is what bounds this kernel, piled up there.)  x is staged in LDS once per workgroup,
+// with zeros behind its end up to a whole strip, so idle lanes add nothing, and read from there, 64 bytes
+// per lane and strip.  The loads of strip s + kDepth are issued as soon as strip s has been worked on; past the
+// wave's last strip they fetch one uniform address instead of nothing, so that the number of loads in flight
+// is the same in every iteration and the compiler can count its waits.  Per value: half a byte-to-float
+// conversion and one FMA (dequantize_symmetric_packed_value_pairs), half a v_cvt_pk, half a v_dot2.
+template <dev::Float kF, int kRows, int kWaves, int kDepth>
+__global__ __launch_bounds__(64 * kWaves) void gemv_w4_b32_kernel(
+    const uint32_t* __restrict__ words, const float* __restrict__ scales, const void* __restrict__ x, void* __restrict__ y,
+    int y_dtype, uint32_t rows, uint32_t blocks_per_row, uint64_t word_pitch, uint32_t scale_stride_row,
+    uint32_t scale_stride_col) {
+    extern __shared__ u32x4 xs[];  // x, 64 bytes per block, whole strips
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t strips = (blocks_per_row + 63u) / 64u;
+    for (uint32_t i = threadIdx.x; i < strips * 256u; i += blockDim.x)
+        xs[i] = i < blocks_per_row * 4u ? static_cast<const u32x4*>(x)[i] : u32x4{0, 0, 0, 0};
+    __syncthreads();
+    const uint32_t row0 = (blockIdx.x * kWaves + wave) * kRows;
+    if (row0 >= rows) return;
+    const uint32_t nrows = min(static_cast<uint32_t>(kRows), rows - row0);
 
-template <dev::Float kF, class FS, int kRows, int kChunks, int kMaxStrips>
-__global__ __launch_bounds__(64 * kMaxStrips) void gemv_w4_b32_kernel(
-    const uint32_t* __restrict__ words, const FS* __restrict__ scales, const void* __restrict__ x, void* __restrict__ y,
-    int y_dtype, uint32_t rows, uint32_t blocks_per_row, uint32_t rows_per_group, uint64_t word_pitch,
-    dev::GlobalScaleLayout<1, 32> scale_at) {
-    static_assert(kChunks == 4, "the pass below is written out for four chunks");
-    constexpr int kPass = kRows * kChunks;
-    using Chunk = RowChunk<FS, kRows>;
-    const uint32_t lane = threadIdx.x & 63u, strip = threadIdx.x >> 6, strips = blockDim.x >> 6;
-    const uint32_t block = strip * 64u + lane;
-    const bool live = block < blocks_per_row;
-    const uint32_t b = live ? block : blocks_per_row - 1;  // idle lanes re-read the row's last block
-    // this lane's 32 values of x, as 16 pairs; nothing waits for them before the first rows are on their way
-    uint32_t xp[16];
-    {
-        const u32x4* xv = static_cast<const u32x4*>(x) + static_cast<uint64_t>(b) * 4;
+    struct Chunk {
+        u32x4 w[kRows];
+        float s[kRows];
+    };
+    // the rows' first bytes, wave-uniform; rows past the end are the last row again
+    const char* wrow[kRows];
+    const char* srow[kRows];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const u32x4 v = xv[j];
-            xp[4 * j] = v[0], xp[4 * j + 1] = v[1], xp[4 * j + 2] = v[2], xp[4 * j + 3] = v[3];
-        }
+    for (int k = 0; k < kRows; k++) {
+        const uint32_t r = row0 + min(static_cast<uint32_t>(k), nrows - 1u);
+        wrow[k] = reinterpret_cast<const char*>(words + static_cast<uint64_t>(r) * word_pitch);
+        srow[k] = reinterpret_cast<const char*>(scales + static_cast<uint64_t>(r) * scale_stride_row);
     }
-    __shared__ float partial[kMaxStrips][kPass];
-    const uint32_t row_begin = blockIdx.x * rows_per_group;
-    const uint32_t row_end = min(row_begin + rows_per_group, rows);
-    const u32x4* const wbase = reinterpret_cast<const u32x4*>(words) + b;
-    const uint64_t wstep = word_pitch / 4;  // row pitch in 16-byte units
-
-    // rows [first, first + kRows) of the pass; rows past the workgroup's end re-read its last row
-    const auto load = [&](Chunk& c, uint32_t first) {
+    const auto load = [&](Chunk& c, uint32_t strip) {
+        const bool real = strip < strips;  // wave-uniform
+        const uint32_t b = min(strip * 64u + lane, blocks_per_row - 1u);  // idle lanes re-read the row's last block
+        const uint32_t woff = real ? b * 16u : 0u, soff = real ? b * scale_stride_col * 4u : 0u;
 #pragma unroll
         for (int k = 0; k < kRows; k++) {
-            const uint32_t r = min(first + k, row_end - 1);
-            c.w[k] = __builtin_nontemporal_load(wbase + r * wstep);
-            c.s[k] = __builtin_nontemporal_load(scales + scale_at.to_source_pos(0, r, b * 32u));
+            c.w[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[k] + woff));
+            c.s[k] = __builtin_nontemporal_load(reinterpret_cast<const float*>(srow[k] + soff));
         }
-        __builtin_amdgcn_sched_barrier(0);  // loads stay where they are written: one chunk ahead of the arithmetic
+        __builtin_amdgcn_sched_barrier(0);  // loads stay where they are written: two strips ahead of the arithmetic
     };
-    // One row's share of this lane, the plain way: words, scale and x read again from memory in rolled loops
-    // (few registers, little code).  Only lanes whose scale is not tame come here.
-    const auto plain_row = [&](uint32_t r) {
-        const uint32_t* wr = words + r * word_pitch + b * 4u;
-        const FS scale = scales[scale_at.to_source_pos(0, r, b * 32u)];
-        const typename Elem<kF>::T* xr = static_cast<const typename Elem<kF>::T*>(x) + b * 32u;
+    // One row's share of this lane, the plain way (rolled loops, operands read again).  Only lanes whose scale
+    // is not tame come here.
+    const auto plain_row = [&](int k, uint32_t strip) {
+        const uint32_t block = strip * 64u + lane;
+        if (block >= blocks_per_row) return 0.0f;
+        const uint32_t* wr = reinterpret_cast<const uint32_t*>(wrow[k]) + block * 4u;
+        const float scale = reinterpret_cast<const float*>(srow[k])[block * scale_stride_col];
+        const typename Elem<kF>::T* xr = static_cast<const typename Elem<kF>::T*>(x) + block * 32u;
         float a = 0.0f;
 #pragma unroll 1
         for (int j = 0; j < 4; j++) {
@@ -150,15 +150,23 @@ __global__ __launch_bounds__(64 * kMaxStrips) void gemv_w4_b32_kernel(
                 a = dot2<kF>(dev::pack_pair<kF>(v[i], v[i + 1]), xpair, a);
             }
         }
-        return live ? a : 0.0f;
+        return a;
     };
-    // rows [first, first + kRows) out of a chunk's registers into acc[0..kRows); rows past the workgroup's end
-    // are skipped (the row numbers are wave-uniform, so these are scalar branches)
-    const auto work = [&](const Chunk& c, uint32_t first, float* acc) {
+    float acc[kRows];
+#pragma unroll
+    for (int k = 0; k < kRows; k++) acc[k] = 0.0f;
+    const auto work = [&](const Chunk& c, uint32_t strip) {
+        // this lane's 32 values of x, as 16 pairs
+        uint32_t xp[16];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const u32x4 v = xs[(strip * 64u + lane) * 4u + j];
+            xp[4 * j] = v[0], xp[4 * j + 1] = v[1], xp[4 * j + 2] = v[2], xp[4 * j + 3] = v[3];
+        }
         bool tame = true;
+        float part[kRows];
 #pragma unroll
         for (int k = 0; k < kRows; k++) {
-            if (k > 0 && first + k >= row_end) break;
             float a = 0.0f;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
@@ -167,51 +175,35 @@ __global__ __launch_bounds__(64 * kMaxStrips) void gemv_w4_b32_kernel(
 #pragma unroll
                 for (int i = 0; i < 4; i++) a = dot2<kF>(pairs[i], xp[4 * j + i], a);
             }
-            acc[k] = live ? a : 0.0f;  // idle lanes worked on a copy of the row's last block
+            part[k] = a;
             tame = tame && dev::pairs_scale_is_tame<kF>(c.s[k]);
         }
         // ordinary scales are all tame: one wave-uniform test per chunk, then straight on
         if (__builtin_amdgcn_ballot_w64(!tame) != 0) {
 #pragma unroll
             for (int k = 0; k < kRows; k++)
-                if (first + k < row_end && !dev::pairs_scale_is_tame<kF>(c.s[k])) acc[k] = plain_row(first + k);
+                if (!dev::pairs_scale_is_tame<kF>(c.s[k])) part[k] = plain_row(k, strip);
         }
+#pragma unroll
+        for (int k = 0; k < kRows; k++) acc[k] += part[k];
         __builtin_amdgcn_sched_barrier(0);
     };
-
-    // Chunks alternate between two register sets; each is re-filled, two chunks ahead, as soon as its rows have
-    // been worked on, also across the end of a pass, so the stream of loads never pauses for a reduction.
-    Chunk ca, cb;
-    load(ca, row_begin);
-    if (row_begin + kRows < row_end) load(cb, row_begin + kRows);
-    for (uint32_t p0 = row_begin; p0 < row_end; p0 += kPass) {
-        // which chunks exist is wave-uniform: scalar branches
-        float acc[kPass];
+    Chunk c[kDepth];
 #pragma unroll
-        for (int k = 0; k < kPass; k++) acc[k] = 0.0f;
-        work(ca, p0, acc);
-        if (p0 + 2 * kRows < row_end) load(ca, p0 + 2 * kRows);
-        if (p0 + kRows < row_end) work(cb, p0 + kRows, acc + kRows);
-        if (p0 + 3 * kRows < row_end) load(cb, p0 + 3 * kRows);
-        if (p0 + 2 * kRows < row_end) work(ca, p0 + 2 * kRows, acc + 2 * kRows);
-        if (p0 + 4 * kRows < row_end) load(ca, p0 + 4 * kRows);  // the next pass's first chunk
-        if (p0 + 3 * kRows < row_end) work(cb, p0 + 3 * kRows, acc + 3 * kRows);
-        if (p0 + 5 * kRows < row_end) load(cb, p0 + 5 * kRows);
-        // the pass's row sums: lane 63 of every wave holds its strip's share
+    for (int d = 0; d < kDepth; d++) load(c[d], d);
+    for (uint32_t strip = 0; strip < strips; strip += kDepth) {
 #pragma unroll
-        for (int k = 0; k < kPass; k++)
-            if (p0 + k < row_end) acc[k] = wave_sum_to_lane63(acc[k]);
-        if (lane == 63) {
-#pragma unroll
-            for (int k = 0; k < kPass; k++) partial[strip][k] = acc[k];
+        for (int d = 0; d < kDepth; d++) {
+            if (d == 0 || strip + d < strips) work(c[d], strip + d);
+            load(c[d], strip + d + kDepth);
         }
-        __syncthreads();
-        if (threadIdx.x < kPass && p0 + threadIdx.x < row_end) {
-            float v = 0.0f;
-            for (uint32_t t = 0; t < strips; t++) v += partial[t][threadIdx.x];
-            store_y(y_dtype, y, p0 + threadIdx.x, v);
-        }
-        __syncthreads();
+    }
+#pragma unroll
+    for (int k = 0; k < kRows; k++) acc[k] = wave_sum_to_lane63(acc[k]);
+    if (lane == 63) {
+#pragma unroll
+        for (int k = 0; k < kRows; k++)
+            if (static_cast<uint32_t>(k) < nrows) store_y(y_dtype, y, row0 + k, acc[k]);
     }
 }
 
@@ -272,27 +264,31 @@ hipError_t launch_general_bits(hipStream_t s, const GemvArgs& a, const dev::Scal
     }
 }
 
-constexpr int kStreamRows = 4, kStreamChunks = 4, kStreamMaxStrips = 16;
+constexpr int kStreamRows = 2, kStreamDepth = 2;
+constexpr uint32_t kStreamMaxStrips = 16;  // x of 16 strips fills 64 KiB of LDS
 
+template <dev::Float kF, int kWaves>
+void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
+    const uint32_t blocks_per_row = a.cols / 32, strips = (blocks_per_row + 63) / 64;
+    const dim3 grid((a.rows + kStreamRows * kWaves - 1) / (kStreamRows * kWaves)), block(64 * kWaves);
+    hipLaunchKernelGGL((gemv_w4_b32_kernel<kF, kStreamRows, kWaves, kStreamDepth>), grid, block, strips * 4096, s,
+                       static_cast<const uint32_t*>(a.words), static_cast<const float*>(a.scales), a.x, a.y, a.y_dtype, a.rows,
+                       blocks_per_row, a.word_pitch, static_cast<uint32_t>(a.scale_stride_row),
+                       static_cast<uint32_t>(a.scale_stride_col));
+}
+
+// Two rows per wave, two strips in flight, four waves (eight rows) per workgroup; eight waves from 16384 columns
+// on, where the 32 KiB and more of x that every workgroup stages weigh more than the smaller workgroup gains.
+// Measured on MI355X (rows / waves / strips in flight; weights [14336, 4096], [28672, 8192], [4096, 11008],
+// [8192, 28672]): 2 / 4 / 2 10.1, 31.3, 9.5, 33.5 us; 2 / 8 / 2 11.2, 33.1, 9.0, 28.9 us; 2 / 4 / 3 10.3, 33.0,
+// 10.1, 33.4 us; 4 / 4 / 2 11.8, 36.5, 10.3, 32.6 us; 1 / 4 / 4 11.4, 34.0, 10.1, 43.3 us; 3 / 4 / 2 10.8, 31.2,
+// 11.7, 34.5 us.
 template <dev::Float kF>
 hipError_t launch_stream(hipStream_t s, const GemvArgs& a) {
-    const uint32_t blocks_per_row = a.cols / 32;
-    const uint32_t strips = (blocks_per_row + 63) / 64;
-    // Seven rows per wave, fewer where that would leave fewer than four waves per SIMD (256 compute units x 4
-    // SIMDs).  Measured on MI355X with 4096 / 8192 / 16384 / 32768 waves per launch: weights [14336, 4096]
-    // 11.5 / 11.7 / 13.4 / 19.4 us, [28672, 8192] 34.5 / 31.7 / 30.0 / 31.5 us: about seven rows per wave in
-    // both, enough rows to pay for a wave's 64 bytes of x per lane and enough waves to even out their ends.
-    const uint64_t row_strips = static_cast<uint64_t>(a.rows) * strips;
-    uint32_t rows_per_group = static_cast<uint32_t>((row_strips + 4095) / 4096);
-    if (rows_per_group < 1) rows_per_group = 1;
-    if (rows_per_group > 7) rows_per_group = 7;
-    const dim3 grid((a.rows + rows_per_group - 1) / rows_per_group), block(64 * strips);
-    dev::GlobalScaleLayout<1, 32> scale_at;
-    scale_at.stride_row = static_cast<uint32_t>(a.scale_stride_row);
-    scale_at.stride_col = static_cast<uint32_t>(a.scale_stride_col);
-    hipLaunchKernelGGL((gemv_w4_b32_kernel<kF, float, kStreamRows, kStreamChunks, kStreamMaxStrips>), grid, block, 0, s,
-                       static_cast<const uint32_t*>(a.words), static_cast<const float*>(a.scales), a.x, a.y, a.y_dtype, a.rows,
-                       blocks_per_row, rows_per_group, a.word_pitch, scale_at);
+    if (a.cols >= 16384)
+        launch_stream_waves<kF, 8>(s, a);
+    else
+        launch_stream_waves<kF, 4>(s, a);
     return hipGetLastError();
 }
 
@@ -301,8 +297,7 @@ hipError_t launch_stream(hipStream_t s, const GemvArgs& a) {
 bool gemv_streams(const GemvArgs& a) {
     return a.dtype != CQ_F32 && a.bits == 4 && a.block_rows == 1 && a.block_cols == 32 && a.param_dtype == CQ_F32 &&
            a.cols % 32 == 0 && a.cols / 32 <= 64u * kStreamMaxStrips && a.word_pitch % 4 == 0 && a.x_aligned16 &&
-           a.words_aligned16 && a.rows < (1u << 26) && static_cast<uint64_t>(a.rows) * a.scale_stride_row < (1ull << 32) &&
-           (a.cols / 32) * a.scale_stride_col < (1ull << 32);
+           a.words_aligned16 && a.scale_stride_row < (1ull << 32) && (a.cols / 32) * a.scale_stride_col < (1ull << 30);
 }
 
 hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a) {

@@ -267,7 +267,8 @@ __device__ __forceinline__ void dequantize_symmetric_packed_value_pairs_tame(uin
             // is d * 2^-9 for every d in 0..15 (denormals, then the first binade, in one linear run), so
             // v_cvt_pk_f32_fp8 turns two digits into floats per instruction; s * 512 takes the 2^-9 back
             typedef float f32x2 __attribute__((ext_vector_type(2)));
-            const uint32_t even = digits & 0x0f0f0f0fu, odd = (digits >> 4) & 0x0f0f0f0fu;
+            // (mask, then bias: each is one three-operand bit operation on gfx950)
+            const uint32_t even = (word & 0x0f0f0f0fu) ^ 0x08080808u, odd = ((word >> 4) & 0x0f0f0f0fu) ^ 0x08080808u;
             const f32x2 e01 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(even), false);
             const f32x2 e23 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(even), true);
             const f32x2 o01 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(odd), false);

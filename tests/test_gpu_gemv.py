@@ -1,6 +1,6 @@
 """cq_gemv_quantized (y = dequantize(W) @ x from the packed weights) against the GEMV over the ORACLE's
 dequantized weights, computed in float64.  Tolerance, stated once: the kernels accumulate in f32, at most
-~180 sequential additions per lane followed by a 6-step tree, each rounding 2^-24 relative, so
+~260 sequential additions per lane followed by a 6-step tree, each rounding 2^-24 relative, so
 |y - y_ref| <= 2e-5 * sum|w * x|; an output of a 16-bit type is the f32 sum rounded once (checked bit for
 bit against the f32 output)."""
 import numpy as np
@@ -12,12 +12,16 @@ from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantParam, QuantSch
 pytestmark = pytest.mark.gpu
 
 CASES = [
-    # elem, value, block, param, rows, cols, word pitch (None: contiguous)     -- first five: the streaming kernel
+    # elem, value, block, param, rows, cols, word pitch (None: contiguous)     -- first nine: the streaming kernel
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 1000, 4096, None),
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 77, 2048, None),
     (ElemType.BF16, QuantValue.E2M1, [32], QuantParam.F32, 130, 11008, None),     # last strip partly idle
     (ElemType.F16, QuantValue.Q4F, [32], QuantParam.F32, 333, 8192, None),
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 64, 4096, 520),         # pitched rows of words
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 50, 8448, None),        # four strips and an eighth
+    (ElemType.F16, QuantValue.Q4S, [32], QuantParam.F32, 21, 16480, None),        # eight waves per workgroup
+    (ElemType.BF16, QuantValue.Q4F, [32], QuantParam.F32, 1, 32768, None),        # one row, the longest it takes
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 9, 32, None),           # one block per row
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.BF16, 100, 1024, None),      # general kernel from here on
     (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, 50, 512, None),
     (ElemType.F32, QuantValue.Q2S, [64], QuantParam.F32, 96, 1024, None),
