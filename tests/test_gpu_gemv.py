@@ -113,6 +113,36 @@ def test_gemv_scales_of_every_kind(oracle, elem):
     assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), float(np.max(np.abs(got - want) / (mag + 1e-30)))
 
 
+def test_gemv_scales_with_strides(oracle):
+    """The scales of a [rows, blocks] layout stored column by column (strides (1, rows)) and with a row pitch:
+    the streaming kernel addresses them through both strides."""
+    import torch
+
+    rows, cols = 37, 2304
+    scheme = QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([32]))
+    rng = np.random.default_rng(11)
+    words = rng.integers(0, 2**32, (rows, cols // 8), dtype=np.uint64).astype(np.uint32)
+    scales = rng.uniform(0.001, 0.02, (rows, cols // 32)).astype(np.float32)
+    deq = oracle.from_bits(oracle.dequantize(words, (rows, cols), scales, ElemType.BF16, scheme), ElemType.BF16).astype(np.float64)
+    xb = oracle.to_bits(rng.normal(0, 1, cols).astype(np.float32), ElemType.BF16)
+    x64 = oracle.from_bits(xb, ElemType.BF16).astype(np.float64)
+    want, mag = deq @ x64, np.abs(deq) @ np.abs(x64)
+    d_words = torch.from_numpy(words.view(np.int32)).cuda()
+    d_x = torch.from_numpy(xb.view(np.int16)).cuda()
+    h = TensorHandleRef.from_torch
+    nb = cols // 32
+    col_major = torch.from_numpy(np.ascontiguousarray(scales.T)).cuda()           # [blocks, rows]
+    pitched = torch.zeros((rows, nb + 5), dtype=torch.float32, device="cuda")
+    pitched[:, :nb] = torch.from_numpy(scales).cuda()
+    for name, h_scales in (("column-major", TensorHandleRef(col_major.data_ptr(), (rows, nb), (1, rows), 4)),
+                           ("pitched", TensorHandleRef(pitched.data_ptr(), (rows, nb), (nb + 5, 1), 4))):
+        y = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
+        matvec.launch_ref(ComputeClient.current(), h(d_words), h_scales, scheme, h(d_x), h(y), ElemType.BF16, ElemType.F32)
+        torch.cuda.synchronize()
+        got = y.cpu().numpy().astype(np.float64)
+        assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), name
+
+
 def test_gemv_argument_checks():
     import torch
 
