@@ -299,25 +299,37 @@ def cpu_baseline(torch, w, path, budget_s=12.0):
 
 def packed_gemv(torch):
     """The consumer side of the packed format: cq_gemv_quantized over 4-bit weights with f32 scales on blocks of
-    32 (configuration 3's weight-load path and four other weights), weights rotated through enough sets that
-    no launch finds them in the Infinity Cache.  HBM roofline on the packed bytes."""
-    from cubek_amd import ComputeClient, ElemType, QuantLevel, QuantScheme, QuantValue, TensorHandleRef, matvec
+    32 (configuration 3's weight-load path and four other weights), then other codes, blocks and scale types on
+    the largest of them; weights rotated through enough sets that no launch finds them in the Infinity Cache.
+    HBM roofline on the packed bytes."""
+    from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantParam, QuantScheme, QuantValue, TensorHandleRef,
+                           matvec)
 
     client = ComputeClient.current()
     h = TensorHandleRef.from_torch
-    scheme = QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([32]))
+    types = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+    cases = [(r, c, "Q4S", 32, "f32", "bf16") for r, c in ((14336, 4096), (4096, 14336), (28672, 8192), (4096, 11008),
+                                                          (8192, 28672))]
+    cases += [(28672, 8192, "Q4S", 128, "f16", "f16"), (28672, 8192, "Q4S", 64, "bf16", "bf16"),
+              (28672, 8192, "Q8S", 32, "f32", "bf16"), (28672, 8192, "Q2S", 64, "f32", "bf16")]
     out = []
-    for rows, cols in ((14336, 4096), (4096, 14336), (28672, 8192), (4096, 11008), (8192, 28672)):
-        b = rows * cols // 2 + rows * cols // 32 * 4 + cols * 2 + rows * 2
+    for rows, cols, value, block, param, elem in cases:
+        scheme = (QuantScheme.default().with_value(QuantValue[value]).with_level(QuantLevel.block([block]))
+                  .with_param(QuantParam[param.upper()]))
+        nq = scheme.num_quants()
+        b = rows * cols // nq * 4 + rows * cols // block * (4 if param == "f32" else 2) + cols * 2 + rows * 2
         sets = max(2, min(16, -(-(1 << 30) // b)))
-        ws = [torch.randint(-2**31, 2**31 - 1, (rows, cols // 8), dtype=torch.int32, device="cuda") for _ in range(sets)]
-        ss = [torch.rand((rows, cols // 32), dtype=torch.float32, device="cuda") * 0.01 + 0.001 for _ in range(sets)]
-        x = torch.randn(cols, device="cuda").to(torch.bfloat16)
-        y = torch.zeros(rows, device="cuda", dtype=torch.bfloat16)
+        ws = [torch.randint(-2**31, 2**31 - 1, (rows, cols // nq), dtype=torch.int32, device="cuda") for _ in range(sets)]
+        ss = [(torch.rand((rows, cols // block), dtype=torch.float32, device="cuda") * 0.01 + 0.001).to(types[param])
+              for _ in range(sets)]
+        x = torch.randn(cols, device="cuda").to(types[elem])
+        y = torch.zeros(rows, device="cuda", dtype=types[elem])
         hw, hs, hx, hy = [h(t) for t in ws], [h(t) for t in ss], h(x), h(y)
-        fn = lambda i: matvec.launch_ref(client, hw[i % sets], hs[i % sets], scheme, hx, hy, ElemType.BF16, ElemType.BF16)
+        et = ElemType[elem.upper()]
+        fn = lambda i: matvec.launch_ref(client, hw[i % sets], hs[i % sets], scheme, hx, hy, et, et)
         ms = sorted(timed_region(torch, fn, 48)[0] for _ in range(3))[1]
-        out.append({"kernel": f"gemv_quantized, q4 blocks of 32, f32 scales, bf16 x and y, weights [{rows}, {cols}]",
+        out.append({"kernel": f"gemv_quantized, {value.lower()[:2]} blocks of {block}, {param} scales, {elem} x and y, "
+                              f"weights [{rows}, {cols}]",
                     "algorithmic_bytes": b, "buffer_sets_rotated": sets, "ms": round(ms, 4),
                     "GBps": round(b / (ms * 1e-3) / 1e9, 1), "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                     "weights_per_s": round(rows * cols / (ms * 1e-3))})

@@ -78,29 +78,34 @@ __device__ __forceinline__ void store_y(int dtype, void* y, uint64_t i, float v)
         static_cast<__bf16*>(y)[i] = static_cast<__bf16>(v);
 }
 
-// ---- streaming kernel: 16-bit float types, 1-D blocks of 32 values, 4-bit codes ---------------------
-// A wave owns kRows rows and walks along them, strip by strip (64 blocks = 2048 columns, a lane per block: four
-// words, one 16-byte load, and one scale per row), so every wave of a launch does the same work whatever the
-// number of strips, and the row sums never leave the wave: six DPP additions per row at its end, no exchange
-// between waves, no barrier after the first.  (With a wave per strip and the strips of a row in one workgroup,
-// 5 to 8 strips all took the time of 8: the waves of a workgroup go round the four SIMDs from the first one, and
-// the arithmetic, which is what bounds this kernel, piled up there.)  x is staged in LDS once per workgroup,
-// with zeros behind its end up to a whole strip, so idle lanes add nothing, and read from there, 64 bytes
-// per lane and strip.  The loads of strip s + kDepth are issued as soon as strip s has been worked on; past the
-// wave's last strip they fetch one uniform address instead of nothing, so that the number of loads in flight
-// is the same in every iteration and the compiler can count its waits.  Per value: half a byte-to-float
-// conversion and one FMA (dequantize_symmetric_packed_value_pairs), half a v_cvt_pk, half a v_dot2.
-template <dev::Float kF, int kRows, int kWaves, int kDepth>
-__global__ __launch_bounds__(64 * kWaves) void gemv_w4_b32_kernel(
-    const uint32_t* __restrict__ words, const float* __restrict__ scales, const void* __restrict__ x, void* __restrict__ y,
-    int y_dtype, uint32_t rows, uint32_t blocks_per_row, uint64_t word_pitch, uint32_t scale_stride_row,
-    uint32_t scale_stride_col) {
-    extern __shared__ u32x4 xs[];  // x, 64 bytes per block, whole strips
+// ---- streaming kernel: 16-bit float types, blocks along the row ---------------------------------------
+// A lane's unit is one 16-byte load of codes: four words, 64 values of 2 bits, 32 of 4 or 16 of 8, under one scale
+// (blocks of 1, 2, 4, ... units).  A wave owns kRows rows and walks along them, strip by strip (64 units, a lane
+// per unit), so every wave of a launch does the same work whatever the number of strips, and the row sums never
+// leave the wave: six DPP additions per row at its end, no exchange between waves, no barrier after the first.
+// (With a wave per strip and the strips of a row in one workgroup, 5 to 8 strips all took the time of 8: the
+// waves of a workgroup go round the four SIMDs from the first one, and the arithmetic, which is what bounds this
+// kernel, piled up there.)  x is staged in LDS once per workgroup, with zeros behind its end up to a whole strip,
+// so idle lanes add nothing, and read from there, a unit's values per lane and strip.  The loads of strip
+// s + kDepth are issued as soon as strip s has been worked on; past the wave's last strip they fetch one uniform
+// address instead of nothing, so that the number of loads in flight is the same in every iteration and the
+// compiler can count its waits.  Per 4-bit value: half a byte-to-float conversion and one FMA
+// (dequantize_symmetric_packed_value_pairs), half a v_cvt_pk, half a v_dot2.
+template <dev::Float kF, class FS, int kBits, int kRows, int kWaves, int kDepth>
+__global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
+    const uint32_t* __restrict__ words, const FS* __restrict__ scales, const void* __restrict__ x, void* __restrict__ y,
+    int y_dtype, uint32_t rows, uint32_t units_per_row, uint32_t units_per_block_log2, uint64_t word_pitch,
+    uint32_t scale_stride_row, uint32_t scale_stride_col) {
+    constexpr uint32_t kVals = 128 / kBits;         // values of a unit
+    constexpr uint32_t kPairs = kVals / 2;          // ... as packed pairs of x
+    constexpr uint32_t kVecs = kPairs / 4;          // ... as 16-byte pieces of x
+    constexpr uint32_t kWordPairs = 16 / kBits;     // pairs out of one word
+    extern __shared__ u32x4 xs[];  // x, kVecs pieces per unit, whole strips
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t strips = (blocks_per_row + 63u) / 64u;
-    for (uint32_t i = threadIdx.x; i < strips * 256u; i += blockDim.x)
-        xs[i] = i < blocks_per_row * 4u ? static_cast<const u32x4*>(x)[i] : u32x4{0, 0, 0, 0};
+    const uint32_t strips = (units_per_row + 63u) / 64u;
+    for (uint32_t i = threadIdx.x; i < strips * 64u * kVecs; i += blockDim.x)
+        xs[i] = i < units_per_row * kVecs ? static_cast<const u32x4*>(x)[i] : u32x4{0, 0, 0, 0};
     __syncthreads();
     const uint32_t row0 = (blockIdx.x * kWaves + wave) * kRows;
     if (row0 >= rows) return;
@@ -108,7 +113,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_w4_b32_kernel(
 
     struct Chunk {
         u32x4 w[kRows];
-        float s[kRows];
+        FS s[kRows];
     };
     // the rows' first bytes, wave-uniform; rows past the end are the last row again
     const char* wrow[kRows];
@@ -119,34 +124,36 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_w4_b32_kernel(
         wrow[k] = reinterpret_cast<const char*>(words + static_cast<uint64_t>(r) * word_pitch);
         srow[k] = reinterpret_cast<const char*>(scales + static_cast<uint64_t>(r) * scale_stride_row);
     }
+    const uint32_t scale_step = scale_stride_col * static_cast<uint32_t>(sizeof(FS));
     const auto load = [&](Chunk& c, uint32_t strip) {
         const bool real = strip < strips;  // wave-uniform
-        const uint32_t b = min(strip * 64u + lane, blocks_per_row - 1u);  // idle lanes re-read the row's last block
-        const uint32_t woff = real ? b * 16u : 0u, soff = real ? b * scale_stride_col * 4u : 0u;
+        const uint32_t u = min(strip * 64u + lane, units_per_row - 1u);  // idle lanes re-read the row's last unit
+        const uint32_t woff = real ? u * 16u : 0u, soff = real ? (u >> units_per_block_log2) * scale_step : 0u;
 #pragma unroll
         for (int k = 0; k < kRows; k++) {
             c.w[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[k] + woff));
-            c.s[k] = __builtin_nontemporal_load(reinterpret_cast<const float*>(srow[k] + soff));
+            c.s[k] = __builtin_nontemporal_load(reinterpret_cast<const FS*>(srow[k] + soff));
         }
-        __builtin_amdgcn_sched_barrier(0);  // loads stay where they are written: two strips ahead of the arithmetic
+        __builtin_amdgcn_sched_barrier(0);  // loads stay where they are written: kDepth strips ahead of the arithmetic
     };
     // One row's share of this lane, the plain way (rolled loops, operands read again).  Only lanes whose scale
     // is not tame come here.
     const auto plain_row = [&](int k, uint32_t strip) {
-        const uint32_t block = strip * 64u + lane;
-        if (block >= blocks_per_row) return 0.0f;
-        const uint32_t* wr = reinterpret_cast<const uint32_t*>(wrow[k]) + block * 4u;
-        const float scale = reinterpret_cast<const float*>(srow[k])[block * scale_stride_col];
-        const typename Elem<kF>::T* xr = static_cast<const typename Elem<kF>::T*>(x) + block * 32u;
+        const uint32_t u = strip * 64u + lane;
+        if (u >= units_per_row) return 0.0f;
+        const uint32_t* wr = reinterpret_cast<const uint32_t*>(wrow[k]) + u * 4u;
+        const FS scale = *reinterpret_cast<const FS*>(srow[k] + (u >> units_per_block_log2) * scale_step);
+        const typename Elem<kF>::T* xr = static_cast<const typename Elem<kF>::T*>(x) + u * kVals;
         float a = 0.0f;
 #pragma unroll 1
         for (int j = 0; j < 4; j++) {
-            float v[8];
-            dev::dequantize_symmetric_packed_value<kF, 4>(wr[j], scale, v);
+            float v[2 * kWordPairs];
+            dev::dequantize_symmetric_packed_value<kF, kBits>(wr[j], scale, v);
 #pragma unroll
-            for (int i = 0; i < 8; i += 2) {
-                const uint32_t xpair = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, xr[8 * j + i])) |
-                                       static_cast<uint32_t>(__builtin_bit_cast(uint16_t, xr[8 * j + i + 1])) << 16;
+            for (uint32_t i = 0; i < 2 * kWordPairs; i += 2) {
+                const uint32_t xpair =
+                    static_cast<uint32_t>(__builtin_bit_cast(uint16_t, xr[2 * kWordPairs * j + i])) |
+                    static_cast<uint32_t>(__builtin_bit_cast(uint16_t, xr[2 * kWordPairs * j + i + 1])) << 16;
                 a = dot2<kF>(dev::pack_pair<kF>(v[i], v[i + 1]), xpair, a);
             }
         }
@@ -156,11 +163,11 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_w4_b32_kernel(
 #pragma unroll
     for (int k = 0; k < kRows; k++) acc[k] = 0.0f;
     const auto work = [&](const Chunk& c, uint32_t strip) {
-        // this lane's 32 values of x, as 16 pairs
-        uint32_t xp[16];
+        // this lane's values of x, as pairs
+        uint32_t xp[kPairs];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const u32x4 v = xs[(strip * 64u + lane) * 4u + j];
+        for (uint32_t j = 0; j < kVecs; j++) {
+            const u32x4 v = xs[(strip * 64u + lane) * kVecs + j];
             xp[4 * j] = v[0], xp[4 * j + 1] = v[1], xp[4 * j + 2] = v[2], xp[4 * j + 3] = v[3];
         }
         bool tame = true;
@@ -170,10 +177,10 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_w4_b32_kernel(
             float a = 0.0f;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                uint32_t pairs[4];
-                dev::dequantize_symmetric_packed_value_pairs_tame<kF, 4>(c.w[k][j], c.s[k], pairs);
+                uint32_t pairs[kWordPairs];
+                dev::dequantize_symmetric_packed_value_pairs_tame<kF, kBits>(c.w[k][j], c.s[k], pairs);
 #pragma unroll
-                for (int i = 0; i < 4; i++) a = dot2<kF>(pairs[i], xp[4 * j + i], a);
+                for (uint32_t i = 0; i < kWordPairs; i++) a = dot2<kF>(pairs[i], xp[kWordPairs * j + i], a);
             }
             part[k] = a;
             tame = tame && dev::pairs_scale_is_tame<kF>(c.s[k]);
@@ -265,44 +272,76 @@ hipError_t launch_general_bits(hipStream_t s, const GemvArgs& a, const dev::Scal
 }
 
 constexpr int kStreamRows = 2, kStreamDepth = 2;
-constexpr uint32_t kStreamMaxStrips = 16;  // x of 16 strips fills 64 KiB of LDS
+constexpr uint32_t kStreamMaxColumns = 32768;  // x of that many columns fills 64 KiB of LDS
 
-template <dev::Float kF, int kWaves>
+uint32_t log2_of(uint32_t v) {
+    uint32_t l = 0;
+    while ((1u << l) < v) l++;
+    return l;
+}
+
+template <dev::Float kF, class FS, int kBits, int kWaves>
 void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
-    const uint32_t blocks_per_row = a.cols / 32, strips = (blocks_per_row + 63) / 64;
+    constexpr uint32_t kVals = 128 / kBits;
+    const uint32_t units_per_row = a.cols / kVals, strips = (units_per_row + 63) / 64;
     const dim3 grid((a.rows + kStreamRows * kWaves - 1) / (kStreamRows * kWaves)), block(64 * kWaves);
-    hipLaunchKernelGGL((gemv_w4_b32_kernel<kF, kStreamRows, kWaves, kStreamDepth>), grid, block, strips * 4096, s,
-                       static_cast<const uint32_t*>(a.words), static_cast<const float*>(a.scales), a.x, a.y, a.y_dtype, a.rows,
-                       blocks_per_row, a.word_pitch, static_cast<uint32_t>(a.scale_stride_row),
-                       static_cast<uint32_t>(a.scale_stride_col));
+    hipLaunchKernelGGL((gemv_stream_kernel<kF, FS, kBits, kStreamRows, kWaves, kStreamDepth>), grid, block,
+                       strips * 64 * kVals * 2, s, static_cast<const uint32_t*>(a.words), static_cast<const FS*>(a.scales), a.x,
+                       a.y, a.y_dtype, a.rows, units_per_row, log2_of(a.block_cols / kVals), a.word_pitch,
+                       static_cast<uint32_t>(a.scale_stride_row), static_cast<uint32_t>(a.scale_stride_col));
 }
 
 // Two rows per wave, two strips in flight, four waves (eight rows) per workgroup; eight waves from 16384 columns
 // on, where the 32 KiB and more of x that every workgroup stages weigh more than the smaller workgroup gains.
-// Measured on MI355X (rows / waves / strips in flight; weights [14336, 4096], [28672, 8192], [4096, 11008],
+// Measured on MI355X (rows / waves / strips in flight; 4-bit weights [14336, 4096], [28672, 8192], [4096, 11008],
 // [8192, 28672]): 2 / 4 / 2 10.1, 31.3, 9.5, 33.5 us; 2 / 8 / 2 11.2, 33.1, 9.0, 28.9 us; 2 / 4 / 3 10.3, 33.0,
 // 10.1, 33.4 us; 4 / 4 / 2 11.8, 36.5, 10.3, 32.6 us; 1 / 4 / 4 11.4, 34.0, 10.1, 43.3 us; 3 / 4 / 2 10.8, 31.2,
 // 11.7, 34.5 us.
-template <dev::Float kF>
-hipError_t launch_stream(hipStream_t s, const GemvArgs& a) {
+template <dev::Float kF, class FS, int kBits>
+void launch_stream_bits(hipStream_t s, const GemvArgs& a) {
     if (a.cols >= 16384)
-        launch_stream_waves<kF, 8>(s, a);
+        launch_stream_waves<kF, FS, kBits, 8>(s, a);
     else
-        launch_stream_waves<kF, 4>(s, a);
+        launch_stream_waves<kF, FS, kBits, 4>(s, a);
+}
+
+// scales typed f32 or like x
+template <dev::Float kF, class Same>
+hipError_t launch_stream(hipStream_t s, const GemvArgs& a) {
+    if (a.param_dtype == CQ_F32) {
+        if (a.bits == 4)
+            launch_stream_bits<kF, float, 4>(s, a);
+        else if (a.bits == 8)
+            launch_stream_bits<kF, float, 8>(s, a);
+        else
+            launch_stream_bits<kF, float, 2>(s, a);
+    } else {
+        if (a.bits == 4)
+            launch_stream_bits<kF, Same, 4>(s, a);
+        else if (a.bits == 8)
+            launch_stream_bits<kF, Same, 8>(s, a);
+        else
+            launch_stream_bits<kF, Same, 2>(s, a);
+    }
     return hipGetLastError();
 }
 
 }  // namespace
 
 bool gemv_streams(const GemvArgs& a) {
-    return a.dtype != CQ_F32 && a.bits == 4 && a.block_rows == 1 && a.block_cols == 32 && a.param_dtype == CQ_F32 &&
-           a.cols % 32 == 0 && a.cols / 32 <= 64u * kStreamMaxStrips && a.word_pitch % 4 == 0 && a.x_aligned16 &&
-           a.words_aligned16 && a.scale_stride_row < (1ull << 32) && (a.cols / 32) * a.scale_stride_col < (1ull << 30);
+    if (a.dtype == CQ_F32 || (a.bits != 2 && a.bits != 4 && a.bits != 8) || a.block_rows != 1) return false;
+    const uint32_t vals = 128 / a.bits;  // values of a 16-byte unit
+    const uint32_t units_per_block = a.block_cols / vals;
+    return a.block_cols % vals == 0 && (units_per_block & (units_per_block - 1)) == 0 && a.cols % a.block_cols == 0 &&
+           (a.param_dtype == CQ_F32 || a.param_dtype == a.dtype) && a.cols <= kStreamMaxColumns && a.word_pitch % 4 == 0 &&
+           a.x_aligned16 && a.words_aligned16 && a.scale_stride_row < (1ull << 32) &&
+           (a.cols / a.block_cols) * a.scale_stride_col < (1ull << 29);
 }
 
 hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a) {
     if (a.rows == 0 || a.cols == 0) return hipSuccess;
-    if (gemv_streams(a)) return a.dtype == CQ_BF16 ? launch_stream<dev::Float::BF16>(s, a) : launch_stream<dev::Float::F16>(s, a);
+    if (gemv_streams(a))
+        return a.dtype == CQ_BF16 ? launch_stream<dev::Float::BF16, __bf16>(s, a) : launch_stream<dev::Float::F16, _Float16>(s, a);
     // the N-D layout of the [rows, cols] matrix, as the reference's scales_layout builds it
     dev::ScalesLayout layout;
     if (a.block_rows != 0) {

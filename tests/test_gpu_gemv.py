@@ -12,7 +12,7 @@ from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantParam, QuantSch
 pytestmark = pytest.mark.gpu
 
 CASES = [
-    # elem, value, block, param, rows, cols, word pitch (None: contiguous)     -- first nine: the streaming kernel
+    # elem, value, block, param, rows, cols, word pitch (None: contiguous)     -- the streaming kernel unless noted
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 1000, 4096, None),
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 77, 2048, None),
     (ElemType.BF16, QuantValue.E2M1, [32], QuantParam.F32, 130, 11008, None),     # last strip partly idle
@@ -22,10 +22,17 @@ CASES = [
     (ElemType.F16, QuantValue.Q4S, [32], QuantParam.F32, 21, 16480, None),        # eight waves per workgroup
     (ElemType.BF16, QuantValue.Q4F, [32], QuantParam.F32, 1, 32768, None),        # one row, the longest it takes
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 9, 32, None),           # one block per row
-    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.BF16, 100, 1024, None),      # general kernel from here on
+    (ElemType.F16, QuantValue.Q4S, [128], QuantParam.F16, 33, 4224, None),        # four units under one f16 scale
+    (ElemType.BF16, QuantValue.Q8S, [32], QuantParam.F32, 45, 2080, None),        # 8-bit codes, two units per block
+    (ElemType.BF16, QuantValue.Q4F, [64], QuantParam.BF16, 19, 16448, 2060),      # bf16 scales, eight waves, pitched
+    (ElemType.F16, QuantValue.Q8F, [16], QuantParam.F32, 70, 1040, None),         # 8-bit codes, a scale per unit
+    (ElemType.BF16, QuantValue.Q2S, [64], QuantParam.F32, 52, 4160, None),        # 2-bit codes
+    (ElemType.F16, QuantValue.Q2F, [128], QuantParam.F16, 17, 8192, None),        # 2-bit codes, two units per block
+    (ElemType.BF16, QuantValue.Q4S, [128], QuantParam.F16, 12, 1024, None),       # scales typed unlike x: general kernel
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.BF16, 100, 1024, None),
     (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, 50, 512, None),
-    (ElemType.F32, QuantValue.Q2S, [64], QuantParam.F32, 96, 1024, None),
-    (ElemType.F32, QuantValue.Q8F, None, QuantParam.F32, 33, 260, None),          # per tensor
+    (ElemType.F32, QuantValue.Q2S, [64], QuantParam.F32, 96, 1024, None),          # general kernel: f32 x,
+    (ElemType.F32, QuantValue.Q8F, None, QuantParam.F32, 33, 260, None),          # per tensor,
     (ElemType.BF16, QuantValue.Q4S, [4, 16], QuantParam.F32, 64, 256, None),      # blocks over both dimensions
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 40, 1056, None),        # cols not a multiple of 64 blocks
 ]
