@@ -126,7 +126,7 @@ FAMILY_NONE, FAMILY_FLAT, FAMILY_FLAT_ROWS, FAMILY_FLAT_LANES, FAMILY_ROWS, FAMI
     FAMILY_PER_ELEMENT = range(8)
 FAMILY_NAMES = ("none", "flat", "flat_rows", "flat_lanes", "rows", "blocks", "transposed", "per_element")
 #: enum cq_op
-OP_QUANTIZE, OP_QUANTIZE_DYNAMIC, OP_DEQUANTIZE, OP_COMPUTE_SCALES = range(4)
+OP_QUANTIZE, OP_QUANTIZE_DYNAMIC, OP_DEQUANTIZE, OP_COMPUTE_SCALES, OP_GEMV = range(5)
 
 
 def plan_kind(op: int, floats, values, scale, out_scale, scheme, elem) -> str:

@@ -1233,7 +1233,7 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
     a.word_pitch = values->strides[0];
     a.x_aligned16 = aligned(x->ptr, 16);
     a.words_aligned16 = aligned(values->ptr, 16);
-    return hip_status(cq::launch_gemv_quantized(stream, a));
+    return CQ_RUN(cq::gemv_streams(a) ? CQ_FAMILY_FLAT : CQ_FAMILY_ROWS, cq::launch_gemv_quantized(stream, a));
 }
 
 cq_status cq_plan_kind(cq_op op, const cq_tensor* floats, const cq_tensor* values, const cq_tensor* scale,
@@ -1253,6 +1253,10 @@ cq_status cq_plan_kind(cq_op op, const cq_tensor* floats, const cq_tensor* value
         case CQ_OP_DEQUANTIZE: st = cq_dequantize(nullptr, values, floats, scale, scheme, dtype); break;
         case CQ_OP_COMPUTE_SCALES:
             st = cq_compute_scales(nullptr, floats, scale, scheme, dtype, workspace, sizeof(workspace));
+            break;
+        case CQ_OP_GEMV:
+            st = cq_gemv_quantized(nullptr, values, scale, scheme, floats, out_scale, dtype,
+                                   out_scale && out_scale->elem_size == 4 ? CQ_F32 : dtype);
             break;
     }
     *family = g_probe.main != CQ_FAMILY_NONE ? g_probe.main : g_probe.aux;

@@ -80,7 +80,8 @@ __device__ __forceinline__ void store_y(int dtype, void* y, uint64_t i, float v)
 
 // ---- streaming kernel: 16-bit float types, blocks along the row ---------------------------------------
 // A lane's unit is one 16-byte load of codes: four words, 64 values of 2 bits, 32 of 4 or 16 of 8, under one scale
-// (blocks of 1, 2, 4, ... units).  A wave owns kRows rows and walks along them, strip by strip (64 units, a lane
+// (blocks of 1, 2, 4, ... units along the row and any number of rows, or one scale for the tensor: a shift of 31
+// and strides of 0).  A wave owns kRows rows and walks along them, strip by strip (64 units, a lane
 // per unit), so every wave of a launch does the same work whatever the number of strips, and the row sums never
 // leave the wave: six DPP additions per row at its end, no exchange between waves, no barrier after the first.
 // (With a wave per strip and the strips of a row in one workgroup, 5 to 8 strips all took the time of 8: the
@@ -94,8 +95,8 @@ __device__ __forceinline__ void store_y(int dtype, void* y, uint64_t i, float v)
 template <dev::Float kF, class FS, int kBits, int kRows, int kWaves, int kDepth>
 __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     const uint32_t* __restrict__ words, const FS* __restrict__ scales, const void* __restrict__ x, void* __restrict__ y,
-    int y_dtype, uint32_t rows, uint32_t units_per_row, uint32_t units_per_block_log2, uint64_t word_pitch,
-    uint32_t scale_stride_row, uint32_t scale_stride_col) {
+    int y_dtype, uint32_t rows, uint32_t units_per_row, uint32_t units_per_block_log2, uint32_t block_rows,
+    uint64_t word_pitch, uint32_t scale_stride_row, uint32_t scale_stride_col) {
     constexpr uint32_t kVals = 128 / kBits;         // values of a unit
     constexpr uint32_t kPairs = kVals / 2;          // ... as packed pairs of x
     constexpr uint32_t kVecs = kPairs / 4;          // ... as 16-byte pieces of x
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     for (int k = 0; k < kRows; k++) {
         const uint32_t r = row0 + min(static_cast<uint32_t>(k), nrows - 1u);
         wrow[k] = reinterpret_cast<const char*>(words + static_cast<uint64_t>(r) * word_pitch);
-        srow[k] = reinterpret_cast<const char*>(scales + static_cast<uint64_t>(r) * scale_stride_row);
+        srow[k] = reinterpret_cast<const char*>(scales + static_cast<uint64_t>(r / block_rows) * scale_stride_row);
     }
     const uint32_t scale_step = scale_stride_col * static_cast<uint32_t>(sizeof(FS));
     const auto load = [&](Chunk& c, uint32_t strip) {
@@ -287,8 +288,9 @@ void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
     const dim3 grid((a.rows + kStreamRows * kWaves - 1) / (kStreamRows * kWaves)), block(64 * kWaves);
     hipLaunchKernelGGL((gemv_stream_kernel<kF, FS, kBits, kStreamRows, kWaves, kStreamDepth>), grid, block,
                        strips * 64 * kVals * 2, s, static_cast<const uint32_t*>(a.words), static_cast<const FS*>(a.scales), a.x,
-                       a.y, a.y_dtype, a.rows, units_per_row, log2_of(a.block_cols / kVals), a.word_pitch,
-                       static_cast<uint32_t>(a.scale_stride_row), static_cast<uint32_t>(a.scale_stride_col));
+                       a.y, a.y_dtype, a.rows, units_per_row, a.block_rows == 0 ? 31u : log2_of(a.block_cols / kVals),
+                       a.block_rows == 0 ? 1u : a.block_rows, a.word_pitch, static_cast<uint32_t>(a.scale_stride_row),
+                       static_cast<uint32_t>(a.scale_stride_col));
 }
 
 // Two rows per wave, two strips in flight, four waves (eight rows) per workgroup; eight waves from 16384 columns
@@ -329,13 +331,16 @@ hipError_t launch_stream(hipStream_t s, const GemvArgs& a) {
 }  // namespace
 
 bool gemv_streams(const GemvArgs& a) {
-    if (a.dtype == CQ_F32 || (a.bits != 2 && a.bits != 4 && a.bits != 8) || a.block_rows != 1) return false;
+    if (a.dtype == CQ_F32 || (a.bits != 2 && a.bits != 4 && a.bits != 8)) return false;
     const uint32_t vals = 128 / a.bits;  // values of a 16-byte unit
-    const uint32_t units_per_block = a.block_cols / vals;
-    return a.block_cols % vals == 0 && (units_per_block & (units_per_block - 1)) == 0 && a.cols % a.block_cols == 0 &&
-           (a.param_dtype == CQ_F32 || a.param_dtype == a.dtype) && a.cols <= kStreamMaxColumns && a.word_pitch % 4 == 0 &&
-           a.x_aligned16 && a.words_aligned16 && a.scale_stride_row < (1ull << 32) &&
-           (a.cols / a.block_cols) * a.scale_stride_col < (1ull << 29);
+    if (a.block_rows != 0) {             // blocks: whole units along the row, a power of two of them
+        const uint32_t units_per_block = a.block_cols / vals;
+        if (a.block_cols % vals != 0 || (units_per_block & (units_per_block - 1)) != 0 || a.cols % a.block_cols != 0 ||
+            a.scale_stride_row >= (1ull << 32) || (a.cols / a.block_cols) * a.scale_stride_col >= (1ull << 29))
+            return false;
+    }
+    return a.cols % vals == 0 && (a.param_dtype == CQ_F32 || a.param_dtype == a.dtype) &&
+           a.cols <= kStreamMaxColumns && a.word_pitch % 4 == 0 && a.x_aligned16 && a.words_aligned16;
 }
 
 hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a) {

@@ -266,7 +266,10 @@ typedef enum cq_op {
     CQ_OP_QUANTIZE = 0,          /* cq_quantize: scale and out_scale given                    */
     CQ_OP_QUANTIZE_DYNAMIC = 1,  /* cq_quantize_dynamic: `scale` ignored (may be NULL)        */
     CQ_OP_DEQUANTIZE = 2,        /* cq_dequantize: `scale` = params, `out_scale` ignored      */
-    CQ_OP_COMPUTE_SCALES = 3     /* cq_compute_scales: `values` and `out_scale` ignored       */
+    CQ_OP_COMPUTE_SCALES = 3,    /* cq_compute_scales: `values` and `out_scale` ignored       */
+    CQ_OP_GEMV = 4               /* cq_gemv_quantized: `floats` = x, `scale` = params, `out_scale` = y (typed `dtype`
+                                    or f32): CQ_FAMILY_FLAT for its streaming kernel, CQ_FAMILY_ROWS for the
+                                    general one (a wave per row, about a third of the rate)  */
 } cq_op;
 
 /* The family of the kernel that would move the value tensors of the call (for CQ_OP_COMPUTE_SCALES: that

@@ -33,7 +33,11 @@ CASES = [
     (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, 50, 512, None),
     (ElemType.F32, QuantValue.Q2S, [64], QuantParam.F32, 96, 1024, None),          # general kernel: f32 x,
     (ElemType.F32, QuantValue.Q8F, None, QuantParam.F32, 33, 260, None),          # per tensor,
-    (ElemType.BF16, QuantValue.Q4S, [4, 16], QuantParam.F32, 64, 256, None),      # blocks over both dimensions
+    (ElemType.BF16, QuantValue.Q4S, [4, 16], QuantParam.F32, 64, 256, None),      # blocks narrower than a unit
+    (ElemType.BF16, QuantValue.Q8S, None, QuantParam.F32, 29, 2064, None),        # streaming again: one scale per tensor
+    (ElemType.F16, QuantValue.Q4F, None, QuantParam.F16, 11, 4128, None),
+    (ElemType.BF16, QuantValue.Q4S, [6, 64], QuantParam.F32, 66, 4160, None),     # blocks of six rows
+    (ElemType.F16, QuantValue.Q8S, [128, 128], QuantParam.F32, 256, 1024, None),  # 128 x 128 weight blocks
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 40, 1056, None),        # cols not a multiple of 64 blocks
 ]
 

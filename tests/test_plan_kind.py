@@ -92,6 +92,39 @@ def test_layouts_land_on_the_family_the_design_claims():
     assert got == {"quantize": "rows", "dequantize": "rows"}
 
 
+def gemv_kind(scheme, elem, rows, cols, pitch=None, s_strides=None, x_offset=0):
+    esz = 4 if elem == F32 else 2
+    wpr = cols // scheme.num_quants()
+    values = t((rows, wpr), 4, (pitch or wpr, 1), 0, 1)
+    sshape = scheme.scales_shape((rows, cols))
+    params = t(sshape, 4 if scheme.param == QuantParam.F32 else 2, s_strides, 0, 3)
+    return _ffi.plan_kind(_ffi.OP_GEMV, t((cols,), esz, None, x_offset, 0), values, params, t((rows,), esz, None, 0, 2), scheme, elem)
+
+
+def test_matrix_vector_products_that_stream():
+    F16 = ElemType.F16
+    # configuration 3's weights and the other shapes of the benchmark
+    for rows, cols in ((14336, 4096), (4096, 14336), (28672, 8192), (4096, 11008), (8192, 28672)):
+        assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, rows, cols) == "flat", (rows, cols)
+    # 2-, 4- and 8-bit codes, larger blocks, scales typed like x, blocks over rows, one scale per tensor, pitched rows
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [128], param=QuantParam.F16), F16, 4096, 4096) == "flat"
+    assert gemv_kind(scheme_of(QuantValue.Q4F, [64], param=QuantParam.BF16), BF16, 4096, 4096, pitch=520) == "flat"
+    assert gemv_kind(scheme_of(QuantValue.Q8S, [16]), BF16, 100, 2064) == "flat"
+    assert gemv_kind(scheme_of(QuantValue.Q2S, [64]), F16, 100, 4160) == "flat"
+    assert gemv_kind(scheme_of(QuantValue.Q8S, [128, 128]), BF16, 256, 1024) == "flat"
+    assert gemv_kind(scheme_of(QuantValue.Q4S, None), BF16, 64, 32768) == "flat"
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 4096, s_strides=(1, 64)) == "flat"
+    # the general kernel: f32 x, scales typed unlike x, blocks narrower than 16 bytes of codes or not a power of two
+    # of them, more than 32768 columns, words or x off 16-byte boundaries
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), F32, 64, 4096) == "rows"
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [32], param=QuantParam.F16), BF16, 64, 4096) == "rows"
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [16]), BF16, 64, 4096) == "rows"
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [96]), BF16, 64, 4032) == "rows"
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 32800) == "rows"
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 4096, pitch=513) == "rows"
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 4096, x_offset=2) == "rows"
+
+
 def test_slow_paths_are_reported():
     e2m1 = scheme_of(QuantValue.E2M1, [32])
     # rows that start on odd multiples of 2 bytes
