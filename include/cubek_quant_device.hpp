@@ -279,19 +279,23 @@ __device__ __forceinline__ void dequantize_symmetric_packed_value_pairs_tame(uin
             out[2] = pack_pair<kF>(__builtin_fmaf(e23[0], s512, nbs), __builtin_fmaf(o23[0], s512, nbs));
             out[3] = pack_pair<kF>(__builtin_fmaf(e23[1], s512, nbs), __builtin_fmaf(o23[1], s512, nbs));
         } else {
-            // field j of every byte, j = 0..3: byte b of (digits >> 2j) & 0x03030303 is value 4b + j
-            uint32_t plane[4];
+            // field j of every byte, j = 0..3: byte b of ((word >> 2j) & 0x03030303) ^ 0x02020202 is the digit of
+            // value 4b + j, and as an e4m3 number it is digit * 2^-9 like the nibbles above
+            typedef float f32x2 __attribute__((ext_vector_type(2)));
+            const float s512 = s * 512.0f;  // exact: s < 2^100
+            f32x2 lo[4], hi[4];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                plane[j] = (digits >> (2 * j)) & 0x03030303u;
-                asm("" : "+v"(plane[j]));  // as above: one conversion instruction per byte
+                const uint32_t plane = ((word >> (2 * j)) & 0x03030303u) ^ 0x02020202u;
+                lo[j] = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(plane), false);
+                hi[j] = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(plane), true);
             }
 #pragma unroll
             for (int b = 0; b < 4; b++) {
-                const float v0 = __builtin_fmaf(static_cast<float>((plane[0] >> (8 * b)) & 0xffu), s, nbs);
-                const float v1 = __builtin_fmaf(static_cast<float>((plane[1] >> (8 * b)) & 0xffu), s, nbs);
-                const float v2 = __builtin_fmaf(static_cast<float>((plane[2] >> (8 * b)) & 0xffu), s, nbs);
-                const float v3 = __builtin_fmaf(static_cast<float>((plane[3] >> (8 * b)) & 0xffu), s, nbs);
+                const float v0 = __builtin_fmaf(b < 2 ? lo[0][b & 1] : hi[0][b & 1], s512, nbs);
+                const float v1 = __builtin_fmaf(b < 2 ? lo[1][b & 1] : hi[1][b & 1], s512, nbs);
+                const float v2 = __builtin_fmaf(b < 2 ? lo[2][b & 1] : hi[2][b & 1], s512, nbs);
+                const float v3 = __builtin_fmaf(b < 2 ? lo[3][b & 1] : hi[3][b & 1], s512, nbs);
                 out[2 * b] = pack_pair<kF>(v0, v1);
                 out[2 * b + 1] = pack_pair<kF>(v2, v3);
             }
