@@ -80,8 +80,8 @@ __device__ __forceinline__ void store_y(int dtype, void* y, uint64_t i, float v)
 
 // ---- streaming kernel: 16-bit float types, blocks along the row ---------------------------------------
 // A lane's unit is one 16-byte load of codes: four words, 64 values of 2 bits, 32 of 4 or 16 of 8, under one scale
-// (blocks of 1, 2, 4, ... units along the row and any number of rows, or one scale for the tensor: a shift of 31
-// and strides of 0).  A wave owns kRows rows and walks along them, strip by strip (64 units, a lane
+// (f32, f16 or bf16; blocks of 1, 2, 4, ... units along the row and any number of rows, or one scale for the
+// tensor: a shift of 31 and strides of 0).  A wave owns kRows rows and walks along them, strip by strip (64 units, a lane
 // per unit), so every wave of a launch does the same work whatever the number of strips, and the row sums never
 // leave the wave: six DPP additions per row at its end, no exchange between waves, no barrier after the first.
 // (With a wave per strip and the strips of a row in one workgroup, 5 to 8 strips all took the time of 8: the
@@ -307,23 +307,22 @@ void launch_stream_bits(hipStream_t s, const GemvArgs& a) {
         launch_stream_waves<kF, FS, kBits, 4>(s, a);
 }
 
-// scales typed f32 or like x
-template <dev::Float kF, class Same>
+template <dev::Float kF, class FS>
+void launch_stream_scales(hipStream_t s, const GemvArgs& a) {
+    if (a.bits == 4)
+        launch_stream_bits<kF, FS, 4>(s, a);
+    else if (a.bits == 8)
+        launch_stream_bits<kF, FS, 8>(s, a);
+    else
+        launch_stream_bits<kF, FS, 2>(s, a);
+}
+
+template <dev::Float kF>
 hipError_t launch_stream(hipStream_t s, const GemvArgs& a) {
-    if (a.param_dtype == CQ_F32) {
-        if (a.bits == 4)
-            launch_stream_bits<kF, float, 4>(s, a);
-        else if (a.bits == 8)
-            launch_stream_bits<kF, float, 8>(s, a);
-        else
-            launch_stream_bits<kF, float, 2>(s, a);
-    } else {
-        if (a.bits == 4)
-            launch_stream_bits<kF, Same, 4>(s, a);
-        else if (a.bits == 8)
-            launch_stream_bits<kF, Same, 8>(s, a);
-        else
-            launch_stream_bits<kF, Same, 2>(s, a);
+    switch (a.param_dtype) {
+        case CQ_F32: launch_stream_scales<kF, float>(s, a); break;
+        case CQ_F16: launch_stream_scales<kF, _Float16>(s, a); break;
+        default: launch_stream_scales<kF, __bf16>(s, a); break;
     }
     return hipGetLastError();
 }
@@ -339,14 +338,14 @@ bool gemv_streams(const GemvArgs& a) {
             a.scale_stride_row >= (1ull << 32) || (a.cols / a.block_cols) * a.scale_stride_col >= (1ull << 29))
             return false;
     }
-    return a.cols % vals == 0 && (a.param_dtype == CQ_F32 || a.param_dtype == a.dtype) &&
+    return a.cols % vals == 0 &&
            a.cols <= kStreamMaxColumns && a.word_pitch % 4 == 0 && a.x_aligned16 && a.words_aligned16;
 }
 
 hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a) {
     if (a.rows == 0 || a.cols == 0) return hipSuccess;
     if (gemv_streams(a))
-        return a.dtype == CQ_BF16 ? launch_stream<dev::Float::BF16, __bf16>(s, a) : launch_stream<dev::Float::F16, _Float16>(s, a);
+        return a.dtype == CQ_BF16 ? launch_stream<dev::Float::BF16>(s, a) : launch_stream<dev::Float::F16>(s, a);
     // the N-D layout of the [rows, cols] matrix, as the reference's scales_layout builds it
     dev::ScalesLayout layout;
     if (a.block_rows != 0) {

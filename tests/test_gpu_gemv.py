@@ -28,7 +28,8 @@ CASES = [
     (ElemType.F16, QuantValue.Q8F, [16], QuantParam.F32, 70, 1040, None),         # 8-bit codes, a scale per unit
     (ElemType.BF16, QuantValue.Q2S, [64], QuantParam.F32, 52, 4160, None),        # 2-bit codes
     (ElemType.F16, QuantValue.Q2F, [128], QuantParam.F16, 17, 8192, None),        # 2-bit codes, two units per block
-    (ElemType.BF16, QuantValue.Q4S, [128], QuantParam.F16, 12, 1024, None),       # scales typed unlike x: general kernel
+    (ElemType.BF16, QuantValue.Q4S, [128], QuantParam.F16, 12, 1024, None),       # f16 scales under bf16 x
+    (ElemType.F16, QuantValue.Q8S, [64], QuantParam.BF16, 31, 2112, None),        # bf16 scales under f16 x
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.BF16, 100, 1024, None),
     (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, 50, 512, None),
     (ElemType.F32, QuantValue.Q2S, [64], QuantParam.F32, 96, 1024, None),          # general kernel: f32 x,
