@@ -49,14 +49,13 @@ def _id(c):
         ("-pitched" if pitch else "")
 
 
-@pytest.mark.parametrize("case", CASES, ids=_id)
-def test_gemv_matches_oracle_dequantized_weights(oracle, case):
+def check_case(oracle, case, seed):
     import torch
 
     elem, value, block, param, rows, cols, pitch = case
     level = QuantLevel.Tensor if block is None else QuantLevel.block(block)
     scheme = QuantScheme.default().with_value(value).with_level(level).with_param(param)
-    rng = np.random.default_rng(rows * 7 + cols)
+    rng = np.random.default_rng(seed)
     w32 = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
     w32[rng.random((rows, cols)) < 0.002] *= 20
     wb = oracle.to_bits(w32, elem)
@@ -87,13 +86,51 @@ def test_gemv_matches_oracle_dequantized_weights(oracle, case):
                       elem, ElemType.F32)
     torch.cuda.synchronize()
     got = y32.cpu().numpy().astype(np.float64)
-    assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), float(np.max(np.abs(got - want) / (mag + 1e-30)))
+    assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), (case, float(np.max(np.abs(got - want) / (mag + 1e-30))))
     if elem != ElemType.F32:  # the same sums, rounded once to the 16-bit type
         y16 = torch.zeros((rows,), dtype=torch.int16, device="cuda")
         matvec.launch_ref(client, h_words, h_scales, scheme, TensorHandleRef.from_torch(d_x),
                           TensorHandleRef.from_torch(y16), elem, elem)
         torch.cuda.synchronize()
-        assert np.array_equal(y16.cpu().numpy().view(np.uint16), oracle.to_bits(y32.cpu().numpy(), elem))
+        assert np.array_equal(y16.cpu().numpy().view(np.uint16), oracle.to_bits(y32.cpu().numpy(), elem)), case
+
+
+@pytest.mark.parametrize("case", CASES, ids=_id)
+def test_gemv_matches_oracle_dequantized_weights(oracle, case):
+    elem, value, block, param, rows, cols, pitch = case
+    check_case(oracle, case, rows * 7 + cols)
+
+
+def test_gemv_random_configurations(oracle):
+    """Sixty drawn cases of the streaming kernel's domain and its edges: every code width, block extents from one
+    16-byte unit up (also over rows), one scale per tensor, every scale type, ragged strips, pitched words."""
+    rng = np.random.default_rng(2024)
+    values = {2: [QuantValue.Q2S, QuantValue.Q2F], 4: [QuantValue.Q4S, QuantValue.Q4F, QuantValue.E2M1],
+              8: [QuantValue.Q8S, QuantValue.Q8F]}
+    for i in range(60):
+        bits = int(rng.choice([2, 4, 8]))
+        unit = 128 // bits
+        elem = [ElemType.BF16, ElemType.F16][int(rng.integers(2))]
+        param = [QuantParam.F32, QuantParam.F16, QuantParam.BF16][int(rng.integers(3))]
+        kind = int(rng.integers(4))
+        units_per_block = int(2 ** rng.integers(0, 3))
+        bc = unit * units_per_block
+        if bc > 255:  # block extents are bytes in the scheme
+            bc, units_per_block = unit, 1
+        blocks = int(rng.integers(1, max(2, 6000 // bc)))
+        cols = bc * blocks
+        rows = int(rng.integers(1, 70))
+        block = [bc]
+        if kind == 0:
+            block = None
+        elif kind == 1:
+            br = int(rng.choice([2, 3, 5]))
+            rows = br * int(rng.integers(1, 20))
+            block = [br, bc]
+        value = values[bits][int(rng.integers(len(values[bits])))]
+        wpr = cols // (32 // bits)
+        pitch = None if rng.random() < 0.6 else wpr + 4 * int(rng.integers(1, 5))
+        check_case(oracle, (elem, value, block, param, rows, cols, pitch), 1000 + i)
 
 
 @pytest.mark.parametrize("elem", [ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
