@@ -1190,16 +1190,21 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
     drop_stale_hip_error();
     cq_status st = check_scheme(scheme);
     if (st != CQ_OK) return st;
-    if (scheme->store != CQ_STORE_U32) return CQ_ERR_UNSUPPORTED_SCHEME;
+    const bool native = scheme->store == CQ_STORE_NATIVE;
+    // the native store holds i8, e4m3, e5m2 bytes or e2m1 pairs (src/quantize.rs:196-219)
+    if (native && scheme->value != CQ_VALUE_Q8F && scheme->value != CQ_VALUE_Q8S && scheme->value != CQ_VALUE_E4M3 &&
+        scheme->value != CQ_VALUE_E5M2 && scheme->value != CQ_VALUE_E2M1)
+        return CQ_ERR_UNSUPPORTED_SCHEME;
     if (!tensor_ok(values) || !tensor_ok(params) || !tensor_ok(x) || !tensor_ok(y) || !valid_dtype(dtype) ||
         !valid_dtype(y_dtype))
         return CQ_ERR_INVALID_ARGUMENT;
     const int pd = param_to_dtype(scheme->param);
     if (values->rank != 2 || x->rank != 1 || y->rank != 1) return CQ_ERR_SHAPE_MISMATCH;
-    if (values->elem_size != 4 || x->elem_size != dtype_size(dtype) || y->elem_size != dtype_size(y_dtype) ||
+    if (values->elem_size != (native ? 1u : 4u) || x->elem_size != dtype_size(dtype) || y->elem_size != dtype_size(y_dtype) ||
         params->elem_size != dtype_size(pd))
         return CQ_ERR_SHAPE_MISMATCH;
-    const uint32_t bits = value_bits(scheme->value), nq = 32u / bits;
+    const uint32_t bits = value_bits(scheme->value);
+    const uint32_t nq = native ? (scheme->value == CQ_VALUE_E2M1 ? 2u : 1u) : 32u / bits;  // values per stored element
     const uint64_t rows = values->shape[0], cols = values->shape[1] * nq;
     if (rows > 0xffffffffull || cols > 0xffffffffull) return CQ_ERR_TOO_LARGE;
     if (x->shape[0] != cols || y->shape[0] != rows) return CQ_ERR_SHAPE_MISMATCH;
@@ -1233,6 +1238,13 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
     a.word_pitch = values->strides[0];
     a.x_aligned16 = aligned(x->ptr, 16);
     a.words_aligned16 = aligned(values->ptr, 16);
+    if (native) {
+        // only the streaming kernel reads the native store: rows of whole 16-byte units on 16-byte boundaries
+        a.native = scheme->value == CQ_VALUE_E4M3 ? 1u : scheme->value == CQ_VALUE_E5M2 ? 2u : scheme->value == CQ_VALUE_E2M1 ? 3u : 0u;
+        if (values->strides[0] % 16 != 0 && rows > 1) return CQ_ERR_UNSUPPORTED_SCHEME;
+        a.word_pitch = values->strides[0] / 4;
+        if (!cq::gemv_streams(a)) return CQ_ERR_UNSUPPORTED_SCHEME;
+    }
     return CQ_RUN(cq::gemv_streams(a) ? CQ_FAMILY_FLAT : CQ_FAMILY_ROWS, cq::launch_gemv_quantized(stream, a));
 }
 

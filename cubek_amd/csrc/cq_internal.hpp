@@ -220,6 +220,7 @@ struct GemvArgs {
     void* y;             // [rows], typed y_dtype
     int dtype, y_dtype, param_dtype;
     uint32_t bits;       // bits per value
+    uint32_t native;     // 0: fields of the U32 store (and i8 bytes); 1 e4m3, 2 e5m2, 3 e2m1x2 of the native store
     uint32_t rows, cols;
     uint64_t word_pitch;
     uint32_t block_rows, block_cols;  // 0, 0: one scale per tensor

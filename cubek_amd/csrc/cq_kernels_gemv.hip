@@ -92,15 +92,23 @@ __device__ __forceinline__ void store_y(int dtype, void* y, uint64_t i, float v)
 // address instead of nothing, so that the number of loads in flight is the same in every iteration and the
 // compiler can count its waits.  Per 4-bit value: half a byte-to-float conversion and one FMA
 // (dequantize_symmetric_packed_value_pairs), half a v_cvt_pk, half a v_dot2.
-template <dev::Float kF, class FS, int kBits, int kRows, int kWaves, int kDepth>
+// kCode: 2, 4 or 8 for fields of that many bits in the U32 store (and the i8 bytes of the native store, which are
+// the same bits), or one of the native encodings below.
+constexpr int kCodeE4M3 = 100, kCodeE5M2 = 101, kCodeE2M1x2 = 102;
+
+template <dev::Float kF, class FS, int kCode, int kRows, int kWaves, int kDepth>
 __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     const uint32_t* __restrict__ words, const FS* __restrict__ scales, const void* __restrict__ x, void* __restrict__ y,
     int y_dtype, uint32_t rows, uint32_t units_per_row, uint32_t units_per_block_log2, uint32_t block_rows,
     uint64_t word_pitch, uint32_t scale_stride_row, uint32_t scale_stride_col) {
-    constexpr uint32_t kVals = 128 / kBits;         // values of a unit
+    constexpr bool kPacked = kCode <= 8;
+    constexpr int kBits = kPacked ? kCode : 8;      // (of the packed fields)
+    constexpr uint32_t kVals = kPacked ? 128 / kBits : (kCode == kCodeE2M1x2 ? 32 : 16);  // values of a unit
     constexpr uint32_t kPairs = kVals / 2;          // ... as packed pairs of x
     constexpr uint32_t kVecs = kPairs / 4;          // ... as 16-byte pieces of x
-    constexpr uint32_t kWordPairs = 16 / kBits;     // pairs out of one word
+    constexpr uint32_t kWordPairs = kVals / 8;      // pairs out of one word
+    constexpr dev::Native kNative = kCode == kCodeE4M3 ? dev::Native::E4M3
+                                    : kCode == kCodeE5M2 ? dev::Native::E5M2 : dev::Native::E2M1x2;
     extern __shared__ u32x4 xs[];  // x, kVecs pieces per unit, whole strips
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -141,7 +149,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     // is not tame come here.
     const auto plain_row = [&](int k, uint32_t strip) {
         const uint32_t u = strip * 64u + lane;
-        if (u >= units_per_row) return 0.0f;
+        if (!kPacked || u >= units_per_row) return 0.0f;
         const uint32_t* wr = reinterpret_cast<const uint32_t*>(wrow[k]) + u * 4u;
         const FS scale = *reinterpret_cast<const FS*>(srow[k] + (u >> units_per_block_log2) * scale_step);
         const typename Elem<kF>::T* xr = static_cast<const typename Elem<kF>::T*>(x) + u * kVals;
@@ -171,26 +179,42 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
             const u32x4 v = xs[(strip * 64u + lane) * kVecs + j];
             xp[4 * j] = v[0], xp[4 * j + 1] = v[1], xp[4 * j + 2] = v[2], xp[4 * j + 3] = v[3];
         }
-        bool tame = true;
         float part[kRows];
+        if constexpr (kPacked) {
+            bool tame = true;
 #pragma unroll
-        for (int k = 0; k < kRows; k++) {
-            float a = 0.0f;
+            for (int k = 0; k < kRows; k++) {
+                float a = 0.0f;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                uint32_t pairs[kWordPairs];
-                dev::dequantize_symmetric_packed_value_pairs_tame<kF, kBits>(c.w[k][j], c.s[k], pairs);
+                for (int j = 0; j < 4; j++) {
+                    uint32_t pairs[kWordPairs];
+                    dev::dequantize_symmetric_packed_value_pairs_tame<kF, kBits>(c.w[k][j], c.s[k], pairs);
 #pragma unroll
-                for (uint32_t i = 0; i < kWordPairs; i++) a = dot2<kF>(pairs[i], xp[kWordPairs * j + i], a);
+                    for (uint32_t i = 0; i < kWordPairs; i++) a = dot2<kF>(pairs[i], xp[kWordPairs * j + i], a);
+                }
+                part[k] = a;
+                tame = tame && dev::pairs_scale_is_tame<kF>(c.s[k]);
             }
-            part[k] = a;
-            tame = tame && dev::pairs_scale_is_tame<kF>(c.s[k]);
-        }
-        // ordinary scales are all tame: one wave-uniform test per chunk, then straight on
-        if (__builtin_amdgcn_ballot_w64(!tame) != 0) {
+            // ordinary scales are all tame: one wave-uniform test per chunk, then straight on
+            if (__builtin_amdgcn_ballot_w64(!tame) != 0) {
 #pragma unroll
-            for (int k = 0; k < kRows; k++)
-                if (!dev::pairs_scale_is_tame<kF>(c.s[k])) part[k] = plain_row(k, strip);
+                for (int k = 0; k < kRows; k++)
+                    if (!dev::pairs_scale_is_tame<kF>(c.s[k])) part[k] = plain_row(k, strip);
+            }
+        } else {
+            // native encodings: the pairs are the plain arithmetic, every scale goes the same way
+#pragma unroll
+            for (int k = 0; k < kRows; k++) {
+                float a = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    uint32_t pairs[kWordPairs];
+                    dev::dequantize_symmetric_native_value_pairs<kF, kNative>(c.w[k][j], c.s[k], pairs);
+#pragma unroll
+                    for (uint32_t i = 0; i < kWordPairs; i++) a = dot2<kF>(pairs[i], xp[kWordPairs * j + i], a);
+                }
+                part[k] = a;
+            }
         }
 #pragma unroll
         for (int k = 0; k < kRows; k++) acc[k] += part[k];
@@ -281,9 +305,11 @@ uint32_t log2_of(uint32_t v) {
     return l;
 }
 
+constexpr uint32_t values_per_unit(int code) { return code <= 8 ? 128 / code : (code == kCodeE2M1x2 ? 32 : 16); }
+
 template <dev::Float kF, class FS, int kBits, int kWaves>
 void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
-    constexpr uint32_t kVals = 128 / kBits;
+    constexpr uint32_t kVals = values_per_unit(kBits);
     const uint32_t units_per_row = a.cols / kVals, strips = (units_per_row + 63) / 64;
     const dim3 grid((a.rows + kStreamRows * kWaves - 1) / (kStreamRows * kWaves)), block(64 * kWaves);
     hipLaunchKernelGGL((gemv_stream_kernel<kF, FS, kBits, kStreamRows, kWaves, kStreamDepth>), grid, block,
@@ -309,7 +335,13 @@ void launch_stream_bits(hipStream_t s, const GemvArgs& a) {
 
 template <dev::Float kF, class FS>
 void launch_stream_scales(hipStream_t s, const GemvArgs& a) {
-    if (a.bits == 4)
+    if (a.native == 1)
+        launch_stream_bits<kF, FS, kCodeE4M3>(s, a);
+    else if (a.native == 2)
+        launch_stream_bits<kF, FS, kCodeE5M2>(s, a);
+    else if (a.native == 3)
+        launch_stream_bits<kF, FS, kCodeE2M1x2>(s, a);
+    else if (a.bits == 4)
         launch_stream_bits<kF, FS, 4>(s, a);
     else if (a.bits == 8)
         launch_stream_bits<kF, FS, 8>(s, a);
@@ -331,7 +363,7 @@ hipError_t launch_stream(hipStream_t s, const GemvArgs& a) {
 
 bool gemv_streams(const GemvArgs& a) {
     if (a.dtype == CQ_F32 || (a.bits != 2 && a.bits != 4 && a.bits != 8)) return false;
-    const uint32_t vals = 128 / a.bits;  // values of a 16-byte unit
+    const uint32_t vals = 128 / a.bits;  // values of a 16-byte unit (native encodings come with their bits)
     if (a.block_rows != 0) {             // blocks: whole units along the row, a power of two of them
         const uint32_t units_per_block = a.block_cols / vals;
         if (a.block_cols % vals != 0 || (units_per_block & (units_per_block - 1)) != 0 || a.cols % a.block_cols != 0 ||

@@ -232,14 +232,18 @@ cq_status cq_into_contiguous_packed(cq_stream_t stream, const cq_tensor* input, 
  * crates/cubek-matmul/src/base.rs:309-317; scale lookup per (row, col),
  * crates/cubek-matmul/src/components/global/memory/layout.rs:371-455), for the matrix-vector case.
  * The kernels are written against include/cubek_quant_device.hpp only.
- *   values : U32-store tensor [rows, cols / num_quants], rows may be pitched (stride 1 along the row)
+ *   values : U32-store tensor [rows, cols / num_quants] of words, or native-store tensor of bytes ([rows, cols]
+ *            for i8 / e4m3 / e5m2, [rows, cols / 2] for e2m1 pairs); rows may be pitched (stride 1 along the row)
  *   params : scales typed scheme->param, shape [1] (per tensor) or [rows / block_rows, cols / block_cols]
  *            for blocks over the last one or two dimensions, any strides
  *   x      : [cols] of `dtype`, contiguous;  y : [rows] of `y_dtype`, contiguous
  * Every weight enters as the value cq_dequantize would produce for `dtype`, F(F(scale) * F(code)); the
  * products are accumulated in f32 (order unspecified) and the sum is rounded once to `y_dtype`.
- * 4-bit codes with f32 scales on 1-D blocks of 32 and a 16-bit `dtype` stream at HBM rate; everything
- * else takes a simple wave-per-row kernel. */
+ * A streaming kernel (HBM- or arithmetic-bound, 45 - 70 % of the HBM peak on large weights) takes a 16-bit
+ * `dtype` with 16-byte aligned rows of codes and x, up to 32768 columns, scales of any type per tensor or on
+ * blocks of 1, 2, 4, ... times 16 bytes of codes along the row (any number of rows): cq_plan_kind(CQ_OP_GEMV)
+ * tells.  Every other U32-store layout takes a simple wave-per-row kernel; every other native-store layout is
+ * CQ_ERR_UNSUPPORTED_SCHEME. */
 cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const cq_tensor* params,
                             const cq_scheme* scheme, const cq_tensor* x, const cq_tensor* y,
                             cq_dtype dtype, cq_dtype y_dtype);

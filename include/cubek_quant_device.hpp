@@ -383,6 +383,42 @@ __device__ __forceinline__ void dequantize_symmetric_native_value(uint32_t word,
     for (int i = 0; i < kN; i++) out[i] = round_to<kF>(s * q[i]);  // F(q) is exact: every stored value fits kF
 }
 
+// dequantize_symmetric_native_value as packed pairs of a 16-bit kF, as they sit in memory: two values out of
+// 32 bits per conversion, one multiplication each (exact in f32: at most 8 significant bits times at most 11),
+// one rounding per pair.  The same operations as the plain function, so every scale is taken (negative, zero,
+// infinite, NaN).  I8 bytes are the 8-bit fields of the U32 store: dequantize_symmetric_packed_value_pairs<kF, 8>.
+template <Float kF, Native kNative, class FS>
+__device__ __forceinline__ void dequantize_symmetric_native_value_pairs(uint32_t word, FS scale, uint32_t* out) {
+    static_assert(kF != Float::F32, "pairs are for the 16-bit types");
+    static_assert(kNative != Native::I8, "I8 bytes: dequantize_symmetric_packed_value_pairs<kF, 8>");
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const float s = round_to<kF>(widen(scale));
+    constexpr int kPairs = native_values_per_word<kNative>() / 2;
+    f32x2 q[kPairs];
+    if constexpr (kNative == Native::E4M3) {
+        q[0] = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(word), false);
+        q[1] = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(word), true);
+    } else if constexpr (kNative == Native::E5M2) {
+        q[0] = __builtin_amdgcn_cvt_pk_f32_bf8(static_cast<int>(word), false);
+        q[1] = __builtin_amdgcn_cvt_pk_f32_bf8(static_cast<int>(word), true);
+    } else {
+        q[0] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0);
+        q[1] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1);
+        q[2] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2);
+        q[3] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3);
+    }
+#pragma unroll
+    for (int i = 0; i < kPairs; i++) {
+        float a = s * q[i][0], b = s * q[i][1];
+        if constexpr (kF == Float::F16) {
+            // pinned: fused with the conversion (v_fma_mixlo_f16, +0 addend) a negative zero product would turn +0
+            asm("" : "+v"(a));
+            asm("" : "+v"(b));
+        }
+        out[i] = pack_pair<kF>(a, b);
+    }
+}
+
 // 32 bits of a native tensor at `position` (in units of 32 bits), scaled by the scale of their first
 // element, as the reference's kernel scales a line (the last block extent must be a multiple of the
 // values per 32 bits).

@@ -6,8 +6,8 @@ bit against the f32 output)."""
 import numpy as np
 import pytest
 
-from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantParam, QuantScheme, QuantValue, TensorHandleRef,
-                       _ffi, matvec)
+from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantParam, QuantScheme, QuantStore, QuantValue,
+                       TensorHandleRef, _ffi, matvec)
 
 pytestmark = pytest.mark.gpu
 
@@ -49,12 +49,14 @@ def _id(c):
         ("-pitched" if pitch else "")
 
 
-def check_case(oracle, case, seed):
+def check_case(oracle, case, seed, native=False):
     import torch
 
     elem, value, block, param, rows, cols, pitch = case
     level = QuantLevel.Tensor if block is None else QuantLevel.block(block)
     scheme = QuantScheme.default().with_value(value).with_level(level).with_param(param)
+    if native:
+        scheme = scheme.with_store(QuantStore.Native)
     rng = np.random.default_rng(seed)
     w32 = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
     w32[rng.random((rows, cols)) < 0.002] *= 20
@@ -70,14 +72,14 @@ def check_case(oracle, case, seed):
     nq = scheme.num_quants()
     wpr = cols // nq
     pitch = pitch or wpr
-    buf = np.zeros((rows, pitch), np.uint32)
+    buf = np.zeros((rows, pitch), np.uint8 if native else np.uint32)  # native: stored elements are bytes
     buf[:, :wpr] = words.reshape(rows, wpr)
-    d_words = torch.from_numpy(buf.view(np.int32)).cuda()
+    d_words = torch.from_numpy(buf if native else buf.view(np.int32)).cuda()
     to16 = lambda a: torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda() if a.dtype == np.uint16 \
         else torch.from_numpy(np.ascontiguousarray(a)).cuda()
     d_scales, d_x = to16(out_scale), to16(xb)
     sshape = (1,) if block is None else tuple(d_scales.shape)
-    h_words = TensorHandleRef(d_words.data_ptr(), (rows, wpr), (pitch, 1), 4)
+    h_words = TensorHandleRef(d_words.data_ptr(), (rows, wpr), (pitch, 1), 1 if native else 4)
     h_scales = TensorHandleRef(d_scales.data_ptr(), sshape, tuple(d_scales.stride()) if block else (1,),
                                d_scales.element_size())
     client = ComputeClient.current()
@@ -99,6 +101,25 @@ def check_case(oracle, case, seed):
 def test_gemv_matches_oracle_dequantized_weights(oracle, case):
     elem, value, block, param, rows, cols, pitch = case
     check_case(oracle, case, rows * 7 + cols)
+
+
+NATIVE_CASES = [
+    # the native store: e4m3 / e5m2 / i8 bytes (16 values per 16-byte unit), e2m1 pairs (32 values)
+    (ElemType.BF16, QuantValue.E4M3, [32], QuantParam.F32, 77, 4128, None),
+    (ElemType.F16, QuantValue.E4M3, [128, 128], QuantParam.F32, 256, 2048, None),   # 128 x 128 weight blocks
+    (ElemType.BF16, QuantValue.E5M2, [16], QuantParam.BF16, 30, 2064, 2096),        # a scale per unit, pitched rows
+    (ElemType.F16, QuantValue.E5M2, None, QuantParam.F16, 21, 16400, None),         # per tensor, eight waves
+    (ElemType.BF16, QuantValue.E2M1, [32], QuantParam.F32, 53, 8448, None),         # e2m1 pairs, a scale per unit
+    (ElemType.F16, QuantValue.E2M1, [64], QuantParam.F16, 18, 1088, None),
+    (ElemType.BF16, QuantValue.Q8S, [32], QuantParam.F32, 45, 2080, None),          # i8 bytes: the 8-bit fields
+    (ElemType.F16, QuantValue.Q8F, [16], QuantParam.BF16, 9, 16, None),             # one unit per row
+]
+
+
+@pytest.mark.parametrize("case", NATIVE_CASES, ids=_id)
+def test_gemv_native_store_matches_oracle_dequantized_weights(oracle, case):
+    elem, value, block, param, rows, cols, pitch = case
+    check_case(oracle, case, rows * 11 + cols, native=True)
 
 
 def test_gemv_random_configurations(oracle):
