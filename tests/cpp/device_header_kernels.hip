@@ -51,6 +51,18 @@ __global__ void dequantize_native_kernel(const uint32_t* words, const FS* scales
     for (int i = 0; i < kN; i++) store_value<kF>(out, p * kN + i, v[i]);
 }
 
+// ... and through dequantize_symmetric_native_value_pairs (16-bit float types; e4m3, e5m2, e2m1x2)
+template <dev::Float kF, dev::Native kNative, class FS>
+__global__ void dequantize_native_pairs_kernel(const uint32_t* words, const FS* scales, dev::ScalesLayout layout,
+                                               uint64_t num_words, void* out) {
+    constexpr int kN = dev::native_values_per_word<kNative>();
+    const uint64_t p = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (p >= num_words) return;
+    uint32_t pairs[kN / 2];
+    dev::dequantize_symmetric_native_value_pairs<kF, kNative>(words[p], scales[layout.to_source_pos(p * kN)], pairs);
+    for (int i = 0; i < kN / 2; i++) static_cast<uint32_t*>(out)[p * (kN / 2) + i] = pairs[i];
+}
+
 // scale index of every element of a [batches, rows, cols] tensor through GlobalScaleLayout
 template <uint32_t kBR, uint32_t kBC>
 __global__ void scale_pos_kernel(dev::GlobalScaleLayout<kBR, kBC> layout, uint32_t batches, uint32_t rows, uint32_t cols,
@@ -129,6 +141,35 @@ int native_store(int native, int param, const uint32_t* words, const void* scale
     return -1;
 }
 
+template <dev::Float kF, dev::Native kNative>
+int native_pairs_param(int param, const uint32_t* words, const void* scales, const dev::ScalesLayout& l, uint64_t n, void* out) {
+    switch (param) {
+        case 0:
+            hipLaunchKernelGGL((dequantize_native_pairs_kernel<kF, kNative, float>), grid_for(n), dim3(256), 0, 0, words,
+                               static_cast<const float*>(scales), l, n, out);
+            return 0;
+        case 1:
+            hipLaunchKernelGGL((dequantize_native_pairs_kernel<kF, kNative, _Float16>), grid_for(n), dim3(256), 0, 0, words,
+                               static_cast<const _Float16*>(scales), l, n, out);
+            return 0;
+        case 2:
+            hipLaunchKernelGGL((dequantize_native_pairs_kernel<kF, kNative, __bf16>), grid_for(n), dim3(256), 0, 0, words,
+                               static_cast<const __bf16*>(scales), l, n, out);
+            return 0;
+    }
+    return -1;
+}
+template <dev::Float kF>
+int native_pairs_store(int native, int param, const uint32_t* words, const void* scales, const dev::ScalesLayout& l,
+                       uint64_t n, void* out) {
+    switch (native) {
+        case 1: return native_pairs_param<kF, dev::Native::E4M3>(param, words, scales, l, n, out);
+        case 2: return native_pairs_param<kF, dev::Native::E5M2>(param, words, scales, l, n, out);
+        case 3: return native_pairs_param<kF, dev::Native::E2M1x2>(param, words, scales, l, n, out);
+    }
+    return -1;
+}
+
 int finish() { return hipGetLastError() == hipSuccess && hipDeviceSynchronize() == hipSuccess ? 0 : -2; }
 
 }  // namespace
@@ -161,6 +202,20 @@ int dh_dequantize_native(int float_type, int native, int param, const uint32_t* 
         case 0: rc = native_store<dev::Float::F32>(native, param, words, scales, l, num_words, out); break;
         case 1: rc = native_store<dev::Float::F16>(native, param, words, scales, l, num_words, out); break;
         case 2: rc = native_store<dev::Float::BF16>(native, param, words, scales, l, num_words, out); break;
+    }
+    return rc ? rc : finish();
+}
+
+// The same through dequantize_symmetric_native_value_pairs: float_type 1 or 2, native 1, 2 or 3.
+int dh_dequantize_native_pairs(int float_type, int native, int param, const uint32_t* words, const void* scales,
+                               const uint64_t* values_shape, uint32_t rank, const uint64_t* scales_strides,
+                               const uint8_t* block, uint32_t block_rank, uint64_t num_words, void* out) {
+    const dev::ScalesLayout l =
+        dev::scales_layout(values_shape, rank, native == 3 ? 2u : 1u, scales_strides, block, block_rank);
+    int rc = -1;
+    switch (float_type) {
+        case 1: rc = native_pairs_store<dev::Float::F16>(native, param, words, scales, l, num_words, out); break;
+        case 2: rc = native_pairs_store<dev::Float::BF16>(native, param, words, scales, l, num_words, out); break;
     }
     return rc ? rc : finish();
 }

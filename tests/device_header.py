@@ -22,6 +22,8 @@ def lib() -> ctypes.CDLL:
         L.dh_dequantize_packed.argtypes = [ctypes.c_int] * 4 + [_vp, _vp] + layout + [ctypes.c_uint64, _vp]
         L.dh_dequantize_native.restype = ctypes.c_int
         L.dh_dequantize_native.argtypes = [ctypes.c_int] * 3 + [_vp, _vp] + layout + [ctypes.c_uint64, _vp]
+        L.dh_dequantize_native_pairs.restype = ctypes.c_int
+        L.dh_dequantize_native_pairs.argtypes = [ctypes.c_int] * 3 + [_vp, _vp] + layout + [ctypes.c_uint64, _vp]
         L.dh_global_scale_pos.restype = ctypes.c_int
         L.dh_global_scale_pos.argtypes = [ctypes.c_uint32] * 8 + [_vp]
         with_nq = [_u64p, ctypes.c_uint32, ctypes.c_uint32, _u64p, _u8p, ctypes.c_uint32]

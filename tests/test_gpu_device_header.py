@@ -101,6 +101,49 @@ def test_pairs_equal_values_for_every_word_pattern():
             assert np.array_equal(outs[0], outs[1]), (elem.name, bits)
 
 
+@pytest.mark.parametrize("case", [c for c in NATIVE if c.elem != ElemType.F32 and _NATIVE_ID[c.scheme.value] != 0],
+                         ids=lambda c: c.name)
+def test_native_pairs_reproduce_the_fixtures(case):
+    """dequantize_symmetric_native_value_pairs for e4m3 / e5m2 / e2m1x2 bytes and the 16-bit float types."""
+    words, scales = _dev(case.words.view(np.uint32)), _dev(case.out_scale)
+    out = _out(case)
+    rc = dh.lib().dh_dequantize_native_pairs(int(case.elem), _NATIVE_ID[case.scheme.value], int(case.scheme.param),
+                                             words.data_ptr(), scales.data_ptr(), *_layout_args(case), words.numel(),
+                                             out.data_ptr())
+    assert rc == 0
+    assert np.array_equal(_bits(out, case.elem), case.deq.reshape(-1))
+
+
+def test_native_pairs_equal_values_for_every_word_pattern():
+    """The pair form against the plain one over scales of every kind (tiny, huge, negative, zero, infinite, NaN)
+    and every byte value in every position (NaN and infinity encodings included), bf16 and f16: identical bits."""
+    import torch
+
+    rng = np.random.default_rng(4)
+    n_words = 1 << 14
+    words = rng.integers(0, 2**32, n_words, dtype=np.uint64).astype(np.uint32)
+    words[:256] = np.arange(256, dtype=np.uint32) * 0x01010101
+    scales = rng.normal(0, 1, n_words // 8).astype(np.float32)
+    # the 256 patterns under an ordinary, a negative and a zero scale; the special scales over random words
+    words[256:512], words[512:768] = words[:256], words[:256]
+    scales[0:32], scales[32:64], scales[64:96] = 0.37, -1.5, -0.0
+    scales[96:110] = [0.0, -0.0, 1e-38, 1e-30, 3e38, 1e30, -1.5, 65504.0, 6e-8, 2.0 ** -100, 2.0 ** 100, 2.0 ** -14,
+                      np.inf, np.nan]
+    dw, ds = _dev(words), _dev(scales)
+    for elem in (ElemType.BF16, ElemType.F16):
+        for native in (1, 2, 3):
+            per_word = 8 if native == 3 else 4
+            stored = (n_words * 4,)  # stored elements: bytes
+            block = 8 * per_word     # one scale per 8 words
+            layout = (dh.u64(stored), 1, dh.u64((1,)), dh.u8((block,)), 1)
+            outs = []
+            for fn in (dh.lib().dh_dequantize_native, dh.lib().dh_dequantize_native_pairs):
+                out = torch.zeros(n_words * per_word, dtype=torch.int16, device="cuda")
+                assert fn(int(elem), native, 0, dw.data_ptr(), ds.data_ptr(), *layout, n_words, out.data_ptr()) == 0
+                outs.append(out.cpu().numpy().view(np.uint16))
+            assert np.array_equal(outs[0], outs[1]), (elem.name, native)
+
+
 def test_global_scale_layout_and_device_scales_layout(oracle):
     """GlobalScaleLayout<BR, BC>::to_source_pos(batch, row, col) == the N-D ScalesLayout of the same tensor
     == 'coordinate / block extent' in numpy; and ScalesLayout evaluated on the device."""
