@@ -555,6 +555,36 @@ def adjacent_kernels(torch):
                     "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
     del xa, ya, words, bscales, hxa, hya, hw, hb
+    # the row kernels: blocks that are not a power of two of 16-byte chunks (24 values of 4 bits), and the headline
+    # scheme with its scales stored column by column
+    for pr, pc, value, block, col_major in ((rows, cols - 8, "Q4S", 24, False), (rows, cols, "E2M1", 32, True)):
+        rscheme = QuantScheme.default().with_value(QuantValue[value]).with_level(QuantLevel.block([block]))
+        nbk = pc // block
+        xr = [torch.randn((pr, pc), device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
+        yr = [torch.empty((pr, pc), device="cuda", dtype=torch.bfloat16) for _ in range(2)]
+        wr = [torch.empty((pr, pc // 8), dtype=torch.int32, device="cuda") for _ in range(sets)]
+        given = [torch.rand((pr, nbk), device="cuda").mul_(0.01).add_(0.01).to(torch.bfloat16) for _ in range(sets)]
+        if col_major:
+            sr = [torch.rand((nbk, pr), device="cuda").mul_(0.01).add_(0.01) for _ in range(sets)]
+            hsr = [TensorHandleRef(h(t).handle, (pr, nbk), (1, pr), 4) for t in sr]
+        else:
+            sr = [torch.rand((pr, nbk), device="cuda").mul_(0.01).add_(0.01) for _ in range(sets)]
+            hsr = [h(t) for t in sr]
+        hxr, hyr, hwr, hgr = [h(t) for t in xr], [h(t) for t in yr], [h(t) for t in wr], [h(t) for t in given]
+        b = pr * pc * 2 + wr[0].numel() * 4 + sr[0].numel() * 4
+        what = f"{value.lower()} blocks of {block}, bf16 [{pr}, {pc}]" + (", scales stored column by column" if col_major else "")
+        calls = [("quantize (given scales)", lambda i: cq_quantize.launch_ref(client, hxr[i % sets], hwr[i % sets], hgr[i % sets],
+                                                                             hsr[i % sets], rscheme, ElemType.BF16)),
+                 ("dequantize", lambda i: cq_dequantize.launch_ref(client, hwr[i % sets], hyr[i % 2], hsr[i % sets], rscheme,
+                                                                   ElemType.BF16))]
+        if not col_major:  # cq_quantize_dynamic writes contiguous scales
+            calls.insert(1, ("quantize_dynamic", lambda i: cq_quantize.launch_dynamic(client, hxr[i % sets], hwr[i % sets],
+                                                                                      hsr[i % sets], rscheme, ElemType.BF16)))
+        for label, fn in calls:
+            ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
+            out.append({"kernel": f"{label}, {what}", "algorithmic_bytes": b, "ms": round(ms, 4),
+                        "GBps": round(b / (ms * 1e-3) / 1e9, 1), "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+        del xr, yr, wr, given, sr, hsr, hxr, hyr, hwr, hgr
     # 4-bit codes of a [rows, cols] weight, 8 per u32 word along cols, viewed transposed as [cols, rows]
     packing = 8
     srcs = [torch.randint(-2**31, 2**31 - 1, (rows, cols // packing), dtype=torch.int32, device="cuda")
