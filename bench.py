@@ -310,17 +310,21 @@ def packed_gemv(torch):
     types = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
     cases = [(r, c, "Q4S", [32], "f32", "bf16", "u32") for r, c in ((14336, 4096), (4096, 14336), (28672, 8192),
                                                                     (4096, 11008), (8192, 28672))]
+    # (the last element: right-hand vectors, 1 unless given)
+    cases += [(28672, 8192, "Q4S", [32], "f32", "bf16", "u32", 4), (14336, 4096, "Q4S", [32], "f32", "bf16", "u32", 4),
+              (28672, 8192, "E4M3", [128, 128], "f32", "bf16", "native", 4)]
     cases += [(28672, 8192, "Q4S", [128], "f16", "f16", "u32"), (28672, 8192, "Q4S", [64], "bf16", "bf16", "u32"),
               (28672, 8192, "Q8S", [32], "f32", "bf16", "u32"), (28672, 8192, "Q2S", [64], "f32", "bf16", "u32"),
               (28672, 8192, "E4M3", [128, 128], "f32", "bf16", "native"), (28672, 8192, "E2M1", [32], "f32", "bf16", "native")]
     out = []
-    for rows, cols, value, block, param, elem, store in cases:
+    for rows, cols, value, block, param, elem, store, *more in cases:
+        vectors = more[0] if more else 1
         scheme = (QuantScheme.default().with_value(QuantValue[value]).with_level(QuantLevel.block(block))
                   .with_param(QuantParam[param.upper()]).with_store(QuantStore.Native if store == "native" else QuantStore.U32))
         nq = scheme.num_quants()
         stored = 4 if store == "u32" else 1  # bytes per stored element
         nscales = (rows // block[0]) * (cols // block[1]) if len(block) == 2 else rows * cols // block[0]
-        b = rows * cols // nq * stored + nscales * (4 if param == "f32" else 2) + cols * 2 + rows * 2
+        b = rows * cols // nq * stored + nscales * (4 if param == "f32" else 2) + (cols * 2 + rows * 2) * vectors
         sets = max(2, min(16, -(-(1 << 30) // b)))
         if store == "u32":
             ws = [torch.randint(-2**31, 2**31 - 1, (rows, cols // nq), dtype=torch.int32, device="cuda") for _ in range(sets)]
@@ -329,18 +333,20 @@ def packed_gemv(torch):
                   for _ in range(sets)]
         sshape = (rows // block[0], cols // block[1]) if len(block) == 2 else (rows, cols // block[0])
         ss = [(torch.rand(sshape, dtype=torch.float32, device="cuda") * 0.01 + 0.001).to(types[param]) for _ in range(sets)]
-        x = torch.randn(cols, device="cuda").to(types[elem])
-        y = torch.zeros(rows, device="cuda", dtype=types[elem])
+        x = torch.randn((vectors, cols) if vectors > 1 else cols, device="cuda").to(types[elem])
+        y = torch.zeros((vectors, rows) if vectors > 1 else rows, device="cuda", dtype=types[elem])
         hw, hs, hx, hy = [h(t) for t in ws], [h(t) for t in ss], h(x), h(y)
         et = ElemType[elem.upper()]
         fn = lambda i: matvec.launch_ref(client, hw[i % sets], hs[i % sets], scheme, hx, hy, et, et)
         ms = sorted(timed_region(torch, fn, 48)[0] for _ in range(3))[1]
         what = f"{value.lower()[:2]} blocks of {block[0]}" if store == "u32" else \
             f"{value.lower()} ({store} store) blocks of {' x '.join(map(str, block))}"
-        out.append({"kernel": f"gemv_quantized, {what}, {param} scales, {elem} x and y, weights [{rows}, {cols}]",
+        out.append({"kernel": f"gemv_quantized, {what}, {param} scales, {elem} x and y, weights [{rows}, {cols}]" +
+                              (f", {vectors} right-hand vectors at once" if vectors > 1 else ""),
                     "algorithmic_bytes": b, "buffer_sets_rotated": sets, "ms": round(ms, 4),
                     "GBps": round(b / (ms * 1e-3) / 1e9, 1), "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                    "weights_per_s": round(rows * cols / (ms * 1e-3))})
+                    "weights_per_s": round(rows * cols / (ms * 1e-3)),
+                    "multiply_adds_per_s": round(rows * cols * vectors / (ms * 1e-3))})
         del ws, ss, hw, hs
     return out
 

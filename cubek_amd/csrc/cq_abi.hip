@@ -1199,7 +1199,10 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
         !valid_dtype(y_dtype))
         return CQ_ERR_INVALID_ARGUMENT;
     const int pd = param_to_dtype(scheme->param);
-    if (values->rank != 2 || x->rank != 1 || y->rank != 1) return CQ_ERR_SHAPE_MISMATCH;
+    // x: [cols] or [vectors, cols]; y: [rows] or [vectors, rows]
+    if (values->rank != 2 || x->rank < 1 || x->rank > 2 || y->rank != x->rank) return CQ_ERR_SHAPE_MISMATCH;
+    const uint32_t last = x->rank - 1;
+    const uint64_t vectors = x->rank == 2 ? x->shape[0] : 1;
     if (values->elem_size != (native ? 1u : 4u) || x->elem_size != dtype_size(dtype) || y->elem_size != dtype_size(y_dtype) ||
         params->elem_size != dtype_size(pd))
         return CQ_ERR_SHAPE_MISMATCH;
@@ -1207,9 +1210,11 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
     const uint32_t nq = native ? (scheme->value == CQ_VALUE_E2M1 ? 2u : 1u) : 32u / bits;  // values per stored element
     const uint64_t rows = values->shape[0], cols = values->shape[1] * nq;
     if (rows > 0xffffffffull || cols > 0xffffffffull) return CQ_ERR_TOO_LARGE;
-    if (x->shape[0] != cols || y->shape[0] != rows) return CQ_ERR_SHAPE_MISMATCH;
-    if ((values->shape[1] != 1 && values->strides[1] != 1) || (cols != 1 && x->strides[0] != 1) ||
-        (rows != 1 && y->strides[0] != 1))
+    if (x->shape[last] != cols || y->shape[last] != rows || (x->rank == 2 && y->shape[0] != vectors))
+        return CQ_ERR_SHAPE_MISMATCH;
+    if (vectors > 0xffffffffull) return CQ_ERR_TOO_LARGE;
+    if ((values->shape[1] != 1 && values->strides[1] != 1) || (cols != 1 && x->strides[last] != 1) ||
+        (rows != 1 && y->strides[last] != 1))
         return CQ_ERR_NON_CONTIGUOUS;
     cq::GemvArgs a{};
     if (scheme->level == CQ_LEVEL_BLOCK) {
@@ -1224,7 +1229,10 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
     } else if (numel(params) < 1) {
         return CQ_ERR_SHAPE_MISMATCH;
     }
-    if (rows == 0) return CQ_OK;
+    if (rows == 0 || vectors == 0) return CQ_OK;
+    a.vectors = static_cast<uint32_t>(vectors);
+    a.x_stride = x->rank == 2 ? x->strides[0] : 0;
+    a.y_stride = y->rank == 2 ? y->strides[0] : 0;
     a.words = values->ptr;
     a.scales = params->ptr;
     a.x = x->ptr;

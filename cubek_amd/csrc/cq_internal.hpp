@@ -225,9 +225,12 @@ struct GemvArgs {
     uint64_t word_pitch;
     uint32_t block_rows, block_cols;  // 0, 0: one scale per tensor
     uint64_t scale_stride_row, scale_stride_col;
+    uint32_t vectors;             // right-hand vectors: x is `vectors` rows of x_stride elements, y of y_stride
+    uint64_t x_stride, y_stride;
     bool x_aligned16, words_aligned16;
 };
 bool gemv_streams(const GemvArgs& a);  // the launch takes the streaming kernel
+uint32_t gemv_vectors_per_launch(const GemvArgs& a, uint32_t remaining);
 hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a);
 
 }  // namespace cq

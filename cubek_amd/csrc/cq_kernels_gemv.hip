@@ -96,11 +96,15 @@ __device__ __forceinline__ void store_y(int dtype, void* y, uint64_t i, float v)
 // the same bits), or one of the native encodings below.
 constexpr int kCodeE4M3 = 100, kCodeE5M2 = 101, kCodeE2M1x2 = 102;
 
-template <dev::Float kF, class FS, int kCode, int kRows, int kWaves, int kDepth>
+// kVectors: 1, or room for that many right-hand vectors at once (x is then `vectors` <= kVectors rows of
+// x_stride elements, y as many rows of y_stride): every dequantized pair is used kVectors times out of its
+// registers, so a batch of vectors costs the weights' traffic and their dequantization once.
+template <dev::Float kF, class FS, int kCode, int kRows, int kWaves, int kDepth, int kVectors>
 __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     const uint32_t* __restrict__ words, const FS* __restrict__ scales, const void* __restrict__ x, void* __restrict__ y,
     int y_dtype, uint32_t rows, uint32_t units_per_row, uint32_t units_per_block_log2, uint32_t block_rows,
-    uint64_t word_pitch, uint32_t scale_stride_row, uint32_t scale_stride_col) {
+    uint64_t word_pitch, uint32_t scale_stride_row, uint32_t scale_stride_col, uint32_t vectors, uint32_t x_stride,
+    uint32_t y_stride) {
     constexpr bool kPacked = kCode <= 8;
     constexpr int kBits = kPacked ? kCode : 8;      // (of the packed fields)
     constexpr uint32_t kVals = kPacked ? 128 / kBits : (kCode == kCodeE2M1x2 ? 32 : 16);  // values of a unit
@@ -109,12 +113,17 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     constexpr uint32_t kWordPairs = kVals / 8;      // pairs out of one word
     constexpr dev::Native kNative = kCode == kCodeE4M3 ? dev::Native::E4M3
                                     : kCode == kCodeE5M2 ? dev::Native::E5M2 : dev::Native::E2M1x2;
-    extern __shared__ u32x4 xs[];  // x, kVecs pieces per unit, whole strips
+    extern __shared__ u32x4 xs[];  // x, kVecs pieces per unit, whole strips; vector after vector
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t strips = (units_per_row + 63u) / 64u;
-    for (uint32_t i = threadIdx.x; i < strips * 64u * kVecs; i += blockDim.x)
-        xs[i] = i < units_per_row * kVecs ? static_cast<const u32x4*>(x)[i] : u32x4{0, 0, 0, 0};
+    const uint32_t xs_vector = strips * 64u * kVecs;  // pieces of one staged vector
+#pragma unroll
+    for (int v = 0; v < kVectors; v++) {
+        const u32x4* xv = reinterpret_cast<const u32x4*>(static_cast<const char*>(x) + static_cast<uint64_t>(v) * x_stride * 2u);
+        for (uint32_t i = threadIdx.x; i < xs_vector; i += blockDim.x)
+            xs[v * xs_vector + i] = (static_cast<uint32_t>(v) < vectors && i < units_per_row * kVecs) ? xv[i] : u32x4{0, 0, 0, 0};
+    }
     __syncthreads();
     const uint32_t row0 = (blockIdx.x * kWaves + wave) * kRows;
     if (row0 >= rows) return;
@@ -147,12 +156,12 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     };
     // One row's share of this lane, the plain way (rolled loops, operands read again).  Only lanes whose scale
     // is not tame come here.
-    const auto plain_row = [&](int k, uint32_t strip) {
+    const auto plain_row = [&](const char* words_of_row, const char* scales_of_row, uint32_t strip, uint32_t v) {
         const uint32_t u = strip * 64u + lane;
-        if (!kPacked || u >= units_per_row) return 0.0f;
-        const uint32_t* wr = reinterpret_cast<const uint32_t*>(wrow[k]) + u * 4u;
-        const FS scale = *reinterpret_cast<const FS*>(srow[k] + (u >> units_per_block_log2) * scale_step);
-        const typename Elem<kF>::T* xr = static_cast<const typename Elem<kF>::T*>(x) + u * kVals;
+        if (!kPacked || u >= units_per_row || v >= vectors) return 0.0f;
+        const uint32_t* wr = reinterpret_cast<const uint32_t*>(words_of_row) + u * 4u;
+        const FS scale = *reinterpret_cast<const FS*>(scales_of_row + (u >> units_per_block_log2) * scale_step);
+        const typename Elem<kF>::T* xr = static_cast<const typename Elem<kF>::T*>(x) + static_cast<uint64_t>(v) * x_stride + u * kVals;
         float a = 0.0f;
 #pragma unroll 1
         for (int j = 0; j < 4; j++) {
@@ -168,10 +177,72 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
         }
         return a;
     };
-    float acc[kRows];
+    float acc[kRows * kVectors];
 #pragma unroll
-    for (int k = 0; k < kRows; k++) acc[k] = 0.0f;
+    for (int k = 0; k < kRows * kVectors; k++) acc[k] = 0.0f;
+    // several vectors: the pairs of the chunk's rows once, then vector after vector against them
+    const auto work_vectors = [&](const Chunk& c, uint32_t strip) {
+        uint32_t pairs[kRows][kPairs];
+        bool tame = true;
+#pragma unroll
+        for (int k = 0; k < kRows; k++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if constexpr (kPacked)
+                    dev::dequantize_symmetric_packed_value_pairs_tame<kF, kBits>(c.w[k][j], c.s[k], &pairs[k][kWordPairs * j]);
+                else
+                    dev::dequantize_symmetric_native_value_pairs<kF, kNative>(c.w[k][j], c.s[k], &pairs[k][kWordPairs * j]);
+            }
+            if constexpr (kPacked) tame = tame && dev::pairs_scale_is_tame<kF>(c.s[k]);
+        }
+        float part[kRows * kVectors];
+#pragma unroll
+        for (int v = 0; v < kVectors; v++) {
+            uint32_t xp[kPairs];
+#pragma unroll
+            for (uint32_t j = 0; j < kVecs; j++) {
+                const u32x4 t = xs[v * xs_vector + (strip * 64u + lane) * kVecs + j];
+                xp[4 * j] = t[0], xp[4 * j + 1] = t[1], xp[4 * j + 2] = t[2], xp[4 * j + 3] = t[3];
+            }
+#pragma unroll
+            for (int k = 0; k < kRows; k++) {
+                float a = 0.0f;
+#pragma unroll
+                for (uint32_t i = 0; i < kPairs; i++) a = dot2<kF>(pairs[k][i], xp[i], a);
+                part[k * kVectors + v] = a;
+            }
+        }
+        // lanes whose scale is not tame: the plain way, one (row, vector) at a time in a rolled loop (one copy of
+        // the code; unrolled, it took the compiler minutes)
+        if (kPacked && __builtin_amdgcn_ballot_w64(!tame) != 0) {
+            uint32_t plain_rows = 0;  // per lane: bit k set, row k's scale is not tame
+#pragma unroll
+            for (int k = 0; k < kRows; k++) plain_rows |= dev::pairs_scale_is_tame<kF>(c.s[k]) ? 0u : 1u << k;
+#pragma unroll 1
+            for (int kv = 0; kv < kRows * kVectors; kv++) {
+                const int k = kv / kVectors;
+                const char* wr = wrow[0];
+                const char* sr = srow[0];
+#pragma unroll
+                for (int t = 1; t < kRows; t++) {
+                    if (k == t) wr = wrow[t], sr = srow[t];
+                }
+                if ((plain_rows >> k) & 1u) {
+                    const float r = plain_row(wr, sr, strip, static_cast<uint32_t>(kv % kVectors));
+#pragma unroll
+                    for (int t = 0; t < kRows * kVectors; t++) part[t] = t == kv ? r : part[t];
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kRows * kVectors; k++) acc[k] += part[k];
+        __builtin_amdgcn_sched_barrier(0);
+    };
     const auto work = [&](const Chunk& c, uint32_t strip) {
+        if constexpr (kVectors > 1) {
+            work_vectors(c, strip);
+            return;
+        }
         // this lane's values of x, as pairs
         uint32_t xp[kPairs];
 #pragma unroll
@@ -199,7 +270,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
             if (__builtin_amdgcn_ballot_w64(!tame) != 0) {
 #pragma unroll
                 for (int k = 0; k < kRows; k++)
-                    if (!dev::pairs_scale_is_tame<kF>(c.s[k])) part[k] = plain_row(k, strip);
+                    if (!dev::pairs_scale_is_tame<kF>(c.s[k])) part[k] = plain_row(wrow[k], srow[k], strip, 0);
             }
         } else {
             // native encodings: the pairs are the plain arithmetic, every scale goes the same way
@@ -231,11 +302,15 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
         }
     }
 #pragma unroll
-    for (int k = 0; k < kRows; k++) acc[k] = wave_sum_to_lane63(acc[k]);
+    for (int k = 0; k < kRows * kVectors; k++) acc[k] = wave_sum_to_lane63(acc[k]);
     if (lane == 63) {
 #pragma unroll
-        for (int k = 0; k < kRows; k++)
-            if (static_cast<uint32_t>(k) < nrows) store_y(y_dtype, y, row0 + k, acc[k]);
+        for (int k = 0; k < kRows; k++) {
+#pragma unroll
+            for (int v = 0; v < kVectors; v++)
+                if (static_cast<uint32_t>(k) < nrows && static_cast<uint32_t>(v) < vectors)
+                    store_y(y_dtype, y, static_cast<uint64_t>(v) * y_stride + row0 + k, acc[k * kVectors + v]);
+        }
     }
 }
 
@@ -307,16 +382,24 @@ uint32_t log2_of(uint32_t v) {
 
 constexpr uint32_t values_per_unit(int code) { return code <= 8 ? 128 / code : (code == kCodeE2M1x2 ? 32 : 16); }
 
-template <dev::Float kF, class FS, int kBits, int kWaves>
+// LDS for x: whole strips, 2 bytes per value, times the vectors staged at once
+uint32_t stream_lds_bytes(const GemvArgs& a, uint32_t vectors) {
+    const uint32_t vals = 128 / a.bits;
+    return (a.cols / vals + 63) / 64 * 64 * vals * 2 * vectors;
+}
+constexpr uint32_t kStreamMaxLds = 65536;
+
+template <dev::Float kF, class FS, int kBits, int kWaves, int kVectors, int kRows = kStreamRows>
 void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
     constexpr uint32_t kVals = values_per_unit(kBits);
-    const uint32_t units_per_row = a.cols / kVals, strips = (units_per_row + 63) / 64;
-    const dim3 grid((a.rows + kStreamRows * kWaves - 1) / (kStreamRows * kWaves)), block(64 * kWaves);
-    hipLaunchKernelGGL((gemv_stream_kernel<kF, FS, kBits, kStreamRows, kWaves, kStreamDepth>), grid, block,
-                       strips * 64 * kVals * 2, s, static_cast<const uint32_t*>(a.words), static_cast<const FS*>(a.scales), a.x,
-                       a.y, a.y_dtype, a.rows, units_per_row, a.block_rows == 0 ? 31u : log2_of(a.block_cols / kVals),
-                       a.block_rows == 0 ? 1u : a.block_rows, a.word_pitch, static_cast<uint32_t>(a.scale_stride_row),
-                       static_cast<uint32_t>(a.scale_stride_col));
+    const uint32_t units_per_row = a.cols / kVals;
+    const dim3 grid((a.rows + kRows * kWaves - 1) / (kRows * kWaves)), block(64 * kWaves);
+    hipLaunchKernelGGL((gemv_stream_kernel<kF, FS, kBits, kRows, kWaves, kStreamDepth, kVectors>), grid, block,
+                       stream_lds_bytes(a, kVectors), s, static_cast<const uint32_t*>(a.words),
+                       static_cast<const FS*>(a.scales), a.x, a.y, a.y_dtype, a.rows, units_per_row,
+                       a.block_rows == 0 ? 31u : log2_of(a.block_cols / kVals), a.block_rows == 0 ? 1u : a.block_rows,
+                       a.word_pitch, static_cast<uint32_t>(a.scale_stride_row), static_cast<uint32_t>(a.scale_stride_col),
+                       a.vectors, static_cast<uint32_t>(a.x_stride), static_cast<uint32_t>(a.y_stride));
 }
 
 // Two rows per wave, two strips in flight, four waves (eight rows) per workgroup; eight waves from 16384 columns
@@ -325,12 +408,22 @@ void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
 // [8192, 28672]): 2 / 4 / 2 10.1, 31.3, 9.5, 33.5 us; 2 / 8 / 2 11.2, 33.1, 9.0, 28.9 us; 2 / 4 / 3 10.3, 33.0,
 // 10.1, 33.4 us; 4 / 4 / 2 11.8, 36.5, 10.3, 32.6 us; 1 / 4 / 4 11.4, 34.0, 10.1, 43.3 us; 3 / 4 / 2 10.8, 31.2,
 // 11.7, 34.5 us.
+// Right-hand vectors at once, and the waves of a workgroup that shares their x, rows per wave.  Measured on MI355X,
+// four vectors on 4-bit [28672, 8192] / [14336, 4096] / [4096, 8192] and e4m3 bytes [28672, 8192] (waves / rows):
+// 8 / 2 56.8, 19.3, 12.2, 57.1 us; 16 / 2 63.5, 19.6, 15.3, 67.9 us; 8 / 4 60.0, 20.1, 17.0, 71.7 us; 4 / 2 79.0,
+// 19.6, 13.0, 82.2 us; 16 / 4 68.6, 22.5, 29.6, 68.3 us.
+constexpr int kBatch = 4, kBatchWaves = 8, kBatchRows = 2;
+constexpr bool batches(int code) { return code == 4 || code == 8 || code == kCodeE4M3 || code == kCodeE2M1x2; }
+
 template <dev::Float kF, class FS, int kBits>
 void launch_stream_bits(hipStream_t s, const GemvArgs& a) {
-    if (a.cols >= 16384)
-        launch_stream_waves<kF, FS, kBits, 8>(s, a);
-    else
-        launch_stream_waves<kF, FS, kBits, 4>(s, a);
+    if (a.vectors > 1) {
+        if constexpr (batches(kBits)) launch_stream_waves<kF, FS, kBits, kBatchWaves, kBatch, kBatchRows>(s, a);
+    } else if (a.cols >= 16384) {
+        launch_stream_waves<kF, FS, kBits, 8, 1>(s, a);
+    } else {
+        launch_stream_waves<kF, FS, kBits, 4, 1>(s, a);
+    }
 }
 
 template <dev::Float kF, class FS>
@@ -374,8 +467,9 @@ bool gemv_streams(const GemvArgs& a) {
            a.cols <= kStreamMaxColumns && a.word_pitch % 4 == 0 && a.x_aligned16 && a.words_aligned16;
 }
 
-hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a) {
-    if (a.rows == 0 || a.cols == 0) return hipSuccess;
+namespace {
+
+hipError_t launch_one(hipStream_t s, const GemvArgs& a) {
     if (gemv_streams(a))
         return a.dtype == CQ_BF16 ? launch_stream<dev::Float::BF16>(s, a) : launch_stream<dev::Float::F16>(s, a);
     // the N-D layout of the [rows, cols] matrix, as the reference's scales_layout builds it
@@ -391,6 +485,34 @@ hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a) {
         case CQ_BF16: return launch_general_bits<dev::Float::BF16>(s, a, layout);
         default: return hipErrorInvalidValue;
     }
+}
+
+uint32_t dtype_bytes(int dtype) { return dtype == CQ_F32 ? 4u : 2u; }
+
+}  // namespace
+
+// How many of the remaining vectors the next launch takes: up to four at once where the streaming kernel applies
+// (4- and 8-bit fields, e4m3 bytes, e2m1 pairs), their x fits the LDS and every one of them starts on a 16-byte
+// boundary; else one.
+uint32_t gemv_vectors_per_launch(const GemvArgs& a, uint32_t remaining) {
+    if (remaining < 2 || !gemv_streams(a) || (a.x_stride * 2) % 16 != 0 || a.bits == 2 || a.native == 2) return 1;
+    if (stream_lds_bytes(a, kBatch) > kStreamMaxLds) return 1;
+    return remaining < kBatch ? remaining : kBatch;
+}
+
+hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a) {
+    if (a.rows == 0 || a.cols == 0) return hipSuccess;
+    for (uint32_t v = 0; v < a.vectors;) {
+        GemvArgs b = a;
+        b.x = static_cast<const char*>(a.x) + static_cast<uint64_t>(v) * a.x_stride * dtype_bytes(a.dtype);
+        b.y = static_cast<char*>(a.y) + static_cast<uint64_t>(v) * a.y_stride * dtype_bytes(a.y_dtype);
+        b.x_aligned16 = (reinterpret_cast<uintptr_t>(b.x) & 15u) == 0;
+        b.vectors = gemv_vectors_per_launch(b, a.vectors - v);
+        const hipError_t e = launch_one(s, b);
+        if (e != hipSuccess) return e;
+        v += b.vectors;
+    }
+    return hipSuccess;
 }
 
 }  // namespace cq

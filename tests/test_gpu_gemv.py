@@ -122,6 +122,50 @@ def test_gemv_native_store_matches_oracle_dequantized_weights(oracle, case):
     check_case(oracle, case, rows * 11 + cols, native=True)
 
 
+@pytest.mark.parametrize("vectors", [2, 3, 4, 7, 8, 11])
+@pytest.mark.parametrize("kind", ["q4-b32", "q8-b64-f16", "e4m3-native", "q4-general"])
+def test_gemv_with_several_right_hand_sides(oracle, kind, vectors):
+    """x [vectors, cols] -> y [vectors, rows]: every row of y is the product with that row of x, whichever way the
+    vectors are taken (up to four or eight at once by the streaming kernel, in turns otherwise)."""
+    import torch
+
+    elem, value, block, param, native, rows, cols = {
+        "q4-b32": (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, False, 70, 4160),
+        "q8-b64-f16": (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, False, 33, 2112),
+        "e4m3-native": (ElemType.BF16, QuantValue.E4M3, [32], QuantParam.F32, True, 41, 1056),
+        "q4-general": (ElemType.BF16, QuantValue.Q4S, [8], QuantParam.F32, False, 20, 512),   # blocks narrower than a unit
+    }[kind]
+    scheme = QuantScheme.default().with_value(value).with_level(QuantLevel.block(block)).with_param(param)
+    if native:
+        scheme = scheme.with_store(QuantStore.Native)
+    rng = np.random.default_rng(vectors * 100 + cols)
+    w32 = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+    wb = oracle.to_bits(w32, elem)
+    scales = oracle.compute_scales(wb, elem, (rows, cols), scheme)
+    words, out_scale = oracle.quantize(wb, elem, (rows, cols), scales, scheme)
+    deq = oracle.from_bits(oracle.dequantize(words, (rows, cols), out_scale, elem, scheme), elem).astype(np.float64)
+    xpitch = cols + 8 * int(rng.integers(0, 3))  # rows of x on 16-byte boundaries, sometimes pitched
+    xb = np.zeros((vectors, xpitch), np.uint16)
+    xb[:, :cols] = oracle.to_bits(rng.normal(0, 1, (vectors, cols)).astype(np.float32), elem).reshape(vectors, cols)
+    x64 = oracle.from_bits(xb[:, :cols].copy(), elem).astype(np.float64).reshape(vectors, cols)
+    want, mag = x64 @ deq.T, np.abs(x64) @ np.abs(deq).T
+    wpr = cols // scheme.num_quants()
+    stored = words.reshape(rows, wpr)
+    d_words = torch.from_numpy(stored if native else stored.view(np.int32)).cuda()
+    to16 = lambda a: torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda() if a.dtype == np.uint16 \
+        else torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    d_scales, d_x = to16(out_scale), to16(xb)
+    h = TensorHandleRef.from_torch
+    h_x = TensorHandleRef(d_x.data_ptr(), (vectors, cols), (xpitch, 1), 2)
+    y = torch.full((vectors, rows + 3), float("nan"), dtype=torch.float32, device="cuda")
+    h_y = TensorHandleRef(y.data_ptr(), (vectors, rows), (rows + 3, 1), 4)
+    matvec.launch_ref(ComputeClient.current(), h(d_words), h(d_scales), scheme, h_x, h_y, elem, ElemType.F32)
+    torch.cuda.synchronize()
+    got = y.cpu().numpy().astype(np.float64)
+    assert np.all(np.isnan(got[:, rows:]))  # nothing written between the rows of y
+    assert np.all(np.abs(got[:, :rows] - want) <= 2e-5 * mag + 1e-30), float(np.max(np.abs(got[:, :rows] - want) / (mag + 1e-30)))
+
+
 def test_gemv_random_configurations(oracle):
     """Sixty drawn cases of the streaming kernel's domain and its edges: every code width, block extents from one
     16-byte unit up (also over rows), one scale per tensor, every scale type, ragged strips, pitched words."""
@@ -168,19 +212,21 @@ def test_gemv_scales_of_every_kind(oracle, elem):
     odd = rng.random(scales.shape) < 0.05
     scales[odd] = rng.choice(np.array([-0.01, 0.0, -0.0, 1e-36, -3.0, 2.0 ** -110, 3000.0, -1e-30], np.float32), int(odd.sum()))
     deq = oracle.from_bits(oracle.dequantize(words, (rows, cols), scales, elem, scheme), elem).astype(np.float64)
-    xb = oracle.to_bits(rng.normal(0, 1, cols).astype(np.float32), elem)
-    x64 = oracle.from_bits(xb, elem).astype(np.float64)
     assert np.all(np.isfinite(deq))
-    want, mag = deq @ x64, np.abs(deq) @ np.abs(x64)
     d_words = torch.from_numpy(words.view(np.int32)).cuda()
     d_scales = torch.from_numpy(scales).cuda()
-    d_x = torch.from_numpy(xb.view(np.int16)).cuda()
-    y = torch.zeros(rows, dtype=torch.float32, device="cuda")
     h = TensorHandleRef.from_torch
-    matvec.launch_ref(ComputeClient.current(), h(d_words), h(d_scales), scheme, h(d_x), h(y), elem, ElemType.F32)
-    torch.cuda.synchronize()
-    got = y.cpu().numpy().astype(np.float64)
-    assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), float(np.max(np.abs(got - want) / (mag + 1e-30)))
+    for vectors in (1, 3):  # one right-hand side, and three at once
+        xb = oracle.to_bits(rng.normal(0, 1, (vectors, cols)).astype(np.float32), elem).reshape(vectors, cols)
+        x64 = oracle.from_bits(xb, elem).astype(np.float64).reshape(vectors, cols)
+        want, mag = x64 @ deq.T, np.abs(x64) @ np.abs(deq).T
+        d_x = torch.from_numpy(xb.view(np.int16)).cuda()
+        y = torch.zeros((vectors, rows), dtype=torch.float32, device="cuda")
+        hx, hy = (h(d_x), h(y)) if vectors > 1 else (h(d_x[0]), h(y[0]))
+        matvec.launch_ref(ComputeClient.current(), h(d_words), h(d_scales), scheme, hx, hy, elem, ElemType.F32)
+        torch.cuda.synchronize()
+        got = y.cpu().numpy().astype(np.float64)
+        assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), (vectors, float(np.max(np.abs(got - want) / (mag + 1e-30))))
 
 
 def test_gemv_scales_with_strides(oracle):
