@@ -125,6 +125,20 @@ def test_matrix_vector_products_that_stream():
     assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 4096, x_offset=2) == "rows"
 
 
+def test_matrix_vector_product_with_several_right_hand_sides():
+    scheme = scheme_of(QuantValue.Q4S, [32])
+    rows, cols = 512, 4096
+    values, params = t((rows, cols // 8), 4, None, 0, 1), t((rows, cols // 32), 4, None, 0, 3)
+    x, y = t((5, cols), 2, None, 0, 0), t((5, rows), 2, None, 0, 2)
+    assert _ffi.plan_kind(_ffi.OP_GEMV, x, values, params, y, scheme, BF16) == "flat"
+    with pytest.raises(_ffi.QuantError) as e:  # as many rows of y as of x
+        _ffi.plan_kind(_ffi.OP_GEMV, x, values, params, t((4, rows), 2, None, 0, 2), scheme, BF16)
+    assert e.value.status == _ffi.ERR_SHAPE_MISMATCH
+    with pytest.raises(_ffi.QuantError) as e:  # a vector against a batch
+        _ffi.plan_kind(_ffi.OP_GEMV, x, values, params, t((rows,), 2, None, 0, 2), scheme, BF16)
+    assert e.value.status == _ffi.ERR_SHAPE_MISMATCH
+
+
 def test_slow_paths_are_reported():
     e2m1 = scheme_of(QuantValue.E2M1, [32])
     # rows that start on odd multiples of 2 bytes
