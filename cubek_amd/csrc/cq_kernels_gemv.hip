@@ -99,7 +99,9 @@ constexpr int kCodeE4M3 = 100, kCodeE5M2 = 101, kCodeE2M1x2 = 102;
 // kVectors: 1, or room for that many right-hand vectors at once (x is then `vectors` <= kVectors rows of
 // x_stride elements, y as many rows of y_stride): every dequantized pair is used kVectors times out of its
 // registers, so a batch of vectors costs the weights' traffic and their dequantization once.
-template <dev::Float kF, class FS, int kCode, int kRows, int kWaves, int kDepth, int kVectors>
+// kSegment (several vectors only): strips of x staged at a time; the workgroup meets at a barrier and stages the next
+// ones when its waves have worked through them (they all do the same work, so nobody waits long).
+template <dev::Float kF, class FS, int kCode, int kRows, int kWaves, int kDepth, int kVectors, int kSegment = 0>
 __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     const uint32_t* __restrict__ words, const FS* __restrict__ scales, const void* __restrict__ x, void* __restrict__ y,
     int y_dtype, uint32_t rows, uint32_t units_per_row, uint32_t units_per_block_log2, uint32_t block_rows,
@@ -117,16 +119,29 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t strips = (units_per_row + 63u) / 64u;
-    const uint32_t xs_vector = strips * 64u * kVecs;  // pieces of one staged vector
+    constexpr bool kSegmented = kVectors > 1;
+    constexpr uint32_t kSegmentOr1 = kSegment > 0 ? kSegment : 1;
+    static_assert(!kSegmented || (kSegment > 0 && kSegment % kDepth == 0), "segments of whole rounds of the ring");
+    const uint32_t xs_vector = (kSegmented ? min(static_cast<uint32_t>(kSegment), strips) : strips) * 64u * kVecs;  // pieces of one staged vector
+    // strips [first, first + xs_vector / (64 * kVecs)) of every vector into LDS, zeros behind the end of x
+    const auto stage = [&](uint32_t first) {
 #pragma unroll
-    for (int v = 0; v < kVectors; v++) {
-        const u32x4* xv = reinterpret_cast<const u32x4*>(static_cast<const char*>(x) + static_cast<uint64_t>(v) * x_stride * 2u);
-        for (uint32_t i = threadIdx.x; i < xs_vector; i += blockDim.x)
-            xs[v * xs_vector + i] = (static_cast<uint32_t>(v) < vectors && i < units_per_row * kVecs) ? xv[i] : u32x4{0, 0, 0, 0};
+        for (int v = 0; v < kVectors; v++) {
+            const u32x4* xv = reinterpret_cast<const u32x4*>(static_cast<const char*>(x) + static_cast<uint64_t>(v) * x_stride * 2u);
+            for (uint32_t i = threadIdx.x; i < xs_vector; i += blockDim.x) {
+                const uint32_t at = first * 64u * kVecs + i;
+                xs[v * xs_vector + i] = (static_cast<uint32_t>(v) < vectors && at < units_per_row * kVecs) ? xv[at] : u32x4{0, 0, 0, 0};
+            }
+        }
+    };
+    if constexpr (!kSegmented) {
+        stage(0);
+        __syncthreads();
     }
-    __syncthreads();
-    const uint32_t row0 = (blockIdx.x * kWaves + wave) * kRows;
-    if (row0 >= rows) return;
+    // (segmented: a wave past the last row goes through the motions on the last row, for the barriers' sake)
+    const bool idle = (blockIdx.x * kWaves + wave) * kRows >= rows;
+    if (!kSegmented && idle) return;
+    const uint32_t row0 = idle ? rows - 1u : (blockIdx.x * kWaves + wave) * kRows;
     const uint32_t nrows = min(static_cast<uint32_t>(kRows), rows - row0);
 
     struct Chunk {
@@ -201,7 +216,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
             uint32_t xp[kPairs];
 #pragma unroll
             for (uint32_t j = 0; j < kVecs; j++) {
-                const u32x4 t = xs[v * xs_vector + (strip * 64u + lane) * kVecs + j];
+                const u32x4 t = xs[v * xs_vector + ((strip % kSegmentOr1) * 64u + lane) * kVecs + j];
                 xp[4 * j] = t[0], xp[4 * j + 1] = t[1], xp[4 * j + 2] = t[2], xp[4 * j + 3] = t[3];
             }
 #pragma unroll
@@ -295,6 +310,13 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
 #pragma unroll
     for (int d = 0; d < kDepth; d++) load(c[d], d);
     for (uint32_t strip = 0; strip < strips; strip += kDepth) {
+        if constexpr (kSegmented) {
+            if (strip % kSegmentOr1 == 0) {
+                if (strip != 0) __syncthreads();  // everybody has read the strips that are about to be replaced
+                stage(strip);
+                __syncthreads();
+            }
+        }
 #pragma unroll
         for (int d = 0; d < kDepth; d++) {
             if (d == 0 || strip + d < strips) work(c[d], strip + d);
@@ -308,7 +330,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
         for (int k = 0; k < kRows; k++) {
 #pragma unroll
             for (int v = 0; v < kVectors; v++)
-                if (static_cast<uint32_t>(k) < nrows && static_cast<uint32_t>(v) < vectors)
+                if (!idle && static_cast<uint32_t>(k) < nrows && static_cast<uint32_t>(v) < vectors)
                     store_y(y_dtype, y, static_cast<uint64_t>(v) * y_stride + row0 + k, acc[k * kVectors + v]);
         }
     }
@@ -387,15 +409,16 @@ uint32_t stream_lds_bytes(const GemvArgs& a, uint32_t vectors) {
     const uint32_t vals = 128 / a.bits;
     return (a.cols / vals + 63) / 64 * 64 * vals * 2 * vectors;
 }
-constexpr uint32_t kStreamMaxLds = 65536;
 
-template <dev::Float kF, class FS, int kBits, int kWaves, int kVectors, int kRows = kStreamRows>
+template <dev::Float kF, class FS, int kBits, int kWaves, int kVectors, int kRows = kStreamRows, int kSegment = 0>
 void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
     constexpr uint32_t kVals = values_per_unit(kBits);
     const uint32_t units_per_row = a.cols / kVals;
     const dim3 grid((a.rows + kRows * kWaves - 1) / (kRows * kWaves)), block(64 * kWaves);
-    hipLaunchKernelGGL((gemv_stream_kernel<kF, FS, kBits, kRows, kWaves, kStreamDepth, kVectors>), grid, block,
-                       stream_lds_bytes(a, kVectors), s, static_cast<const uint32_t*>(a.words),
+    const uint32_t strips = (units_per_row + 63) / 64;
+    const uint32_t lds = kSegment > 0 ? (strips < kSegment ? strips : kSegment) * 64 * kVals * 2 * kVectors : stream_lds_bytes(a, 1);
+    hipLaunchKernelGGL((gemv_stream_kernel<kF, FS, kBits, kRows, kWaves, kStreamDepth, kVectors, kSegment>), grid, block,
+                       lds, s, static_cast<const uint32_t*>(a.words),
                        static_cast<const FS*>(a.scales), a.x, a.y, a.y_dtype, a.rows, units_per_row,
                        a.block_rows == 0 ? 31u : log2_of(a.block_cols / kVals), a.block_rows == 0 ? 1u : a.block_rows,
                        a.word_pitch, static_cast<uint32_t>(a.scale_stride_row), static_cast<uint32_t>(a.scale_stride_col),
@@ -412,13 +435,16 @@ void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
 // four vectors on 4-bit [28672, 8192] / [14336, 4096] / [4096, 8192] and e4m3 bytes [28672, 8192] (waves / rows):
 // 8 / 2 56.8, 19.3, 12.2, 57.1 us; 16 / 2 63.5, 19.6, 15.3, 67.9 us; 8 / 4 60.0, 20.1, 17.0, 71.7 us; 4 / 2 79.0,
 // 19.6, 13.0, 82.2 us; 16 / 4 68.6, 22.5, 29.6, 68.3 us.
-constexpr int kBatch = 4, kBatchWaves = 8, kBatchRows = 2;
+// Strips of x staged at a time (64 KiB of LDS for four vectors of 4-bit units): 4; with 2, [28672, 8192] took 63.0
+// instead of 57.4 us (e4m3 bytes 72.4 instead of 60.5 us), with 8 (half as many 4-bit workgroups per compute
+// unit) 83.3 us.
+constexpr int kBatch = 4, kBatchWaves = 8, kBatchRows = 2, kBatchSegment = 4;
 constexpr bool batches(int code) { return code == 4 || code == 8 || code == kCodeE4M3 || code == kCodeE2M1x2; }
 
 template <dev::Float kF, class FS, int kBits>
 void launch_stream_bits(hipStream_t s, const GemvArgs& a) {
     if (a.vectors > 1) {
-        if constexpr (batches(kBits)) launch_stream_waves<kF, FS, kBits, kBatchWaves, kBatch, kBatchRows>(s, a);
+        if constexpr (batches(kBits)) launch_stream_waves<kF, FS, kBits, kBatchWaves, kBatch, kBatchRows, kBatchSegment>(s, a);
     } else if (a.cols >= 16384) {
         launch_stream_waves<kF, FS, kBits, 8, 1>(s, a);
     } else {
@@ -492,11 +518,9 @@ uint32_t dtype_bytes(int dtype) { return dtype == CQ_F32 ? 4u : 2u; }
 }  // namespace
 
 // How many of the remaining vectors the next launch takes: up to four at once where the streaming kernel applies
-// (4- and 8-bit fields, e4m3 bytes, e2m1 pairs), their x fits the LDS and every one of them starts on a 16-byte
-// boundary; else one.
+// (4- and 8-bit fields, e4m3 bytes, e2m1 pairs) and every one of them starts on a 16-byte boundary; else one.
 uint32_t gemv_vectors_per_launch(const GemvArgs& a, uint32_t remaining) {
     if (remaining < 2 || !gemv_streams(a) || (a.x_stride * 2) % 16 != 0 || a.bits == 2 || a.native == 2) return 1;
-    if (stream_lds_bytes(a, kBatch) > kStreamMaxLds) return 1;
     return remaining < kBatch ? remaining : kBatch;
 }
 

@@ -123,7 +123,7 @@ def test_gemv_native_store_matches_oracle_dequantized_weights(oracle, case):
 
 
 @pytest.mark.parametrize("vectors", [2, 3, 4, 7, 8, 11])
-@pytest.mark.parametrize("kind", ["q4-b32", "q8-b64-f16", "e4m3-native", "q4-general"])
+@pytest.mark.parametrize("kind", ["q4-b32", "q8-b64-f16", "e4m3-native", "q4-general", "q4-wide", "e2m1-native-wide"])
 def test_gemv_with_several_right_hand_sides(oracle, kind, vectors):
     """x [vectors, cols] -> y [vectors, rows]: every row of y is the product with that row of x, whichever way the
     vectors are taken (up to four or eight at once by the streaming kernel, in turns otherwise)."""
@@ -134,6 +134,8 @@ def test_gemv_with_several_right_hand_sides(oracle, kind, vectors):
         "q8-b64-f16": (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, False, 33, 2112),
         "e4m3-native": (ElemType.BF16, QuantValue.E4M3, [32], QuantParam.F32, True, 41, 1056),
         "q4-general": (ElemType.BF16, QuantValue.Q4S, [8], QuantParam.F32, False, 20, 512),   # blocks narrower than a unit
+        "q4-wide": (ElemType.BF16, QuantValue.Q4S, [64], QuantParam.BF16, False, 19, 18560),   # five segments of x, the last short
+        "e2m1-native-wide": (ElemType.F16, QuantValue.E2M1, [32], QuantParam.F32, True, 10, 10304),
     }[kind]
     scheme = QuantScheme.default().with_value(value).with_level(QuantLevel.block(block)).with_param(param)
     if native:
