@@ -394,7 +394,7 @@ hipError_t launch_general_bits(hipStream_t s, const GemvArgs& a, const dev::Scal
 }
 
 constexpr int kStreamRows = 2, kStreamDepth = 2;
-constexpr uint32_t kStreamMaxColumns = 32768;  // x of that many columns fills 64 KiB of LDS
+[[maybe_unused]] constexpr uint32_t kStreamMaxColumns = 32768;  // x of that many columns fills 64 KiB of LDS
 
 uint32_t log2_of(uint32_t v) {
     uint32_t l = 0;
@@ -441,9 +441,9 @@ void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
 constexpr int kBatch = 4, kBatchWaves = 8, kBatchRows = 2, kBatchSegment = 4;
 constexpr bool batches(int code) { return code == 4 || code == 8 || code == kCodeE4M3 || code == kCodeE2M1x2; }
 
-template <dev::Float kF, class FS, int kBits>
+template <dev::Float kF, class FS, int kBits, bool kBatched>
 void launch_stream_bits(hipStream_t s, const GemvArgs& a) {
-    if (a.vectors > 1) {
+    if constexpr (kBatched) {
         if constexpr (batches(kBits)) launch_stream_waves<kF, FS, kBits, kBatchWaves, kBatch, kBatchRows, kBatchSegment>(s, a);
     } else if (a.cols >= 16384) {
         launch_stream_waves<kF, FS, kBits, 8, 1>(s, a);
@@ -452,34 +452,55 @@ void launch_stream_bits(hipStream_t s, const GemvArgs& a) {
     }
 }
 
-template <dev::Float kF, class FS>
+template <dev::Float kF, class FS, bool kBatched>
 void launch_stream_scales(hipStream_t s, const GemvArgs& a) {
     if (a.native == 1)
-        launch_stream_bits<kF, FS, kCodeE4M3>(s, a);
+        launch_stream_bits<kF, FS, kCodeE4M3, kBatched>(s, a);
     else if (a.native == 2)
-        launch_stream_bits<kF, FS, kCodeE5M2>(s, a);
+        launch_stream_bits<kF, FS, kCodeE5M2, kBatched>(s, a);
     else if (a.native == 3)
-        launch_stream_bits<kF, FS, kCodeE2M1x2>(s, a);
+        launch_stream_bits<kF, FS, kCodeE2M1x2, kBatched>(s, a);
     else if (a.bits == 4)
-        launch_stream_bits<kF, FS, 4>(s, a);
+        launch_stream_bits<kF, FS, 4, kBatched>(s, a);
     else if (a.bits == 8)
-        launch_stream_bits<kF, FS, 8>(s, a);
+        launch_stream_bits<kF, FS, 8, kBatched>(s, a);
     else
-        launch_stream_bits<kF, FS, 2>(s, a);
+        launch_stream_bits<kF, FS, 2, kBatched>(s, a);
 }
 
-template <dev::Float kF>
-hipError_t launch_stream(hipStream_t s, const GemvArgs& a) {
-    switch (a.param_dtype) {
-        case CQ_F32: launch_stream_scales<kF, float>(s, a); break;
-        case CQ_F16: launch_stream_scales<kF, _Float16>(s, a); break;
-        default: launch_stream_scales<kF, __bf16>(s, a); break;
-    }
+template <class FS, bool kBatched>
+hipError_t launch_stream_floats(hipStream_t s, const GemvArgs& a) {
+    if (a.dtype == CQ_BF16)
+        launch_stream_scales<dev::Float::BF16, FS, kBatched>(s, a);
+    else
+        launch_stream_scales<dev::Float::F16, FS, kBatched>(s, a);
     return hipGetLastError();
 }
 
 }  // namespace
 
+// The streaming kernels sit in three objects, so that a process loads the code of the kind it uses (the first launch
+// out of an object loads all of it): one right-hand side with f32 scales, with f16 / bf16 scales, several at once.
+// CQ_GEMV_PART names the one being compiled; without it everything lands in one object.
+#if !defined(CQ_GEMV_PART) || CQ_GEMV_PART == 0
+hipError_t gemv_stream_f32_scales(hipStream_t s, const GemvArgs& a) { return launch_stream_floats<float, false>(s, a); }
+#endif
+#if !defined(CQ_GEMV_PART) || CQ_GEMV_PART == 1
+hipError_t gemv_stream_16bit_scales(hipStream_t s, const GemvArgs& a) {
+    return a.param_dtype == CQ_F16 ? launch_stream_floats<_Float16, false>(s, a) : launch_stream_floats<__bf16, false>(s, a);
+}
+#endif
+#if !defined(CQ_GEMV_PART) || CQ_GEMV_PART == 2
+hipError_t gemv_stream_batched(hipStream_t s, const GemvArgs& a) {
+    switch (a.param_dtype) {
+        case CQ_F32: return launch_stream_floats<float, true>(s, a);
+        case CQ_F16: return launch_stream_floats<_Float16, true>(s, a);
+        default: return launch_stream_floats<__bf16, true>(s, a);
+    }
+}
+#endif
+
+#if !defined(CQ_GEMV_PART) || CQ_GEMV_PART == 0
 bool gemv_streams(const GemvArgs& a) {
     if (a.dtype == CQ_F32 || (a.bits != 2 && a.bits != 4 && a.bits != 8)) return false;
     const uint32_t vals = 128 / a.bits;  // values of a 16-byte unit (native encodings come with their bits)
@@ -496,8 +517,10 @@ bool gemv_streams(const GemvArgs& a) {
 namespace {
 
 hipError_t launch_one(hipStream_t s, const GemvArgs& a) {
-    if (gemv_streams(a))
-        return a.dtype == CQ_BF16 ? launch_stream<dev::Float::BF16>(s, a) : launch_stream<dev::Float::F16>(s, a);
+    if (gemv_streams(a)) {
+        if (a.vectors > 1) return gemv_stream_batched(s, a);
+        return a.param_dtype == CQ_F32 ? gemv_stream_f32_scales(s, a) : gemv_stream_16bit_scales(s, a);
+    }
     // the N-D layout of the [rows, cols] matrix, as the reference's scales_layout builds it
     dev::ScalesLayout layout;
     if (a.block_rows != 0) {
@@ -538,5 +561,7 @@ hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a) {
     }
     return hipSuccess;
 }
+
+#endif  // part 0
 
 }  // namespace cq
