@@ -278,4 +278,20 @@ inline void into_contiguous_packed_ref(const ComputeClient& client, const Tensor
 }
 }  // namespace contiguous
 
+namespace matvec {
+// The matrix-vector case of a matmul with a quantized operand (MatmulInputHandle::Quantized,
+// crates/cubek-matmul/src/base.rs:309-317): y = dequantize(values, params) * x with the weights read once in
+// their stored form.  `values` [rows, cols / num_quants] (U32 store) or the byte tensor of the native store,
+// `x` [cols] or [vectors, cols] of `elem`, `y` [rows] or [vectors, rows] of `y_elem`.
+inline void launch_ref(const ComputeClient& client, const TensorHandleRef& values, const TensorHandleRef& params,
+                       const scheme::QuantScheme& scheme, const TensorHandleRef& x, const TensorHandleRef& y, ElemType elem,
+                       ElemType y_elem) {
+    cq_tensor v = values.as_c(), p = params.as_c(), xs = x.as_c(), ys = y.as_c();
+    cq_scheme c = scheme.to_c();
+    detail::check(cq_gemv_quantized(client.stream, &v, &p, &c, &xs, &ys, static_cast<cq_dtype>(elem),
+                                    static_cast<cq_dtype>(y_elem)),
+                  scheme);
+}
+}  // namespace matvec
+
 }  // namespace cubek_quant
