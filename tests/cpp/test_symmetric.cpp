@@ -241,6 +241,43 @@ static void test_reduce_max_abs() {
     report("reduce::invalid_axis_and_mismatch_shape", bad_axis && bad_shape);
 }
 
+// matvec::launch_ref against the dequantized weights times x on the host (f32 throughout)
+static void test_matvec() {
+    ComputeClient client;
+    const size_t m = 16, n = 64, block_size = 32;
+    std::vector<float> data(m * n), xs(n);
+    for (size_t i = 0; i < m * n; i++) data[i] = std::sin(static_cast<float>(i) * 0.37f);
+    for (size_t i = 0; i < n; i++) xs[i] = std::cos(static_cast<float>(i) * 0.11f);
+    QuantScheme scheme = QuantScheme::default_()
+                             .with_level(QuantLevel::block({static_cast<uint8_t>(block_size)}))
+                             .with_value(QuantValue::Q8S)
+                             .with_store(QuantStore::U32)
+                             .with_param(QuantParam::F32);
+    DeviceBuffer<float> input(data), x(xs), scale(m * n / block_size), restored(m * n), y(m);
+    DeviceBuffer<uint32_t> words(m * n / scheme.num_quants());
+    auto t_in = TensorHandleRef::contiguous(input.ptr, {m, n}, 4);
+    auto t_words = TensorHandleRef::contiguous(words.ptr, {m, n / scheme.num_quants()}, 4);
+    auto t_scale = TensorHandleRef::contiguous(scale.ptr, {m, n / block_size}, 4);
+    auto t_restored = TensorHandleRef::contiguous(restored.ptr, {m, n}, 4);
+    auto t_x = TensorHandleRef::contiguous(x.ptr, {n}, 4);
+    auto t_y = TensorHandleRef::contiguous(y.ptr, {m}, 4);
+    quantize::launch_dynamic(client, t_in, t_words, t_scale, scheme, ElemType::F32);
+    dequantize::launch_ref(client, t_words, t_restored, t_scale, scheme, ElemType::F32);
+    matvec::launch_ref(client, t_words, t_scale, scheme, t_x, t_y, ElemType::F32, ElemType::F32);
+    HIP_OK(hipDeviceSynchronize());
+    const std::vector<float> w = restored.read(), got = y.read();
+    bool ok = true;
+    for (size_t r = 0; r < m; r++) {
+        double want = 0.0, mag = 0.0;
+        for (size_t c = 0; c < n; c++) {
+            want += static_cast<double>(w[r * n + c]) * xs[c];
+            mag += std::fabs(static_cast<double>(w[r * n + c]) * xs[c]);
+        }
+        ok = ok && std::fabs(got[r] - want) <= 2e-5 * mag;
+    }
+    report("matvec::launch_ref", ok);
+}
+
 int main() {
     int devices = 0;
     if (hipGetDeviceCount(&devices) != hipSuccess || devices == 0) {
@@ -259,6 +296,7 @@ int main() {
         }
     test_error_behaviour();
     test_reduce_max_abs();
+    test_matvec();
     std::printf("%d failure(s)\n", failures);
     return failures == 0 ? 0 : 1;
 }

@@ -16,4 +16,4 @@ def test_reference_suite_through_cpp_host_layer():
     print(proc.stdout)
     lines = [l for l in proc.stdout.splitlines() if l.startswith(("PASS", "FAIL"))]
     assert proc.returncode == 0, proc.stdout
-    assert len([l for l in lines if l.startswith("PASS")]) == 24 + 4 + 2 and not [l for l in lines if l.startswith("FAIL")]
+    assert len([l for l in lines if l.startswith("PASS")]) == 24 + 4 + 2 + 1 and not [l for l in lines if l.startswith("FAIL")]
