@@ -49,7 +49,7 @@ def _id(c):
         ("-pitched" if pitch else "")
 
 
-def check_case(oracle, case, seed, native=False):
+def check_case(oracle, case, seed, native=False, vectors=1):
     import torch
 
     elem, value, block, param, rows, cols, pitch = case
@@ -64,10 +64,10 @@ def check_case(oracle, case, seed, native=False):
     scales = oracle.compute_scales(wb, elem, (rows, cols), scheme)
     words, out_scale = oracle.quantize(wb, elem, (rows, cols), scales, scheme)
     deq = oracle.from_bits(oracle.dequantize(words, (rows, cols), out_scale, elem, scheme), elem).astype(np.float64)
-    xb = oracle.to_bits(rng.normal(0, 1, cols).astype(np.float32), elem)
-    x64 = oracle.from_bits(xb, elem).astype(np.float64)
-    want = deq @ x64
-    mag = np.abs(deq) @ np.abs(x64)
+    xb = oracle.to_bits(rng.normal(0, 1, (vectors, cols)).astype(np.float32), elem).reshape(vectors, cols)
+    x64 = oracle.from_bits(xb, elem).astype(np.float64).reshape(vectors, cols)
+    want = x64 @ deq.T           # [vectors, rows]
+    mag = np.abs(x64) @ np.abs(deq).T
 
     nq = scheme.num_quants()
     wpr = cols // nq
@@ -82,19 +82,21 @@ def check_case(oracle, case, seed, native=False):
     h_words = TensorHandleRef(d_words.data_ptr(), (rows, wpr), (pitch, 1), 1 if native else 4)
     h_scales = TensorHandleRef(d_scales.data_ptr(), sshape, tuple(d_scales.stride()) if block else (1,),
                                d_scales.element_size())
+    # one right-hand side as a vector, several as the rows of a matrix
+    h_x = TensorHandleRef.from_torch(d_x) if vectors > 1 else TensorHandleRef.from_torch(d_x[0])
     client = ComputeClient.current()
-    y32 = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
-    matvec.launch_ref(client, h_words, h_scales, scheme, TensorHandleRef.from_torch(d_x), TensorHandleRef.from_torch(y32),
-                      elem, ElemType.F32)
+    y32 = torch.full((vectors, rows), float("nan"), dtype=torch.float32, device="cuda")
+    h_y = lambda t: TensorHandleRef.from_torch(t) if vectors > 1 else TensorHandleRef.from_torch(t[0])
+    matvec.launch_ref(client, h_words, h_scales, scheme, h_x, h_y(y32), elem, ElemType.F32)
     torch.cuda.synchronize()
     got = y32.cpu().numpy().astype(np.float64)
-    assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), (case, float(np.max(np.abs(got - want) / (mag + 1e-30))))
+    assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), (case, vectors, float(np.max(np.abs(got - want) / (mag + 1e-30))))
     if elem != ElemType.F32:  # the same sums, rounded once to the 16-bit type
-        y16 = torch.zeros((rows,), dtype=torch.int16, device="cuda")
-        matvec.launch_ref(client, h_words, h_scales, scheme, TensorHandleRef.from_torch(d_x),
-                          TensorHandleRef.from_torch(y16), elem, elem)
+        y16 = torch.zeros((vectors, rows), dtype=torch.int16, device="cuda")
+        matvec.launch_ref(client, h_words, h_scales, scheme, h_x, h_y(y16), elem, elem)
         torch.cuda.synchronize()
-        assert np.array_equal(y16.cpu().numpy().view(np.uint16), oracle.to_bits(y32.cpu().numpy(), elem)), case
+        assert np.array_equal(y16.cpu().numpy().view(np.uint16).reshape(-1), oracle.to_bits(y32.cpu().numpy().reshape(-1), elem)), \
+            (case, vectors)
 
 
 @pytest.mark.parametrize("case", CASES, ids=_id)
@@ -169,12 +171,15 @@ def test_gemv_with_several_right_hand_sides(oracle, kind, vectors):
 
 
 def test_gemv_random_configurations(oracle):
-    """Sixty drawn cases of the streaming kernel's domain and its edges: every code width, block extents from one
-    16-byte unit up (also over rows), one scale per tensor, every scale type, ragged strips, pitched words."""
+    """Sixty drawn cases (CQ_RANDOM_GEMV=N: N) of the streaming kernel's domain and its edges: every code width,
+    block extents from one 16-byte unit up (also over rows), one scale per tensor, every scale type, ragged strips,
+    pitched words, one to six right-hand sides, both stores."""
+    import os
+
     rng = np.random.default_rng(2024)
     values = {2: [QuantValue.Q2S, QuantValue.Q2F], 4: [QuantValue.Q4S, QuantValue.Q4F, QuantValue.E2M1],
               8: [QuantValue.Q8S, QuantValue.Q8F]}
-    for i in range(60):
+    for i in range(int(os.environ.get("CQ_RANDOM_GEMV", "60"))):
         bits = int(rng.choice([2, 4, 8]))
         unit = 128 // bits
         elem = [ElemType.BF16, ElemType.F16][int(rng.integers(2))]
@@ -197,7 +202,12 @@ def test_gemv_random_configurations(oracle):
         value = values[bits][int(rng.integers(len(values[bits])))]
         wpr = cols // (32 // bits)
         pitch = None if rng.random() < 0.6 else wpr + 4 * int(rng.integers(1, 5))
-        check_case(oracle, (elem, value, block, param, rows, cols, pitch), 1000 + i)
+        vectors = int(rng.choice([1, 1, 1, 2, 4, 5, 6]))
+        # every third case in the native store, where the value has one (bytes: the pitch counts bytes)
+        native = i % 3 == 2 and value in (QuantValue.Q8S, QuantValue.Q8F, QuantValue.E2M1)
+        if native:
+            pitch = None if pitch is None else (cols // (2 if value == QuantValue.E2M1 else 1)) + 16 * int(rng.integers(1, 4))
+        check_case(oracle, (elem, value, block, param, rows, cols, pitch), 1000 + i, native=native, vectors=vectors)
 
 
 @pytest.mark.parametrize("elem", [ElemType.BF16, ElemType.F16], ids=lambda e: e.name)
