@@ -99,8 +99,9 @@ constexpr int kCodeE4M3 = 100, kCodeE5M2 = 101, kCodeE2M1x2 = 102;
 // kVectors: 1, or room for that many right-hand vectors at once (x is then `vectors` <= kVectors rows of
 // x_stride elements, y as many rows of y_stride): every dequantized pair is used kVectors times out of its
 // registers, so a batch of vectors costs the weights' traffic and their dequantization once.
-// kSegment (several vectors only): strips of x staged at a time; the workgroup meets at a barrier and stages the next
-// ones when its waves have worked through them (they all do the same work, so nobody waits long).
+// kSegment (several vectors, or rows too long for the LDS): strips of x staged at a time; the workgroup meets at a
+// barrier and stages the next ones when its waves have worked through them (they all do the same work, so nobody
+// waits long).  0: all of x at once.
 template <dev::Float kF, class FS, int kCode, int kRows, int kWaves, int kDepth, int kVectors, int kSegment = 0>
 __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     const uint32_t* __restrict__ words, const FS* __restrict__ scales, const void* __restrict__ x, void* __restrict__ y,
@@ -119,9 +120,10 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t strips = (units_per_row + 63u) / 64u;
-    constexpr bool kSegmented = kVectors > 1;
+    constexpr bool kSegmented = kSegment > 0;
     constexpr uint32_t kSegmentOr1 = kSegment > 0 ? kSegment : 1;
-    static_assert(!kSegmented || (kSegment > 0 && kSegment % kDepth == 0), "segments of whole rounds of the ring");
+    static_assert(kVectors == 1 || kSegmented, "several vectors are staged in segments");
+    static_assert(kSegment % kDepth == 0, "segments of whole rounds of the ring");
     const uint32_t xs_vector = (kSegmented ? min(static_cast<uint32_t>(kSegment), strips) : strips) * 64u * kVecs;  // pieces of one staged vector
     // strips [first, first + xs_vector / (64 * kVecs)) of every vector into LDS, zeros behind the end of x
     const auto stage = [&](uint32_t first) {
@@ -262,7 +264,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
         uint32_t xp[kPairs];
 #pragma unroll
         for (uint32_t j = 0; j < kVecs; j++) {
-            const u32x4 v = xs[(strip * 64u + lane) * kVecs + j];
+            const u32x4 v = xs[((kSegmented ? strip % kSegmentOr1 : strip) * 64u + lane) * kVecs + j];
             xp[4 * j] = v[0], xp[4 * j + 1] = v[1], xp[4 * j + 2] = v[2], xp[4 * j + 3] = v[3];
         }
         float part[kRows];
@@ -441,10 +443,15 @@ void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
 constexpr int kBatch = 4, kBatchWaves = 8, kBatchRows = 2, kBatchSegment = 4;
 constexpr bool batches(int code) { return code == 4 || code == 8 || code == kCodeE4M3 || code == kCodeE2M1x2; }
 
+constexpr int kWideSegment = 16;  // strips of x at a time where a row has more than kStreamMaxColumns values
+
 template <dev::Float kF, class FS, int kBits, bool kBatched>
 void launch_stream_bits(hipStream_t s, const GemvArgs& a) {
     if constexpr (kBatched) {
-        if constexpr (batches(kBits)) launch_stream_waves<kF, FS, kBits, kBatchWaves, kBatch, kBatchRows, kBatchSegment>(s, a);
+        if (a.vectors == 1)  // one right-hand side, rows too long for the LDS
+            launch_stream_waves<kF, FS, kBits, 8, 1, kStreamRows, kWideSegment * int(values_per_unit(4)) / int(values_per_unit(kBits))>(s, a);
+        else if constexpr (batches(kBits))
+            launch_stream_waves<kF, FS, kBits, kBatchWaves, kBatch, kBatchRows, kBatchSegment>(s, a);
     } else if (a.cols >= 16384) {
         launch_stream_waves<kF, FS, kBits, 8, 1>(s, a);
     } else {
@@ -510,15 +517,14 @@ bool gemv_streams(const GemvArgs& a) {
             a.scale_stride_row >= (1ull << 32) || (a.cols / a.block_cols) * a.scale_stride_col >= (1ull << 29))
             return false;
     }
-    return a.cols % vals == 0 &&
-           a.cols <= kStreamMaxColumns && a.word_pitch % 4 == 0 && a.x_aligned16 && a.words_aligned16;
+    return a.cols % vals == 0 && a.cols < (1u << 26) && a.word_pitch % 4 == 0 && a.x_aligned16 && a.words_aligned16;
 }
 
 namespace {
 
 hipError_t launch_one(hipStream_t s, const GemvArgs& a) {
     if (gemv_streams(a)) {
-        if (a.vectors > 1) return gemv_stream_batched(s, a);
+        if (a.vectors > 1 || a.cols > kStreamMaxColumns) return gemv_stream_batched(s, a);
         return a.param_dtype == CQ_F32 ? gemv_stream_f32_scales(s, a) : gemv_stream_16bit_scales(s, a);
     }
     // the N-D layout of the [rows, cols] matrix, as the reference's scales_layout builds it

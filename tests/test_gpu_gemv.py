@@ -22,6 +22,8 @@ CASES = [
     (ElemType.F16, QuantValue.Q4S, [32], QuantParam.F32, 21, 16480, None),        # eight waves per workgroup
     (ElemType.BF16, QuantValue.Q4F, [32], QuantParam.F32, 1, 32768, None),        # one row, the longest it takes
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 9, 32, None),           # one block per row
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 11, 53248, None),       # rows longer than the LDS holds of x
+    (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, 5, 40000, None),         # ... 8-bit codes, two segments
     (ElemType.F16, QuantValue.Q4S, [128], QuantParam.F16, 33, 4224, None),        # four units under one f16 scale
     (ElemType.BF16, QuantValue.Q8S, [32], QuantParam.F32, 45, 2080, None),        # 8-bit codes, two units per block
     (ElemType.BF16, QuantValue.Q4F, [64], QuantParam.BF16, 19, 16448, 2060),      # bf16 scales, eight waves, pitched

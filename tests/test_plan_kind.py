@@ -114,13 +114,13 @@ def test_matrix_vector_products_that_stream():
     assert gemv_kind(scheme_of(QuantValue.Q8S, [128, 128]), BF16, 256, 1024) == "flat"
     assert gemv_kind(scheme_of(QuantValue.Q4S, None), BF16, 64, 32768) == "flat"
     assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 4096, s_strides=(1, 64)) == "flat"
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 53248) == "flat"  # rows longer than the LDS holds of x
     assert gemv_kind(scheme_of(QuantValue.Q4S, [32], param=QuantParam.F16), BF16, 64, 4096) == "flat"
     # the general kernel: f32 x, blocks narrower than 16 bytes of codes or not a power of two
-    # of them, more than 32768 columns, words or x off 16-byte boundaries
+    # of them, words or x off 16-byte boundaries
     assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), F32, 64, 4096) == "rows"
     assert gemv_kind(scheme_of(QuantValue.Q4S, [16]), BF16, 64, 4096) == "rows"
     assert gemv_kind(scheme_of(QuantValue.Q4S, [96]), BF16, 64, 4032) == "rows"
-    assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 32800) == "rows"
     assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 4096, pitch=513) == "rows"
     assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 4096, x_offset=2) == "rows"
 
