@@ -441,7 +441,7 @@ void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
 // instead of 57.4 us (e4m3 bytes 72.4 instead of 60.5 us), with 8 (half as many 4-bit workgroups per compute
 // unit) 83.3 us.
 constexpr int kBatch = 4, kBatchWaves = 8, kBatchRows = 2, kBatchSegment = 4;
-constexpr bool batches(int code) { return code == 4 || code == 8 || code == kCodeE4M3 || code == kCodeE2M1x2; }
+constexpr bool batches(int code) { return code != 2; }  // (64 values per unit: their pairs alone would fill the registers)
 
 constexpr int kWideSegment = 16;  // strips of x at a time where a row has more than kStreamMaxColumns values
 
@@ -547,9 +547,9 @@ uint32_t dtype_bytes(int dtype) { return dtype == CQ_F32 ? 4u : 2u; }
 }  // namespace
 
 // How many of the remaining vectors the next launch takes: up to four at once where the streaming kernel applies
-// (4- and 8-bit fields, e4m3 bytes, e2m1 pairs) and every one of them starts on a 16-byte boundary; else one.
+// (all but the 2-bit fields) and every one of them starts on a 16-byte boundary; else one.
 uint32_t gemv_vectors_per_launch(const GemvArgs& a, uint32_t remaining) {
-    if (remaining < 2 || !gemv_streams(a) || (a.x_stride * 2) % 16 != 0 || a.bits == 2 || a.native == 2) return 1;
+    if (remaining < 2 || !gemv_streams(a) || (a.x_stride * 2) % 16 != 0 || a.bits == 2) return 1;
     return remaining < kBatch ? remaining : kBatch;
 }
 

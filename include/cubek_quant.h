@@ -243,8 +243,8 @@ cq_status cq_into_contiguous_packed(cq_stream_t stream, const cq_tensor* input, 
  * A streaming kernel (HBM- or arithmetic-bound, 45 - 70 % of the HBM peak on large weights) takes a 16-bit
  * `dtype` with 16-byte aligned rows of codes and x, scales of any type per tensor or on
  * blocks of 1, 2, 4, ... times 16 bytes of codes along the row (any number of rows): cq_plan_kind(CQ_OP_GEMV)
- * tells.  Four right-hand sides go through it at once (4- and 8-bit fields, e4m3 bytes, e2m1 pairs; rows of x
- * on 16-byte boundaries), so that the weights are read and dequantized once for the four; more, or others, are
+ * tells.  Four right-hand sides go through it at once (all but 2-bit fields; rows of x on 16-byte
+ * boundaries), so that the weights are read and dequantized once for the four; more, or others, are
  * computed in turns.  Every other U32-store layout takes a simple
  * wave-per-row kernel; every other native-store layout is CQ_ERR_UNSUPPORTED_SCHEME. */
 cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const cq_tensor* params,

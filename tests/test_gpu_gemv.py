@@ -127,7 +127,8 @@ def test_gemv_native_store_matches_oracle_dequantized_weights(oracle, case):
 
 
 @pytest.mark.parametrize("vectors", [2, 3, 4, 7, 8, 11])
-@pytest.mark.parametrize("kind", ["q4-b32", "q8-b64-f16", "e4m3-native", "q4-general", "q4-wide", "e2m1-native-wide"])
+@pytest.mark.parametrize("kind", ["q4-b32", "q8-b64-f16", "e4m3-native", "q4-general", "q4-wide", "e2m1-native-wide",
+                                  "e5m2-native", "q2-in-turns"])
 def test_gemv_with_several_right_hand_sides(oracle, kind, vectors):
     """x [vectors, cols] -> y [vectors, rows]: every row of y is the product with that row of x, whichever way the
     vectors are taken (up to four or eight at once by the streaming kernel, in turns otherwise)."""
@@ -138,6 +139,8 @@ def test_gemv_with_several_right_hand_sides(oracle, kind, vectors):
         "q8-b64-f16": (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, False, 33, 2112),
         "e4m3-native": (ElemType.BF16, QuantValue.E4M3, [32], QuantParam.F32, True, 41, 1056),
         "q4-general": (ElemType.BF16, QuantValue.Q4S, [8], QuantParam.F32, False, 20, 512),   # blocks narrower than a unit
+        "e5m2-native": (ElemType.F16, QuantValue.E5M2, [64], QuantParam.F32, True, 26, 2112),
+        "q2-in-turns": (ElemType.BF16, QuantValue.Q2S, [64], QuantParam.F32, False, 14, 1088),   # 2-bit: one vector per launch
         "q4-wide": (ElemType.BF16, QuantValue.Q4S, [64], QuantParam.BF16, False, 19, 18560),   # five segments of x, the last short
         "e2m1-native-wide": (ElemType.F16, QuantValue.E2M1, [32], QuantParam.F32, True, 10, 10304),
     }[kind]
