@@ -234,6 +234,7 @@ uint32_t gemv_vectors_per_launch(const GemvArgs& a, uint32_t remaining);
 hipError_t gemv_stream_f32_scales(hipStream_t s, const GemvArgs& a);    // the streaming kernels, by object
 hipError_t gemv_stream_16bit_scales(hipStream_t s, const GemvArgs& a);
 hipError_t gemv_stream_batched(hipStream_t s, const GemvArgs& a);
+hipError_t gemv_stream_f32_x(hipStream_t s, const GemvArgs& a);
 hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a);
 
 }  // namespace cq

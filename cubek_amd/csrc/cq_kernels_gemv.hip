@@ -111,8 +111,11 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     constexpr bool kPacked = kCode <= 8;
     constexpr int kBits = kPacked ? kCode : 8;      // (of the packed fields)
     constexpr uint32_t kVals = kPacked ? 128 / kBits : (kCode == kCodeE2M1x2 ? 32 : 16);  // values of a unit
+    constexpr bool kWide32 = kF == dev::Float::F32;  // x in f32: no pairs, the plain dequantization and one FMA per value
     constexpr uint32_t kPairs = kVals / 2;          // ... as packed pairs of x
-    constexpr uint32_t kVecs = kPairs / 4;          // ... as 16-byte pieces of x
+    constexpr uint32_t kVecs = kWide32 ? kVals / 4 : kPairs / 4;  // ... as 16-byte pieces of x
+    constexpr uint32_t kWordVals = kVals / 4;       // values out of one word
+    static_assert(!kWide32 || kVectors == 1, "several vectors at once: 16-bit float types");
     constexpr uint32_t kWordPairs = kVals / 8;      // pairs out of one word
     constexpr dev::Native kNative = kCode == kCodeE4M3 ? dev::Native::E4M3
                                     : kCode == kCodeE5M2 ? dev::Native::E5M2 : dev::Native::E2M1x2;
@@ -129,7 +132,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     const auto stage = [&](uint32_t first) {
 #pragma unroll
         for (int v = 0; v < kVectors; v++) {
-            const u32x4* xv = reinterpret_cast<const u32x4*>(static_cast<const char*>(x) + static_cast<uint64_t>(v) * x_stride * 2u);
+            const u32x4* xv = reinterpret_cast<const u32x4*>(static_cast<const char*>(x) + static_cast<uint64_t>(v) * x_stride * (kWide32 ? 4u : 2u));
             for (uint32_t i = threadIdx.x; i < xs_vector; i += blockDim.x) {
                 const uint32_t at = first * 64u * kVecs + i;
                 xs[v * xs_vector + i] = (static_cast<uint32_t>(v) < vectors && at < units_per_row * kVecs) ? xv[at] : u32x4{0, 0, 0, 0};
@@ -174,139 +177,175 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     // One row's share of this lane, the plain way (rolled loops, operands read again).  Only lanes whose scale
     // is not tame come here.
     const auto plain_row = [&](const char* words_of_row, const char* scales_of_row, uint32_t strip, uint32_t v) {
-        const uint32_t u = strip * 64u + lane;
-        if (!kPacked || u >= units_per_row || v >= vectors) return 0.0f;
-        const uint32_t* wr = reinterpret_cast<const uint32_t*>(words_of_row) + u * 4u;
-        const FS scale = *reinterpret_cast<const FS*>(scales_of_row + (u >> units_per_block_log2) * scale_step);
-        const typename Elem<kF>::T* xr = static_cast<const typename Elem<kF>::T*>(x) + static_cast<uint64_t>(v) * x_stride + u * kVals;
-        float a = 0.0f;
-#pragma unroll 1
-        for (int j = 0; j < 4; j++) {
-            float v[2 * kWordPairs];
-            dev::dequantize_symmetric_packed_value<kF, kBits>(wr[j], scale, v);
-#pragma unroll
-            for (uint32_t i = 0; i < 2 * kWordPairs; i += 2) {
-                const uint32_t xpair =
-                    static_cast<uint32_t>(__builtin_bit_cast(uint16_t, xr[2 * kWordPairs * j + i])) |
-                    static_cast<uint32_t>(__builtin_bit_cast(uint16_t, xr[2 * kWordPairs * j + i + 1])) << 16;
-                a = dot2<kF>(dev::pack_pair<kF>(v[i], v[i + 1]), xpair, a);
+        if constexpr (kWide32) {
+            return 0.0f;  // (f32 x: the main path is the plain one)
+        } else {
+            const uint32_t u = strip * 64u + lane;
+            if (!kPacked || u >= units_per_row || v >= vectors) return 0.0f;
+            const uint32_t* wr = reinterpret_cast<const uint32_t*>(words_of_row) + u * 4u;
+            const FS scale = *reinterpret_cast<const FS*>(scales_of_row + (u >> units_per_block_log2) * scale_step);
+            const typename Elem<kF>::T* xr = static_cast<const typename Elem<kF>::T*>(x) + static_cast<uint64_t>(v) * x_stride + u * kVals;
+            float a = 0.0f;
+    #pragma unroll 1
+            for (int j = 0; j < 4; j++) {
+                float v[2 * kWordPairs];
+                dev::dequantize_symmetric_packed_value<kF, kBits>(wr[j], scale, v);
+    #pragma unroll
+                for (uint32_t i = 0; i < 2 * kWordPairs; i += 2) {
+                    const uint32_t xpair =
+                        static_cast<uint32_t>(__builtin_bit_cast(uint16_t, xr[2 * kWordPairs * j + i])) |
+                        static_cast<uint32_t>(__builtin_bit_cast(uint16_t, xr[2 * kWordPairs * j + i + 1])) << 16;
+                    a = dot2<kF>(dev::pack_pair<kF>(v[i], v[i + 1]), xpair, a);
+                }
             }
+            return a;
         }
-        return a;
     };
     float acc[kRows * kVectors];
 #pragma unroll
     for (int k = 0; k < kRows * kVectors; k++) acc[k] = 0.0f;
     // several vectors: the pairs of the chunk's rows once, then vector after vector against them
     const auto work_vectors = [&](const Chunk& c, uint32_t strip) {
-        uint32_t pairs[kRows][kPairs];
-        bool tame = true;
-#pragma unroll
-        for (int k = 0; k < kRows; k++) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if constexpr (kPacked)
-                    dev::dequantize_symmetric_packed_value_pairs_tame<kF, kBits>(c.w[k][j], c.s[k], &pairs[k][kWordPairs * j]);
-                else
-                    dev::dequantize_symmetric_native_value_pairs<kF, kNative>(c.w[k][j], c.s[k], &pairs[k][kWordPairs * j]);
-            }
-            if constexpr (kPacked) tame = tame && dev::pairs_scale_is_tame<kF>(c.s[k]);
-        }
-        float part[kRows * kVectors];
-#pragma unroll
-        for (int v = 0; v < kVectors; v++) {
-            uint32_t xp[kPairs];
-#pragma unroll
-            for (uint32_t j = 0; j < kVecs; j++) {
-                const u32x4 t = xs[v * xs_vector + ((strip % kSegmentOr1) * 64u + lane) * kVecs + j];
-                xp[4 * j] = t[0], xp[4 * j + 1] = t[1], xp[4 * j + 2] = t[2], xp[4 * j + 3] = t[3];
-            }
-#pragma unroll
+        if constexpr (kVectors > 1) {
+            uint32_t pairs[kRows][kPairs];
+            bool tame = true;
+    #pragma unroll
             for (int k = 0; k < kRows; k++) {
-                float a = 0.0f;
-#pragma unroll
-                for (uint32_t i = 0; i < kPairs; i++) a = dot2<kF>(pairs[k][i], xp[i], a);
-                part[k * kVectors + v] = a;
-            }
-        }
-        // lanes whose scale is not tame: the plain way, one (row, vector) at a time in a rolled loop (one copy of
-        // the code; unrolled, it took the compiler minutes)
-        if (kPacked && __builtin_amdgcn_ballot_w64(!tame) != 0) {
-            uint32_t plain_rows = 0;  // per lane: bit k set, row k's scale is not tame
-#pragma unroll
-            for (int k = 0; k < kRows; k++) plain_rows |= dev::pairs_scale_is_tame<kF>(c.s[k]) ? 0u : 1u << k;
-#pragma unroll 1
-            for (int kv = 0; kv < kRows * kVectors; kv++) {
-                const int k = kv / kVectors;
-                const char* wr = wrow[0];
-                const char* sr = srow[0];
-#pragma unroll
-                for (int t = 1; t < kRows; t++) {
-                    if (k == t) wr = wrow[t], sr = srow[t];
+    #pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if constexpr (kPacked)
+                        dev::dequantize_symmetric_packed_value_pairs_tame<kF, kBits>(c.w[k][j], c.s[k], &pairs[k][kWordPairs * j]);
+                    else
+                        dev::dequantize_symmetric_native_value_pairs<kF, kNative>(c.w[k][j], c.s[k], &pairs[k][kWordPairs * j]);
                 }
-                if ((plain_rows >> k) & 1u) {
-                    const float r = plain_row(wr, sr, strip, static_cast<uint32_t>(kv % kVectors));
-#pragma unroll
-                    for (int t = 0; t < kRows * kVectors; t++) part[t] = t == kv ? r : part[t];
+                if constexpr (kPacked) tame = tame && dev::pairs_scale_is_tame<kF>(c.s[k]);
+            }
+            float part[kRows * kVectors];
+    #pragma unroll
+            for (int v = 0; v < kVectors; v++) {
+                uint32_t xp[kPairs];
+    #pragma unroll
+                for (uint32_t j = 0; j < kVecs; j++) {
+                    const u32x4 t = xs[v * xs_vector + ((strip % kSegmentOr1) * 64u + lane) * kVecs + j];
+                    xp[4 * j] = t[0], xp[4 * j + 1] = t[1], xp[4 * j + 2] = t[2], xp[4 * j + 3] = t[3];
+                }
+    #pragma unroll
+                for (int k = 0; k < kRows; k++) {
+                    float a = 0.0f;
+    #pragma unroll
+                    for (uint32_t i = 0; i < kPairs; i++) a = dot2<kF>(pairs[k][i], xp[i], a);
+                    part[k * kVectors + v] = a;
                 }
             }
+            // lanes whose scale is not tame: the plain way, one (row, vector) at a time in a rolled loop (one copy of
+            // the code; unrolled, it took the compiler minutes)
+            if (kPacked && __builtin_amdgcn_ballot_w64(!tame) != 0) {
+                uint32_t plain_rows = 0;  // per lane: bit k set, row k's scale is not tame
+    #pragma unroll
+                for (int k = 0; k < kRows; k++) plain_rows |= dev::pairs_scale_is_tame<kF>(c.s[k]) ? 0u : 1u << k;
+    #pragma unroll 1
+                for (int kv = 0; kv < kRows * kVectors; kv++) {
+                    const int k = kv / kVectors;
+                    const char* wr = wrow[0];
+                    const char* sr = srow[0];
+    #pragma unroll
+                    for (int t = 1; t < kRows; t++) {
+                        if (k == t) wr = wrow[t], sr = srow[t];
+                    }
+                    if ((plain_rows >> k) & 1u) {
+                        const float r = plain_row(wr, sr, strip, static_cast<uint32_t>(kv % kVectors));
+    #pragma unroll
+                        for (int t = 0; t < kRows * kVectors; t++) part[t] = t == kv ? r : part[t];
+                    }
+                }
+            }
+    #pragma unroll
+            for (int k = 0; k < kRows * kVectors; k++) acc[k] += part[k];
+            __builtin_amdgcn_sched_barrier(0);
         }
-#pragma unroll
-        for (int k = 0; k < kRows * kVectors; k++) acc[k] += part[k];
-        __builtin_amdgcn_sched_barrier(0);
     };
     const auto work = [&](const Chunk& c, uint32_t strip) {
-        if constexpr (kVectors > 1) {
-            work_vectors(c, strip);
-            return;
-        }
-        // this lane's values of x, as pairs
-        uint32_t xp[kPairs];
+        if constexpr (kWide32) {
+            // this lane's values of x
+            float xf[kVals];
 #pragma unroll
-        for (uint32_t j = 0; j < kVecs; j++) {
-            const u32x4 v = xs[((kSegmented ? strip % kSegmentOr1 : strip) * 64u + lane) * kVecs + j];
-            xp[4 * j] = v[0], xp[4 * j + 1] = v[1], xp[4 * j + 2] = v[2], xp[4 * j + 3] = v[3];
-        }
-        float part[kRows];
-        if constexpr (kPacked) {
-            bool tame = true;
+            for (uint32_t j = 0; j < kVecs; j++) {
+                const u32x4 t = xs[((kSegmented ? strip % kSegmentOr1 : strip) * 64u + lane) * kVecs + j];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t bits = t[i];  // (a bit cast of the element expression itself reads element 0)
+                    xf[4 * j + i] = __builtin_bit_cast(float, bits);
+                }
+            }
 #pragma unroll
             for (int k = 0; k < kRows; k++) {
                 float a = 0.0f;
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    uint32_t pairs[kWordPairs];
-                    dev::dequantize_symmetric_packed_value_pairs_tame<kF, kBits>(c.w[k][j], c.s[k], pairs);
+                    float v[kWordVals];
+                    if constexpr (kPacked)
+                        dev::dequantize_symmetric_packed_value<kF, kBits>(c.w[k][j], c.s[k], v);
+                    else
+                        dev::dequantize_symmetric_native_value<kF, kNative>(c.w[k][j], c.s[k], v);
 #pragma unroll
-                    for (uint32_t i = 0; i < kWordPairs; i++) a = dot2<kF>(pairs[i], xp[kWordPairs * j + i], a);
+                    for (uint32_t i = 0; i < kWordVals; i++) a = __builtin_fmaf(v[i], xf[kWordVals * j + i], a);
                 }
-                part[k] = a;
-                tame = tame && dev::pairs_scale_is_tame<kF>(c.s[k]);
+                acc[k] += a;
             }
-            // ordinary scales are all tame: one wave-uniform test per chunk, then straight on
-            if (__builtin_amdgcn_ballot_w64(!tame) != 0) {
-#pragma unroll
-                for (int k = 0; k < kRows; k++)
-                    if (!dev::pairs_scale_is_tame<kF>(c.s[k])) part[k] = plain_row(wrow[k], srow[k], strip, 0);
-            }
+            __builtin_amdgcn_sched_barrier(0);
         } else {
-            // native encodings: the pairs are the plain arithmetic, every scale goes the same way
-#pragma unroll
-            for (int k = 0; k < kRows; k++) {
-                float a = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    uint32_t pairs[kWordPairs];
-                    dev::dequantize_symmetric_native_value_pairs<kF, kNative>(c.w[k][j], c.s[k], pairs);
-#pragma unroll
-                    for (uint32_t i = 0; i < kWordPairs; i++) a = dot2<kF>(pairs[i], xp[kWordPairs * j + i], a);
-                }
-                part[k] = a;
+            if constexpr (kVectors > 1) {
+                work_vectors(c, strip);
+                return;
             }
+            // this lane's values of x, as pairs
+            uint32_t xp[kPairs];
+    #pragma unroll
+            for (uint32_t j = 0; j < kVecs; j++) {
+                const u32x4 v = xs[((kSegmented ? strip % kSegmentOr1 : strip) * 64u + lane) * kVecs + j];
+                xp[4 * j] = v[0], xp[4 * j + 1] = v[1], xp[4 * j + 2] = v[2], xp[4 * j + 3] = v[3];
+            }
+            float part[kRows];
+            if constexpr (kPacked) {
+                bool tame = true;
+    #pragma unroll
+                for (int k = 0; k < kRows; k++) {
+                    float a = 0.0f;
+    #pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        uint32_t pairs[kWordPairs];
+                        dev::dequantize_symmetric_packed_value_pairs_tame<kF, kBits>(c.w[k][j], c.s[k], pairs);
+    #pragma unroll
+                        for (uint32_t i = 0; i < kWordPairs; i++) a = dot2<kF>(pairs[i], xp[kWordPairs * j + i], a);
+                    }
+                    part[k] = a;
+                    tame = tame && dev::pairs_scale_is_tame<kF>(c.s[k]);
+                }
+                // ordinary scales are all tame: one wave-uniform test per chunk, then straight on
+                if (__builtin_amdgcn_ballot_w64(!tame) != 0) {
+    #pragma unroll
+                    for (int k = 0; k < kRows; k++)
+                        if (!dev::pairs_scale_is_tame<kF>(c.s[k])) part[k] = plain_row(wrow[k], srow[k], strip, 0);
+                }
+            } else {
+                // native encodings: the pairs are the plain arithmetic, every scale goes the same way
+    #pragma unroll
+                for (int k = 0; k < kRows; k++) {
+                    float a = 0.0f;
+    #pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        uint32_t pairs[kWordPairs];
+                        dev::dequantize_symmetric_native_value_pairs<kF, kNative>(c.w[k][j], c.s[k], pairs);
+    #pragma unroll
+                        for (uint32_t i = 0; i < kWordPairs; i++) a = dot2<kF>(pairs[i], xp[kWordPairs * j + i], a);
+                    }
+                    part[k] = a;
+                }
+            }
+    #pragma unroll
+            for (int k = 0; k < kRows; k++) acc[k] += part[k];
+            __builtin_amdgcn_sched_barrier(0);
         }
-#pragma unroll
-        for (int k = 0; k < kRows; k++) acc[k] += part[k];
-        __builtin_amdgcn_sched_barrier(0);
     };
     Chunk c[kDepth];
 #pragma unroll
@@ -409,7 +448,7 @@ constexpr uint32_t values_per_unit(int code) { return code <= 8 ? 128 / code : (
 // LDS for x: whole strips, 2 bytes per value, times the vectors staged at once
 uint32_t stream_lds_bytes(const GemvArgs& a, uint32_t vectors) {
     const uint32_t vals = 128 / a.bits;
-    return (a.cols / vals + 63) / 64 * 64 * vals * 2 * vectors;
+    return (a.cols / vals + 63) / 64 * 64 * vals * (a.dtype == CQ_F32 ? 4 : 2) * vectors;
 }
 
 template <dev::Float kF, class FS, int kBits, int kWaves, int kVectors, int kRows = kStreamRows, int kSegment = 0>
@@ -418,7 +457,8 @@ void launch_stream_waves(hipStream_t s, const GemvArgs& a) {
     const uint32_t units_per_row = a.cols / kVals;
     const dim3 grid((a.rows + kRows * kWaves - 1) / (kRows * kWaves)), block(64 * kWaves);
     const uint32_t strips = (units_per_row + 63) / 64;
-    const uint32_t lds = kSegment > 0 ? (strips < kSegment ? strips : kSegment) * 64 * kVals * 2 * kVectors : stream_lds_bytes(a, 1);
+    const uint32_t lds = kSegment > 0 ? (strips < kSegment ? strips : kSegment) * 64 * kVals * (kF == dev::Float::F32 ? 4 : 2) * kVectors
+                                      : stream_lds_bytes(a, 1);
     hipLaunchKernelGGL((gemv_stream_kernel<kF, FS, kBits, kRows, kWaves, kStreamDepth, kVectors, kSegment>), grid, block,
                        lds, s, static_cast<const uint32_t*>(a.words),
                        static_cast<const FS*>(a.scales), a.x, a.y, a.y_dtype, a.rows, units_per_row,
@@ -449,8 +489,9 @@ template <dev::Float kF, class FS, int kBits, bool kBatched>
 void launch_stream_bits(hipStream_t s, const GemvArgs& a) {
     if constexpr (kBatched) {
         if (a.vectors == 1)  // one right-hand side, rows too long for the LDS
-            launch_stream_waves<kF, FS, kBits, 8, 1, kStreamRows, kWideSegment * int(values_per_unit(4)) / int(values_per_unit(kBits))>(s, a);
-        else if constexpr (batches(kBits))
+            launch_stream_waves<kF, FS, kBits, 8, 1, kStreamRows,
+                                kWideSegment * int(values_per_unit(4)) / int(values_per_unit(kBits)) / (kF == dev::Float::F32 ? 2 : 1)>(s, a);
+        else if constexpr (batches(kBits) && kF != dev::Float::F32)
             launch_stream_waves<kF, FS, kBits, kBatchWaves, kBatch, kBatchRows, kBatchSegment>(s, a);
     } else if (a.cols >= 16384) {
         launch_stream_waves<kF, FS, kBits, 8, 1>(s, a);
@@ -487,7 +528,8 @@ hipError_t launch_stream_floats(hipStream_t s, const GemvArgs& a) {
 }  // namespace
 
 // The streaming kernels sit in three objects, so that a process loads the code of the kind it uses (the first launch
-// out of an object loads all of it): one right-hand side with f32 scales, with f16 / bf16 scales, several at once.
+// out of an object loads all of it): one right-hand side with f32 scales, with f16 / bf16 scales, several at once
+// (and rows too long for the LDS), x in f32.
 // CQ_GEMV_PART names the one being compiled; without it everything lands in one object.
 #if !defined(CQ_GEMV_PART) || CQ_GEMV_PART == 0
 hipError_t gemv_stream_f32_scales(hipStream_t s, const GemvArgs& a) { return launch_stream_floats<float, false>(s, a); }
@@ -507,9 +549,20 @@ hipError_t gemv_stream_batched(hipStream_t s, const GemvArgs& a) {
 }
 #endif
 
+#if !defined(CQ_GEMV_PART) || CQ_GEMV_PART == 3
+// x in f32 (f32 scales): the plain dequantization and one FMA per value
+hipError_t gemv_stream_f32_x(hipStream_t s, const GemvArgs& a) {
+    if (a.cols > kStreamMaxColumns / 2)
+        launch_stream_scales<dev::Float::F32, float, true>(s, a);
+    else
+        launch_stream_scales<dev::Float::F32, float, false>(s, a);
+    return hipGetLastError();
+}
+#endif
+
 #if !defined(CQ_GEMV_PART) || CQ_GEMV_PART == 0
 bool gemv_streams(const GemvArgs& a) {
-    if (a.dtype == CQ_F32 || (a.bits != 2 && a.bits != 4 && a.bits != 8)) return false;
+    if ((a.bits != 2 && a.bits != 4 && a.bits != 8) || (a.dtype == CQ_F32 && a.param_dtype != CQ_F32)) return false;
     const uint32_t vals = 128 / a.bits;  // values of a 16-byte unit (native encodings come with their bits)
     if (a.block_rows != 0) {             // blocks: whole units along the row, a power of two of them
         const uint32_t units_per_block = a.block_cols / vals;
@@ -524,6 +577,7 @@ namespace {
 
 hipError_t launch_one(hipStream_t s, const GemvArgs& a) {
     if (gemv_streams(a)) {
+        if (a.dtype == CQ_F32) return gemv_stream_f32_x(s, a);
         if (a.vectors > 1 || a.cols > kStreamMaxColumns) return gemv_stream_batched(s, a);
         return a.param_dtype == CQ_F32 ? gemv_stream_f32_scales(s, a) : gemv_stream_16bit_scales(s, a);
     }
@@ -549,7 +603,7 @@ uint32_t dtype_bytes(int dtype) { return dtype == CQ_F32 ? 4u : 2u; }
 // How many of the remaining vectors the next launch takes: up to four at once where the streaming kernel applies
 // (all but the 2-bit fields) and every one of them starts on a 16-byte boundary; else one.
 uint32_t gemv_vectors_per_launch(const GemvArgs& a, uint32_t remaining) {
-    if (remaining < 2 || !gemv_streams(a) || (a.x_stride * 2) % 16 != 0 || a.bits == 2) return 1;
+    if (remaining < 2 || !gemv_streams(a) || (a.x_stride * 2) % 16 != 0 || a.bits == 2 || a.dtype == CQ_F32) return 1;
     return remaining < kBatch ? remaining : kBatch;
 }
 

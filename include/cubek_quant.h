@@ -241,7 +241,7 @@ cq_status cq_into_contiguous_packed(cq_stream_t stream, const cq_tensor* input, 
  * Every weight enters as the value cq_dequantize would produce for `dtype`, F(F(scale) * F(code)); the
  * products are accumulated in f32 (order unspecified) and the sum is rounded once to `y_dtype`.
  * A streaming kernel (HBM- or arithmetic-bound, 45 - 70 % of the HBM peak on large weights) takes a 16-bit
- * `dtype` with 16-byte aligned rows of codes and x, scales of any type per tensor or on
+ * `dtype` (f32 as well where the scales are f32) with 16-byte aligned rows of codes and x, scales of any type per tensor or on
  * blocks of 1, 2, 4, ... times 16 bytes of codes along the row (any number of rows): cq_plan_kind(CQ_OP_GEMV)
  * tells.  Four right-hand sides go through it at once (all but 2-bit fields; rows of x on 16-byte
  * boundaries), so that the weights are read and dequantized once for the four; more, or others, are

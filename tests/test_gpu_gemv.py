@@ -34,8 +34,11 @@ CASES = [
     (ElemType.F16, QuantValue.Q8S, [64], QuantParam.BF16, 31, 2112, None),        # bf16 scales under f16 x
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.BF16, 100, 1024, None),
     (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, 50, 512, None),
-    (ElemType.F32, QuantValue.Q2S, [64], QuantParam.F32, 96, 1024, None),          # general kernel: f32 x,
-    (ElemType.F32, QuantValue.Q8F, None, QuantParam.F32, 33, 260, None),          # per tensor,
+    (ElemType.F32, QuantValue.Q2S, [64], QuantParam.F32, 96, 1024, None),          # x in f32: streaming again
+    (ElemType.F32, QuantValue.Q4S, [32], QuantParam.F32, 75, 4160, 524),
+    (ElemType.F32, QuantValue.Q8F, [16], QuantParam.F32, 31, 17008, None),         # ... rows too long for the LDS
+    (ElemType.F32, QuantValue.Q4S, [32], QuantParam.BF16, 20, 1024, None),         # f32 x under bf16 scales: general kernel
+    (ElemType.F32, QuantValue.Q8F, None, QuantParam.F32, 33, 260, None),          # general: 260 values are not whole units
     (ElemType.BF16, QuantValue.Q4S, [4, 16], QuantParam.F32, 64, 256, None),      # blocks narrower than a unit
     (ElemType.BF16, QuantValue.Q8S, None, QuantParam.F32, 29, 2064, None),        # streaming again: one scale per tensor
     (ElemType.F16, QuantValue.Q4F, None, QuantParam.F16, 11, 4128, None),
@@ -117,6 +120,8 @@ NATIVE_CASES = [
     (ElemType.F16, QuantValue.E2M1, [64], QuantParam.F16, 18, 1088, None),
     (ElemType.BF16, QuantValue.Q8S, [32], QuantParam.F32, 45, 2080, None),          # i8 bytes: the 8-bit fields
     (ElemType.F16, QuantValue.Q8F, [16], QuantParam.BF16, 9, 16, None),             # one unit per row
+    (ElemType.F32, QuantValue.E4M3, [32], QuantParam.F32, 37, 2080, None),          # x in f32
+    (ElemType.F32, QuantValue.E2M1, [64], QuantParam.F32, 12, 4160, None),
 ]
 
 

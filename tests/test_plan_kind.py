@@ -116,9 +116,10 @@ def test_matrix_vector_products_that_stream():
     assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 4096, s_strides=(1, 64)) == "flat"
     assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 53248) == "flat"  # rows longer than the LDS holds of x
     assert gemv_kind(scheme_of(QuantValue.Q4S, [32], param=QuantParam.F16), BF16, 64, 4096) == "flat"
-    # the general kernel: f32 x, blocks narrower than 16 bytes of codes or not a power of two
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), F32, 64, 4096) == "flat"  # x in f32 (with f32 scales)
+    # the general kernel: f32 x with 16-bit scales, blocks narrower than 16 bytes of codes or not a power of two
     # of them, words or x off 16-byte boundaries
-    assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), F32, 64, 4096) == "rows"
+    assert gemv_kind(scheme_of(QuantValue.Q4S, [32], param=QuantParam.F16), F32, 64, 4096) == "rows"
     assert gemv_kind(scheme_of(QuantValue.Q4S, [16]), BF16, 64, 4096) == "rows"
     assert gemv_kind(scheme_of(QuantValue.Q4S, [96]), BF16, 64, 4032) == "rows"
     assert gemv_kind(scheme_of(QuantValue.Q4S, [32]), BF16, 64, 4096, pitch=513) == "rows"
