@@ -183,7 +183,7 @@ def test_gemv_with_several_right_hand_sides(oracle, kind, vectors):
 def test_gemv_random_configurations(oracle):
     """Sixty drawn cases (CQ_RANDOM_GEMV=N: N) of the streaming kernel's domain and its edges: every code width,
     block extents from one 16-byte unit up (also over rows), one scale per tensor, every scale type, ragged strips,
-    pitched words, one to six right-hand sides, both stores."""
+    pitched words, one to six right-hand sides, both stores, x in all three float types."""
     import os
 
     rng = np.random.default_rng(2024)
@@ -192,8 +192,10 @@ def test_gemv_random_configurations(oracle):
     for i in range(int(os.environ.get("CQ_RANDOM_GEMV", "60"))):
         bits = int(rng.choice([2, 4, 8]))
         unit = 128 // bits
-        elem = [ElemType.BF16, ElemType.F16][int(rng.integers(2))]
+        elem = [ElemType.BF16, ElemType.F16, ElemType.BF16, ElemType.F32][int(rng.integers(4))]
         param = [QuantParam.F32, QuantParam.F16, QuantParam.BF16][int(rng.integers(3))]
+        if elem == ElemType.F32 and rng.random() < 0.8:
+            param = QuantParam.F32  # (f32 x streams under f32 scales; the rest goes to the general kernel)
         kind = int(rng.integers(4))
         units_per_block = int(2 ** rng.integers(0, 3))
         bc = unit * units_per_block
@@ -215,6 +217,8 @@ def test_gemv_random_configurations(oracle):
         vectors = int(rng.choice([1, 1, 1, 2, 4, 5, 6]))
         # every third case in the native store, where the value has one (bytes: the pitch counts bytes)
         native = i % 3 == 2 and value in (QuantValue.Q8S, QuantValue.Q8F, QuantValue.E2M1)
+        if native and elem == ElemType.F32:
+            param = QuantParam.F32  # the native store only streams, and f32 x streams under f32 scales
         if native:
             pitch = None if pitch is None else (cols // (2 if value == QuantValue.E2M1 else 1)) + 16 * int(rng.integers(1, 4))
         check_case(oracle, (elem, value, block, param, rows, cols, pitch), 1000 + i, native=native, vectors=vectors)
