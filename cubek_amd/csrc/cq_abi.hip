@@ -580,13 +580,20 @@ static_assert(CQ_STATIC_SCRATCH_BYTES >= cq::kMaxPartials * sizeof(float), "the 
 constexpr int kMaxDevices = 64;
 std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
-// Device address of `scratch` on the current device, resolved on the first call per device (threads that
-// race here resolve the same address).
-cq_status static_scratch(void** ptr) {
+// Device address of `scratch` on the device the launches will run on, resolved on the first call per device
+// (threads that race here resolve the same address).  hipGetSymbolAddress answers for the current device, so a
+// stream that lives on another device is refused: its kernels would be handed this device's address.
+cq_status static_scratch(hipStream_t stream, void** ptr) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return hip_status(e);
     if (dev < 0 || dev >= kMaxDevices) return CQ_ERR_INVALID_ARGUMENT;
+    if (stream != nullptr) {  // the null stream is the current device's
+        hipDevice_t stream_dev = -1;
+        e = hipStreamGetDevice(stream, &stream_dev);
+        if (e != hipSuccess) return hip_status(e);
+        if (static_cast<int>(stream_dev) != dev) return CQ_ERR_INVALID_ARGUMENT;
+    }
     void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (p == nullptr) {
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
@@ -1143,7 +1150,7 @@ cq_status cq_quantize_dynamic_static(cq_stream_t stream, const cq_tensor* input,
     }
     if (cq_workspace_bytes(scheme, n) > CQ_STATIC_SCRATCH_BYTES) return CQ_ERR_SCRATCH_TOO_SMALL;
     void* ws = nullptr;
-    st = static_scratch(&ws);
+    st = static_scratch(stream, &ws);
     if (st != CQ_OK) return st;
     return quantize_dynamic(stream, input, output, out_scale, scheme, input_dtype, ws, CQ_STATIC_SCRATCH_BYTES);
 }

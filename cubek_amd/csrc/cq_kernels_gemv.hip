@@ -204,6 +204,9 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
     float acc[kRows * kVectors];
 #pragma unroll
     for (int k = 0; k < kRows * kVectors; k++) acc[k] = 0.0f;
+    // Lanes past the end of a row's last strip hold the row's last unit again (see `load`) against zeros of x: their
+    // share is dropped, not added, because an infinite or NaN scale in that unit would turn the zeros into NaN.
+    const auto lane_holds = [&](uint32_t strip) { return strip * 64u + lane < units_per_row; };
     // several vectors: the pairs of the chunk's rows once, then vector after vector against them
     const auto work_vectors = [&](const Chunk& c, uint32_t strip) {
         if constexpr (kVectors > 1) {
@@ -260,7 +263,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
                 }
             }
     #pragma unroll
-            for (int k = 0; k < kRows * kVectors; k++) acc[k] += part[k];
+            for (int k = 0; k < kRows * kVectors; k++) acc[k] += lane_holds(strip) ? part[k] : 0.0f;
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -290,7 +293,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
 #pragma unroll
                     for (uint32_t i = 0; i < kWordVals; i++) a = __builtin_fmaf(v[i], xf[kWordVals * j + i], a);
                 }
-                acc[k] += a;
+                acc[k] += lane_holds(strip) ? a : 0.0f;
             }
             __builtin_amdgcn_sched_barrier(0);
         } else {
@@ -343,7 +346,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_stream_kernel(
                 }
             }
     #pragma unroll
-            for (int k = 0; k < kRows; k++) acc[k] += part[k];
+            for (int k = 0; k < kRows; k++) acc[k] += lane_holds(strip) ? part[k] : 0.0f;
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -570,6 +573,7 @@ bool gemv_streams(const GemvArgs& a) {
             a.scale_stride_row >= (1ull << 32) || (a.cols / a.block_cols) * a.scale_stride_col >= (1ull << 29))
             return false;
     }
+    if (a.x_stride >= (1ull << 32) || a.y_stride >= (1ull << 32)) return false;  // the kernels take them as 32-bit numbers
     return a.cols % vals == 0 && a.cols < (1u << 26) && a.word_pitch % 4 == 0 && a.x_aligned16 && a.words_aligned16;
 }
 
@@ -607,8 +611,19 @@ uint32_t gemv_vectors_per_launch(const GemvArgs& a, uint32_t remaining) {
     return remaining < kBatch ? remaining : kBatch;
 }
 
+// an empty sum: every y is zero
+__global__ void gemv_zero_kernel(void* y, int y_dtype, uint32_t rows, uint32_t vectors, uint64_t y_stride) {
+    const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    for (uint32_t v = 0; v < vectors; v++) store_y(y_dtype, y, static_cast<uint64_t>(v) * y_stride + r, 0.0f);
+}
+
 hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a) {
-    if (a.rows == 0 || a.cols == 0) return hipSuccess;
+    if (a.rows == 0) return hipSuccess;
+    if (a.cols == 0) {
+        hipLaunchKernelGGL(gemv_zero_kernel, dim3((a.rows + 255) / 256), dim3(256), 0, s, a.y, a.y_dtype, a.rows, a.vectors, a.y_stride);
+        return hipGetLastError();
+    }
     for (uint32_t v = 0; v < a.vectors;) {
         GemvArgs b = a;
         b.x = static_cast<const char*>(a.x) + static_cast<uint64_t>(v) * a.x_stride * dtype_bytes(a.dtype);

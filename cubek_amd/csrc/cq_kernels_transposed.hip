@@ -895,11 +895,14 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
     const uint32_t cols = a.segments * a.segment;
     uint32_t seg_magic = 0, seg_shift = 0;
     magic_of(a.segment, &seg_magic, &seg_shift);
+    const uint32_t tile_cols = 32u * (32u / static_cast<uint32_t>(bits));  // 128 bytes of codes per row
+    // A tile stores the scales of the blocks that start in it, as one run per row: blocks divide the tile's columns
+    // (a block of 96 columns would straddle two tiles of 256; such layouts take the kernels below).
     bool tiles = cols < (1u << 31) && a.pitch_f * F::kBytes < (1u << 25) && runs_of_16_bytes<F>(a, a.input) && a.segment % kTilePart == 0 && (kScale == 1 || a.segment == kTilePart) &&
+                 (a.tensor_level || tile_cols % a.segment == 0) &&
                  (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0 && a.vrow % 4 == 0 &&
                  (cols / (32u / static_cast<uint32_t>(bits))) % 4 == 0 && a.batches <= 65535;
     for (uint32_t k = 0; k < a.num_batch_dims; k++) tiles = tiles && a.batch_v[k] % 4 == 0;
-    const uint32_t tile_cols = 32u * (32u / static_cast<uint32_t>(bits));  // 128 bytes of codes per row
     const uint64_t tile_count = static_cast<uint64_t>((a.rows + 64 * kTileRowsPerThread<F> - 1) / (64 * kTileRowsPerThread<F>)) *
                                 ((cols + tile_cols - 1) / tile_cols);
     const dim3 tile_grid(static_cast<uint32_t>((tile_count + 7) / 8 * 8), 1, a.batches);  // see tile_place()

@@ -18,8 +18,9 @@
  *     reference leaves to its JIT backend and its tests do not observe: round() is round-half-to-even,
  *     clamp() is max(lo, min(x, hi)) with minNum/maxNum, so a NaN quotient (NaN element, NaN scale, 0/0)
  *     quantizes to q_max; abs-max ignores NaN elements; a zero result keeps the sign IEEE gives it;
- *   - calls are re-entrant and thread safe: the library keeps no state besides the
- *     per-thread code behind cq_last_hip_error().
+ *   - calls are re-entrant and thread safe.  The library's state is the per-thread code behind
+ *     cq_last_hip_error() and, for cq_quantize_dynamic_static only, one scratch array per GPU inside the
+ *     library's device code, shared by all calls of that entry point on that GPU (see there).
  */
 #ifndef CUBEK_QUANT_H
 #define CUBEK_QUANT_H
@@ -185,8 +186,9 @@ size_t cq_workspace_bytes(const cq_scheme* scheme, uint64_t num_elements);
  * runs on holds its copy until the process ends.  The call allocates and frees nothing.
  *   - a call whose scheme and size need more scratch than the array holds returns
  *     CQ_ERR_SCRATCH_TOO_SMALL (cq_workspace_bytes() tells the need; today no scheme exceeds it);
- *   - the device that is current when the call is made must be the stream's device; the first call
- *     on a device looks the array's address up and must not run under stream capture;
+ *   - the device that is current when the call is made must be the stream's device: a stream of
+ *     another device returns CQ_ERR_INVALID_ARGUMENT (the array's address is per device); the first
+ *     call on a device looks the array's address up and must not run under stream capture;
  *   - all calls on one GPU share that GPU's array: two calls that overlap in time on one GPU
  *     (different streams, or threads) race on it.  Calls on one stream do not overlap. */
 #define CQ_STATIC_SCRATCH_BYTES 1024

@@ -43,7 +43,9 @@ __device__ __forceinline__ float widen(__bf16 s) { return static_cast<float>(s);
 struct FastDivmod {
     uint32_t divisor = 1, magic = 0x80000001u, shift = 31;  // default: division by 1
     FastDivmod() = default;
-    __host__ __device__ explicit FastDivmod(uint32_t d) : divisor(d) {
+    // d == 0 (a dimension of an empty tensor, which no position ever indexes) keeps the division by 1
+    __host__ __device__ explicit FastDivmod(uint32_t d) : divisor(d == 0 ? 1u : d) {
+        if (d == 0) return;
         uint32_t s = 0;
         while ((1ull << s) < d) s++;
         magic = static_cast<uint32_t>((1ull << (31 + s)) / d + 1);

@@ -43,3 +43,14 @@ def test_scales_layout_matches_brute_force_and_oracle(oracle):
     big = (dh.u64((1 << 20, 1 << 10)), 2, 4, dh.u64((128, 1)), dh.u8((32,)), 1)
     for e in ((1 << 31) - 1, 1 << 31, (1 << 32) - 5, (1 << 32) - 1):
         assert L.dh_host_scale_pos(*big, e) == (e // 4096) * 128 + (e % 4096) // 32
+
+
+def test_scales_layout_of_an_empty_tensor_is_built_without_dividing_by_zero():
+    """A zero-sized dimension must not reach the magic-number division on the host (1 << k) / 0; such a layout is
+    never indexed, and a divisor of 0 stands for the division by 1."""
+    L = dh.lib()
+    assert L.dh_host_fast_div(12345, 0) == 12345
+    empty = (dh.u64((0, 8)), 2, 4, dh.u64((1, 1)), dh.u8((32,)), 1)
+    assert L.dh_host_scale_pos(*empty, 0) == 0
+    empty_last = (dh.u64((4, 0)), 2, 4, dh.u64((1, 1)), dh.u8((32,)), 1)
+    assert L.dh_host_scale_pos(*empty_last, 0) == 0

@@ -285,6 +285,77 @@ def test_gemv_scales_with_strides(oracle):
         assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), name
 
 
+@pytest.mark.parametrize("kind", ["e4m3-native", "q4-f32-x", "q4-bf16", "q4-bf16-four-vectors"])
+def test_gemv_infinite_scale_in_a_rows_last_unit(oracle, kind):
+    """Rows whose last strip is partly filled (cols / values per unit is not a multiple of 64), with an infinite scale
+    on the last block of one row and +-0 codes elsewhere in it: the lanes past the row's end must contribute nothing
+    (they hold the last unit again against zeros of x, and Inf * 0 is NaN).  The row with the infinite scale sums to
+    +-Inf or NaN exactly where the float64 product over the oracle's dequantized weights does; every other row is
+    finite and within the tolerance."""
+    import torch
+
+    native = kind == "e4m3-native"
+    elem = ElemType.F32 if kind == "q4-f32-x" else ElemType.BF16
+    vectors = 4 if kind.endswith("four-vectors") else 1
+    value = QuantValue.E4M3 if native else QuantValue.Q4S
+    scheme = QuantScheme.default().with_value(value).with_level(QuantLevel.block([32]))
+    if native:
+        scheme = scheme.with_store(QuantStore.Native)
+    rows, cols = 6, 2080   # 65 units of 32 values (130 of 16 for the bytes): the last strip holds one or two units
+    rng = np.random.default_rng(21)
+    nq = scheme.num_quants()
+    if native:
+        stored = rng.integers(0, 120, (rows, cols), dtype=np.uint8) | (rng.integers(0, 2, (rows, cols), dtype=np.uint8) << 7)
+    else:
+        stored = rng.integers(0, 2**32, (rows, cols // nq), dtype=np.uint64).astype(np.uint32)
+    scales = rng.uniform(0.001, 0.02, (rows, cols // 32)).astype(np.float32)
+    scales[2, -1] = np.inf
+    # that block's codes are all +3 (e4m3: 1.0) and x is +1 there, so row 2 sums to +Inf, not to NaN
+    if native:
+        stored[2, -32:] = 0x38
+    else:
+        stored[2, -(32 // nq):] = 0x33333333
+    deq = oracle.from_bits(oracle.dequantize(stored, (rows, cols), scales, elem, scheme), elem).astype(np.float64)
+    xb = oracle.to_bits(rng.normal(0, 1, (vectors, cols)).astype(np.float32), elem).reshape(vectors, cols)
+    xb[:, -32:] = oracle.to_bits(np.ones(32, np.float32), elem)
+    x64 = oracle.from_bits(xb, elem).astype(np.float64).reshape(vectors, cols)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want, mag = x64 @ deq.T, np.abs(x64) @ np.abs(deq).T
+    d_stored = torch.from_numpy(stored if native else stored.view(np.int32)).cuda()
+    d_scales = torch.from_numpy(scales).cuda()
+    d_x = torch.from_numpy(xb.view(np.int16) if elem != ElemType.F32 else xb).cuda()
+    h = TensorHandleRef.from_torch
+    y = torch.zeros((vectors, rows), dtype=torch.float32, device="cuda")
+    hx, hy = (h(d_x), h(y)) if vectors > 1 else (h(d_x[0]), h(y[0]))
+    matvec.launch_ref(ComputeClient.current(), h(d_stored), h(d_scales), scheme, hx, hy, elem, ElemType.F32)
+    torch.cuda.synchronize()
+    got = y.cpu().numpy().astype(np.float64)
+    finite = np.isfinite(want)
+    assert np.all(want[:, 2] == np.inf) and finite[:, [0, 1, 3, 4, 5]].all()
+    assert np.all(np.abs(got - want)[finite] <= (2e-5 * mag + 1e-30)[finite]), kind
+    assert np.array_equal(np.isnan(got), np.isnan(want)), (kind, got[:, 2], want[:, 2])
+    assert np.array_equal(got[~finite & ~np.isnan(want)], want[~finite & ~np.isnan(want)]), (kind, got[:, 2], want[:, 2])
+
+
+def test_gemv_without_columns_gives_zeros():
+    """cols == 0: every sum is empty, y is written with zeros (one vector and three)."""
+    import torch
+
+    scheme = QuantScheme.default().with_value(QuantValue.Q4S)
+    h = TensorHandleRef
+    w = torch.zeros(4, dtype=torch.int32, device="cuda")
+    s = torch.ones(1, dtype=torch.float32, device="cuda")
+    x = torch.zeros(4, dtype=torch.bfloat16, device="cuda")
+    for vectors in (1, 3):
+        y = torch.full((vectors, 7), float("nan"), dtype=torch.float32, device="cuda")
+        h_x = h(x.data_ptr(), (0,), (1,), 2) if vectors == 1 else h(x.data_ptr(), (vectors, 0), (0, 1), 2)
+        h_y = h.from_torch(y[0]) if vectors == 1 else h.from_torch(y)
+        matvec.launch_ref(ComputeClient.current(), h(w.data_ptr(), (7, 0), (0, 1), 4), h.from_torch(s), scheme, h_x, h_y,
+                          ElemType.BF16, ElemType.F32)
+        torch.cuda.synchronize()
+        assert torch.equal(y, torch.zeros_like(y)), vectors
+
+
 def test_gemv_argument_checks():
     import torch
 

@@ -286,6 +286,10 @@ LARGE_TRANSPOSED_SCHEMES = {
     "q8s_block32": QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([32])),
     "q4s_block64": QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([64])),
     "e5m2_native_tensor": QuantScheme.default().with_value(QuantValue.E5M2).with_store(QuantStore.Native),
+    "q4s_block96": QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([96])),
+    "q8s_block96": QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([96])),
+    "q8s_block160": QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([160])),
+    "q2s_block192": QuantScheme.default().with_value(QuantValue.Q2S).with_level(QuantLevel.block([192])),
 }
 
 
@@ -307,6 +311,17 @@ def test_large_transposed_floats_match_the_contiguous_path(gpu, elem, rows, cols
 def test_transposed_tiles_with_ragged_edges_match_the_contiguous_path(gpu, elem, rows, cols, names):
     """Transposed float tensors of thousands of 64 x 256-byte tiles whose last tiles are cut short along both
     axes (the sizes at which whole tiles go through shared memory), against the contiguous kernels."""
+    transposed_against_contiguous(gpu, elem, rows, cols, names)
+
+
+@pytest.mark.parametrize("elem,rows,cols,names", [
+    (ElemType.BF16, 4128, 8640, ("q4s_block96", "q8s_block96", "q8s_block160", "q2s_block192")),
+    (ElemType.F32, 2064, 8640, ("q4s_block96", "q8s_block160")),
+], ids=["bf16", "f32"])
+def test_large_transposed_floats_with_blocks_that_straddle_tiles(gpu, elem, rows, cols, names):
+    """Blocks of 96, 160 and 192 columns on transposed tensors of more than a thousand tiles: these extents do not
+    divide the 128 / 256 / 512 columns of a tile, so a block may start in one tile and end in the next.  out_scale
+    (given scales) and the codes must equal the contiguous path's."""
     transposed_against_contiguous(gpu, elem, rows, cols, names)
 
 

@@ -317,3 +317,29 @@ def test_native_store_agrees_with_packed_store(oracle, elem):
                 assert set(np.unique(np.abs(ints))) >= {0, 1, 2, 3, 4, 5, 6}  # the data reach every integer
                 on_grid = np.abs(ints) != 5
                 assert np.array_equal(yp[on_grid], yn[on_grid])
+
+
+@pytest.mark.parametrize("elem,value,block,shape", [
+    (ElemType.F32, QuantValue.Q8S, None, (37, 52)),        # 481 words: odd, not a multiple of the 64-word slices
+    (ElemType.BF16, QuantValue.Q4S, 8, (131, 72)),         # 1179 words
+    (ElemType.F16, QuantValue.Q2S, 16, (5, 7, 48)),        # 105 words, rank 3
+    (ElemType.BF16, QuantValue.E2M1, 32, (3, 64)),         # 24 words: fewer than one slice
+], ids=["f32_q8s_tensor", "bf16_q4s_b8", "f16_q2s_b16_rank3", "bf16_e2m1_b32_tiny"])
+def test_threaded_drivers_equal_the_single_threaded_functions(oracle, elem, value, block, shape):
+    """cqo_quantize_packed_mt / cqo_dequantize_packed_mt cut the words into slices for 1 - 17 threads: every word
+    and every out_scale entry must come out as from one call over the whole range (a dropped or doubled slice, or a
+    slice that starts at the wrong word, changes the result)."""
+    rng = np.random.default_rng(len(shape) * 100 + int(value))
+    level = QuantLevel.Tensor if block is None else QuantLevel.block([block])
+    scheme = QuantScheme.default().with_value(value).with_level(level)
+    x = oracle.to_bits(rng.normal(0, 1, shape).astype(np.float32), elem)
+    scale = oracle.compute_scales(x, elem, shape, scheme)
+    words, out_scale = oracle.quantize(x, elem, shape, scale, scheme)
+    deq = oracle.dequantize(words, shape, out_scale, elem, scheme)
+    assert np.count_nonzero(words) > words.size // 2
+    for threads in range(1, 18):
+        w_mt, os_mt = oracle.quantize(x, elem, shape, scale, scheme, threads=threads)
+        assert gc.bits_equal(w_mt, words), threads
+        assert gc.bits_equal(os_mt, out_scale), threads
+        d_mt = oracle.dequantize(words, shape, out_scale, elem, scheme, threads=threads)
+        assert gc.bits_equal(d_mt, deq), threads

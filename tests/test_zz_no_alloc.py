@@ -84,3 +84,27 @@ def test_static_scratch_rejects_bad_arguments():
     s = QuantScheme.default().to_c()
     assert lib.cq_quantize_dynamic_static(None, None, None, None, ctypes.byref(s), 0) == _ffi.ERR_INVALID_ARGUMENT
     assert lib.cq_quantize_dynamic_static(None, None, None, None, None, 0) == _ffi.ERR_INVALID_ARGUMENT
+
+
+def test_static_scratch_on_a_stream_of_its_own():
+    """A non-default stream of the current device: the entry point asks the stream for its device before it resolves
+    the scratch array (a stream of another device would be refused with an invalid-argument status; one GPU cannot
+    show that).  Same codes and scale as on the default stream."""
+    import torch
+
+    scheme = QuantScheme.default().with_value(QuantValue.Q8S)
+    h = TensorHandleRef.from_torch
+    shape = (256, 1024)
+    x = (torch.randn(shape, generator=torch.Generator(device="cpu").manual_seed(3)) * 0.02).to(torch.bfloat16).cuda()
+    outs = []
+    side = torch.cuda.Stream()
+    for stream in (None, side):
+        words = torch.full(scheme.packed_shape(shape), -1, dtype=torch.int32, device="cuda")
+        scales = torch.full((1,), -1.0, dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        client = ComputeClient.current() if stream is None else ComputeClient(stream.cuda_stream)
+        qz.launch_dynamic_static(client, h(x), h(words), h(scales), scheme, ElemType.BF16)
+        torch.cuda.synchronize()
+        outs.append((words, scales))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1].view(torch.int32), outs[1][1].view(torch.int32))
+    assert float(outs[0][1][0]) > 0
