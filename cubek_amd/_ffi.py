@@ -123,8 +123,8 @@ def make_tensor(ptr: int, shape: Sequence[int], strides: Sequence[int], elem_siz
 
 #: enum cq_kernel_family
 FAMILY_NONE, FAMILY_FLAT, FAMILY_FLAT_ROWS, FAMILY_FLAT_LANES, FAMILY_ROWS, FAMILY_BLOCKS, FAMILY_TRANSPOSED, \
-    FAMILY_PER_ELEMENT = range(8)
-FAMILY_NAMES = ("none", "flat", "flat_rows", "flat_lanes", "rows", "blocks", "transposed", "per_element")
+    FAMILY_PER_ELEMENT, FAMILY_STAGED = range(9)
+FAMILY_NAMES = ("none", "flat", "flat_rows", "flat_lanes", "rows", "blocks", "transposed", "per_element", "staged")
 #: enum cq_op
 OP_QUANTIZE, OP_QUANTIZE_DYNAMIC, OP_DEQUANTIZE, OP_COMPUTE_SCALES, OP_GEMV = range(5)
 

@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cstdlib>
 #include <cstring>
 #include <utility>
 
@@ -226,13 +227,15 @@ cq_status make_plan(const cq_scheme* s, const cq_tensor* floats, int dtype, cons
 
 // Can the flat kernels take this launch?  (contiguous scales, 1-D blocks along
 // the last axis that map onto lane groups, 16-byte aligned float tensor)
+// `reads_scales`: the launch reads its scales (given, stored, dequantize): blocks of any whole number of chunks;
+// a fused abs-max takes a power of two of them
 bool flat_ok(const Plan& p, int dtype, const cq_tensor* floats, const cq_tensor* values,
-             const cq_tensor* scale_a, const cq_tensor* scale_b) {
+             const cq_tensor* scale_a, const cq_tensor* scale_b, bool reads_scales) {
     if (p.vs.on || !aligned(floats->ptr, 16) || !aligned(values->ptr, 8)) return false;
     if (p.tensor_level) return true;
     if (!p.last_dim_blocks) return false;
     if (!is_contiguous(scale_a) || (scale_b && !is_contiguous(scale_b))) return false;
-    return cq::flat_block_supported(dtype, p.block_last);
+    return reads_scales ? cq::flat_block_supported_with_scales(dtype, p.block_last) : cq::flat_block_supported(dtype, p.block_last);
 }
 
 // Rows of a tensor as the flat kernels take them: the last dimension contiguous, the rows in front of
@@ -356,7 +359,8 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     // blocks along the last dimension, or (where the scales are given) over the last two: the rows of a block
     // read the same row of scales
     const uint32_t br = scales ? p.layout.block[last - 1] : 1;
-    if (scales && (!(p.last_dim_blocks || (given_scales && scales_rows_ok(p))) || !cq::flat_block_supported(dtype, p.block_last) ||
+    if (scales && (!(p.last_dim_blocks || (given_scales && scales_rows_ok(p))) ||
+                   !(given_scales ? cq::flat_block_supported_with_scales(dtype, p.block_last) : cq::flat_block_supported(dtype, p.block_last)) ||
                    !rows_contiguous(scale_a) || (scale_b && !rows_contiguous(scale_b))))
         return false;
     a->scale_rows = br;
@@ -533,6 +537,80 @@ bool transposed_args(const Plan& p, const cq_scheme* s, int dtype, const cq_tens
     return true;
 }
 
+// Blocks that are not a power-of-two number of lanes, fused abs-max (or given scales): contiguous tensors and
+// scales, one run of blocks (see cq_kernels_staged.hip).  Fills `a` except the data pointers.
+bool pieces_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
+               const cq_tensor* scale_a, const cq_tensor* scale_b, cq::PiecesArgs* a) {
+    if (p.vs.on || p.tensor_level || !p.last_dim_blocks) return false;
+    if (!aligned(floats->ptr, 16) || !aligned(values->ptr, 4)) return false;
+    if (!is_contiguous(scale_a) || (scale_b && !is_contiguous(scale_b))) return false;
+    *a = cq::PiecesArgs{};
+    if (!cq::pieces_supported(dtype, static_cast<int>(p.bits), p.block_last, &a->per, &a->group_log2)) return false;
+    const uint64_t per_chunk = 16 / dtype_size(dtype);
+    a->num_chunks = p.n / per_chunk;
+    if ((p.n * p.bits) % 32 != 0) return false;  // whole words of codes
+    a->param_dtype = param_to_dtype(s->param);
+    a->encoding = flat_encoding(s);
+    a->range = p.range;
+    return true;
+}
+
+// The leading dimensions of a scale tensor as one dimension of rows with a stride of its own (any stride along
+// the last dimension).  False where they do not step uniformly.
+bool scale_rows_and_columns(const cq_tensor* t, uint64_t* row_stride, uint64_t* col_stride) {
+    const uint32_t last = t->rank - 1;
+    *col_stride = t->strides[last];
+    *row_stride = 0;
+    uint64_t expect = 0;
+    bool any = false;
+    for (int d = static_cast<int>(last) - 1; d >= 0; d--) {
+        if (t->shape[d] == 1) continue;
+        if (!any) {
+            any = true;
+            *row_stride = t->strides[d];
+        } else if (t->strides[d] != expect) {
+            return false;
+        }
+        expect = t->strides[d] * t->shape[d];
+    }
+    return true;
+}
+
+// Rows of whole chunks with one pitch per value tensor, 1-D blocks of a power-of-two number of lanes, and scale
+// tensors with a stride along the rows and another along the block columns, neither of which need be 1 (stored
+// column by column, say): the tile kernels that move the scales through LDS (cq_kernels_staged.hip).  The launches
+// before this one have taken the scale tensors whose last dimension is contiguous.  Fills `t` except the data
+// pointers and scale_in_dtype.
+bool scale_tiles_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor* floats, const cq_tensor* values,
+                    const cq_tensor* scale_a, const cq_tensor* scale_b, cq::ScaleTileArgs* t) {
+    if (p.tensor_level || !p.last_dim_blocks || !cq::flat_block_supported(dtype, p.block_last)) return false;
+    const uint32_t last = p.rank - 1;
+    const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
+    const uint32_t stored = s->store == CQ_STORE_U32 ? 4u : 1u;
+    RowLevels lf, lv;
+    if (!row_levels(floats, &lf) || !row_levels(values, &lv) || lf.levels > 1 || lv.levels > 1 || lf.rows != lv.rows) return false;
+    const uint64_t cols = p.shape[last];
+    const uint64_t chunk_elems = per_chunk > 32u / p.bits ? per_chunk : 32u / p.bits;  // whole chunks and whole words of codes
+    if (cols == 0 || cols % chunk_elems || cols / per_chunk >= (1ull << 31) || lf.rows >= (1ull << 31)) return false;
+    const uint32_t chunk_bytes = per_chunk * p.bits / 8;
+    const uint32_t stored_align = chunk_bytes >= 8 ? 8u : 4u;
+    if (!aligned(floats->ptr, 16) || (lf.inner * elem) % 16 || !aligned(values->ptr, stored_align) || (lv.inner * stored) % stored_align)
+        return false;
+    *t = cq::ScaleTileArgs{};
+    if (!scale_rows_and_columns(scale_a, &t->sa_row, &t->sa_col)) return false;
+    if (scale_b && !scale_rows_and_columns(scale_b, &t->sb_row, &t->sb_col)) return false;
+    t->rows = static_cast<uint32_t>(lf.rows);
+    t->row_chunks = static_cast<uint32_t>(cols / per_chunk);
+    const uint32_t group = p.block_last / per_chunk;
+    while ((1u << t->group_log2) < group) t->group_log2++;
+    t->float_pitch = lf.inner * elem;
+    t->stored_pitch = lv.inner * stored;
+    t->param_dtype = param_to_dtype(s->param);
+    t->encoding = flat_encoding(s);
+    t->range = p.range;
+    return true;
+}
+
 // A tensor whose elements fill a buffer without gaps or overlap (a permutation of a contiguous
 // layout): order-free reductions may read the buffer front to back.
 bool is_dense_permutation(const cq_tensor* t) {
@@ -677,7 +755,15 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     const uint64_t per_chunk = 16 / dtype_size(input_dtype);
     uint64_t flat_words = 0;
     const bool streaming = !wraps_its_field(scheme);
-    if (streaming && flat_ok(p, input_dtype, input, output, scale, out_scale)) {
+    cq::PiecesArgs pc;  // EXPERIMENT
+    if (streaming && getenv("CQ_PIECES_GIVEN") && pieces_ok(p, scheme, input_dtype, input, output, scale, out_scale, &pc)) {
+        pc.input = input->ptr;
+        pc.output = output->ptr;
+        pc.scale_in = scale->ptr;
+        pc.scale_out = out_scale->ptr;
+        return CQ_RUN(CQ_FAMILY_STAGED, cq::launch_quantize_pieces(stream, input_dtype, static_cast<int>(p.bits), pc));
+    }
+    if (streaming && flat_ok(p, input_dtype, input, output, scale, out_scale, true)) {
         cq::FlatArgs a{};
         a.input = input->ptr;
         a.output = output->ptr;
@@ -710,6 +796,15 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
         return CQ_RUN(cq::flat_family(fr, input_dtype), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Given, fr));
+    }
+    cq::ScaleTileArgs ts;
+    if (streaming && flat_words == 0 && scale_tiles_ok(p, scheme, input_dtype, input, output, scale, out_scale, &ts)) {
+        ts.input = input->ptr;
+        ts.output = output->ptr;
+        ts.scale_in = scale->ptr;
+        ts.scale_in_dtype = input_dtype;
+        ts.scale_out = out_scale->ptr;
+        return CQ_RUN(CQ_FAMILY_STAGED, cq::launch_quantize_scale_tiles(stream, input_dtype, static_cast<int>(p.bits), ts));
     }
     cq::RowArgs r;
     if (streaming && flat_words == 0 && rows_args(p, scheme, input_dtype, input, output, &r)) {
@@ -760,7 +855,7 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
     uint64_t flat_words = 0;
     // blocks that split a word: only the per-element kernel scales a whole word by its first element's block
     const bool streaming = !p.block_splits_words;
-    if (streaming && flat_ok(p, output_dtype, output, values, params, nullptr)) {
+    if (streaming && flat_ok(p, output_dtype, output, values, params, nullptr, true)) {
         cq::FlatArgs a{};
         a.input = values->ptr;
         a.output = output->ptr;
@@ -787,6 +882,13 @@ cq_status cq_dequantize(cq_stream_t stream, const cq_tensor* values, const cq_te
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
         return CQ_RUN(cq::flat_family(fr, output_dtype), cq::launch_dequantize_flat(stream, output_dtype, p.bits, fr));
+    }
+    cq::ScaleTileArgs ts;
+    if (streaming && flat_words == 0 && scale_tiles_ok(p, scheme, output_dtype, output, values, params, nullptr, &ts)) {
+        ts.input = values->ptr;
+        ts.output = output->ptr;
+        ts.scale_in = params->ptr;
+        return CQ_RUN(CQ_FAMILY_STAGED, cq::launch_dequantize_scale_tiles(stream, output_dtype, static_cast<int>(p.bits), ts));
     }
     cq::RowArgs r;
     if (streaming && flat_words == 0 && rows_args(p, scheme, output_dtype, output, values, &r)) {
@@ -976,7 +1078,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         g.word_end = p.n / p.nq;
         return CQ_RUN(CQ_FAMILY_PER_ELEMENT, cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
     }
-    const bool flat = flat_ok(p, input_dtype, input, output, out_scale, nullptr);
+    const bool flat = flat_ok(p, input_dtype, input, output, out_scale, nullptr, false);
 
     // fused single pass: abs-max, scale, quantize, pack in registers (whole 32-bit words of codes: lanes that
     // share a word store it together)
@@ -1007,6 +1109,23 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         fr.encoding = flat_encoding(scheme);
         fr.range = p.range;
         return CQ_RUN(cq::flat_family(fr, input_dtype), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, fr));
+    }
+
+    // 1-D blocks that are not a power-of-two number of lanes, on one contiguous run: a lane holds a whole piece of its block
+    cq::PiecesArgs pc;
+    if (pieces_ok(p, scheme, input_dtype, input, output, out_scale, nullptr, &pc)) {
+        pc.input = input->ptr;
+        pc.output = output->ptr;
+        pc.scale_out = out_scale->ptr;
+        return CQ_RUN(CQ_FAMILY_STAGED, cq::launch_quantize_pieces(stream, input_dtype, static_cast<int>(p.bits), pc));
+    }
+    // scale tensors whose last dimension is not the contiguous one: the scales of a tile leave through LDS
+    cq::ScaleTileArgs ts;
+    if (scale_tiles_ok(p, scheme, input_dtype, input, output, out_scale, out_scale, &ts)) {
+        ts.input = input->ptr;
+        ts.output = output->ptr;
+        ts.scale_out = out_scale->ptr;
+        return CQ_RUN(CQ_FAMILY_STAGED, cq::launch_quantize_scale_tiles(stream, input_dtype, static_cast<int>(p.bits), ts));
     }
 
     // blocks over the last two dimensions (or 1-D blocks on layouts the flat kernel refuses): one

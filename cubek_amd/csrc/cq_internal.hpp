@@ -53,11 +53,14 @@ struct FlatArgs {
     uint64_t in_outer, out_outer, scale_in_outer, scale_out_outer;
     LaneLevels lanes;     // lanes.levels > 0: `rows` rows of num_chunks chunks addressed lane by lane instead
     uint32_t scale_rows;  // rows > 1, given scales: blocks of this many rows share a row of scales (0 or 1: one)
-    uint32_t block;       // elements per block, 0 = per-tensor
+    uint32_t block;       // elements per block, 0 = per-tensor.  Launches that read their scales (given, stored,
+                          // dequantize) take any whole number of 16-byte chunks, lane by lane where that number is
+                          // not a power of two up to 32; a fused abs-max takes the powers of two
     int param_dtype;      // cq_dtype of the stored scales
     int encoding;         // 0 two's-complement fields (U32 store, native i8); 1 e4m3, 2 e5m2 bytes; 3 e2m1 nibbles
     Range range;
     uint32_t whole_grid = 0;  // set between the launchers' objects only: whole tiles of the run to launch
+    uint32_t any_group = 0;   // set by the launchers: chunks per block where the lane-wise kernels divide by it (see `block`)
 };
 
 enum class ScaleSource { Given, Dynamic, Partials, Stored };  // Stored: lane-wise launches only (FlatArgs::lanes)
@@ -67,6 +70,8 @@ hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource 
 hipError_t launch_dequantize_flat(hipStream_t s, int dtype, int bits, const FlatArgs& a);
 hipError_t launch_scales_flat(hipStream_t s, int dtype, const FlatArgs& a);  // block abs-max -> scales typed like input
 bool flat_block_supported(int dtype, uint32_t block);
+// any whole number of 16-byte chunks: what the flat launches that read their scales take
+bool flat_block_supported_with_scales(int dtype, uint32_t block);
 // the cq_kernel_family a flat launch with these arguments runs on (whole tiles of a run, whole steps of
 // pitched rows, or lane by lane)
 uint32_t flat_family(const FlatArgs& a, int f_dtype);
@@ -170,6 +175,42 @@ hipError_t launch_quantize_blocks_dynamic(hipStream_t s, int dtype, int bits, co
 // per-tensor abs-max partials (same contract as launch_absmax_partials)
 hipError_t launch_absmax_partials_rows(hipStream_t s, int dtype, const RowArgs& a, float* partials,
                                        uint32_t* num_partials);
+
+// Streaming kernels that stage values or scales through LDS (cq_kernels_staged.hip).
+//
+// Pieces: one contiguous run of blocks whose extent is not a power-of-two number of lanes (24, 40, 48 ... values).
+// A block is `per` << group_log2 chunks of 16 bytes: 2^group_log2 neighbouring lanes hold it, `per` (odd) chunks each.
+struct PiecesArgs {
+    const void* input;     // floats
+    void* output;          // stored words
+    const void* scale_in;  // given scales, typed like the input (NULL: the block abs-max is computed in the launch)
+    void* scale_out;       // out_scale typed param_dtype (may be NULL with given scales)
+    int param_dtype, encoding;
+    Range range;
+    uint64_t num_chunks;   // 16-byte chunks of the run: a whole number of blocks
+    uint32_t per, group_log2;
+};
+bool pieces_supported(int dtype, int bits, uint32_t block, uint32_t* per, uint32_t* group_log2);
+hipError_t launch_quantize_pieces(hipStream_t s, int dtype, int bits, const PiecesArgs& a);
+
+// Scale tiles: rows of 16-byte chunks (one uniform pitch per tensor) with 1-D blocks of a power-of-two number of
+// lanes, whose scale tensors have any two strides (stored column by column, with a column stride, ...).  A
+// workgroup takes 32 rows x 64 chunks and moves the tile's scales through LDS, so that the accesses to a scale
+// tensor run along whichever of its two dimensions is closer in memory.
+struct ScaleTileArgs {
+    const void* input;     // floats (quantize) / stored words (dequantize)
+    void* output;
+    const void* scale_in;  // quantize: given scales typed scale_in_dtype, or NULL (abs-max in the launch); dequantize: params
+    void* scale_out;       // quantize: out_scale typed param_dtype, or NULL
+    int scale_in_dtype, param_dtype, encoding;
+    Range range;
+    uint32_t rows, row_chunks;          // rows of the launch, 16-byte chunks of floats per row
+    uint32_t group_log2;                // lanes per block, 2^0 .. 2^5
+    uint64_t float_pitch, stored_pitch; // bytes from row to row
+    uint64_t sa_row, sa_col, sb_row, sb_col;  // strides (elements) of scale_in / scale_out along rows and block columns
+};
+hipError_t launch_quantize_scale_tiles(hipStream_t s, int dtype, int bits, const ScaleTileArgs& a);
+hipError_t launch_dequantize_scale_tiles(hipStream_t s, int dtype, int bits, const ScaleTileArgs& a);
 
 // Transposed float tensors: the memory-fastest dimension is the second to last logical one.
 // Blocks run along the last dimension only (or one scale per tensor).

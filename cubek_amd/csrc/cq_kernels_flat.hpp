@@ -238,6 +238,10 @@ struct LaneRows {
     // for every lane
     uint32_t whole_rows;
     uint32_t group_log2;    // lanes per block as a power of two, for the kernels that take it at run time (kGroupRt)
+    // lanes per block where that is not a power of two (0: it is): blocks of 24 or 40 values ...  Only launches that
+    // read their scales come with it (a fused abs-max needs the power of two for its butterfly): chunk / group_any
+    // as a multiplication and a shift
+    uint32_t group_any, group_magic, group_shift;
     // Tile order (0 = as numbered).  Where whole tiles fit the innermost level and the next level lies closer in
     // memory in the tensor that is read (heads next to each other behind positions, rows of 512 bytes and more),
     // workgroups that run together take the same tile of neighbouring entries of that level: slabs of order_inner x order_outer tiles are walked
@@ -474,11 +478,24 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
     static_assert(kScaleSrc != kScaleStored || kGroup != 0, "stored scales are read back per block only");
     constexpr int kDiv = kGroup <= 0 ? 1 : kGroup;
     constexpr bool kRtGroup = kGroup == kGroupRt;
-    uint32_t group_log2 = 0;
-    if constexpr (kRtGroup) group_log2 = geo.rows.group_log2;
-    // chunk -> its block, and whether it starts one
-    const auto block_of = [&](auto c) { return kRtGroup ? c >> group_log2 : c / kDiv; };
-    const auto starts_block = [&](auto c) { return kRtGroup ? (c & ((1u << group_log2) - 1u)) == 0 : (c % kDiv) == 0; };
+    uint32_t group_log2 = 0, group_any = 0, group_magic = 0, group_shift = 0;
+    if constexpr (kRtGroup) {
+        group_log2 = geo.rows.group_log2;
+        if constexpr (!kDynamic) group_any = geo.rows.group_any, group_magic = geo.rows.group_magic, group_shift = geo.rows.group_shift;
+    }
+    // chunk -> its block, and whether it starts one (group_any is the same for the whole launch: scalar branches)
+    const auto block_of = [&](auto c) {
+        if constexpr (kRtGroup)
+            return group_any != 0 ? static_cast<decltype(c)>(magic_div(static_cast<uint32_t>(c), group_magic, group_shift)) : c >> group_log2;
+        else
+            return c / kDiv;
+    };
+    const auto starts_block = [&](auto c) {
+        if constexpr (kRtGroup)
+            return group_any != 0 ? c == block_of(c) * group_any : (c & ((1u << group_log2) - 1u)) == 0;
+        else
+            return (c % kDiv) == 0;
+    };
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;  // 64, 32, 16 or 8
     // chunks of less than a word of codes in a launch of whole tiles dealt out wave by wave: the words are stored
@@ -702,7 +719,8 @@ __device__ __forceinline__ void dequantize_flat_body(const Geo& geo, int param_d
             w0[u] = w >> ((static_cast<uint32_t>(c) & (kLanesPerWord - 1)) * kChunkBits);
         }
         auto si = kGroup == 0 ? 0 : c / (kGroup <= 0 ? 1 : kGroup);
-        if constexpr (kGroup == kGroupRt) si = c >> geo.rows.group_log2;
+        if constexpr (kGroup == kGroupRt)
+            si = geo.rows.group_any != 0 ? magic_div(c, geo.rows.group_magic, geo.rows.group_shift) : c >> geo.rows.group_log2;
         if constexpr (kParam == CQ_F32)
             sc[u] = F32::load(at.scale_in(u), si);  // a plain load: streamed, the launch takes 4 % longer
         else

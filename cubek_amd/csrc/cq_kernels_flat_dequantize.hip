@@ -16,7 +16,7 @@ hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
     auto out = static_cast<char*>(a.output);
     constexpr int kU = kUnrollD<F, kBits, kGroup>;
     [[maybe_unused]] constexpr uint64_t kInChunk = F::kPerChunk * kBits / 8;  // stored bytes per chunk
-    [[maybe_unused]] constexpr uint64_t kDiv = kGroup == 0 ? 1 : kGroup;
+    [[maybe_unused]] const uint64_t div = kGroup == 0 ? 1 : (a.any_group != 0 ? a.any_group : kGroup);  // chunks per scale
     [[maybe_unused]] const uint64_t param_bytes = kGroup == 0 ? 0 : (a.param_dtype == CQ_F32 ? 4 : 2);
 #if CQ_TU_SAME
     // this object: the whole tiles of a contiguous run, parameters typed like the tensor
@@ -51,8 +51,8 @@ hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
             hipLaunchKernelGGL((dequantize_flat_lanes_kernel<F, kBits, lanes_group(kGroup), kU, kThreads, kEnc>), dim3(grid), dim3(kThreads), 0,
                                s, reinterpret_cast<const uint32_t*>(in + off.chunks * kInChunk),
                                reinterpret_cast<u32x4*>(out + off.chunks * 16),
-                               static_cast<const char*>(a.scale_in) + off.chunks / kDiv * param_bytes, a.param_dtype, tile_begin,
-                               with_group(rows, kGroup));
+                               static_cast<const char*>(a.scale_in) + off.chunks / div * param_bytes, a.param_dtype, tile_begin,
+                               with_group(rows, kGroup, a.any_group));
         });
     return e != hipSuccess ? e : same;
 #endif
@@ -83,7 +83,9 @@ hipError_t CQ_DEQUANTIZE_FLAT_SAME_TU(CQ_TU_FLOAT)(hipStream_t s, int bits, cons
 hipError_t CQ_DEQUANTIZE_FLAT_TU(CQ_TU_FLOAT)(hipStream_t s, int bits, const FlatArgs& a) {
 #endif
     int g = group_of(CQ_TU_FLOAT::kDtype, a.block);
-    CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (dequantize_launch<CQ_TU_FLOAT, kB, kG>(s, a))))
+    FlatArgs b = a;
+    if (g < 0 && (b.any_group = any_group_of(CQ_TU_FLOAT::kDtype, a.block)) != 0) g = shape_group_of(b.any_group);  // lane by lane
+    CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (dequantize_launch<CQ_TU_FLOAT, kB, kG>(s, b))))
 }
 
 }  // namespace cq

@@ -79,6 +79,16 @@ int group_of(int dtype, uint32_t block) {
     return g <= 32 ? static_cast<int>(g) : -1;
 }
 
+// Chunks per block of a block size that group_of() refuses although it is a whole number of chunks (not a power of
+// two, or more than 32): the lane-wise kernels divide by it, for launches that read their scales.  0: none.
+uint32_t any_group_of(int dtype, uint32_t block) {
+    const uint32_t per_chunk = dtype == CQ_F32 ? 4u : 8u;
+    if (block == 0 || block % per_chunk != 0 || group_of(dtype, block) >= 0) return 0;
+    return block / per_chunk;
+}
+// the power-of-two group whose launch shape (loads in flight) a launch with any_group_of() chunks per block takes
+inline int shape_group_of(uint32_t any_group) { return any_group <= 8 ? 8 : 16; }
+
 // Launch shapes from a sweep on MI355X (batches of back-to-back launches,
 // 117 MB - 470 MB tensors): quantize is best with four 16-byte loads in flight
 // per lane; dequantize, which is store-dominated, with two 16-byte stores per lane
@@ -120,9 +130,11 @@ FlatRows flat_rows(const FlatArgs& a) {
 // The lane-wise kernels take the lanes per block at run time (one instantiation for every block size); one scale
 // per tensor (kGroup 0) stays a kernel of its own.
 constexpr int lanes_group(int group) { return group == 0 ? 0 : kGroupRt; }
-inline LaneRows with_group(LaneRows r, int group) {
+inline LaneRows with_group(LaneRows r, int group, uint32_t any_group = 0) {
     r.group_log2 = 0;
     while ((1 << r.group_log2) < group) r.group_log2++;
+    r.group_any = any_group;
+    if (any_group != 0) magic_of(any_group, &r.group_magic, &r.group_shift);
     return r;
 }
 // the most chunks a tile of the lane-wise kernels holds (threads x the deepest unroll in use)
@@ -268,7 +280,7 @@ hipError_t launch_flat(const FlatArgs& a, int f_dtype, int unroll, WholeFn whole
         const LaneRows lr = lane_rows_of_rows(a);
         const uint32_t tiles = static_cast<uint32_t>((static_cast<uint64_t>(lr.total_chunks) + tile - 1) / tile);
         // whole steps: a tile is `unroll` steps in both numberings, so the ragged last tile can go lane by lane
-        const uint32_t full = p32 && a.num_chunks % kThreads == 0 ? static_cast<uint32_t>(lr.total_chunks / tile) : 0u;
+        const uint32_t full = p32 && a.any_group == 0 && a.num_chunks % kThreads == 0 ? static_cast<uint32_t>(lr.total_chunks / tile) : 0u;
         if (full > 0) {
             whole(full, 0ull);
             if ((e = hipGetLastError()) != hipSuccess) return e;
@@ -280,13 +292,14 @@ hipError_t launch_flat(const FlatArgs& a, int f_dtype, int unroll, WholeFn whole
         return e;
     }
     // one contiguous run
-    const uint64_t full = p32 || a.param_dtype == f_dtype ? a.num_chunks / tile : 0;
+    const uint64_t full = (p32 || a.param_dtype == f_dtype) && a.any_group == 0 ? a.num_chunks / tile : 0;
     if (full > 0) {
         whole(static_cast<uint32_t>(full), 0ull);
         if ((e = hipGetLastError()) != hipSuccess) return e;
     }
-    // the rest lane by lane, in pieces the 32-bit chunk numbers of those kernels can hold
-    const uint64_t piece = (1ull << 30);  // a multiple of every tile and every block
+    // the rest lane by lane, in pieces the 32-bit chunk numbers of those kernels can hold: a multiple of every tile and
+    // every power-of-two block, or of whole blocks and whole words of codes
+    const uint64_t piece = a.any_group == 0 ? (1ull << 30) : (1ull << 30) / (4ull * a.any_group) * (4ull * a.any_group);
     for (uint64_t begin = full * tile; begin < a.num_chunks; begin += piece) {
         const uint64_t n = a.num_chunks - begin < piece ? a.num_chunks - begin : piece;
         lanes(lane_rows_of_run(n), 0u, static_cast<uint32_t>((n + tile - 1) / tile), RunOffsets{begin});
@@ -314,13 +327,13 @@ hipError_t quantize_launch_src(hipStream_t s, ScaleSource src, const FlatArgs& a
         // tensors).  Larger outputs stream past the caches.
         {
             const uint64_t chunks = a.num_chunks * (a.rows > 1 ? a.rows : 1);
-            const uint64_t scales = kGroup == 0 ? 0 : chunks / kGroup * (a.param_dtype == CQ_F32 ? 4 : 2);
+            const uint64_t scales = kGroup == 0 ? 0 : chunks / (a.any_group != 0 ? a.any_group : kGroup) * (a.param_dtype == CQ_F32 ? 4 : 2);
             qp.keep = chunks * kOutChunk + scales <= kKeepOutputBytes ? 1u : 0u;
         }
         // bytes per scale of the two scale tensors (per-tensor launches and the partials never move their pointers)
         [[maybe_unused]] const uint64_t scale_in_bytes = kGroup == 0 ? 0 : (kSrc == kScaleStored ? (a.param_dtype == CQ_F32 ? 4 : 2) : F::kBytes);
         [[maybe_unused]] const uint64_t scale_out_bytes = kGroup == 0 ? 0 : (a.param_dtype == CQ_F32 ? 4 : 2);
-        [[maybe_unused]] constexpr uint64_t kDiv = kGroup == 0 ? 1 : kGroup;
+        [[maybe_unused]] const uint64_t div = kGroup == 0 ? 1 : (a.any_group != 0 ? a.any_group : kGroup);  // chunks per scale
 #if CQ_TU_SAME
         // this object: the whole tiles of a contiguous run, parameters typed like the tensor
         if constexpr (kSrc != kScaleStored && F::kBytes == 2) {
@@ -356,13 +369,13 @@ hipError_t quantize_launch_src(hipStream_t s, ScaleSource src, const FlatArgs& a
                 }
             },
             [&](const LaneRows& rows, uint32_t tile_begin, uint32_t grid, RunOffsets off) {
-                const uint64_t scales = off.chunks / kDiv;
+                const uint64_t scales = off.chunks / div;
                 const void* scale_in = a.scale_in == nullptr ? nullptr : static_cast<const char*>(a.scale_in) + scales * scale_in_bytes;
                 void* scale_out = a.scale_out == nullptr ? nullptr : static_cast<char*>(a.scale_out) + scales * scale_out_bytes;
                 hipLaunchKernelGGL((quantize_flat_lanes_kernel<F, kBits, lanes_group(kGroup), kSrc, kWide, kUnrollQ, kThreads, kEnc>),
                                    dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in + off.chunks * 16),
                                    reinterpret_cast<uint32_t*>(out + off.chunks * kOutChunk), scale_in, scale_out,
-                                   a.param_dtype, qp, a.num_partials, tile_begin, with_group(rows, kGroup));
+                                   a.param_dtype, qp, a.num_partials, tile_begin, with_group(rows, kGroup, a.any_group));
             });
         return e != hipSuccess ? e : same;
 #endif

@@ -20,7 +20,11 @@ hipError_t CQ_QUANTIZE_FLAT_SAME_TU(CQ_TU_FLOAT, CQ_TU_GIVEN)(hipStream_t s, int
 hipError_t CQ_QUANTIZE_FLAT_TU(CQ_TU_FLOAT, CQ_TU_GIVEN)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a) {
 #endif
     int g = group_of(CQ_TU_FLOAT::kDtype, a.block);
-    CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (quantize_launch<CQ_TU_FLOAT, kB, kG, CQ_TU_GIVEN != 0>(s, src, a))))
+    FlatArgs b = a;
+    // blocks of another whole number of chunks: lane by lane, for the launches that read their scales
+    if (g < 0 && (src == ScaleSource::Given || src == ScaleSource::Stored) && (b.any_group = any_group_of(CQ_TU_FLOAT::kDtype, a.block)) != 0)
+        g = shape_group_of(b.any_group);
+    CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (quantize_launch<CQ_TU_FLOAT, kB, kG, CQ_TU_GIVEN != 0>(s, src, b))))
 }
 
 }  // namespace cq

@@ -268,7 +268,10 @@ typedef enum cq_kernel_family {
     CQ_FAMILY_ROWS = 4,        /* contiguous last dimension, any blocks and strides (35 - 70 %)                */
     CQ_FAMILY_BLOCKS = 5,      /* fused abs-max + quantize for blocks over the last two dimensions (55 - 70 %) */
     CQ_FAMILY_TRANSPOSED = 6,  /* float tensor whose contiguous dimension is the second to last (45 - 70 %)    */
-    CQ_FAMILY_PER_ELEMENT = 7  /* everything else, one thread per stored element (3 - 30 %)                    */
+    CQ_FAMILY_PER_ELEMENT = 7, /* everything else, one thread per stored element (3 - 30 %)                    */
+    CQ_FAMILY_STAGED = 8       /* streaming kernels with one trip through LDS: fused abs-max over blocks that are
+                                  not a power-of-two number of lanes (24, 40, 48 values), scale tensors stored along
+                                  another dimension than the last                                              */
 } cq_kernel_family;
 
 typedef enum cq_op {

@@ -1,0 +1,340 @@
+"""The streaming kernels that stage values or scales through LDS (cq_kernels_staged.hip), bit for bit against
+the oracle through the C ABI:
+
+* blocks that are not a power-of-two number of 16-byte chunks (24, 40, 48, 72, 120 ... values): fused dynamic
+  quantize on the pieces kernel, given scales and dequantize lane by lane with a division by the block's chunks;
+* scale tensors with any two strides (stored column by column, padded, with a column stride), on tiles of
+  32 rows x 64 chunks whose edges are cut short both ways.
+
+Every case also checks that nothing outside the outputs' views is written."""
+import numpy as np
+import pytest
+
+from cubek_amd import (ComputeClient, ElemType, QuantLevel, QuantParam, QuantScheme, QuantStore, QuantValue,
+                       TensorHandleRef, _ffi)
+from cubek_amd import dequantize as dq
+from cubek_amd import quantize as qz
+
+pytestmark = pytest.mark.gpu
+
+ELEMS = [ElemType.BF16, ElemType.F16, ElemType.F32]
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import gpu_harness
+
+    return gpu_harness
+
+
+def same_bits(a, b):
+    a, b = np.ascontiguousarray(a).reshape(-1), np.ascontiguousarray(b).reshape(-1)
+    return a.shape == b.shape and np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+def scheme_of(value, store, block, param=QuantParam.F32):
+    return (QuantScheme.default().with_value(value).with_store(store).with_param(param)
+            .with_level(QuantLevel.block(list(block))))
+
+
+def plan_family(op, scheme, elem, floats, values, scale, out_scale=None):
+    return _ffi.plan_kind(op, floats, values, scale, out_scale, scheme, elem)
+
+
+# (shape, block, value, store): blocks of 3, 5, 6, 7, 9, 12, 15, 17 and 31 chunks of a 16-bit type; rows that make the
+# last wave ragged; several workgroups
+PIECES = [
+    ((64, 4104), (24,), QuantValue.Q8S, QuantStore.U32),
+    ((7, 33, 120), (40,), QuantValue.Q4S, QuantStore.U32),
+    ((1000, 48), (48,), QuantValue.Q2S, QuantStore.U32),
+    ((129, 1008), (56,), QuantValue.E2M1, QuantStore.U32),
+    ((31, 2160), (72,), QuantValue.Q8F, QuantStore.U32),
+    ((300, 96), (96,), QuantValue.Q4F, QuantStore.U32),
+    ((77, 1080), (120,), QuantValue.E4M3, QuantStore.Native),
+    ((50, 2040), (136,), QuantValue.E5M2, QuantStore.Native),
+    ((9, 4960), (248,), QuantValue.E2M1, QuantStore.Native),
+    ((2000, 24), (24,), QuantValue.Q8S, QuantStore.Native),
+    ((5, 240), (80,), QuantValue.Q2F, QuantStore.U32),
+]
+
+
+@pytest.mark.parametrize("elem", ELEMS, ids=lambda e: e.name)
+@pytest.mark.parametrize("case", PIECES, ids=lambda c: f"{c[2].name}_{c[3].name}_b{c[1][0]}")
+def test_blocks_of_an_odd_number_of_chunks(gpu, oracle, elem, case):
+    shape, block, value, store = case
+    rng = np.random.default_rng(sum(shape) + block[0] + int(elem))
+    for param in (QuantParam.F32, QuantParam.F16 if elem == ElemType.BF16 else QuantParam.BF16):
+        scheme = scheme_of(value, store, block, param)
+        x32 = rng.normal(0, 1.5, shape).astype(np.float32)
+        x32[rng.random(shape) < 0.002] = np.nan
+        x32.reshape(-1)[:block[0]] = 0.0           # an all-zero block: scale 0, 0/0 -> q_max
+        x = oracle.to_bits(x32, elem)
+        s_ref = oracle.compute_scales(x, elem, shape, scheme)
+        w_ref, os_ref = oracle.quantize(x, elem, shape, s_ref, scheme)
+        w_dyn, os_dyn = gpu.quantize_dynamic(x, elem, shape, scheme)
+        assert same_bits(w_dyn, w_ref) and same_bits(os_dyn, os_ref), (param, "dynamic")
+        w_gpu, os_gpu = gpu.quantize(x, elem, shape, s_ref, scheme)
+        assert same_bits(w_gpu, w_ref) and same_bits(os_gpu, os_ref), (param, "given")
+        y_ref = oracle.dequantize(w_ref, shape, os_ref, elem, scheme)
+        y_gpu = gpu.dequantize(w_ref, shape, os_ref, elem, scheme)
+        ok = ~np.isnan(oracle.from_bits(y_ref, elem)).reshape(-1)
+        assert same_bits(y_gpu.reshape(-1)[ok], y_ref.reshape(-1)[ok]), (param, "dequantize")
+        assert np.isnan(oracle.from_bits(y_gpu, elem)).reshape(-1)[~ok].all()
+
+
+def test_odd_blocks_take_the_staged_and_the_lane_wise_kernels():
+    """cq_plan_kind: contiguous bf16 [512, 4104] with blocks of 24: the fused quantize runs on the staged family,
+    given scales and dequantize lane by lane; f32 blocks of 252 values (63 chunks: more than a wave's LDS share holds)
+    stay with the block kernel."""
+    import torch
+
+    h = TensorHandleRef.from_torch
+    for elem, dt, shape, block, dynamic in ((ElemType.BF16, torch.bfloat16, (512, 4104), 24, "staged"),
+                                            (ElemType.F32, torch.float32, (64, 2520), 252, "blocks")):
+        scheme = scheme_of(QuantValue.Q8S, QuantStore.U32, (block,))
+        x = torch.zeros(shape, dtype=dt, device="cuda")
+        w = torch.zeros(scheme.packed_shape(shape), dtype=torch.int32, device="cuda")
+        s = torch.zeros(scheme.scales_shape(shape), dtype=torch.float32, device="cuda")
+        sf = torch.zeros(scheme.scales_shape(shape), dtype=dt, device="cuda")
+        assert plan_family(_ffi.OP_QUANTIZE_DYNAMIC, scheme, elem, h(x), h(w), None, h(s)) == dynamic
+        assert plan_family(_ffi.OP_QUANTIZE, scheme, elem, h(x), h(w), h(sf), h(s)) == "flat_lanes"
+        assert plan_family(_ffi.OP_DEQUANTIZE, scheme, elem, h(x), h(w), h(s)) == "flat_lanes"
+
+
+def test_pieces_with_unaligned_codes_and_more_than_one_workgroup(gpu, oracle):
+    """The stored tensor starts 4 bytes into its allocation (no 16-byte stores), 70 000 blocks of 24 bf16 values
+    (274 waves of the pieces kernel, the last one ragged)."""
+    import torch
+
+    elem, shape = ElemType.BF16, (70000, 24)
+    scheme = scheme_of(QuantValue.Q4S, QuantStore.U32, (24,))
+    rng = np.random.default_rng(77)
+    x = oracle.to_bits(rng.normal(0, 0.3, shape).astype(np.float32), elem)
+    s_ref = oracle.compute_scales(x, elem, shape, scheme)
+    w_ref, os_ref = oracle.quantize(x, elem, shape, s_ref, scheme)
+    pshape = scheme.packed_shape(shape)
+    buf = torch.full((int(np.prod(pshape)) + 2,), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+    view = buf[1:-1].view(pshape)
+    assert view.data_ptr() % 16 == 4
+    os_ = torch.zeros(scheme.scales_shape(shape), dtype=torch.float32, device="cuda")
+    dx = gpu.to_dev(x.reshape(shape))
+    h = TensorHandleRef.from_torch
+    qz.launch_dynamic(ComputeClient.current(), h(dx), h(view), h(os_), scheme, elem)
+    torch.cuda.synchronize()
+    got = buf.cpu().numpy().view(np.uint32)
+    assert got[0] == 0x5A5A5A5A and got[-1] == 0x5A5A5A5A
+    assert np.array_equal(got[1:-1], w_ref.reshape(-1))
+    assert same_bits(os_.cpu().numpy(), os_ref)
+
+
+# ---- scale tensors with two strides ----------------------------------------------------------------------------
+
+def strided_buffer(rng, shape, strides, fill, dtype):
+    """A buffer that holds a [rows, cols] view with the given strides (elements), filled with `fill` elsewhere."""
+    reach = 1 + sum((n - 1) * st for n, st in zip(shape, strides))
+    return np.full(reach, fill, dtype=dtype)
+
+
+def place(buf, values, strides):
+    rows, cols = values.shape
+    idx = (np.arange(rows)[:, None] * strides[0] + np.arange(cols)[None, :] * strides[1]).reshape(-1)
+    buf[idx] = values.reshape(-1)
+    return idx
+
+
+SCALE_LAYOUTS = {
+    "column_major": lambda rows, nb: (1, rows),
+    "column_major_padded": lambda rows, nb: (1, rows + 3),
+    "column_stride_2": lambda rows, nb: (2 * nb + 1, 2),
+    "both_strided": lambda rows, nb: (3, 3 * rows + 2),
+}
+# (rows, cols, block, value, store): tiles cut short along rows (33, 70, 5) and along the row (cols / chunk not a
+# multiple of 64), every width of codes
+TILE_CASES = [
+    (70, 1056, 32, QuantValue.E2M1, QuantStore.U32),
+    (33, 2048, 64, QuantValue.Q8S, QuantStore.U32),
+    (128, 512, 16, QuantValue.Q4S, QuantStore.U32),
+    (5, 4160, 32, QuantValue.Q2S, QuantStore.U32),
+    (40, 1280, 128, QuantValue.E4M3, QuantStore.Native),
+    (64, 640, 32, QuantValue.E2M1, QuantStore.Native),
+    (37, 768, 128, QuantValue.Q8F, QuantStore.Native),
+]
+
+
+@pytest.mark.parametrize("elem", ELEMS, ids=lambda e: e.name)
+@pytest.mark.parametrize("layout", sorted(SCALE_LAYOUTS))
+@pytest.mark.parametrize("case", TILE_CASES, ids=lambda c: f"{c[3].name}_{c[4].name}_{c[0]}x{c[1]}_b{c[2]}")
+def test_scale_tensors_with_two_strides(gpu, oracle, elem, layout, case):
+    import torch
+
+    rows, cols, block, value, store = case
+    if elem == ElemType.F32 and block > 128:
+        block = 128  # 32 lanes of four values at most
+    shape = (rows, cols)
+    nb = cols // block
+    rng = np.random.default_rng(rows * 31 + cols + int(elem))
+    param = {ElemType.BF16: QuantParam.F32, ElemType.F16: QuantParam.F16, ElemType.F32: QuantParam.BF16}[elem]
+    scheme = scheme_of(value, store, (block,), param)
+    pe = gpu.param_elem(scheme)
+    x32 = rng.normal(0, 0.7, shape).astype(np.float32)
+    x32[rng.random(shape) < 0.001] = np.nan
+    x = oracle.to_bits(x32, elem)
+    s_ref = oracle.compute_scales(x, elem, shape, scheme)                  # [rows, nb], typed elem
+    w_ref, os_ref = oracle.quantize(x, elem, shape, s_ref, scheme)         # out_scale typed param
+    y_ref = oracle.dequantize(w_ref, shape, os_ref, elem, scheme)
+    sstr = SCALE_LAYOUTS[layout](rows, nb)
+    ostr = SCALE_LAYOUTS["column_major" if layout != "column_major" else "column_stride_2"](rows, nb)
+    client = ComputeClient.current()
+    h = TensorHandleRef.from_torch
+    hs = lambda t, strides: TensorHandleRef(t.data_ptr(), (rows, nb), tuple(strides), t.element_size())
+    stored_np = np.uint32 if store == QuantStore.U32 else np.uint8
+    pshape = scheme.packed_shape(shape)
+    dx = gpu.to_dev(x.reshape(shape))
+    sent16, sent32 = np.uint16(0x7B7B), np.float32(-777.0)
+    sent = lambda e: sent32 if e == ElemType.F32 else sent16
+    np_of = lambda e: np.float32 if e == ElemType.F32 else np.uint16
+
+    def fresh_out_scale(strides):
+        buf = strided_buffer(rng, (rows, nb), strides, sent(pe), np_of(pe))
+        return gpu.to_dev(buf)
+
+    def check_out_scale(t, strides, what):
+        got = gpu.to_host(t)
+        want = strided_buffer(rng, (rows, nb), strides, sent(pe), np_of(pe))
+        place(want, np.asarray(os_ref).reshape(rows, nb), strides)
+        assert same_bits(got, want), (layout, what)
+
+    # the plan: nothing of this runs one thread per element or on the row kernels
+    sin_buf = strided_buffer(rng, (rows, nb), sstr, sent(elem), np_of(elem))
+    place(sin_buf, np.asarray(s_ref).reshape(rows, nb), sstr)
+    d_sin = gpu.to_dev(sin_buf)
+    d_w = torch.zeros(pshape, dtype=torch.int32 if store == QuantStore.U32 else torch.uint8, device="cuda")
+    d_os = fresh_out_scale(ostr)
+    assert plan_family(_ffi.OP_QUANTIZE, scheme, elem, h(dx), h(d_w), hs(d_sin, sstr), hs(d_os, ostr)) == "staged"
+    assert plan_family(_ffi.OP_QUANTIZE_DYNAMIC, scheme, elem, h(dx), h(d_w), None, hs(d_os, ostr)) == "staged"
+    assert plan_family(_ffi.OP_DEQUANTIZE, scheme, elem, h(dx), h(d_w), hs(d_os, ostr)) == "staged"
+
+    # given scales in one layout, out_scale in another
+    qz.launch_ref(client, h(dx), h(d_w), hs(d_sin, sstr), hs(d_os, ostr), scheme, elem)
+    torch.cuda.synchronize()
+    assert same_bits(gpu.to_host(d_w).view(stored_np), w_ref), (layout, "given")
+    check_out_scale(d_os, ostr, "given out_scale")
+
+    # fused abs-max, out_scale in the first layout
+    d_w2 = torch.zeros_like(d_w)
+    d_os2 = fresh_out_scale(sstr)
+    qz.launch_dynamic(client, h(dx), h(d_w2), hs(d_os2, sstr), scheme, elem)
+    torch.cuda.synchronize()
+    assert same_bits(gpu.to_host(d_w2).view(stored_np), w_ref), (layout, "dynamic")
+    check_out_scale(d_os2, sstr, "dynamic out_scale")
+
+    # dequantize from either
+    for t, strides in ((d_os, ostr), (d_os2, sstr)):
+        d_y = torch.zeros(shape, dtype=gpu.storage_dtype(elem), device="cuda")
+        dq.launch_ref(client, h(d_w), h(d_y), hs(t, strides), scheme, elem)
+        torch.cuda.synchronize()
+        y_gpu = gpu.to_host(d_y)
+        ok = ~np.isnan(oracle.from_bits(y_ref, elem)).reshape(-1)
+        assert same_bits(y_gpu.reshape(-1)[ok], y_ref.reshape(-1)[ok]), (layout, "dequantize")
+        assert np.isnan(oracle.from_bits(y_gpu, elem)).reshape(-1)[~ok].all()
+
+
+def test_scale_tiles_on_pitched_rows(gpu, oracle):
+    """Value tensors with a row pitch of their own (a [100, 1024] view of [100, 1040] floats, codes in rows of 136
+    words) under scales stored column by column: the padding keeps its bytes."""
+    import torch
+
+    elem, rows, cols, block = ElemType.BF16, 100, 1024, 32
+    scheme = scheme_of(QuantValue.Q4S, QuantStore.U32, (block,))
+    nb = cols // block
+    rng = np.random.default_rng(9)
+    x = oracle.to_bits(rng.normal(0, 1, (rows, cols)).astype(np.float32), elem)
+    s_ref = oracle.compute_scales(x, elem, (rows, cols), scheme)
+    w_ref, os_ref = oracle.quantize(x, elem, (rows, cols), s_ref, scheme)
+    y_ref = oracle.dequantize(w_ref, (rows, cols), os_ref, elem, scheme)
+    xbuf = np.full((rows, cols + 16), 0x7F7F, dtype=np.uint16)
+    xbuf[:, :cols] = x.reshape(rows, cols)
+    d_x = gpu.to_dev(xbuf)
+    d_w = torch.full((rows, 136), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+    d_os = torch.full((nb, rows), -5.0, dtype=torch.float32, device="cuda")
+    hx = TensorHandleRef(d_x.data_ptr(), (rows, cols), (cols + 16, 1), 2)
+    hw = TensorHandleRef(d_w.data_ptr(), (rows, cols // 8), (136, 1), 4)
+    hos = TensorHandleRef(d_os.data_ptr(), (rows, nb), (1, rows), 4)
+    client = ComputeClient.current()
+    assert plan_family(_ffi.OP_QUANTIZE_DYNAMIC, scheme, elem, hx, hw, None, hos) == "staged"
+    qz.launch_dynamic(client, hx, hw, hos, scheme, elem)
+    torch.cuda.synchronize()
+    got_w = d_w.cpu().numpy().view(np.uint32)
+    assert np.array_equal(got_w[:, :cols // 8], w_ref.reshape(rows, -1)) and np.all(got_w[:, cols // 8:] == 0x5A5A5A5A)
+    assert same_bits(d_os.cpu().numpy().T, os_ref)
+    d_y = torch.full((rows, cols + 16), 0x7777, dtype=torch.int16, device="cuda")
+    hy = TensorHandleRef(d_y.data_ptr(), (rows, cols), (cols + 16, 1), 2)
+    dq.launch_ref(client, hw, hy, hos, scheme, elem)
+    torch.cuda.synchronize()
+    got_y = d_y.cpu().numpy().view(np.uint16)
+    assert np.array_equal(got_y[:, :cols], y_ref.reshape(rows, cols)) and np.all(got_y[:, cols:] == 0x7777)
+
+
+@pytest.mark.parametrize("what", ["blocks_of_24", "column_major_scales"])
+def test_staged_kernels_at_full_size_match_the_flat_kernels(gpu, what):
+    """bf16 [28672, 8184] with blocks of 24 and [28672, 8192] with scales stored column by column: thousands of
+    workgroups.  Given scales / dequantize of the odd blocks run lane by lane and were checked against the oracle
+    above; here the fused quantize must give the same codes and scales as that path, and the column-major launches
+    the same as the contiguous-scale (flat) ones."""
+    import torch
+
+    h = TensorHandleRef.from_torch
+    client = ComputeClient.current()
+    g = torch.Generator(device="cuda").manual_seed(5)
+    if what == "blocks_of_24":
+        rows, cols, block = 28672, 8184, 24
+        scheme = scheme_of(QuantValue.Q4S, QuantStore.U32, (block,))
+        x = torch.randn((rows, cols), generator=g, device="cuda", dtype=torch.float32).mul_(0.02).to(torch.bfloat16)
+        w1 = torch.zeros(scheme.packed_shape((rows, cols)), dtype=torch.int32, device="cuda")
+        s1 = torch.zeros(scheme.scales_shape((rows, cols)), dtype=torch.float32, device="cuda")
+        qz.launch_dynamic(client, h(x), h(w1), h(s1), scheme, ElemType.BF16)
+        # the same scales, given (typed like the input: they are bf16 values already)
+        w2, s2 = torch.zeros_like(w1), torch.zeros_like(s1)
+        qz.launch_ref(client, h(x), h(w2), h(s1.to(torch.bfloat16)), h(s2), scheme, ElemType.BF16)
+        torch.cuda.synchronize()
+        assert torch.equal(w1, w2) and torch.equal(s1.view(torch.int32), s2.view(torch.int32))
+        # scales against torch: F(2 * absmax / 14) with the division in f32
+        amax = x.view(rows, cols // block, block).abs().amax(dim=2).float()
+        want = ((2 * amax) / 14.0).to(torch.bfloat16).float()
+        assert torch.equal(s1, want)
+        # codes and dequantized values against the same formulas in torch (bf16 arithmetic = the f32 operation rounded
+        # once): clamp(rint(bf16(x / d)), -7, 7) and bf16(scale * code)
+        y = torch.empty_like(x)
+        dq.launch_ref(client, h(w1), h(y), h(s1), scheme, ElemType.BF16)
+        torch.cuda.synchronize()
+        shifts = torch.arange(8, device="cuda", dtype=torch.int32) * 4
+        codes = (w1.unsqueeze(-1) >> shifts) & 15
+        codes = torch.where(codes >= 8, codes - 16, codes).reshape(rows, cols)
+        d = s1.repeat_interleave(block, dim=1)
+        want_codes = (x.float() / d).to(torch.bfloat16).float().round().clamp(-7, 7).to(torch.int32)
+        assert torch.equal(codes, want_codes)
+        assert torch.equal((codes.float() * d).to(torch.bfloat16).view(torch.int16), y.view(torch.int16))
+    else:
+        rows, cols, block = 28672, 8192, 32
+        scheme = scheme_of(QuantValue.E2M1, QuantStore.U32, (block,))
+        nb = cols // block
+        x = torch.randn((rows, cols), generator=g, device="cuda", dtype=torch.float32).mul_(0.02).to(torch.bfloat16)
+        w1 = torch.zeros(scheme.packed_shape((rows, cols)), dtype=torch.int32, device="cuda")
+        s1 = torch.zeros((rows, nb), dtype=torch.float32, device="cuda")
+        qz.launch_dynamic(client, h(x), h(w1), h(s1), scheme, ElemType.BF16)         # flat
+        col = lambda t: TensorHandleRef(t.data_ptr(), (rows, nb), (1, rows), t.element_size())
+        w2 = torch.zeros_like(w1)
+        s2 = torch.zeros((nb, rows), dtype=torch.float32, device="cuda")
+        qz.launch_dynamic(client, h(x), h(w2), col(s2), scheme, ElemType.BF16)       # tiles
+        torch.cuda.synchronize()
+        assert torch.equal(w1, w2) and torch.equal(s1.view(torch.int32), s2.t().contiguous().view(torch.int32))
+        w3 = torch.zeros_like(w1)
+        s3 = torch.zeros((nb, rows), dtype=torch.float32, device="cuda")
+        sin = s2.to(torch.bfloat16)
+        qz.launch_ref(client, h(x), h(w3), col(sin), col(s3), scheme, ElemType.BF16)
+        y1, y2 = torch.empty_like(x), torch.empty_like(x)
+        dq.launch_ref(client, h(w1), h(y1), h(s1), scheme, ElemType.BF16)
+        dq.launch_ref(client, h(w1), h(y2), col(s2), scheme, ElemType.BF16)
+        torch.cuda.synchronize()
+        assert torch.equal(w1, w3) and torch.equal(s2.view(torch.int32), s3.view(torch.int32))
+        assert torch.equal(y1.view(torch.int16), y2.view(torch.int16))

@@ -84,11 +84,20 @@ def test_layouts_land_on_the_family_the_design_claims():
     # transposed float tensor
     got = kinds(e2m1, BF16, (rows, cols), f_strides=(1, rows))
     assert got == {"quantize": "transposed", "dynamic": "transposed", "dequantize": "transposed", "scales": "transposed"}
-    # blocks that are not a power-of-two number of lanes: row kernels (fused block kernel for dynamic)
+    # blocks that are not a power-of-two number of lanes: the fused quantize stages its floats through LDS so that a
+    # lane holds a whole piece of its block; launches that read their scales run lane by lane and divide by the block
     got = kinds(scheme_of(QuantValue.Q4S, [24]), BF16, (8192, 8184))
-    assert got == {"quantize": "rows", "dynamic": "blocks", "dequantize": "rows", "scales": "rows"}
-    # scales stored column-major: row kernels
-    got = kinds(e2m1, BF16, (8192, 8192), s_strides=(1, 8192), ops=("quantize", "dequantize"))
+    assert got == {"quantize": "flat_lanes", "dynamic": "staged", "dequantize": "flat_lanes", "scales": "rows"}
+    # ... on pitched rows the fused quantize stays with the block kernel
+    got = kinds(scheme_of(QuantValue.Q4S, [24]), BF16, (8192, 8184), f_strides=(8192, 1))
+    assert got == {"quantize": "flat_lanes", "dynamic": "blocks", "dequantize": "flat_lanes", "scales": "rows"}
+    # scales stored column-major: tiles of 32 rows whose scales pass through LDS
+    got = kinds(e2m1, BF16, (8192, 8192), s_strides=(1, 8192), ops=("quantize", "dynamic", "dequantize"))
+    assert got == {"quantize": "staged", "dynamic": "staged", "dequantize": "staged"}
+    # ... also on pitched rows; 2-D blocks under such scales stay with the row kernels
+    got = kinds(e2m1, BF16, (8192, 8192), f_strides=(8256, 1), s_strides=(1, 8192), ops=("quantize", "dynamic", "dequantize"))
+    assert got == {"quantize": "staged", "dynamic": "staged", "dequantize": "staged"}
+    got = kinds(scheme_of(QuantValue.E2M1, [4, 32]), BF16, (8192, 8192), s_strides=(1, 2048), ops=("quantize", "dequantize"))
     assert got == {"quantize": "rows", "dequantize": "rows"}
 
 
