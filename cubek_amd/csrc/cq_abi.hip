@@ -6,7 +6,6 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
-#include <cstdlib>
 #include <cstring>
 #include <utility>
 
@@ -755,8 +754,10 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     const uint64_t per_chunk = 16 / dtype_size(input_dtype);
     uint64_t flat_words = 0;
     const bool streaming = !wraps_its_field(scheme);
-    cq::PiecesArgs pc;  // EXPERIMENT
-    if (streaming && getenv("CQ_PIECES_GIVEN") && pieces_ok(p, scheme, input_dtype, input, output, scale, out_scale, &pc)) {
+    // blocks that are not a power-of-two number of lanes on one contiguous run: the kernel of the fused quantize,
+    // reading its scales (bf16 [28672, 8184], blocks of 24: 104 us against 114 us lane by lane)
+    cq::PiecesArgs pc;
+    if (streaming && pieces_ok(p, scheme, input_dtype, input, output, scale, out_scale, &pc)) {
         pc.input = input->ptr;
         pc.output = output->ptr;
         pc.scale_in = scale->ptr;

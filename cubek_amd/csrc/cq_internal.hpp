@@ -195,7 +195,7 @@ hipError_t launch_quantize_pieces(hipStream_t s, int dtype, int bits, const Piec
 
 // Scale tiles: rows of 16-byte chunks (one uniform pitch per tensor) with 1-D blocks of a power-of-two number of
 // lanes, whose scale tensors have any two strides (stored column by column, with a column stride, ...).  A
-// workgroup takes 32 rows x 64 chunks and moves the tile's scales through LDS, so that the accesses to a scale
+// workgroup takes 16 rows x 64 chunks and moves the tile's scales through LDS, so that the accesses to a scale
 // tensor run along whichever of its two dimensions is closer in memory.
 struct ScaleTileArgs {
     const void* input;     // floats (quantize) / stored words (dequantize)

@@ -4,7 +4,7 @@ the oracle through the C ABI:
 * blocks that are not a power-of-two number of 16-byte chunks (24, 40, 48, 72, 120 ... values): fused dynamic
   quantize on the pieces kernel, given scales and dequantize lane by lane with a division by the block's chunks;
 * scale tensors with any two strides (stored column by column, padded, with a column stride), on tiles of
-  32 rows x 64 chunks whose edges are cut short both ways.
+  16 rows x 64 chunks whose edges are cut short both ways.
 
 Every case also checks that nothing outside the outputs' views is written."""
 import numpy as np
@@ -83,21 +83,21 @@ def test_blocks_of_an_odd_number_of_chunks(gpu, oracle, elem, case):
 
 
 def test_odd_blocks_take_the_staged_and_the_lane_wise_kernels():
-    """cq_plan_kind: contiguous bf16 [512, 4104] with blocks of 24: the fused quantize runs on the staged family,
-    given scales and dequantize lane by lane; f32 blocks of 252 values (63 chunks: more than a wave's LDS share holds)
+    """cq_plan_kind: contiguous bf16 [512, 4104] with blocks of 24: quantize (fused or with given scales) runs on
+    the staged family, dequantize lane by lane; f32 blocks of 252 values (63 chunks: more than a wave's LDS share holds)
     stay with the block kernel."""
     import torch
 
     h = TensorHandleRef.from_torch
-    for elem, dt, shape, block, dynamic in ((ElemType.BF16, torch.bfloat16, (512, 4104), 24, "staged"),
-                                            (ElemType.F32, torch.float32, (64, 2520), 252, "blocks")):
+    for elem, dt, shape, block, dynamic, given in ((ElemType.BF16, torch.bfloat16, (512, 4104), 24, "staged", "staged"),
+                                                   (ElemType.F32, torch.float32, (64, 2520), 252, "blocks", "flat_lanes")):
         scheme = scheme_of(QuantValue.Q8S, QuantStore.U32, (block,))
         x = torch.zeros(shape, dtype=dt, device="cuda")
         w = torch.zeros(scheme.packed_shape(shape), dtype=torch.int32, device="cuda")
         s = torch.zeros(scheme.scales_shape(shape), dtype=torch.float32, device="cuda")
         sf = torch.zeros(scheme.scales_shape(shape), dtype=dt, device="cuda")
         assert plan_family(_ffi.OP_QUANTIZE_DYNAMIC, scheme, elem, h(x), h(w), None, h(s)) == dynamic
-        assert plan_family(_ffi.OP_QUANTIZE, scheme, elem, h(x), h(w), h(sf), h(s)) == "flat_lanes"
+        assert plan_family(_ffi.OP_QUANTIZE, scheme, elem, h(x), h(w), h(sf), h(s)) == given
         assert plan_family(_ffi.OP_DEQUANTIZE, scheme, elem, h(x), h(w), h(s)) == "flat_lanes"
 
 
@@ -125,6 +125,62 @@ def test_pieces_with_unaligned_codes_and_more_than_one_workgroup(gpu, oracle):
     assert got[0] == 0x5A5A5A5A and got[-1] == 0x5A5A5A5A
     assert np.array_equal(got[1:-1], w_ref.reshape(-1))
     assert same_bits(os_.cpu().numpy(), os_ref)
+
+
+@pytest.mark.parametrize("elem", ELEMS, ids=lambda e: e.name)
+@pytest.mark.parametrize("value,block,cols", [(QuantValue.Q4S, 24, 1176), (QuantValue.Q8S, 40, 4120), (QuantValue.Q2S, 48, 96)],
+                         ids=["q4s_b24", "q8s_b40", "q2s_b48"])
+def test_odd_blocks_on_pitched_rows(gpu, oracle, elem, value, block, cols):
+    """Rows with a pitch of their own in all three tensors: given scales and dequantize run lane by lane with the
+    division by the block's chunks, the fused quantize on the block kernel.  The padding keeps its bytes."""
+    import torch
+
+    rows = 37
+    scheme = scheme_of(value, QuantStore.U32, (block,))
+    nq, nb = scheme.num_quants(), cols // block
+    rng = np.random.default_rng(block + cols + int(elem))
+    x = oracle.to_bits(rng.normal(0, 1, (rows, cols)).astype(np.float32), elem)
+    s_ref = oracle.compute_scales(x, elem, (rows, cols), scheme)
+    w_ref, os_ref = oracle.quantize(x, elem, (rows, cols), s_ref, scheme)
+    y_ref = oracle.dequantize(w_ref, (rows, cols), os_ref, elem, scheme)
+    esz = 4 if elem == ElemType.F32 else 2
+    pad = 32 // esz
+    fill = np.float32(777.0) if elem == ElemType.F32 else np.uint16(0x7777)
+    xbuf = np.full((rows, cols + pad), fill, dtype=x.dtype)
+    xbuf[:, :cols] = x.reshape(rows, cols)
+    sbuf = np.full((rows, nb + 3), fill, dtype=x.dtype)
+    sbuf[:, :nb] = np.asarray(s_ref).reshape(rows, nb)
+    d_x, d_s = gpu.to_dev(xbuf), gpu.to_dev(sbuf)
+    wcols = cols // nq
+    d_w = torch.full((rows, wcols + 4), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+    d_os = torch.full((rows, nb + 1), -5.0, dtype=torch.float32, device="cuda")
+    hx = TensorHandleRef(d_x.data_ptr(), (rows, cols), (cols + pad, 1), esz)
+    hs = TensorHandleRef(d_s.data_ptr(), (rows, nb), (nb + 3, 1), esz)
+    hw = TensorHandleRef(d_w.data_ptr(), (rows, wcols), (wcols + 4, 1), 4)
+    hos = TensorHandleRef(d_os.data_ptr(), (rows, nb), (nb + 1, 1), 4)
+    client = ComputeClient.current()
+    assert plan_family(_ffi.OP_QUANTIZE, scheme, elem, hx, hw, hs, hos) == "flat_lanes"
+    assert plan_family(_ffi.OP_DEQUANTIZE, scheme, elem, hx, hw, hos) == "flat_lanes"
+
+    def check_stored(what):
+        got_w = d_w.cpu().numpy().view(np.uint32)
+        assert np.array_equal(got_w[:, :wcols], w_ref.reshape(rows, -1)) and np.all(got_w[:, wcols:] == 0x5A5A5A5A), what
+        got_s = d_os.cpu().numpy()
+        assert same_bits(got_s[:, :nb], os_ref) and np.all(got_s[:, nb:] == -5.0), what
+
+    qz.launch_ref(client, hx, hw, hs, hos, scheme, elem)
+    torch.cuda.synchronize()
+    check_stored("given")
+    d_w.fill_(0x5A5A5A5A)
+    d_os.fill_(-5.0)
+    qz.launch_dynamic(client, hx, hw, hos, scheme, elem)
+    torch.cuda.synchronize()
+    check_stored("dynamic")
+    d_y = gpu.to_dev(np.full((rows, cols + pad), fill, dtype=x.dtype))
+    dq.launch_ref(client, hw, TensorHandleRef(d_y.data_ptr(), (rows, cols), (cols + pad, 1), esz), hos, scheme, elem)
+    torch.cuda.synchronize()
+    got_y = gpu.to_host(d_y)
+    assert same_bits(got_y[:, :cols], y_ref.reshape(rows, cols)) and np.all(got_y[:, cols:] == fill)
 
 
 # ---- scale tensors with two strides ----------------------------------------------------------------------------

@@ -84,10 +84,10 @@ def test_layouts_land_on_the_family_the_design_claims():
     # transposed float tensor
     got = kinds(e2m1, BF16, (rows, cols), f_strides=(1, rows))
     assert got == {"quantize": "transposed", "dynamic": "transposed", "dequantize": "transposed", "scales": "transposed"}
-    # blocks that are not a power-of-two number of lanes: the fused quantize stages its floats through LDS so that a
-    # lane holds a whole piece of its block; launches that read their scales run lane by lane and divide by the block
+    # blocks that are not a power-of-two number of lanes: quantize stages its floats through LDS so that a lane holds
+    # a whole piece of its block; dequantize (and quantize on pitched rows) runs lane by lane and divides by the block
     got = kinds(scheme_of(QuantValue.Q4S, [24]), BF16, (8192, 8184))
-    assert got == {"quantize": "flat_lanes", "dynamic": "staged", "dequantize": "flat_lanes", "scales": "rows"}
+    assert got == {"quantize": "staged", "dynamic": "staged", "dequantize": "flat_lanes", "scales": "rows"}
     # ... on pitched rows the fused quantize stays with the block kernel
     got = kinds(scheme_of(QuantValue.Q4S, [24]), BF16, (8192, 8184), f_strides=(8192, 1))
     assert got == {"quantize": "flat_lanes", "dynamic": "blocks", "dequantize": "flat_lanes", "scales": "rows"}
