@@ -15,9 +15,10 @@ the host's share of an eager call bounds them).
 
 value      = algorithmic bytes of one step / wall time per step  (GB/s, 1e9)
              algorithmic bytes = input once + codes once + scales once, per direction
-roofline   = the quantize kernel alone: algorithmic bytes / its average launch duration
-             over a region of K back-to-back launches between two HIP events on the
-             launch stream, against the 8 TB/s HBM peak
+roofline   = the quantize kernel alone: algorithmic bytes / its launch duration, against the 8 TB/s HBM peak.
+             Duration = the median over 50 regions of back-to-back launches, each between two HIP events on
+             the launch stream (timed_median); the average over one region of K launches stands beside it.
+             roofline.per_config holds the same fraction for the three launches of every configuration
 cpu_baseline = the CPU oracle (oracle/cq_oracle.c, the scalar restatement of the
              reference algorithm) on a bounded row sample of the same tensor, best of three
              runs on every hardware thread the job may use
@@ -188,6 +189,36 @@ def timed_region(torch, fn, launches, warmup=3):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     return a.elapsed_time(b) / launches, wall * 1e3 / launches
+
+
+def timed_median(torch, fn, regions=50, warmup=10, region_us=1000.0):
+    """The timing protocol of the per-kernel figures: `warmup` untimed launches, then `regions` (>= 50) regions of
+    back-to-back launches, each bracketed by HIP events recorded on the launch stream (all regions are enqueued
+    first, one synchronize at the end).  A region holds as many launches as fill about `region_us` microseconds
+    (2 .. 256), so that the ~2.5 us an event pair adds stay near 0.3 % of a sample.  Returns the median, mean and
+    minimum of the per-launch times of the regions, in ms, and the launches per region."""
+    for i in range(warmup):
+        fn(i)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(8):
+        fn(i)
+    b.record()
+    torch.cuda.synchronize()
+    est_us = max(a.elapsed_time(b) / 8 * 1e3, 0.5)
+    per = int(min(256, max(2, -(-region_us // est_us))))
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(regions + 1)]
+    events[0].record()
+    k = 0
+    for r in range(regions):
+        for _ in range(per):
+            fn(k)
+            k += 1
+        events[r + 1].record()
+    torch.cuda.synchronize()
+    samples = sorted(events[r].elapsed_time(events[r + 1]) / per for r in range(regions))
+    return {"median_ms": samples[len(samples) // 2], "mean_ms": sum(samples) / len(samples), "min_ms": samples[0],
+            "regions": regions, "launches_per_region": per}
 
 
 def graph_region(torch, paths, method, launches=32, replays=5):
@@ -561,8 +592,9 @@ def adjacent_kernels(torch):
                     "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
     del xa, ya, words, bscales, hxa, hya, hw, hb
-    # the row kernels: blocks that are not a power of two of 16-byte chunks (24 values of 4 bits), and the headline
-    # scheme with its scales stored column by column
+    # the kernels that stage through LDS: blocks that are not a power of two of 16-byte chunks (24 values of 4 bits),
+    # and the headline scheme with its scales stored column by column (given scales: read row by row, out_scale
+    # written column by column)
     for pr, pc, value, block, col_major in ((rows, cols - 8, "Q4S", 24, False), (rows, cols, "E2M1", 32, True)):
         rscheme = QuantScheme.default().with_value(QuantValue[value]).with_level(QuantLevel.block([block]))
         nbk = pc // block
@@ -583,9 +615,8 @@ def adjacent_kernels(torch):
                                                                              hsr[i % sets], rscheme, ElemType.BF16)),
                  ("dequantize", lambda i: cq_dequantize.launch_ref(client, hwr[i % sets], hyr[i % 2], hsr[i % sets], rscheme,
                                                                    ElemType.BF16))]
-        if not col_major:  # cq_quantize_dynamic writes contiguous scales
-            calls.insert(1, ("quantize_dynamic", lambda i: cq_quantize.launch_dynamic(client, hxr[i % sets], hwr[i % sets],
-                                                                                      hsr[i % sets], rscheme, ElemType.BF16)))
+        calls.insert(1, ("quantize_dynamic", lambda i: cq_quantize.launch_dynamic(client, hxr[i % sets], hwr[i % sets],
+                                                                                  hsr[i % sets], rscheme, ElemType.BF16)))
         for label, fn in calls:
             ms = sorted(timed_region(torch, fn, 24)[0] for _ in range(3))[1]
             out.append({"kernel": f"{label}, {what}", "algorithmic_bytes": b, "ms": round(ms, 4),
@@ -681,9 +712,12 @@ def main():
 
     # timed region: exactly K steps between synchronize() calls
     ev_ms, ms_per_step = timed_region(torch, step, args.steps, warmup=args.warmup)
-    # the two kernels of the step, each as its own region of K back-to-back launches
+    # the two kernels of the step, each alone: the average over one region of K back-to-back launches (what a
+    # rocprofv3 kernel trace of this command averages), and the median of 50 event-timed regions
     q_ms, _ = timed_region(torch, lambda i: paths[i % len(paths)].quantize_dynamic(), args.steps)
     d_ms, _ = timed_region(torch, lambda i: paths[i % len(paths)].dequantize(), args.steps)
+    q_med = timed_median(torch, lambda i: paths[i % len(paths)].quantize_dynamic())
+    d_med = timed_median(torch, lambda i: paths[i % len(paths)].dequantize())
 
     yardstick = copy_yardstick(torch, x)
     if args.copy_probe:
@@ -692,8 +726,8 @@ def main():
         torch.cuda.synchronize()
 
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
-    q_gbps = q_bytes / (q_ms * 1e-3) / 1e9
-    d_gbps = q_bytes / (d_ms * 1e-3) / 1e9
+    q_gbps = q_bytes / (q_med["median_ms"] * 1e-3) / 1e9
+    d_gbps = q_bytes / (d_med["median_ms"] * 1e-3) / 1e9
     traffic_table = measured_traffic()
     traffic = traffic_table.get(args.workload, {}).get("quantize_dynamic")
 
@@ -711,13 +745,20 @@ def main():
                       "Cache, so fewer bytes than these cross the HBM interface; `roofline` and `roofline_dequantize` time "
                       "each kernel alone on operands from HBM",
         "elements_per_s": round(2 * n / (ms_per_step * 1e-3)),
+        # achieved / frac: algorithmic bytes over the MEDIAN launch duration of 50 event-timed regions; the average
+        # over one region of K launches (and the regions' mean) stand beside it
         "roofline": {"bound": "hbm", "kernel": "quantize_flat_kernel (fused abs-max+scale+quantize+pack)",
                      "achieved": round(q_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(q_gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "algorithmic_bytes_per_launch": q_bytes, "avg_launch_ms": round(q_ms, 4)},
+                     "algorithmic_bytes_per_launch": q_bytes, "median_launch_ms": round(q_med["median_ms"], 4),
+                     "avg_launch_ms": round(q_ms, 4), "mean_of_regions_ms": round(q_med["mean_ms"], 4),
+                     "frac_at_avg": round(q_bytes / (q_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "regions": q_med["regions"], "launches_per_region": q_med["launches_per_region"]},
         "roofline_dequantize": {"bound": "hbm", "kernel": "dequantize_flat_kernel", "achieved": round(d_gbps, 1),
                                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(d_gbps / HBM_PEAK_GBPS, 4),
-                                "algorithmic_bytes_per_launch": q_bytes, "avg_launch_ms": round(d_ms, 4)},
+                                "algorithmic_bytes_per_launch": q_bytes, "median_launch_ms": round(d_med["median_ms"], 4),
+                                "avg_launch_ms": round(d_ms, 4),
+                                "frac_at_avg": round(q_bytes / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
     }
 
     result["copy_yardstick"] = yardstick
@@ -745,8 +786,10 @@ def main():
                 meth = {"quantize_dynamic": "quantize_dynamic", "quantize_given_scales": "quantize_given",
                         "dequantize": "dequantize"}[label]
                 fn = lambda i, m=meth: getattr(ps[i % len(ps)], m)()
-                med_ms = sorted(timed_region(torch, fn, 32)[0] for _ in range(3))[1]
-                row[label] = {"ms": round(med_ms, 4), "GBps": round(b / (med_ms * 1e-3) / 1e9, 1),
+                med = timed_median(torch, fn)
+                med_ms = med["median_ms"]
+                row[label] = {"ms": round(med_ms, 4), "mean_ms": round(med["mean_ms"], 4),
+                              "GBps": round(b / (med_ms * 1e-3) / 1e9, 1),
                               "frac_hbm_peak": round(b / (med_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                               "traffic": traffic_table.get(name, {}).get(label)}
                 if med_ms < 0.016:  # within four host enqueue times: also as a replayed HIP graph
@@ -763,6 +806,14 @@ def main():
             table.append(row)
             del ps, p, xi
         result["per_config"] = table
+        # the same fractions where a reader of `roofline` alone finds them: [fused dynamic quantize, quantize with
+        # given scales, dequantize] per configuration, median of 50 regions each, and the smallest cell of the three
+        # configurations the 70 % target speaks of
+        short = {"quantize_dynamic": "dynamic", "quantize_given_scales": "given", "dequantize": "dequantize"}
+        result["roofline"]["per_config"] = {
+            row["workload"]: {short[k]: row[k]["frac_hbm_peak"] for k in short} for row in table}
+        result["roofline"]["min_frac_cfg3_5"] = min(
+            row[k]["frac_hbm_peak"] for row in table if row["workload"] in ("cfg3", "cfg4", "cfg5") for k in short)
         result["adjacent_kernels"] = adjacent_kernels(torch) + packed_gemv(torch)
 
     print(json.dumps(result))
