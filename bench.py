@@ -648,6 +648,75 @@ def adjacent_kernels(torch):
     return out
 
 
+def corner_layouts(torch):
+    """Layouts that ran one thread per stored element before they had kernels of their own, on the headline tensor's
+    size: rows that start on odd multiples of 2 bytes, a stored tensor whose last dimension is not the contiguous one,
+    E4M3 in the u32 store (codes that wrap their field), and an abs-max whose output is strided."""
+    from cubek_amd import ComputeClient, ElemType, QuantLevel, QuantScheme, QuantValue, TensorHandleRef, _ffi
+    from cubek_amd import dequantize as cq_dequantize
+    from cubek_amd import quantize as cq_quantize
+    from cubek_amd import reduce as cq_reduce
+
+    client = ComputeClient.current()
+    h = TensorHandleRef.from_torch
+    rows, cols = WORKLOADS["cfg5"]["shape"]
+    sets = 4
+    out = []
+
+    def record(label, b, fn, family):
+        ms = sorted(timed_region(torch, fn, 12, warmup=2)[0] for _ in range(3))[1]
+        out.append({"kernel": label, "family": family, "algorithmic_bytes": b, "ms": round(ms, 4),
+                    "GBps": round(b / (ms * 1e-3) / 1e9, 1), "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+
+    scheme = QuantScheme.default().with_value(QuantValue.E2M1).with_level(QuantLevel.block([32]))
+    words = [torch.empty((rows, cols // 8), dtype=torch.int32, device="cuda") for _ in range(sets)]
+    scales = [torch.empty((rows, cols // 32), dtype=torch.float32, device="cuda") for _ in range(sets)]
+    hw, hs = [h(t) for t in words], [h(t) for t in scales]
+    b = rows * cols * 2 + rows * cols // 2 + rows * cols // 32 * 4
+    # 1. rows of cols + 1 elements: every other row starts on an odd multiple of 2 bytes
+    xo = [torch.randn((rows, cols + 1), device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
+    yo = [torch.empty((rows, cols + 1), device="cuda", dtype=torch.bfloat16) for _ in range(2)]
+    odd = lambda t: TensorHandleRef(h(t).handle, (rows, cols), (cols + 1, 1), 2)
+    hxo, hyo = [odd(t) for t in xo], [odd(t) for t in yo]
+    fam = _ffi.plan_kind(_ffi.OP_QUANTIZE_DYNAMIC, hxo[0], hw[0], None, hs[0], scheme, ElemType.BF16)
+    record(f"quantize_dynamic, e2m1 blocks of 32, bf16 rows [{rows}, {cols}] with a pitch of {cols + 1} elements", b,
+           lambda i: cq_quantize.launch_dynamic(client, hxo[i % sets], hw[i % sets], hs[i % sets], scheme, ElemType.BF16), fam)
+    fam = _ffi.plan_kind(_ffi.OP_DEQUANTIZE, hyo[0], hw[0], hs[0], None, scheme, ElemType.BF16)
+    record(f"dequantize, e2m1 blocks of 32, bf16 rows [{rows}, {cols}] with a pitch of {cols + 1} elements", b,
+           lambda i: cq_dequantize.launch_ref(client, hw[i % sets], hyo[i % 2], hs[i % sets], scheme, ElemType.BF16), fam)
+    del xo, yo, hxo, hyo
+    # 2. the stored tensor transposed in memory: word (r, w) at w * rows + r
+    xs = [torch.randn((rows, cols), device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
+    ys = [torch.empty((rows, cols), device="cuda", dtype=torch.bfloat16) for _ in range(2)]
+    hx, hy = [h(t) for t in xs], [h(t) for t in ys]
+    hwt = [TensorHandleRef(h(t).handle, (rows, cols // 8), (1, rows), 4) for t in words]
+    fam = _ffi.plan_kind(_ffi.OP_QUANTIZE_DYNAMIC, hx[0], hwt[0], None, hs[0], scheme, ElemType.BF16)
+    record(f"quantize_dynamic, e2m1 blocks of 32, bf16 [{rows}, {cols}], stored tensor with strides (1, {rows})", b,
+           lambda i: cq_quantize.launch_dynamic(client, hx[i % sets], hwt[i % sets], hs[i % sets], scheme, ElemType.BF16), fam)
+    fam = _ffi.plan_kind(_ffi.OP_DEQUANTIZE, hy[0], hwt[0], hs[0], None, scheme, ElemType.BF16)
+    record(f"dequantize, e2m1 blocks of 32, bf16 [{rows}, {cols}], stored tensor with strides (1, {rows})", b,
+           lambda i: cq_dequantize.launch_ref(client, hwt[i % sets], hy[i % 2], hs[i % sets], scheme, ElemType.BF16), fam)
+    # 3. E4M3 in the u32 store
+    e4 = QuantScheme.default().with_value(QuantValue.E4M3).with_level(QuantLevel.block([32]))
+    w8 = [torch.empty((rows, cols // 4), dtype=torch.int32, device="cuda") for _ in range(sets)]
+    hw8 = [h(t) for t in w8]
+    b8 = rows * cols * 2 + rows * cols + rows * cols // 32 * 4
+    fam = _ffi.plan_kind(_ffi.OP_QUANTIZE_DYNAMIC, hx[0], hw8[0], None, hs[0], e4, ElemType.BF16)
+    record(f"quantize_dynamic, e4m3 in the u32 store (fields wrap), blocks of 32, bf16 [{rows}, {cols}]", b8,
+           lambda i: cq_quantize.launch_dynamic(client, hx[i % sets], hw8[i % sets], hs[i % sets], e4, ElemType.BF16), fam)
+    del w8, hw8
+    # 4. abs-max along the rows into column 1 of a [rows, 4] tensor, and along the columns into every other element
+    for axis, oshape, ostr in ((1, (rows, 1), (4, 1)), (0, (1, cols), (2 * cols, 2))):
+        o = torch.zeros(rows * 4 if axis == 1 else cols * 2, device="cuda", dtype=torch.bfloat16)
+        ho = TensorHandleRef(o.data_ptr() + (2 if axis == 1 else 0), oshape, ostr, 2)
+        nbytes = cq_reduce.workspace_bytes(hx[0], axis, ElemType.BF16)
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+        record(f"reduce_max_abs axis {axis} of bf16 [{rows}, {cols}] into an output with strides {ostr}", rows * cols * 2,
+               lambda i: cq_reduce.max_abs(client, hx[i % sets], ho, axis, ElemType.BF16, ws.data_ptr() if nbytes else 0, nbytes),
+               "-")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -660,6 +729,8 @@ def main():
                     help="run only the abs-max / re-pack kernels on the headline tensor (for profiling)")
     ap.add_argument("--gemv-only", action="store_true",
                     help="run only the matrix-vector product over packed weights (for profiling)")
+    ap.add_argument("--corners-only", action="store_true",
+                    help="run only the layouts that used to run one thread per element (for profiling)")
     ap.add_argument("--matrix", action="store_true",
                     help="run only the float type x value x store matrix on the headline shape (reported only)")
     ap.add_argument("--copy-probe", action="store_true",
@@ -678,7 +749,10 @@ def main():
     torch.cuda.set_device(0)
 
     if args.adjacent_only:
-        print(json.dumps({"adjacent_kernels": adjacent_kernels(torch) + packed_gemv(torch)}))
+        print(json.dumps({"adjacent_kernels": adjacent_kernels(torch) + corner_layouts(torch) + packed_gemv(torch)}))
+        return
+    if args.corners_only:
+        print(json.dumps({"adjacent_kernels": corner_layouts(torch)}))
         return
     if args.gemv_only:
         print(json.dumps({"adjacent_kernels": packed_gemv(torch)}))
@@ -814,7 +888,7 @@ def main():
             row["workload"]: {short[k]: row[k]["frac_hbm_peak"] for k in short} for row in table}
         result["roofline"]["min_frac_cfg3_5"] = min(
             row[k]["frac_hbm_peak"] for row in table if row["workload"] in ("cfg3", "cfg4", "cfg5") for k in short)
-        result["adjacent_kernels"] = adjacent_kernels(torch) + packed_gemv(torch)
+        result["adjacent_kernels"] = adjacent_kernels(torch) + corner_layouts(torch) + packed_gemv(torch)
 
     print(json.dumps(result))
 

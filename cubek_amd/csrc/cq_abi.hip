@@ -346,9 +346,10 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
     const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
     const uint32_t stored = s->store == CQ_STORE_U32 ? 4u : 1u;
     const auto rows_contiguous = [&](const cq_tensor* t) { return t->shape[last] == 1 || t->strides[last] == 1; };
-    // 16-byte loads and 8-byte stores at any multiple of 4 bytes: the hardware takes them, at some cost in
-    // cache lines crossed, and whole-chunk alignment is what the other flat launches are for
-    if (!rows_contiguous(floats) || !aligned(floats->ptr, 4)) return false;
+    // 16-byte accesses to the floats at any multiple of their element size (rows that start on odd multiples of
+    // 2 bytes included), 8-byte stores of codes at any multiple of 4 bytes: global memory takes unaligned accesses,
+    // at some cost in cache lines crossed, and whole-chunk alignment is what the other flat launches are for
+    if (!rows_contiguous(floats) || !aligned(floats->ptr, elem)) return false;
     if (values && (!rows_contiguous(values) || !aligned(values->ptr, 4))) return false;  // NULL: scales only
     const uint64_t cols = p.shape[last];
     // whole chunks and whole 32-bit words of codes (lanes that share a word store it together)
@@ -372,7 +373,7 @@ bool lane_rows_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tensor*
         const uint64_t in = floats->strides[d] * elem, out = values ? values->strides[d] * stored : in;
         const uint64_t scale_in = scales ? scale_a->strides[d] * scale_a_size : 0;
         const uint64_t scale_out = scales && scale_b ? scale_b->strides[d] * scale_b_size : 0;
-        if (in == 0 || out == 0 || in % 4 || out % 4) return false;  // broadcast or misaligned rows
+        if (in == 0 || out == 0 || out % 4) return false;  // broadcast rows, or codes off their words
         const uint32_t k = l.levels;
         // entries of the level inside this one as the scales count them: blocks of rows at the innermost level
         const uint64_t scale_count = k == 1 && br > 1 ? l.count[0] / br : (k > 0 ? l.count[k - 1] : 0);
@@ -419,9 +420,10 @@ void scale_in_to_out(cq::FlatArgs* a) {
     }
 }
 
-// E4M3 / E5M2 in the U32 store: the reference packs the rounded integer (up to +-448 / +-57344) into an 8-bit
-// field with `i32 & mask` (src/quantize.rs:75), so most codes wrap.  Faithfully reproduced, but only by the
-// per-element kernels: no streaming kernel is built for a combination nobody can use.
+// E4M3 / E5M2 in the U32 store: the reference sends every U32 scheme to quantize_packed (src/quantize.rs:185-191),
+// which packs the rounded integer (up to +-448 / +-57344) into an 8-bit field with `i32 & mask` (src/quantize.rs:75),
+// so most codes wrap.  The flat launches take them lane by lane (the one geometry compiled with wrapping fields);
+// the row, block, tile and transposed kernels do not, and such layouts run per element.
 bool wraps_its_field(const cq_scheme* s) {
     return s->store == CQ_STORE_U32 && (s->value == CQ_VALUE_E4M3 || s->value == CQ_VALUE_E5M2);
 }
@@ -587,12 +589,22 @@ bool scale_tiles_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tenso
     const uint32_t elem = dtype_size(dtype), per_chunk = 16u / elem;
     const uint32_t stored = s->store == CQ_STORE_U32 ? 4u : 1u;
     RowLevels lf, lv;
-    if (!row_levels(floats, &lf) || !row_levels(values, &lv) || lf.levels > 1 || lv.levels > 1 || lf.rows != lv.rows) return false;
+    if (!row_levels(floats, &lf) || lf.levels > 1) return false;
+    // the stored tensor: rows with one pitch, or (words of the U32 store) a stride along the last dimension as well,
+    // in which case the codes of a tile pass through LDS like its scales
+    uint64_t stored_col = 1;
+    if (row_levels(values, &lv)) {
+        if (lv.levels > 1 || lf.rows != lv.rows) return false;
+    } else {
+        uint64_t v_row = 0;
+        if (s->store != CQ_STORE_U32 || !scale_rows_and_columns(values, &v_row, &stored_col) || stored_col == 0) return false;
+        lv = RowLevels{1, lf.rows, lf.rows, v_row, 0};
+    }
     const uint64_t cols = p.shape[last];
     const uint64_t chunk_elems = per_chunk > 32u / p.bits ? per_chunk : 32u / p.bits;  // whole chunks and whole words of codes
     if (cols == 0 || cols % chunk_elems || cols / per_chunk >= (1ull << 31) || lf.rows >= (1ull << 31)) return false;
     const uint32_t chunk_bytes = per_chunk * p.bits / 8;
-    const uint32_t stored_align = chunk_bytes >= 8 ? 8u : 4u;
+    const uint32_t stored_align = chunk_bytes >= 8 && stored_col == 1 ? 8u : 4u;  // (staged codes leave word by word)
     if (!aligned(floats->ptr, 16) || (lf.inner * elem) % 16 || !aligned(values->ptr, stored_align) || (lv.inner * stored) % stored_align)
         return false;
     *t = cq::ScaleTileArgs{};
@@ -604,6 +616,7 @@ bool scale_tiles_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tenso
     while ((1u << t->group_log2) < group) t->group_log2++;
     t->float_pitch = lf.inner * elem;
     t->stored_pitch = lv.inner * stored;
+    t->stored_col = stored_col;
     t->param_dtype = param_to_dtype(s->param);
     t->encoding = flat_encoding(s);
     t->range = p.range;
@@ -753,7 +766,8 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
     const bool native = scheme->store == CQ_STORE_NATIVE;
     const uint64_t per_chunk = 16 / dtype_size(input_dtype);
     uint64_t flat_words = 0;
-    const bool streaming = !wraps_its_field(scheme);
+    const bool wraps = wraps_its_field(scheme);  // the flat launches take such fields (lane by lane), the others do not
+    const bool streaming = !wraps;
     // blocks that are not a power-of-two number of lanes on one contiguous run: the kernel of the fused quantize,
     // reading its scales (bf16 [28672, 8184], blocks of 24: 104 us against 114 us lane by lane)
     cq::PiecesArgs pc;
@@ -764,8 +778,9 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         pc.scale_out = out_scale->ptr;
         return CQ_RUN(CQ_FAMILY_STAGED, cq::launch_quantize_pieces(stream, input_dtype, static_cast<int>(p.bits), pc));
     }
-    if (streaming && flat_ok(p, input_dtype, input, output, scale, out_scale, true)) {
+    if (flat_ok(p, input_dtype, input, output, scale, out_scale, true)) {
         cq::FlatArgs a{};
+        a.lanes_only = wraps;
         a.input = input->ptr;
         a.output = output->ptr;
         a.scale_in = scale->ptr;
@@ -783,10 +798,11 @@ cq_status cq_quantize(cq_stream_t stream, const cq_tensor* input, const cq_tenso
         flat_words = a.num_chunks * per_chunk / p.nq;
     }
     cq::FlatArgs fr{};
-    if (streaming && flat_words == 0 && (flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
+    if (flat_words == 0 && (flat_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
                                          dtype_size(pd), true, &fr) ||
                             lane_rows_ok(p, scheme, input_dtype, input, output, scale, dtype_size(input_dtype), out_scale,
                                          dtype_size(pd), true, &fr))) {
+        fr.lanes_only = wraps;
         fr.input = input->ptr;
         fr.output = output->ptr;
         fr.scale_in = scale->ptr;
@@ -1065,20 +1081,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
 
     const uint64_t per_chunk = 16 / dtype_size(input_dtype);
     const bool native = scheme->store == CQ_STORE_NATIVE;
-    if (wraps_its_field(scheme)) {
-        // scales into out_scale, then the per-element quantize reading them back
-        st = produce_scales(stream, p, scheme, input, input_dtype, out_scale, pd, workspace, workspace_bytes);
-        if (st != CQ_OK) return st;
-        cq::GenericArgs g = generic_args(p, scheme);
-        g.input = input->ptr;
-        g.output = output->ptr;
-        g.scale_in = out_scale->ptr;
-        g.scale_in_dtype = pd;
-        g.scale_out = nullptr;
-        g.word_begin = 0;
-        g.word_end = p.n / p.nq;
-        return CQ_RUN(CQ_FAMILY_PER_ELEMENT, cq::launch_quantize_generic(stream, input_dtype, p.bits, g));
-    }
+    const bool wraps = wraps_its_field(scheme);  // the flat launches take such fields (lane by lane), the others do not
     const bool flat = flat_ok(p, input_dtype, input, output, out_scale, nullptr, false);
 
     // fused single pass: abs-max, scale, quantize, pack in registers (whole 32-bit words of codes: lanes that
@@ -1094,6 +1097,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
         a.range = p.range;
+        a.lanes_only = wraps;
         return CQ_RUN(cq::flat_family(a, input_dtype), cq::launch_quantize_flat(stream, input_dtype, p.bits, cq::ScaleSource::Dynamic, a));
     }
 
@@ -1105,6 +1109,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         fr.output = output->ptr;
         fr.scale_out = out_scale->ptr;
         scale_in_to_out(&fr);
+        fr.lanes_only = wraps;
         fr.block = p.block_last;
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
@@ -1114,7 +1119,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
 
     // 1-D blocks that are not a power-of-two number of lanes, on one contiguous run: a lane holds a whole piece of its block
     cq::PiecesArgs pc;
-    if (pieces_ok(p, scheme, input_dtype, input, output, out_scale, nullptr, &pc)) {
+    if (!wraps && pieces_ok(p, scheme, input_dtype, input, output, out_scale, nullptr, &pc)) {
         pc.input = input->ptr;
         pc.output = output->ptr;
         pc.scale_out = out_scale->ptr;
@@ -1122,7 +1127,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
     }
     // scale tensors whose last dimension is not the contiguous one: the scales of a tile leave through LDS
     cq::ScaleTileArgs ts;
-    if (scale_tiles_ok(p, scheme, input_dtype, input, output, out_scale, out_scale, &ts)) {
+    if (!wraps && scale_tiles_ok(p, scheme, input_dtype, input, output, out_scale, out_scale, &ts)) {
         ts.input = input->ptr;
         ts.output = output->ptr;
         ts.scale_out = out_scale->ptr;
@@ -1143,6 +1148,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
             f2.input = input->ptr;
             f2.output = output->ptr;
             f2.scale_in = out_scale->ptr;
+            f2.lanes_only = wraps;
             f2.block = p.block_last;
             f2.param_dtype = pd;
             f2.encoding = flat_encoding(scheme);
@@ -1152,7 +1158,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
     }
 
     cq::RowArgs rb;
-    if (!p.tensor_level && scales_rows_ok(p) && rows_args(p, scheme, input_dtype, input, output, &rb) &&
+    if (!wraps && !p.tensor_level && scales_rows_ok(p) && rows_args(p, scheme, input_dtype, input, output, &rb) &&
         cq::blocks_dynamic_supported(input_dtype, static_cast<int>(p.bits), rb)) {
         rb.input = input->ptr;
         rb.output = output->ptr;
@@ -1161,7 +1167,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
     }
 
     cq::TransposedArgs tr;
-    const bool transposed = !flat && transposed_args(p, scheme, input_dtype, input, output, &tr);
+    const bool transposed = !wraps && !flat && transposed_args(p, scheme, input_dtype, input, output, &tr);
     if (transposed && !p.tensor_level) {  // each thread owns whole blocks: one launch
         tr.input = input->ptr;
         tr.output = output->ptr;
@@ -1190,6 +1196,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         a.num_partials = num_partials;
         a.scale_out = out_scale->ptr;
         a.num_chunks = flat_chunks;
+        a.lanes_only = wraps;
         a.block = 0;
         a.param_dtype = pd;
         a.encoding = flat_encoding(scheme);
@@ -1208,6 +1215,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         fr.scale_in = workspace;
         fr.num_partials = num_partials;
         fr.scale_out = out_scale->ptr;
+        fr.lanes_only = wraps;
         fr.block = 0;
         fr.param_dtype = pd;
         fr.encoding = flat_encoding(scheme);
@@ -1220,7 +1228,7 @@ static cq_status quantize_dynamic(cq_stream_t stream, const cq_tensor* input, co
         if (st != CQ_OK) return st;
     }
     cq::RowArgs r;
-    if (flat_words == 0 && rows_args(p, scheme, input_dtype, input, output, &r)) {
+    if (!wraps && flat_words == 0 && rows_args(p, scheme, input_dtype, input, output, &r)) {
         r.input = input->ptr;
         r.output = output->ptr;
         r.scale_in = out_scale->ptr;
@@ -1497,7 +1505,8 @@ cq_status cq_reduce_max_abs(cq_stream_t stream, const cq_tensor* input, const cq
     a.rank = input->rank;
     a.axis = axis;
     a.out_contiguous = is_contiguous(output);
-    a.contiguous = is_contiguous(input) && a.out_contiguous;
+    a.in_contiguous = is_contiguous(input);
+    a.contiguous = a.in_contiguous && a.out_contiguous;
     reduce_view(input, axis, &a.outer, &a.len, &a.inner);
     if (a.outer == 0 || a.inner == 0) return CQ_OK;  // no outputs
     return hip_status(cq::launch_reduce_max_abs(stream, dtype, a));

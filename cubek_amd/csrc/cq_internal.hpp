@@ -61,6 +61,7 @@ struct FlatArgs {
     Range range;
     uint32_t whole_grid = 0;  // set between the launchers' objects only: whole tiles of the run to launch
     uint32_t any_group = 0;   // set by the launchers: chunks per block where the lane-wise kernels divide by it (see `block`)
+    bool lanes_only = false;  // set by the launchers: no whole-tile kernel exists for this launch (fields that wrap)
 };
 
 enum class ScaleSource { Given, Dynamic, Partials, Stored };  // Stored: lane-wise launches only (FlatArgs::lanes)
@@ -133,6 +134,7 @@ struct ReduceArgs {
     uint64_t shape[CQ_MAX_RANK];
     uint64_t in_strides[CQ_MAX_RANK], out_strides[CQ_MAX_RANK];
     bool contiguous;         // input and output are contiguous row-major
+    bool in_contiguous;      // the input is
     bool out_contiguous;     // the output is
     uint64_t outer, len, inner;  // the contiguous view [outer, len, inner] around the axis
 };
@@ -207,6 +209,8 @@ struct ScaleTileArgs {
     uint32_t rows, row_chunks;          // rows of the launch, 16-byte chunks of floats per row
     uint32_t group_log2;                // lanes per block, 2^0 .. 2^5
     uint64_t float_pitch, stored_pitch; // bytes from row to row
+    uint64_t stored_col;                // stored elements from one to the next along the last dimension; other than 1
+                                        // (words of the U32 store only): the codes of a tile pass through LDS too
     uint64_t sa_row, sa_col, sb_row, sb_col;  // strides (elements) of scale_in / scale_out along rows and block columns
 };
 hipError_t launch_quantize_scale_tiles(hipStream_t s, int dtype, int bits, const ScaleTileArgs& a);

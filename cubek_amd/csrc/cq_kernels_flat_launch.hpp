@@ -79,6 +79,9 @@ int group_of(int dtype, uint32_t block) {
     return g <= 32 ? static_cast<int>(g) : -1;
 }
 
+// two's-complement fields of a value range wider than 8 bits (E4M3 / E5M2 in the U32 store)
+inline bool fields_wrap(const FlatArgs& a) { return a.encoding == 0 && (a.range.hi > 127.0f || a.range.lo < -128.0f); }
+
 // Chunks per block of a block size that group_of() refuses although it is a whole number of chunks (not a power of
 // two, or more than 32): the lane-wise kernels divide by it, for launches that read their scales.  0: none.
 uint32_t any_group_of(int dtype, uint32_t block) {
@@ -280,7 +283,7 @@ hipError_t launch_flat(const FlatArgs& a, int f_dtype, int unroll, WholeFn whole
         const LaneRows lr = lane_rows_of_rows(a);
         const uint32_t tiles = static_cast<uint32_t>((static_cast<uint64_t>(lr.total_chunks) + tile - 1) / tile);
         // whole steps: a tile is `unroll` steps in both numberings, so the ragged last tile can go lane by lane
-        const uint32_t full = p32 && a.any_group == 0 && a.num_chunks % kThreads == 0 ? static_cast<uint32_t>(lr.total_chunks / tile) : 0u;
+        const uint32_t full = p32 && a.any_group == 0 && !a.lanes_only && a.num_chunks % kThreads == 0 ? static_cast<uint32_t>(lr.total_chunks / tile) : 0u;
         if (full > 0) {
             whole(full, 0ull);
             if ((e = hipGetLastError()) != hipSuccess) return e;
@@ -292,7 +295,7 @@ hipError_t launch_flat(const FlatArgs& a, int f_dtype, int unroll, WholeFn whole
         return e;
     }
     // one contiguous run
-    const uint64_t full = (p32 || a.param_dtype == f_dtype) && a.any_group == 0 ? a.num_chunks / tile : 0;
+    const uint64_t full = (p32 || a.param_dtype == f_dtype) && a.any_group == 0 && !a.lanes_only ? a.num_chunks / tile : 0;
     if (full > 0) {
         whole(static_cast<uint32_t>(full), 0ull);
         if ((e = hipGetLastError()) != hipSuccess) return e;
@@ -336,7 +339,7 @@ hipError_t quantize_launch_src(hipStream_t s, ScaleSource src, const FlatArgs& a
         [[maybe_unused]] const uint64_t div = kGroup == 0 ? 1 : (a.any_group != 0 ? a.any_group : kGroup);  // chunks per scale
 #if CQ_TU_SAME
         // this object: the whole tiles of a contiguous run, parameters typed like the tensor
-        if constexpr (kSrc != kScaleStored && F::kBytes == 2) {
+        if constexpr (kSrc != kScaleStored && F::kBytes == 2 && !kWide) {
             hipLaunchKernelGGL((quantize_flat_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc, F::kDtype>),
                                dim3(a.whole_grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
                                reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0ull,
@@ -350,7 +353,7 @@ hipError_t quantize_launch_src(hipStream_t s, ScaleSource src, const FlatArgs& a
         const hipError_t e = launch_flat(
             a, F::kDtype, kUnrollQ,
             [&](uint32_t grid, uint64_t) {
-                if constexpr (kSrc != kScaleStored) {
+                if constexpr (kSrc != kScaleStored && !kWide) {  // (fields that wrap: lane by lane only)
                     if (a.param_dtype != CQ_F32) {  // a contiguous run, parameters typed like the tensor
                         FlatArgs b = a;
                         b.whole_grid = grid;
@@ -401,8 +404,16 @@ template <class F, int kBits, int kGroup, bool kGiven>
 hipError_t quantize_launch(hipStream_t s, ScaleSource src, const FlatArgs& a) {
     switch (a.encoding) {
         case kEncInt:
-            // value ranges wider than their field (E4M3 / E5M2 in the U32 store) never come here
-            if (kBits == 8 && (a.range.hi > 127.0f || a.range.lo < -128.0f)) return hipErrorInvalidValue;
+            // value ranges wider than their field (E4M3 / E5M2 in the U32 store): fields wrap like the reference's
+            // `i32 & mask` (src/quantize.rs:75), lane by lane only (FlatArgs::lanes_only, set by the caller)
+            if (fields_wrap(a)) {
+                if constexpr (kBits == 8) {
+                    if (!a.lanes_only) return hipErrorInvalidValue;
+                    return quantize_launch_enc<F, 8, kGroup, true, kEncInt, kGiven>(s, src, a);
+                } else {
+                    return hipErrorInvalidValue;
+                }
+            }
             return quantize_launch_enc<F, kBits, kGroup, false, kEncInt, kGiven>(s, src, a);
         case kEncE4M3:
             if constexpr (kBits == 8) return quantize_launch_enc<F, 8, kGroup, false, kEncE4M3, kGiven>(s, src, a);

@@ -21,6 +21,7 @@ hipError_t CQ_QUANTIZE_FLAT_TU(CQ_TU_FLOAT, CQ_TU_GIVEN)(hipStream_t s, int bits
 #endif
     int g = group_of(CQ_TU_FLOAT::kDtype, a.block);
     FlatArgs b = a;
+    b.lanes_only = fields_wrap(a);
     // blocks of another whole number of chunks: lane by lane, for the launches that read their scales
     if (g < 0 && (src == ScaleSource::Given || src == ScaleSource::Stored) && (b.any_group = any_group_of(CQ_TU_FLOAT::kDtype, a.block)) != 0)
         g = shape_group_of(b.any_group);

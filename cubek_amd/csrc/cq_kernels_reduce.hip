@@ -378,6 +378,28 @@ __global__ __launch_bounds__(kThreads) void reduce_strided_kernel(const void* __
     if (lane == 0) F::store(out, out_off, m);
 }
 
+// Output element i of a contiguous result -> its place in a strided output tensor.
+template <class F>
+__global__ __launch_bounds__(kThreads) void scatter_outputs_kernel(const void* __restrict__ packed, void* __restrict__ out,
+                                                                   StridedReduce r, uint64_t num_out) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (i >= num_out) return;
+    uint64_t rem = i, out_off = 0;
+    for (int d = static_cast<int>(r.rank) - 1; d >= 0; d--) {
+        if (static_cast<uint32_t>(d) == r.axis) continue;
+        const uint64_t c = rem % r.shape[d];
+        rem /= r.shape[d];
+        out_off += c * r.out_strides[d];
+    }
+    if constexpr (F::kBytes == 4)
+        static_cast<uint32_t*>(out)[out_off] = static_cast<const uint32_t*>(packed)[i];
+    else
+        static_cast<uint16_t*>(out)[out_off] = static_cast<const uint16_t*>(packed)[i];
+}
+
+// bytes of the workspace that hold the contiguous result of a launch whose output tensor is strided
+inline uint64_t packed_outputs_bytes(uint64_t num_out, uint64_t elem_bytes) { return (num_out * elem_bytes + 255) / 256 * 256; }
+
 inline dim3 blocks(uint64_t n, uint64_t per_block) { return dim3(static_cast<uint32_t>((n + per_block - 1) / per_block)); }
 inline uint64_t round_up(uint64_t v, uint64_t m) { return (v + m - 1) / m * m; }
 inline uint32_t pow2_at_least(uint64_t v, uint32_t cap) {
@@ -520,6 +542,38 @@ bool strided_levels(const ReduceArgs& a, ReduceLevels* r, uint64_t* len_stride) 
 template <class F>
 hipError_t reduce_dispatch(hipStream_t s, const ReduceArgs& a) {
     constexpr uint64_t kN = F::kPerChunk;
+    // A strided output (one column of a matrix, every other element): the kernels below write a contiguous result
+    // into the front of the workspace, and one more small launch puts every element in its place.  Without that much
+    // workspace the launch runs one wave (or lane) per output.
+    if (!a.out_contiguous) {
+        const uint64_t num_out = a.outer * a.inner, front = packed_outputs_bytes(num_out, F::kBytes);
+        if (a.workspace != nullptr && a.workspace_bytes >= front && num_out != 0) {
+            ReduceArgs b = a;
+            b.output = a.workspace;
+            b.out_contiguous = true;
+            b.contiguous = a.in_contiguous;
+            uint64_t acc = 1;
+            for (int d = static_cast<int>(a.rank) - 1; d >= 0; d--) {
+                b.out_strides[d] = acc;
+                if (static_cast<uint32_t>(d) != a.axis) acc *= a.shape[d];
+            }
+            b.workspace = static_cast<char*>(a.workspace) + front;
+            b.workspace_bytes = a.workspace_bytes - front;
+            if (b.workspace_bytes == 0) b.workspace = nullptr;
+            const hipError_t e = reduce_dispatch<F>(s, b);
+            if (e != hipSuccess) return e;
+            StridedReduce r{};
+            r.rank = a.rank;
+            r.axis = a.axis;
+            for (uint32_t d = 0; d < a.rank; d++) {
+                r.shape[d] = static_cast<uint32_t>(a.shape[d]);
+                r.out_strides[d] = a.out_strides[d];
+            }
+            hipLaunchKernelGGL((scatter_outputs_kernel<F>), blocks(num_out, kThreads), dim3(kThreads), 0, s, a.workspace, a.output, r,
+                               num_out);
+            return hipGetLastError();
+        }
+    }
     ReducePlan p;
     if (a.contiguous && (reinterpret_cast<uintptr_t>(a.input) & 15u) == 0) p = plan_reduce(a.outer, a.len, a.inner, kN);
     ReduceLevels levels;
@@ -658,7 +712,8 @@ hipError_t reduce_dispatch(hipStream_t s, const ReduceArgs& a) {
 uint64_t reduce_workspace_bytes(uint64_t outer, uint64_t len, uint64_t inner, int dtype) {
     const ReducePlan p = plan_reduce(outer, len, inner, dtype == CQ_F32 ? 4 : 8);
     const uint64_t slices = p.slices > p.lane_slices ? p.slices : p.lane_slices;  // either kernel set may run
-    return slices > 1 ? slices * p.pitch * sizeof(float) : 0;
+    // ... and room for the contiguous result of a launch whose output tensor turns out to be strided
+    return (slices > 1 ? slices * p.pitch * sizeof(float) : 0) + packed_outputs_bytes(outer * inner, dtype == CQ_F32 ? 4 : 2);
 }
 
 hipError_t launch_reduce_max_abs(hipStream_t s, int dtype, const ReduceArgs& a) {

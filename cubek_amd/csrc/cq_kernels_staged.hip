@@ -182,13 +182,26 @@ __device__ __forceinline__ TilePlace tile_place(uint32_t col_tiles, uint32_t ct_
     return TilePlace{row_tile * Shape::kTileRows, (blockIdx.x - row_tile * col_tiles) * Shape::kTileChunks};
 }
 
-// LDS: one float per block of the tile, rows one entry further apart than they are long
-template <class F, int kBits, int kEnc, bool kDynamic, class Shape>
+// Word `idx` of a tile's codes, numbered along the dimension that is closer in memory in the stored tensor.
+struct TileWord {
+    uint32_t row, wc;
+};
+template <int kTileRows, int kTileWords>
+__device__ __forceinline__ TileWord tile_word(uint32_t idx, bool rows_fastest) {
+    if (rows_fastest) return TileWord{idx % kTileRows, idx / kTileRows};
+    return TileWord{idx / kTileWords, idx % kTileWords};
+}
+
+// LDS: one float per block of the tile, rows one entry further apart than they are long.
+// kStageCodes: the stored tensor's last dimension is not the contiguous one (words of the U32 store `stored_col`
+// apart): the tile's words pass through a second LDS image and leave along the dimension that is closer in memory.
+template <class F, int kBits, int kEnc, bool kDynamic, class Shape, bool kStageCodes>
 __global__ __launch_bounds__(kThreads) void quantize_scale_tiles_kernel(ScaleTileArgs a, QuantParams qp, uint32_t col_tiles,
                                                                        uint32_t ct_magic, uint32_t ct_shift) {
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;
     constexpr int kUnroll = Shape::kUnroll, kIters = Shape::kIters, kTileRows = Shape::kTileRows;
+    constexpr int kTileWords = Shape::kTileChunks * kChunkBits / 32, kWordPitch = kTileWords + 1;
     extern __shared__ float lds_scale[];  // given: the divisors F(FS(scale)); else the scales FS(F(scale)) on their way out
     const uint32_t t = threadIdx.x, lane = t & (kWave - 1), wave = t / kWave;
     const uint32_t wave_row = wave / Shape::kColWaves, tile_chunk = (wave % Shape::kColWaves) * kWave + lane;
@@ -200,6 +213,7 @@ __global__ __launch_bounds__(kThreads) void quantize_scale_tiles_kernel(ScaleTil
     const uint32_t cl = col_live ? c : a.row_chunks - 1;  // lanes past the end re-read the row's last chunk
     const char* const in = static_cast<const char*>(a.input);
     char* const out = static_cast<char*>(a.output);
+    [[maybe_unused]] uint32_t* const lds_words = reinterpret_cast<uint32_t*>(lds_scale + kTileRows * pitch);
 
     // the loads of iteration it + 1 go out before the arithmetic of iteration it
     u32x4 raw[2][kUnroll];
@@ -256,20 +270,42 @@ __global__ __launch_bounds__(kThreads) void quantize_scale_tiles_kernel(ScaleTil
             uint32_t w[2];
             quantize_chunk<F, kBits, kEnc>(v, d, divisor_is_tame(d), qp, w);
             char* const out_row = out + static_cast<uint64_t>(row) * a.stored_pitch;
+            uint32_t* const image_row = lds_words + tile_row * kWordPitch;
             if constexpr (kChunkBits == 64) {
-                if (live) stream_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(out_row) + c);
+                if constexpr (kStageCodes)
+                    image_row[2 * tile_chunk] = w[0], image_row[2 * tile_chunk + 1] = w[1];
+                else if (live)
+                    stream_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(out_row) + c);
             } else if constexpr (kChunkBits == 32) {
-                if (live) stream_store(w[0], reinterpret_cast<uint32_t*>(out_row) + c);
+                if constexpr (kStageCodes)
+                    image_row[tile_chunk] = w[0];
+                else if (live)
+                    stream_store(w[0], reinterpret_cast<uint32_t*>(out_row) + c);
             } else {
                 constexpr int kLanesPerWord = 32 / kChunkBits;  // 2 or 4: rows are whole words
                 const uint32_t sub = lane & (kLanesPerWord - 1);
                 const uint32_t word = group_or<kLanesPerWord>(w[0] << (sub * kChunkBits));
-                if (live && sub == 0) stream_store(word, reinterpret_cast<uint32_t*>(out_row) + c / kLanesPerWord);
+                if constexpr (kStageCodes) {
+                    if (sub == 0) image_row[tile_chunk / kLanesPerWord] = word;
+                } else if (live && sub == 0) {
+                    stream_store(word, reinterpret_cast<uint32_t*>(out_row) + c / kLanesPerWord);
+                }
             }
         }
     }
+    if constexpr (kDynamic || kStageCodes) __syncthreads();
+    if constexpr (kStageCodes) {
+        const uint32_t w0 = place.c0 * kChunkBits / 32, row_words = a.row_chunks * kChunkBits / 32;
+        const uint64_t pitch_words = a.stored_pitch / 4;
+        const bool rows_fastest = pitch_words <= a.stored_col;
+        for (uint32_t idx = t; idx < kTileRows * kTileWords; idx += kThreads) {
+            const TileWord e = tile_word<kTileRows, kTileWords>(idx, rows_fastest);
+            const uint32_t gr = place.r0 + e.row, gw = w0 + e.wc;
+            if (gr < a.rows && gw < row_words)
+                stream_store(lds_words[e.row * kWordPitch + e.wc], reinterpret_cast<uint32_t*>(out) + gr * pitch_words + gw * a.stored_col);
+        }
+    }
     if constexpr (kDynamic) {
-        __syncthreads();
         const bool rows_fastest = a.sb_row <= a.sb_col;
         for (uint32_t idx = t; idx < kTileRows * bcols; idx += kThreads) {
             const TileScale e = tile_scale<kTileRows>(idx, rows_fastest, bcols_log2);
@@ -280,12 +316,13 @@ __global__ __launch_bounds__(kThreads) void quantize_scale_tiles_kernel(ScaleTil
     }
 }
 
-template <class F, int kBits, int kEnc, class Shape>
+template <class F, int kBits, int kEnc, class Shape, bool kStageCodes>
 __global__ __launch_bounds__(kThreads) void dequantize_scale_tiles_kernel(ScaleTileArgs a, uint32_t col_tiles, uint32_t ct_magic,
                                                                          uint32_t ct_shift) {
     constexpr int kN = F::kPerChunk;
     constexpr int kChunkBits = kN * kBits;
     constexpr int kUnroll = Shape::kUnroll, kIters = Shape::kIters, kTileRows = Shape::kTileRows;
+    constexpr int kTileWords = Shape::kTileChunks * kChunkBits / 32, kWordPitch = kTileWords + 1;
     extern __shared__ float lds_scale[];
     const uint32_t t = threadIdx.x, lane = t & (kWave - 1), wave = t / kWave;
     const uint32_t wave_row = wave / Shape::kColWaves, tile_chunk = (wave % Shape::kColWaves) * kWave + lane;
@@ -298,15 +335,25 @@ __global__ __launch_bounds__(kThreads) void dequantize_scale_tiles_kernel(ScaleT
     const char* const in = static_cast<const char*>(a.input);
     char* const out = static_cast<char*>(a.output);
 
+    [[maybe_unused]] uint32_t* const lds_words = reinterpret_cast<uint32_t*>(lds_scale + kTileRows * pitch);
     // the loads of iteration it + 1 go out before the arithmetic of iteration it
     uint32_t w0[2][kUnroll], w1[2][kUnroll];
     const auto load = [&](int it) {
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
-            const uint32_t row = place.r0 + (it * kUnroll + u) * Shape::kRowWaves + wave_row;
+            const uint32_t tile_row = (it * kUnroll + u) * Shape::kRowWaves + wave_row;
+            const uint32_t row = place.r0 + tile_row;
             const char* const in_row = in + static_cast<uint64_t>(row < a.rows ? row : a.rows - 1) * a.stored_pitch;
             w1[it & 1][u] = 0;
-            if constexpr (kChunkBits == 64) {
+            if constexpr (kStageCodes) {  // out of the tile's image in LDS (after the barrier below)
+                const uint32_t* const image_row = lds_words + tile_row * kWordPitch;
+                if constexpr (kChunkBits == 64)
+                    w0[it & 1][u] = image_row[2 * tile_chunk], w1[it & 1][u] = image_row[2 * tile_chunk + 1];
+                else if constexpr (kChunkBits == 32)
+                    w0[it & 1][u] = image_row[tile_chunk];
+                else
+                    w0[it & 1][u] = image_row[tile_chunk / (32 / kChunkBits)];
+            } else if constexpr (kChunkBits == 64) {
                 const u32x2 w = stream_load(reinterpret_cast<const u32x2*>(in_row) + cl);
                 w0[it & 1][u] = w[0];
                 w1[it & 1][u] = w[1];
@@ -318,7 +365,20 @@ __global__ __launch_bounds__(kThreads) void dequantize_scale_tiles_kernel(ScaleT
             }
         }
     };
-    load(0);
+    if constexpr (kStageCodes) {
+        // the tile's words, read along the dimension that is closer in memory in the stored tensor
+        const uint32_t word0 = place.c0 * kChunkBits / 32, row_words = a.row_chunks * kChunkBits / 32;
+        const uint64_t pitch_words = a.stored_pitch / 4;
+        const bool rows_fastest = pitch_words <= a.stored_col;
+        for (uint32_t idx = t; idx < kTileRows * kTileWords; idx += kThreads) {
+            const TileWord e = tile_word<kTileRows, kTileWords>(idx, rows_fastest);
+            const uint32_t gr = place.r0 + e.row, gw = word0 + e.wc;
+            const bool ok = gr < a.rows && gw < row_words;
+            lds_words[e.row * kWordPitch + e.wc] = stream_load(reinterpret_cast<const uint32_t*>(in) + (ok ? gr * pitch_words + gw * a.stored_col : 0));
+        }
+    } else {
+        load(0);
+    }
     {
         const bool rows_fastest = a.sa_row <= a.sa_col;
         for (uint32_t idx = t; idx < kTileRows * bcols; idx += kThreads) {
@@ -330,6 +390,7 @@ __global__ __launch_bounds__(kThreads) void dequantize_scale_tiles_kernel(ScaleT
         }
         __syncthreads();
     }
+    if constexpr (kStageCodes) load(0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int it = 0; it < kIters; it++) {
@@ -427,26 +488,33 @@ TileGrid tile_grid(const ScaleTileArgs& a) {
     g.lds = Shape::kTileRows * ((Shape::kTileChunks >> a.group_log2) + 1) * static_cast<uint32_t>(sizeof(float));
     return g;
 }
+// LDS of the image of a tile's words (staged codes)
+template <class Shape>
+uint32_t tile_words_lds(uint32_t chunk_bits) {
+    return Shape::kTileRows * (Shape::kTileChunks * chunk_bits / 32 + 1) * 4u;
+}
 
-template <class F, int kBits, int kEnc, class Shape>
+template <class F, int kBits, int kEnc, class Shape, bool kStageCodes>
 hipError_t quantize_scale_tiles_shape(hipStream_t s, const ScaleTileArgs& a) {
     const TileGrid g = tile_grid<Shape>(a);
     if (!g.ok) return hipErrorInvalidValue;
     const QuantParams qp = quant_params(a.range);
+    const uint32_t lds = g.lds + (kStageCodes ? tile_words_lds<Shape>(F::kPerChunk * kBits) : 0u);
     if (a.scale_in == nullptr)
-        hipLaunchKernelGGL((quantize_scale_tiles_kernel<F, kBits, kEnc, true, Shape>), dim3(g.grid), dim3(kThreads), g.lds, s, a, qp,
-                           g.col_tiles, g.magic, g.shift);
+        hipLaunchKernelGGL((quantize_scale_tiles_kernel<F, kBits, kEnc, true, Shape, kStageCodes>), dim3(g.grid), dim3(kThreads), lds, s,
+                           a, qp, g.col_tiles, g.magic, g.shift);
     else
-        hipLaunchKernelGGL((quantize_scale_tiles_kernel<F, kBits, kEnc, false, Shape>), dim3(g.grid), dim3(kThreads), g.lds, s, a, qp,
-                           g.col_tiles, g.magic, g.shift);
+        hipLaunchKernelGGL((quantize_scale_tiles_kernel<F, kBits, kEnc, false, Shape, kStageCodes>), dim3(g.grid), dim3(kThreads), lds, s,
+                           a, qp, g.col_tiles, g.magic, g.shift);
     return hipGetLastError();
 }
-template <class F, int kBits, int kEnc, class Shape>
+template <class F, int kBits, int kEnc, class Shape, bool kStageCodes>
 hipError_t dequantize_scale_tiles_shape(hipStream_t s, const ScaleTileArgs& a) {
     const TileGrid g = tile_grid<Shape>(a);
     if (!g.ok) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((dequantize_scale_tiles_kernel<F, kBits, kEnc, Shape>), dim3(g.grid), dim3(kThreads), g.lds, s, a, g.col_tiles,
-                       g.magic, g.shift);
+    const uint32_t lds = g.lds + (kStageCodes ? tile_words_lds<Shape>(F::kPerChunk * kBits) : 0u);
+    hipLaunchKernelGGL((dequantize_scale_tiles_kernel<F, kBits, kEnc, Shape, kStageCodes>), dim3(g.grid), dim3(kThreads), lds, s, a,
+                       g.col_tiles, g.magic, g.shift);
     return hipGetLastError();
 }
 
@@ -456,15 +524,30 @@ hipError_t dequantize_scale_tiles_shape(hipStream_t s, const ScaleTileArgs& a) {
 // (107 us / 96 us).
 using QuantizeTile = TileShape<16, 1, 4>;
 using DequantizeTile = TileShape<16, 1, 4>;
+// Staged codes (a stored tensor whose last dimension is not the contiguous one; words of the U32 store only): 32 rows,
+// so that the runs along the rows are whole 128-byte lines
+using StagedCodesTile = TileShape<32, 1, 4>;
 
 template <class F, int kBits, int kEnc>
 hipError_t quantize_scale_tiles(hipStream_t s, const ScaleTileArgs& a) {
-    return quantize_scale_tiles_shape<F, kBits, kEnc, QuantizeTile>(s, a);
+    if (a.stored_col != 1) {
+        if constexpr (kEnc == kEncInt)
+            return quantize_scale_tiles_shape<F, kBits, kEnc, StagedCodesTile, true>(s, a);
+        else
+            return hipErrorInvalidValue;
+    }
+    return quantize_scale_tiles_shape<F, kBits, kEnc, QuantizeTile, false>(s, a);
 }
 
 template <class F, int kBits, int kEnc>
 hipError_t dequantize_scale_tiles(hipStream_t s, const ScaleTileArgs& a) {
-    return dequantize_scale_tiles_shape<F, kBits, kEnc, DequantizeTile>(s, a);
+    if (a.stored_col != 1) {
+        if constexpr (kEnc == kEncInt)
+            return dequantize_scale_tiles_shape<F, kBits, kEnc, StagedCodesTile, true>(s, a);
+        else
+            return hipErrorInvalidValue;
+    }
+    return dequantize_scale_tiles_shape<F, kBits, kEnc, DequantizeTile, false>(s, a);
 }
 
 }  // namespace

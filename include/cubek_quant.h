@@ -204,8 +204,10 @@ cq_status cq_quantize_dynamic_static(cq_stream_t stream, const cq_tensor* input,
  *   input  : float tensor of dtype `dtype`, any strides
  *   output : same dtype, same shape except extent 1 on `axis`
  *            (anything else: CQ_ERR_SHAPE_MISMATCH, ReduceError::MismatchShape)
- *   workspace : optional device scratch of cq_reduce_workspace_bytes() bytes; lets
- *            reductions with few outputs spread one output over many workgroups
+ *   workspace : optional device scratch of cq_reduce_workspace_bytes() bytes (16-byte aligned); lets
+ *            reductions with few outputs spread one output over many workgroups, and gives an
+ *            output tensor that is not contiguous the streaming kernels too (they leave a
+ *            contiguous result in the workspace, which one more small launch puts in place)
  * NaN elements are ignored; an axis of extent 0 yields 0. */
 cq_status cq_reduce_max_abs(cq_stream_t stream, const cq_tensor* input, const cq_tensor* output,
                             uint32_t axis, cq_dtype dtype, void* workspace, size_t workspace_bytes);

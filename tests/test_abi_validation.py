@@ -135,8 +135,9 @@ def test_reduce_checks():
     assert status(lambda: cq_reduce.max_abs(CLIENT, x, t((4, 2), 4), 1, ElemType.F32)) == _ffi.ERR_SHAPE_MISMATCH
     assert status(lambda: cq_reduce.max_abs(CLIENT, x, t((4,), 4), 1, ElemType.F32)) == _ffi.ERR_SHAPE_MISMATCH
     assert status(lambda: cq_reduce.max_abs(CLIENT, x, t((4, 1), 2), 1, ElemType.F32)) == _ffi.ERR_SHAPE_MISMATCH
-    assert cq_reduce.workspace_bytes(t((8192, 8192), 2), 1, ElemType.BF16) == 0           # enough rows already
-    assert cq_reduce.workspace_bytes(t((64, 1 << 20), 2), 1, ElemType.BF16) > 0           # rows cut into slices
+    # enough rows already: only the room for a contiguous result, should the output tensor be strided
+    assert cq_reduce.workspace_bytes(t((8192, 8192), 2), 1, ElemType.BF16) == 8192 * 2
+    assert cq_reduce.workspace_bytes(t((64, 1 << 20), 2), 1, ElemType.BF16) > 256         # rows cut into slices
     assert cq_reduce.workspace_bytes(t((64, 1 << 20), 2), 1, ElemType.BF16) <= (64 << 21) // 32
 
 

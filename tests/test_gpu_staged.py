@@ -331,6 +331,56 @@ def test_scale_tiles_on_pitched_rows(gpu, oracle):
     assert np.array_equal(got_y[:, :cols], y_ref.reshape(rows, cols)) and np.all(got_y[:, cols:] == 0x7777)
 
 
+@pytest.mark.parametrize("elem", ELEMS, ids=lambda e: e.name)
+@pytest.mark.parametrize("value,block", [(QuantValue.Q8S, 32), (QuantValue.E2M1, 64), (QuantValue.Q2S, 128)],
+                         ids=["q8s_b32", "e2m1_b64", "q2s_b128"])
+@pytest.mark.parametrize("v_layout", ["transposed", "transposed_padded", "column_stride_3"])
+def test_stored_tensor_whose_last_dimension_is_not_contiguous(gpu, oracle, elem, value, block, v_layout):
+    """Words of the U32 store with a stride along the last dimension (the stored tensor transposed in memory, with
+    padded columns, or every third word of its rows): the codes of a tile pass through LDS.  70 rows x 4224 columns:
+    tiles cut short both ways.  Quantize (fused and with given scales) and dequantize against the oracle; the bytes
+    between the words keep their value."""
+    import torch
+
+    rows, cols = 70, 4224
+    if elem == ElemType.F32 and block == 128:
+        block = 64
+    scheme = scheme_of(value, QuantStore.U32, (block,))
+    nq, nb = scheme.num_quants(), cols // block
+    wcols = cols // nq
+    vstr = {"transposed": (1, rows), "transposed_padded": (1, rows + 5), "column_stride_3": (3 * wcols + 2, 3)}[v_layout]
+    rng = np.random.default_rng(rows + block + int(elem))
+    x = oracle.to_bits(rng.normal(0, 1, (rows, cols)).astype(np.float32), elem)
+    s_ref = oracle.compute_scales(x, elem, (rows, cols), scheme)
+    w_ref, os_ref = oracle.quantize(x, elem, (rows, cols), s_ref, scheme)
+    y_ref = oracle.dequantize(w_ref, (rows, cols), os_ref, elem, scheme)
+    reach = 1 + (rows - 1) * vstr[0] + (wcols - 1) * vstr[1]
+    idx = (np.arange(rows)[:, None] * vstr[0] + np.arange(wcols)[None, :] * vstr[1]).reshape(-1)
+    want_buf = np.full(reach, 0x5A5A5A5A, dtype=np.uint32)
+    want_buf[idx] = np.asarray(w_ref).reshape(-1)
+    d_x, d_s = gpu.to_dev(x.reshape(rows, cols)), gpu.to_dev(np.asarray(s_ref).reshape(rows, nb))
+    h = TensorHandleRef.from_torch
+    client = ComputeClient.current()
+    for what in ("dynamic", "given"):
+        d_w = torch.full((reach,), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+        d_os = torch.zeros((rows, nb), dtype=torch.float32, device="cuda")
+        hw = TensorHandleRef(d_w.data_ptr(), (rows, wcols), vstr, 4)
+        if what == "dynamic":
+            assert plan_family(_ffi.OP_QUANTIZE_DYNAMIC, scheme, elem, h(d_x), hw, None, h(d_os)) == "staged"
+            qz.launch_dynamic(client, h(d_x), hw, h(d_os), scheme, elem)
+        else:
+            assert plan_family(_ffi.OP_QUANTIZE, scheme, elem, h(d_x), hw, h(d_s), h(d_os)) == "staged"
+            qz.launch_ref(client, h(d_x), hw, h(d_s), h(d_os), scheme, elem)
+        torch.cuda.synchronize()
+        assert np.array_equal(d_w.cpu().numpy().view(np.uint32), want_buf), (v_layout, what)
+        assert same_bits(d_os.cpu().numpy(), os_ref), (v_layout, what)
+    d_y = torch.zeros((rows, cols), dtype=gpu.storage_dtype(elem), device="cuda")
+    assert plan_family(_ffi.OP_DEQUANTIZE, scheme, elem, h(d_y), hw, h(d_os)) == "staged"
+    dq.launch_ref(client, hw, h(d_y), h(d_os), scheme, elem)
+    torch.cuda.synchronize()
+    assert same_bits(gpu.to_host(d_y), y_ref), v_layout
+
+
 @pytest.mark.parametrize("what", ["blocks_of_24", "column_major_scales"])
 def test_staged_kernels_at_full_size_match_the_flat_kernels(gpu, what):
     """bf16 [28672, 8184] with blocks of 24 and [28672, 8192] with scales stored column by column: thousands of

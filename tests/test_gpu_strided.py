@@ -113,6 +113,9 @@ SCHEMES = [
     ("q4s_block128", QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([128]))),
     ("e4m3_native_block64", QuantScheme.default().with_value(QuantValue.E4M3).with_store(QuantStore.Native)
      .with_level(QuantLevel.block([64]))),
+    # value ranges wider than their 8-bit field in the u32 store: the codes wrap (src/quantize.rs:75)
+    ("e4m3_u32_block32", QuantScheme.default().with_value(QuantValue.E4M3).with_level(QuantLevel.block([32]))),
+    ("e5m2_u32_tensor", QuantScheme.default().with_value(QuantValue.E5M2)),
 ]
 
 

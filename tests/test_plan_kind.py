@@ -151,15 +151,28 @@ def test_matrix_vector_product_with_several_right_hand_sides():
 
 def test_slow_paths_are_reported():
     e2m1 = scheme_of(QuantValue.E2M1, [32])
-    # rows that start on odd multiples of 2 bytes
+    # rows that start on odd multiples of 2 bytes: lane by lane (16-byte accesses off their alignment); rows that are
+    # not whole words of codes stay per element
     got = kinds(e2m1, BF16, (8192, 8192), f_strides=(8193, 1), ops=("quantize", "dynamic", "dequantize"))
+    assert set(got.values()) == {"flat_lanes"}
+    got = kinds(scheme_of(QuantValue.Q8S), BF16, (8192, 8196), f_strides=(8197, 1), ops=("quantize", "dynamic", "dequantize"))
     assert set(got.values()) == {"per_element"}
-    # a quantized tensor whose last dimension is not the contiguous one
-    got = kinds(e2m1, BF16, (4096, 4096), v_strides=(1, 4096), ops=("quantize", "dequantize"))
+    # a quantized tensor whose last dimension is not the contiguous one: words of the u32 store pass through LDS
+    # (the staged tiles); bytes of the native store go one thread per element
+    got = kinds(e2m1, BF16, (4096, 4096), v_strides=(1, 4096), ops=("quantize", "dynamic", "dequantize"))
+    assert set(got.values()) == {"staged"}
+    native = scheme_of(QuantValue.E4M3, [32], store=QuantStore.Native)
+    got = kinds(native, BF16, (4096, 4096), v_strides=(1, 4096), ops=("quantize", "dequantize"))
     assert set(got.values()) == {"per_element"}
-    # E4M3 in the u32 store (codes wrap their field): per-element quantize, streaming dequantize
-    got = kinds(scheme_of(QuantValue.E4M3, [32]), BF16, (4096, 4096), ops=("quantize", "dynamic", "dequantize"))
-    assert got == {"quantize": "per_element", "dynamic": "per_element", "dequantize": "flat"}
+    # E4M3 / E5M2 in the u32 store (codes wrap their 8-bit field): quantize lane by lane, streaming dequantize; under
+    # layouts of the other families (a transposed float tensor) per element
+    for value in (QuantValue.E4M3, QuantValue.E5M2):
+        got = kinds(scheme_of(value, [32]), BF16, (4096, 4096), ops=("quantize", "dynamic", "dequantize"))
+        assert got == {"quantize": "flat_lanes", "dynamic": "flat_lanes", "dequantize": "flat"}
+        got = kinds(scheme_of(value), F32, (4096, 4096), f_strides=(4160, 1), ops=("quantize", "dynamic", "dequantize"))
+        assert got == {"quantize": "flat_lanes", "dynamic": "flat_lanes", "dequantize": "flat_rows"}
+        got = kinds(scheme_of(value, [32]), BF16, (4096, 4096), f_strides=(1, 4096), ops=("quantize", "dynamic", "dequantize"))
+        assert got == {"quantize": "per_element", "dynamic": "per_element", "dequantize": "transposed"}
     # blocks smaller than a packed word on dequantize
     got = kinds(scheme_of(QuantValue.Q8S, [2]), BF16, (4096, 4096), ops=("dequantize",))
     assert got == {"dequantize": "per_element"}
