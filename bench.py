@@ -717,6 +717,56 @@ def corner_layouts(torch):
     return out
 
 
+def per_tensor_passes(torch):
+    """Where the time of a per-tensor dynamic quantize goes, at sizes that fit the 256 MB Infinity Cache: the two
+    passes timed apart through the public entry points (cq_compute_scales = pass 1 + the scale; cq_quantize with that
+    scale = what pass 2 does), the second one on a tensor that has left the caches (eight rotated inputs) and right
+    behind pass 1 on the same tensor, and cq_quantize_dynamic itself.  q8 of bf16."""
+    from cubek_amd import ComputeClient, ElemType, QuantLevel, QuantScheme, QuantValue, TensorHandleRef
+    from cubek_amd import quantize as cq_quantize
+
+    client = ComputeClient.current()
+    h = TensorHandleRef.from_torch
+    scheme = QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.Tensor)
+    out = []
+    for rows, cols in ((4096, 4096), (8192, 4096), (8192, 8192)):
+        sets = 8
+        xs = [torch.randn((rows, cols), device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
+        words = [torch.empty((rows, cols // 4), dtype=torch.int32, device="cuda") for _ in range(2)]
+        sc_in = [torch.ones((1,), dtype=torch.bfloat16, device="cuda") for _ in range(sets)]
+        sc_out = [torch.empty((1,), dtype=torch.float32, device="cuda") for _ in range(2)]
+        ws_bytes = cq_quantize.workspace_bytes(scheme, rows * cols)
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device="cuda")
+        hx, hw, hsi, hso = [h(t) for t in xs], [h(t) for t in words], [h(t) for t in sc_in], [h(t) for t in sc_out]
+        pass1 = lambda i: cq_quantize.compute_scales(client, hx[i % sets], hsi[i % sets], scheme, ElemType.BF16, ws.data_ptr(), ws_bytes)
+        pass2 = lambda i: cq_quantize.launch_ref(client, hx[i % sets], hw[i % 2], hsi[i % sets], hso[i % 2], scheme, ElemType.BF16)
+
+        def pair(i):
+            pass1(i)
+            pass2(i)
+        dyn = lambda i: cq_quantize.launch_dynamic(client, hx[i % sets], hw[i % 2], hso[i % 2], scheme, ElemType.BF16,
+                                                   ws.data_ptr(), ws_bytes)
+        again = lambda i: cq_quantize.compute_scales(client, hx[0], hsi[0], scheme, ElemType.BF16, ws.data_ptr(), ws_bytes)
+        t = {k: sorted(timed_region(torch, f, 32)[0] for _ in range(3))[1]
+             for k, f in (("pass1", pass1), ("pass1_again", again), ("pass2_cold", pass2), ("pair", pair), ("dynamic", dyn))}
+        mib = rows * cols * 2 >> 20
+        b = rows * cols * 3 + 4
+        out.append({"kernel": f"per-tensor q8 of bf16 [{rows}, {cols}] ({mib} MiB), the two passes apart",
+                    "algorithmic_bytes": b, "ms": round(t["dynamic"], 4),
+                    "GBps": round(b / (t["dynamic"] * 1e-3) / 1e9, 1),
+                    "frac_hbm_peak": round(b / (t["dynamic"] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                    "pass1_abs_max_and_scale_ms": round(t["pass1"], 4),
+                    "pass1_GBps_on_the_input": round(rows * cols * 2 / (t["pass1"] * 1e-3) / 1e9, 1),
+                    # the same launches on ONE tensor, over and over: what a read gains from finding its operand
+                    # in the Infinity Cache
+                    "pass1_on_the_same_tensor_again_ms": round(t["pass1_again"], 4),
+                    "pass2_on_a_cold_tensor_ms": round(t["pass2_cold"], 4),
+                    "pass2_behind_pass1_ms": round(t["pair"] - t["pass1"], 4),
+                    "both_passes_as_two_calls_ms": round(t["pair"], 4)})
+        del xs, words, hx, hw
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -749,10 +799,10 @@ def main():
     torch.cuda.set_device(0)
 
     if args.adjacent_only:
-        print(json.dumps({"adjacent_kernels": adjacent_kernels(torch) + corner_layouts(torch) + packed_gemv(torch)}))
+        print(json.dumps({"adjacent_kernels": adjacent_kernels(torch) + corner_layouts(torch) + per_tensor_passes(torch) + packed_gemv(torch)}))
         return
     if args.corners_only:
-        print(json.dumps({"adjacent_kernels": corner_layouts(torch)}))
+        print(json.dumps({"adjacent_kernels": corner_layouts(torch) + per_tensor_passes(torch)}))
         return
     if args.gemv_only:
         print(json.dumps({"adjacent_kernels": packed_gemv(torch)}))
@@ -888,7 +938,7 @@ def main():
             row["workload"]: {short[k]: row[k]["frac_hbm_peak"] for k in short} for row in table}
         result["roofline"]["min_frac_cfg3_5"] = min(
             row[k]["frac_hbm_peak"] for row in table if row["workload"] in ("cfg3", "cfg4", "cfg5") for k in short)
-        result["adjacent_kernels"] = adjacent_kernels(torch) + corner_layouts(torch) + packed_gemv(torch)
+        result["adjacent_kernels"] = adjacent_kernels(torch) + corner_layouts(torch) + per_tensor_passes(torch) + packed_gemv(torch)
 
     print(json.dumps(result))
 
