@@ -34,9 +34,11 @@ bool flat_block_supported_with_scales(int dtype, uint32_t block) { return group_
 uint32_t flat_family(const FlatArgs& a, int f_dtype) {
     const bool p32 = a.param_dtype == CQ_F32 || a.output == nullptr;  // scale production has no stored parameters
     if (a.lanes.levels > 0 || any_group_of(f_dtype, a.block) != 0 || a.lanes_only) return CQ_FAMILY_FLAT_LANES;
-    if (a.rows > 1) return p32 && a.num_chunks % kThreads == 0 ? CQ_FAMILY_FLAT_ROWS : CQ_FAMILY_FLAT_LANES;
-    return (p32 || a.param_dtype == f_dtype) && a.num_chunks >= static_cast<uint64_t>(kThreads) * 4 ? CQ_FAMILY_FLAT
-                                                                                                     : CQ_FAMILY_FLAT_LANES;
+    const int group = group_of(f_dtype, a.block);
+    if (a.rows > 1) return p32 && whole_steps_for(group) && a.num_chunks % kThreads == 0 ? CQ_FAMILY_FLAT_ROWS : CQ_FAMILY_FLAT_LANES;
+    return (p32 || a.param_dtype == f_dtype) && whole_tiles_for(group) && a.num_chunks >= static_cast<uint64_t>(kThreads) * 4
+               ? CQ_FAMILY_FLAT
+               : CQ_FAMILY_FLAT_LANES;
 }
 
 hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource src, const FlatArgs& a) {

@@ -20,7 +20,7 @@ hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
     [[maybe_unused]] const uint64_t param_bytes = kGroup == 0 ? 0 : (a.param_dtype == CQ_F32 ? 4 : 2);
 #if CQ_TU_SAME
     // this object: the whole tiles of a contiguous run, parameters typed like the tensor
-    if constexpr (F::kBytes == 2) {
+    if constexpr (F::kBytes == 2 && whole_tiles_for(kGroup)) {
         hipLaunchKernelGGL((dequantize_flat_kernel<F, kBits, kGroup, kU, kThreads, kEnc, F::kDtype>), dim3(a.whole_grid),
                            dim3(kThreads), 0, s, reinterpret_cast<const uint32_t*>(in), reinterpret_cast<u32x4*>(out), a.scale_in,
                            0ull, static_cast<uint64_t>(a.whole_grid) * kThreads * kU);
@@ -38,13 +38,15 @@ hipError_t dequantize_launch_enc(hipStream_t s, const FlatArgs& a) {
                 b.whole_grid = grid;
                 same = dequantize_flat_same<F>(s, kBits, b);
             } else if (a.rows > 1) {
-                hipLaunchKernelGGL((dequantize_flat_rows_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(grid), dim3(kThreads),
-                                   0, s, reinterpret_cast<const uint32_t*>(in), reinterpret_cast<u32x4*>(out), a.scale_in, 0u,
-                                   flat_rows(a));
+                if constexpr (whole_steps_for(kGroup))
+                    hipLaunchKernelGGL((dequantize_flat_rows_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(grid), dim3(kThreads),
+                                       0, s, reinterpret_cast<const uint32_t*>(in), reinterpret_cast<u32x4*>(out), a.scale_in, 0u,
+                                       flat_rows(a));
             } else {
-                hipLaunchKernelGGL((dequantize_flat_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(grid), dim3(kThreads), 0,
-                                   s, reinterpret_cast<const uint32_t*>(in), reinterpret_cast<u32x4*>(out), a.scale_in, 0ull,
-                                   static_cast<uint64_t>(grid) * kThreads * kU);
+                if constexpr (whole_tiles_for(kGroup))
+                    hipLaunchKernelGGL((dequantize_flat_kernel<F, kBits, kGroup, kU, kThreads, kEnc>), dim3(grid), dim3(kThreads), 0,
+                                       s, reinterpret_cast<const uint32_t*>(in), reinterpret_cast<u32x4*>(out), a.scale_in, 0ull,
+                                       static_cast<uint64_t>(grid) * kThreads * kU);
             }
         },
         [&](const LaneRows& rows, uint32_t tile_begin, uint32_t grid, RunOffsets off) {

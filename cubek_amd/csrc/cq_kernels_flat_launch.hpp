@@ -92,6 +92,13 @@ uint32_t any_group_of(int dtype, uint32_t block) {
 // the power-of-two group whose launch shape (loads in flight) a launch with any_group_of() chunks per block takes
 inline int shape_group_of(uint32_t any_group) { return any_group <= 8 ? 8 : 16; }
 
+// Which lane groups (16-byte chunks per block) have kernels over whole tiles of a contiguous run, and over whole
+// steps of pitched rows: one scale per tensor and blocks of 4 to 32 (4 to 16) chunks, i.e. 32 - 256 values of a 16-bit
+// type, 16 - 128 of f32.  Blocks of one or two chunks run lane by lane: a kernel per block size, float type, code
+// width and scale source is what makes the library large and its first launch slow.
+constexpr bool whole_tiles_for(int group) { return group == 0 || group >= 4; }
+constexpr bool whole_steps_for(int group) { return group == 0 || (group >= 4 && group <= 16); }
+
 // Launch shapes from a sweep on MI355X (batches of back-to-back launches,
 // 117 MB - 470 MB tensors): quantize is best with four 16-byte loads in flight
 // per lane; dequantize, which is store-dominated, with two 16-byte stores per lane
@@ -274,6 +281,7 @@ template <class WholeFn, class LanesFn>
 hipError_t launch_flat(const FlatArgs& a, int f_dtype, int unroll, WholeFn whole, LanesFn lanes) {
     const uint64_t tile = static_cast<uint64_t>(kThreads) * unroll;
     const bool p32 = a.param_dtype == CQ_F32;
+    const int group = group_of(f_dtype, a.block);
     hipError_t e = hipSuccess;
     if (a.lanes.levels > 0) {
         lanes(lane_rows(a, unroll), 0u, lanes_grid(a, unroll), RunOffsets{0});
@@ -283,7 +291,8 @@ hipError_t launch_flat(const FlatArgs& a, int f_dtype, int unroll, WholeFn whole
         const LaneRows lr = lane_rows_of_rows(a);
         const uint32_t tiles = static_cast<uint32_t>((static_cast<uint64_t>(lr.total_chunks) + tile - 1) / tile);
         // whole steps: a tile is `unroll` steps in both numberings, so the ragged last tile can go lane by lane
-        const uint32_t full = p32 && a.any_group == 0 && !a.lanes_only && a.num_chunks % kThreads == 0 ? static_cast<uint32_t>(lr.total_chunks / tile) : 0u;
+        const uint32_t full = p32 && a.any_group == 0 && !a.lanes_only && whole_steps_for(group) && a.num_chunks % kThreads == 0
+                                  ? static_cast<uint32_t>(lr.total_chunks / tile) : 0u;
         if (full > 0) {
             whole(full, 0ull);
             if ((e = hipGetLastError()) != hipSuccess) return e;
@@ -295,7 +304,7 @@ hipError_t launch_flat(const FlatArgs& a, int f_dtype, int unroll, WholeFn whole
         return e;
     }
     // one contiguous run
-    const uint64_t full = (p32 || a.param_dtype == f_dtype) && a.any_group == 0 && !a.lanes_only ? a.num_chunks / tile : 0;
+    const uint64_t full = (p32 || a.param_dtype == f_dtype) && a.any_group == 0 && !a.lanes_only && whole_tiles_for(group) ? a.num_chunks / tile : 0;
     if (full > 0) {
         whole(static_cast<uint32_t>(full), 0ull);
         if ((e = hipGetLastError()) != hipSuccess) return e;
@@ -339,7 +348,7 @@ hipError_t quantize_launch_src(hipStream_t s, ScaleSource src, const FlatArgs& a
         [[maybe_unused]] const uint64_t div = kGroup == 0 ? 1 : (a.any_group != 0 ? a.any_group : kGroup);  // chunks per scale
 #if CQ_TU_SAME
         // this object: the whole tiles of a contiguous run, parameters typed like the tensor
-        if constexpr (kSrc != kScaleStored && F::kBytes == 2 && !kWide) {
+        if constexpr (kSrc != kScaleStored && F::kBytes == 2 && !kWide && whole_tiles_for(kGroup)) {
             hipLaunchKernelGGL((quantize_flat_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc, F::kDtype>),
                                dim3(a.whole_grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
                                reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0ull,
@@ -359,15 +368,17 @@ hipError_t quantize_launch_src(hipStream_t s, ScaleSource src, const FlatArgs& a
                         b.whole_grid = grid;
                         same = quantize_flat_same<F>(kSrc == kScaleGivenF, s, kBits, src, b);
                     } else if (a.rows > 1) {
-                        hipLaunchKernelGGL((quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
-                                           dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
-                                           reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0u, qp, a.num_partials,
-                                           flat_rows(a));
+                        if constexpr (whole_steps_for(kGroup))
+                            hipLaunchKernelGGL((quantize_flat_rows_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
+                                               dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
+                                               reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0u, qp, a.num_partials,
+                                               flat_rows(a));
                     } else {
-                        hipLaunchKernelGGL((quantize_flat_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
-                                           dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
-                                           reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0ull,
-                                           static_cast<uint64_t>(grid) * kThreads * kUnrollQ, qp, a.num_partials);
+                        if constexpr (whole_tiles_for(kGroup))
+                            hipLaunchKernelGGL((quantize_flat_kernel<F, kBits, kGroup, kSrc, kWide, kUnrollQ, kThreads, kEnc>),
+                                               dim3(grid), dim3(kThreads), 0, s, reinterpret_cast<const u32x4*>(in),
+                                               reinterpret_cast<uint32_t*>(out), a.scale_in, a.scale_out, 0ull,
+                                               static_cast<uint64_t>(grid) * kThreads * kUnrollQ, qp, a.num_partials);
                     }
                 }
             },
