@@ -191,21 +191,24 @@ def timed_region(torch, fn, launches, warmup=3):
     return a.elapsed_time(b) / launches, wall * 1e3 / launches
 
 
-def timed_median(torch, fn, regions=50, warmup=10, region_us=1000.0):
+def timed_median(torch, fn, regions=50, warmup=10, region_us=2000.0):
     """The timing protocol of the per-kernel figures: `warmup` untimed launches, then `regions` (>= 50) regions of
     back-to-back launches, each bracketed by HIP events recorded on the launch stream (all regions are enqueued
     first, one synchronize at the end).  A region holds as many launches as fill about `region_us` microseconds
-    (2 .. 256), so that the ~2.5 us an event pair adds stay near 0.3 % of a sample.  Returns the median, mean and
+    (2 .. 256), so that what an event between two launches costs (its own ~2.5 us, and the next launch no longer
+    starting while the last one drains) stays a small share of a sample.  Returns the median, mean and
     minimum of the per-launch times of the regions, in ms, and the launches per region."""
     for i in range(warmup):
         fn(i)
-    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    a.record()
-    for i in range(8):
-        fn(i)
-    b.record()
-    torch.cuda.synchronize()
-    est_us = max(a.elapsed_time(b) / 8 * 1e3, 0.5)
+    est_us = float("inf")
+    for _ in range(3):  # the shortest of three probes: the first one after an idle spell can read several times too long
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(8):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+        est_us = min(est_us, max(a.elapsed_time(b) / 8 * 1e3, 0.5))
     per = int(min(256, max(2, -(-region_us // est_us))))
     events = [torch.cuda.Event(enable_timing=True) for _ in range(regions + 1)]
     events[0].record()
