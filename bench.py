@@ -708,6 +708,15 @@ def corner_layouts(torch):
     record(f"quantize_dynamic, e4m3 in the u32 store (fields wrap), blocks of 32, bf16 [{rows}, {cols}]", b8,
            lambda i: cq_quantize.launch_dynamic(client, hx[i % sets], hw8[i % sets], hs[i % sets], e4, ElemType.BF16), fam)
     del w8, hw8
+    # 3b. the extension value E2M1_OCP (e2m1 nibbles rounded once from the quotient; not a scheme of the reference) in the
+    # u32 store, contiguous: the headline kernels with the e2m1 conversion instead of the integer packing
+    oc = QuantScheme.default().with_value(QuantValue.E2M1_OCP).with_level(QuantLevel.block([32]))
+    fam = _ffi.plan_kind(_ffi.OP_QUANTIZE_DYNAMIC, hx[0], hw[0], None, hs[0], oc, ElemType.BF16)
+    record(f"quantize_dynamic, e2m1_ocp (extension) blocks of 32, u32 store, bf16 [{rows}, {cols}]", b,
+           lambda i: cq_quantize.launch_dynamic(client, hx[i % sets], hw[i % sets], hs[i % sets], oc, ElemType.BF16), fam)
+    fam = _ffi.plan_kind(_ffi.OP_DEQUANTIZE, hy[0], hw[0], hs[0], None, oc, ElemType.BF16)
+    record(f"dequantize, e2m1_ocp (extension) blocks of 32, u32 store, bf16 [{rows}, {cols}]", b,
+           lambda i: cq_dequantize.launch_ref(client, hw[i % sets], hy[i % 2], hs[i % sets], oc, ElemType.BF16), fam)
     # 4. abs-max along the rows into column 1 of a [rows, 4] tensor, and along the columns into every other element
     for axis, oshape, ostr in ((1, (rows, 1), (4, 1)), (0, (1, cols), (2 * cols, 2))):
         o = torch.zeros(rows * 4 if axis == 1 else cols * 2, device="cuda", dtype=torch.bfloat16)

@@ -56,7 +56,7 @@ int param_to_dtype(uint8_t p) { return p == CQ_PARAM_F32 ? CQ_F32 : (p == CQ_PAR
 uint32_t value_bits(uint8_t v) {
     switch (v) {
         case CQ_VALUE_Q8F: case CQ_VALUE_Q8S: case CQ_VALUE_E4M3: case CQ_VALUE_E5M2: return 8;
-        case CQ_VALUE_Q4F: case CQ_VALUE_Q4S: case CQ_VALUE_E2M1: return 4;
+        case CQ_VALUE_Q4F: case CQ_VALUE_Q4S: case CQ_VALUE_E2M1: case CQ_VALUE_E2M1_OCP: return 4;
         case CQ_VALUE_Q2F: case CQ_VALUE_Q2S: return 2;
         default: return 0;
     }
@@ -77,7 +77,7 @@ cq_status check_scheme(const cq_scheme* s) {
         // the native arm of launch_ref accepts only these values (src/quantize.rs:192-219)
         switch (s->value) {
             case CQ_VALUE_Q8F: case CQ_VALUE_Q8S: case CQ_VALUE_E4M3: case CQ_VALUE_E5M2:
-            case CQ_VALUE_E2M1: break;
+            case CQ_VALUE_E2M1: case CQ_VALUE_E2M1_OCP: break;
             default: return CQ_ERR_UNSUPPORTED_SCHEME;
         }
     }
@@ -123,7 +123,7 @@ struct Plan {
 
 uint32_t stored_nq(const cq_scheme* s) {
     if (s->store == CQ_STORE_U32) return 32u / value_bits(s->value);
-    return s->value == CQ_VALUE_E2M1 ? 2u : 1u;
+    return (s->value == CQ_VALUE_E2M1 || s->value == CQ_VALUE_E2M1_OCP) ? 2u : 1u;
 }
 
 // Line size the reference would pick for the native quantize kernel (src/quantize.rs:234-240,
@@ -154,6 +154,7 @@ cq_status make_plan(const cq_scheme* s, const cq_tensor* floats, int dtype, cons
     p->bits = value_bits(s->value);
     p->nq = stored_nq(s);
     if (cq_value_range(s->value, &p->range.lo, &p->range.hi) != CQ_OK) return CQ_ERR_INVALID_ARGUMENT;
+    p->range.unrounded = s->value == CQ_VALUE_E2M1_OCP ? 1u : 0u;
     if (floats->elem_size != dtype_size(dtype)) return CQ_ERR_SHAPE_MISMATCH;
     if (values->elem_size != (s->store == CQ_STORE_U32 ? 4u : 1u)) return CQ_ERR_SHAPE_MISMATCH;
     if (scale_a->elem_size != scale_a_size || (scale_b && scale_b->elem_size != scale_b_size))
@@ -430,6 +431,8 @@ bool wraps_its_field(const cq_scheme* s) {
 
 // Stored encoding of the flat kernels (cq::Encoding) and the field width they see.
 int flat_encoding(const cq_scheme* s) {
+    // the extension value holds e2m1 nibbles in both stores; eight of them in a word lie as the native store's bytes do
+    if (s->value == CQ_VALUE_E2M1_OCP) return 3;
     if (s->store == CQ_STORE_U32) return 0;
     switch (s->value) {
         case CQ_VALUE_E4M3: return 1;
@@ -597,7 +600,8 @@ bool scale_tiles_ok(const Plan& p, const cq_scheme* s, int dtype, const cq_tenso
         if (lv.levels > 1 || lf.rows != lv.rows) return false;
     } else {
         uint64_t v_row = 0;
-        if (s->store != CQ_STORE_U32 || !scale_rows_and_columns(values, &v_row, &stored_col) || stored_col == 0) return false;
+        // (two's-complement fields only: the kernels that stage codes are not compiled for the float encodings)
+        if (s->store != CQ_STORE_U32 || flat_encoding(s) != 0 || !scale_rows_and_columns(values, &v_row, &stored_col) || stored_col == 0) return false;
         lv = RowLevels{1, lf.rows, lf.rows, v_row, 0};
     }
     const uint64_t cols = p.shape[last];
@@ -736,7 +740,7 @@ cq_status cq_value_range(uint8_t value, float* lo, float* hi) {
         case CQ_VALUE_Q4S: *lo = -7.f; *hi = 7.f; break;
         case CQ_VALUE_Q2F: *lo = -2.f; *hi = 1.f; break;
         case CQ_VALUE_Q2S: *lo = -1.f; *hi = 1.f; break;
-        case CQ_VALUE_E2M1: *lo = -6.f; *hi = 6.f; break;
+        case CQ_VALUE_E2M1: case CQ_VALUE_E2M1_OCP: *lo = -6.f; *hi = 6.f; break;
         case CQ_VALUE_E4M3: *lo = -448.f; *hi = 448.f; break;
         case CQ_VALUE_E5M2: *lo = -57344.f; *hi = 57344.f; break;
         default: return CQ_ERR_INVALID_ARGUMENT;
@@ -1328,7 +1332,7 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
     const bool native = scheme->store == CQ_STORE_NATIVE;
     // the native store holds i8, e4m3, e5m2 bytes or e2m1 pairs (src/quantize.rs:196-219)
     if (native && scheme->value != CQ_VALUE_Q8F && scheme->value != CQ_VALUE_Q8S && scheme->value != CQ_VALUE_E4M3 &&
-        scheme->value != CQ_VALUE_E5M2 && scheme->value != CQ_VALUE_E2M1)
+        scheme->value != CQ_VALUE_E5M2 && scheme->value != CQ_VALUE_E2M1 && scheme->value != CQ_VALUE_E2M1_OCP)
         return CQ_ERR_UNSUPPORTED_SCHEME;
     if (!tensor_ok(values) || !tensor_ok(params) || !tensor_ok(x) || !tensor_ok(y) || !valid_dtype(dtype) ||
         !valid_dtype(y_dtype))
@@ -1342,7 +1346,7 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
         params->elem_size != dtype_size(pd))
         return CQ_ERR_SHAPE_MISMATCH;
     const uint32_t bits = value_bits(scheme->value);
-    const uint32_t nq = native ? (scheme->value == CQ_VALUE_E2M1 ? 2u : 1u) : 32u / bits;  // values per stored element
+    const uint32_t nq = stored_nq(scheme);  // values per stored element
     const uint64_t rows = values->shape[0], cols = values->shape[1] * nq;
     if (rows > 0xffffffffull || cols > 0xffffffffull) return CQ_ERR_TOO_LARGE;
     if (x->shape[last] != cols || y->shape[last] != rows || (x->rank == 2 && y->shape[0] != vectors))
@@ -1383,9 +1387,15 @@ cq_status cq_gemv_quantized(cq_stream_t stream, const cq_tensor* values, const c
     a.words_aligned16 = aligned(values->ptr, 16);
     if (native) {
         // only the streaming kernel reads the native store: rows of whole 16-byte units on 16-byte boundaries
-        a.native = scheme->value == CQ_VALUE_E4M3 ? 1u : scheme->value == CQ_VALUE_E5M2 ? 2u : scheme->value == CQ_VALUE_E2M1 ? 3u : 0u;
+        a.native = scheme->value == CQ_VALUE_E4M3 ? 1u : scheme->value == CQ_VALUE_E5M2 ? 2u
+                   : (scheme->value == CQ_VALUE_E2M1 || scheme->value == CQ_VALUE_E2M1_OCP) ? 3u : 0u;
         if (values->strides[0] % 16 != 0 && rows > 1) return CQ_ERR_UNSUPPORTED_SCHEME;
         a.word_pitch = values->strides[0] / 4;
+        if (!cq::gemv_streams(a)) return CQ_ERR_UNSUPPORTED_SCHEME;
+    } else if (scheme->value == CQ_VALUE_E2M1_OCP) {
+        // e2m1 nibbles in u32 words are the native store's bytes: the same kernel, the pitch already in words
+        a.native = 3u;
+        if (values->strides[0] % 4 != 0 && rows > 1) return CQ_ERR_UNSUPPORTED_SCHEME;
         if (!cq::gemv_streams(a)) return CQ_ERR_UNSUPPORTED_SCHEME;
     }
     return CQ_RUN(cq::gemv_streams(a) ? CQ_FAMILY_FLAT : CQ_FAMILY_ROWS, cq::launch_gemv_quantized(stream, a));

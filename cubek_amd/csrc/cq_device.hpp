@@ -265,6 +265,7 @@ __device__ __forceinline__ uint32_t group_or(uint32_t v) {
 struct QuantParams {
     float lo, hi;         // q_min, q_max
     float width, rwidth;  // q_max - q_min and its correctly rounded reciprocal
+    uint32_t unrounded = 0;  // Range::unrounded
     uint32_t keep = 0;    // the flat quantize kernels: codes leave through output_store(keep = true): they stay in the
                           // Infinity Cache for the kernel that reads them next
 };
@@ -365,7 +366,11 @@ __device__ __forceinline__ float scale_from_absmax_tame(float amax, const QuantP
 // Negation commutes with every step (multiply, RNE rounding, rint).
 // kNegated = false gives the codes themselves: the last rounding takes its operand negated (a source
 // modifier), which the conversions to fp8 / fp4 cannot do for theirs.
-template <class F, int kN, bool kNegated = true>
+// kRint = false leaves out the integer rounding (the extension value CQ_VALUE_E2M1_OCP, whose one rounding is the cast
+// to e2m1 that follows): the results are the clamped quotients in F.  The bf16 and f16 arguments above hold for the
+// quotient itself; the f32 shortcut is about rint and is skipped.  Quotients too small for x * rcp(d) to be trusted
+// (below the normal range) are far below 1/4, where every value casts to a zero of its sign.
+template <class F, int kN, bool kNegated = true, bool kRint = true>
 __device__ __forceinline__ void quantize_values_neg(const float* x, float d, bool d_tame, float lo,
                                                     float hi, float* qn) {
     constexpr float kSign = kNegated ? 1.0f : -1.0f;
@@ -378,8 +383,12 @@ __device__ __forceinline__ void quantize_values_neg(const float* x, float d, boo
                 const float a = neg_clamp_of_neg(x[i] * nr, nhi, nlo);
                 const float b = neg_clamp_of_neg(x[i + 1] * nr, nhi, nlo);
                 const uint32_t p = BF16::pack2(a, b);
-                qn[i] = __builtin_rintf(kSign * bits_f32(p << 16));
-                qn[i + 1] = __builtin_rintf(kSign * bits_f32(p & 0xffff0000u));
+                qn[i] = kSign * bits_f32(p << 16);
+                qn[i + 1] = kSign * bits_f32(p & 0xffff0000u);
+                if constexpr (kRint) {
+                    qn[i] = __builtin_rintf(qn[i]);
+                    qn[i + 1] = __builtin_rintf(qn[i + 1]);
+                }
             }
             return;
         }
@@ -392,11 +401,12 @@ __device__ __forceinline__ void quantize_values_neg(const float* x, float d, boo
                 const float tn = neg_clamp_of_neg(x[i] * nr, nhi_t, nlo_t);  // -t
                 const float e = __builtin_fmaf(tn, d, x[i]);                 // x - t*d
                 const float qn1 = __builtin_fmaf(e, nr, tn);                 // -(t + e*r)
-                qn[i] = __builtin_rintf(kSign * F16::round(neg_clamp_of_neg(qn1, nhi, nlo)));
+                qn[i] = kSign * F16::round(neg_clamp_of_neg(qn1, nhi, nlo));
+                if constexpr (kRint) qn[i] = __builtin_rintf(qn[i]);
             }
             return;
         }
-    } else if constexpr (F::kDtype == CQ_F32) {
+    } else if constexpr (F::kDtype == CQ_F32 && kRint) {
         if (d_tame) {
             const float nr = -__builtin_amdgcn_rcpf(d);
             const float nhi_q = -(hi + 0.25f), nlo_q = -(lo - 0.25f);
@@ -414,7 +424,23 @@ __device__ __forceinline__ void quantize_values_neg(const float* x, float d, boo
         }
     }
 #pragma unroll
-    for (int i = 0; i < kN; i++) qn[i] = -kSign * quantize_exact<F>(x[i], d, lo, hi);
+    for (int i = 0; i < kN; i++)
+        qn[i] = -kSign * (kRint ? quantize_exact<F>(x[i], d, lo, hi) : clamp_code(F::round(x[i] / d), lo, hi));
+}
+
+// The codes of kN values for the stored encoding kEnc: negated integer-valued floats for the two's-complement fields,
+// the codes themselves for the float encodings; for e2m1 nibbles a launch may ask for the unrounded quotients
+// (`unrounded`, the same for the whole launch: a scalar branch).  kEnc is an Encoding, declared below.
+template <class F, int kN, int kEnc>
+__device__ __forceinline__ void quantize_codes(const float* x, float d, bool d_tame, float lo, float hi,
+                                               bool unrounded, float* qn) {
+    if constexpr (kEnc == 3) {  // kEncE2M1
+        if (unrounded) {
+            quantize_values_neg<F, kN, false, false>(x, d, d_tame, lo, hi, qn);
+            return;
+        }
+    }
+    quantize_values_neg<F, kN, kEnc == 0>(x, d, d_tame, lo, hi, qn);
 }
 
 // ---- bit packing -----------------------------------------------------------

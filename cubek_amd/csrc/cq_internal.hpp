@@ -20,6 +20,7 @@ struct Layout {
 
 struct Range {
     float lo, hi;
+    uint32_t unrounded = 0;  // CQ_VALUE_E2M1_OCP: the clamped quotient goes to the e2m1 cast without the integer rounding
 };
 
 // Rows that each lane finds for itself (short rows, leading dimensions with strides of their own):

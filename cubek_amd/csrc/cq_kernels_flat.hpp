@@ -634,7 +634,7 @@ __device__ __forceinline__ void quantize_flat_body(const Geo& geo, int param_dty
         uint32_t w[2];
         const auto by_value = [&](bool d_tame) {
             float qn[kN];  // negated codes
-            quantize_values_neg<F, kN, kEnc == kEncInt>(v, d, d_tame, qp.lo, qp.hi, qn);
+            quantize_codes<F, kN, kEnc>(v, d, d_tame, qp.lo, qp.hi, qp.unrounded != 0, qn);
             if constexpr (kEnc == kEncInt)
                 pack_chunk_neg<kBits, kN, kWide>(qn, w);
             else

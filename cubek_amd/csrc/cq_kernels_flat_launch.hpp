@@ -265,6 +265,7 @@ QuantParams quant_params(const Range& r) {
     p.hi = r.hi;
     p.width = r.hi - r.lo;
     p.rwidth = 1.0f / p.width;  // IEEE division on the host: correctly rounded
+    p.unrounded = r.unrounded;
     return p;
 }
 

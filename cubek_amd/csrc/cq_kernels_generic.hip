@@ -67,6 +67,16 @@ __device__ __forceinline__ float fetch_divisor(const GenericArgs& a, uint64_t el
     return F::round(s_fs);
 }
 
+__device__ __forceinline__ float decode_native(int value, uint32_t b);
+
+// The extension value CQ_VALUE_E2M1_OCP: the clamped quotient in F, cast once to e2m1 (nearest, ties to the even code;
+// the sign bit is the float's).
+template <class F>
+__device__ __forceinline__ uint32_t quantize_e2m1_unrounded(float x, float d, float lo, float hi) {
+    const float c = clamp_code(F::round(x / d), lo, hi);
+    return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, c, 0.0f, 1.0f, 0) & 0xfu;
+}
+
 template <class F>
 __global__ __launch_bounds__(kThreads) void quantize_generic_kernel(GenericArgs a, int bits) {
     uint64_t p = a.word_begin + static_cast<uint64_t>(blockIdx.x) * kThreads + threadIdx.x;
@@ -77,7 +87,12 @@ __global__ __launch_bounds__(kThreads) void quantize_generic_kernel(GenericArgs 
     const ValuePos vp = value_pos(a.vs, p, nq);
     uint32_t w = 0;
     for (uint32_t i = 0; i < nq; i++) {
-        float q = quantize_exact<F>(F::load(a.input, vp.f + i * vp.step), d, a.range.lo, a.range.hi);
+        const float x = F::load(a.input, vp.f + i * vp.step);
+        if (a.value == CQ_VALUE_E2M1_OCP) {
+            w |= quantize_e2m1_unrounded<F>(x, d, a.range.lo, a.range.hi) << (i * bits);
+            continue;
+        }
+        float q = quantize_exact<F>(x, d, a.range.lo, a.range.hi);
         w |= (static_cast<uint32_t>(static_cast<int32_t>(q)) & mask) << (i * bits);
     }
     static_cast<uint32_t*>(a.output)[vp.v] = w;
@@ -95,7 +110,8 @@ __global__ __launch_bounds__(kThreads) void dequantize_generic_kernel(GenericArg
     const uint32_t w = static_cast<const uint32_t*>(a.input)[vp.v];
     for (uint32_t i = 0; i < nq; i++) {
         int32_t v = static_cast<int32_t>(w << (32 - bits - i * bits)) >> (32 - bits);
-        F::store(a.output, vp.f + i * vp.step, s * static_cast<float>(v));
+        const float q = a.value == CQ_VALUE_E2M1_OCP ? decode_native(CQ_VALUE_E2M1, (w >> (i * bits)) & 0xfu) : static_cast<float>(v);
+        F::store(a.output, vp.f + i * vp.step, s * q);
     }
 }
 
@@ -155,7 +171,7 @@ __device__ __forceinline__ float decode_native(int value, uint32_t b) {
     switch (value) {
         case CQ_VALUE_E4M3: return __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(b), 0);
         case CQ_VALUE_E5M2: return __builtin_amdgcn_cvt_f32_bf8(static_cast<int>(b), 0);
-        case CQ_VALUE_E2M1: {
+        case CQ_VALUE_E2M1: case CQ_VALUE_E2M1_OCP: {
             uint32_t m = b & 7u;
             uint32_t bits = m == 0 ? 0u : (m == 1 ? 0x3f000000u : (((m >> 1) + 126u) << 23) | ((m & 1u) << 22));
             return bits_f32(bits | ((b & 8u) << 28));
@@ -170,12 +186,17 @@ __global__ __launch_bounds__(kThreads) void quantize_native_kernel(GenericArgs a
     uint64_t j = a.word_begin + static_cast<uint64_t>(blockIdx.x) * kThreads + threadIdx.x;
     if (j >= a.word_end) return;
     uint8_t* out = static_cast<uint8_t*>(a.output);
-    if (a.value == CQ_VALUE_E2M1) {
+    if (a.value == CQ_VALUE_E2M1 || a.value == CQ_VALUE_E2M1_OCP) {
         const ValuePos vp = value_pos(a.vs, j, 2);
         uint32_t byte = 0;
         for (uint32_t h = 0; h < 2; h++) {
             float d = fetch_divisor<F>(a, 2 * j + h);
-            float c = quantize_exact<F>(F::load(a.input, vp.f + h * vp.step), d, a.range.lo, a.range.hi);
+            const float x = F::load(a.input, vp.f + h * vp.step);
+            if (a.value == CQ_VALUE_E2M1_OCP) {
+                byte |= quantize_e2m1_unrounded<F>(x, d, a.range.lo, a.range.hi) << (4 * h);
+                continue;
+            }
+            float c = quantize_exact<F>(x, d, a.range.lo, a.range.hi);
             byte |= encode_native(a.value, c) << (4 * h);
         }
         out[vp.v] = static_cast<uint8_t>(byte);
@@ -192,7 +213,7 @@ template <class F>
 __global__ __launch_bounds__(kThreads) void dequantize_native_kernel(GenericArgs a) {
     uint64_t j = a.word_begin + static_cast<uint64_t>(blockIdx.x) * kThreads + threadIdx.x;
     if (j >= a.word_end) return;
-    const uint32_t per = a.value == CQ_VALUE_E2M1 ? 2u : 1u;
+    const uint32_t per = (a.value == CQ_VALUE_E2M1 || a.value == CQ_VALUE_E2M1_OCP) ? 2u : 1u;
     const ValuePos vp = value_pos(a.vs, j, per);
     const uint8_t b = static_cast<const uint8_t*>(a.input)[vp.v];
     for (uint32_t h = 0; h < per; h++) {

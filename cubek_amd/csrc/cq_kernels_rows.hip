@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(RowArgs a) {
         for (int i = 0; i < U::kChunks; i++) {
             float v[kN], qn[kN];
             F::unpack(raw[u][i], v);
-            quantize_values_neg<F, kN, kEnc == kEncInt>(v, d, tame, a.range.lo, a.range.hi, qn);
+            quantize_codes<F, kN, kEnc>(v, d, tame, a.range.lo, a.range.hi, a.range.unrounded != 0, qn);
             uint32_t cw[2] = {0, 0};
             if constexpr (kEnc == kEncInt)
                 pack_chunk_neg<kBits, kN, kWide>(qn, cw);
@@ -356,7 +356,7 @@ __global__ __launch_bounds__(kThreads) void quantize_blocks_kernel(RowArgs a, Bl
                 const bool row_live = rr < br;  // the same for every lane of a word
                 float v[kN], qn[kN];
                 F::unpack(raw[c][k], v);
-                quantize_values_neg<F, kN, kEnc == kEncInt>(v, d, tame, qp.lo, qp.hi, qn);
+                quantize_codes<F, kN, kEnc>(v, d, tame, qp.lo, qp.hi, qp.unrounded != 0, qn);
                 uint32_t w[2] = {0, 0};
                 if constexpr (kEnc == kEncInt)
                     pack_chunk_neg<kBits, kN, kWide>(qn, w);
@@ -597,6 +597,7 @@ hipError_t quantize_blocks(hipStream_t s, int bits, const RowArgs& a) {
     qp.hi = a.range.hi;
     qp.width = a.range.hi - a.range.lo;
     qp.rwidth = 1.0f / qp.width;  // IEEE division on the host: correctly rounded
+    qp.unrounded = a.range.unrounded;
     const bool wide = a.range.hi > 127.0f || a.range.lo < -128.0f;
     switch (a.encoding) {
         case kEncInt:

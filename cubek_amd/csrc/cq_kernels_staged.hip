@@ -35,6 +35,7 @@ QuantParams quant_params(const Range& r) {
     p.hi = r.hi;
     p.width = r.hi - r.lo;
     p.rwidth = 1.0f / p.width;  // IEEE division on the host: correctly rounded
+    p.unrounded = r.unrounded;
     return p;
 }
 
@@ -50,7 +51,7 @@ __device__ __forceinline__ void quantize_chunk(const float* v, float d, bool tam
         }
     }
     float qn[kN];
-    quantize_values_neg<F, kN, kEnc == kEncInt>(v, d, tame, qp.lo, qp.hi, qn);
+    quantize_codes<F, kN, kEnc>(v, d, tame, qp.lo, qp.hi, qp.unrounded != 0, qn);
     if constexpr (kEnc == kEncInt)
         pack_chunk_neg<kBits, kN, false>(qn, w);
     else

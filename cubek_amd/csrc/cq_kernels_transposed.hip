@@ -164,7 +164,7 @@ __device__ __forceinline__ void quantize_piece_words(const float* v, float d, bo
 #pragma unroll
         for (int i = 0; i < U::kChunks; i++) {
             float qn[kN];
-            quantize_values_neg<F, kN, kEnc == kEncInt>(v + u * U::kV + i * kN, d, tame, qp.lo, qp.hi, qn);
+            quantize_codes<F, kN, kEnc>(v + u * U::kV + i * kN, d, tame, qp.lo, qp.hi, qp.unrounded != 0, qn);
             uint32_t cw[2] = {0, 0};
             if constexpr (kEnc == kEncInt)
                 pack_chunk_neg<kBits, kN, kWide>(qn, cw);
@@ -867,6 +867,7 @@ hipError_t quantize_transposed(hipStream_t s, int bits, const TransposedArgs& a)
     qp.hi = a.range.hi;
     qp.width = a.range.hi - a.range.lo;
     qp.rwidth = 1.0f / qp.width;  // IEEE division on the host: correctly rounded
+    qp.unrounded = a.range.unrounded;
     const bool wide = a.range.hi > 127.0f || a.range.lo < -128.0f;
     // Quads of lanes wherever the runs are 8-byte aligned: blocks of 64 / 128 columns are read once
     // instead of twice, blocks of 32 cost a quarter of the store requests (4-bit codes of a transposed

@@ -26,12 +26,15 @@ class QuantValue(enum.IntEnum):
     E2M1 = 6
     E4M3 = 7
     E5M2 = 8
+    #: extension without a counterpart in the reference: OCP FP4 rounded once, straight to the e2m1 grid
+    #: (0.5 and 1.5 occur), e2m1 nibbles in either store; never what the E2M1 value of the reference produces
+    E2M1_OCP = 9
 
     def size_bits(self) -> int:
         """Bits of one quantized value (call sites src/quantize.rs:62)."""
         if self in (QuantValue.Q8F, QuantValue.Q8S, QuantValue.E4M3, QuantValue.E5M2):
             return 8
-        if self in (QuantValue.Q4F, QuantValue.Q4S, QuantValue.E2M1):
+        if self in (QuantValue.Q4F, QuantValue.Q4S, QuantValue.E2M1, QuantValue.E2M1_OCP):
             return 4
         return 2
 
@@ -55,6 +58,7 @@ _RANGES = {
     QuantValue.E2M1: (-6.0, 6.0),
     QuantValue.E4M3: (-448.0, 448.0),
     QuantValue.E5M2: (-57344.0, 57344.0),
+    QuantValue.E2M1_OCP: (-6.0, 6.0),
 }
 
 
@@ -192,7 +196,7 @@ class QuantScheme:
 
     def native_packing(self) -> int:
         """Values per stored element of the native store (2 for e2m1 bytes)."""
-        return 2 if (self.store == QuantStore.Native and self.value == QuantValue.E2M1) else 1
+        return 2 if (self.store == QuantStore.Native and self.value in (QuantValue.E2M1, QuantValue.E2M1_OCP)) else 1
 
     def num_quants(self) -> int:
         """Values per stored element: 32/size_bits for the U32 store

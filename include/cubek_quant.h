@@ -74,7 +74,15 @@ typedef enum cq_value {
     CQ_VALUE_Q2S = 5,
     CQ_VALUE_E2M1 = 6,
     CQ_VALUE_E4M3 = 7,
-    CQ_VALUE_E5M2 = 8
+    CQ_VALUE_E5M2 = 8,
+    /* Extension with no counterpart in the reference (never produced by, and never to be passed as, E2M1):
+     * OCP microscaling FP4.  The quotient x / scale is clamped to [-6, 6] in the tensor's float type and
+     * rounded ONCE, to the nearest of {0, 0.5, 1, 1.5, 2, 3, 4, 6} (ties to the even code), without the
+     * integer rounding the reference applies first (src/quantize.rs:33-43), so 0.5 and 1.5 occur.  Both stores
+     * hold e2m1 nibbles: eight per u32 word, value i in bits [4i, 4i+4), or two per byte, value 2k in the low
+     * nibble; the two layouts are the same bytes.  Dequantize decodes the nibble and multiplies by the scale.
+     * The scale rule is the common one: 2 * absmax / (6 - -6) = absmax / 6. */
+    CQ_VALUE_E2M1_OCP = 9
 } cq_value;
 
 typedef enum cq_param { /* QuantParam: dtype of the stored scales */

@@ -35,7 +35,8 @@ struct LaunchError : std::runtime_error {
 
 namespace scheme {
 
-enum class QuantValue : uint8_t { Q8F = 0, Q8S, Q4F, Q4S, Q2F, Q2S, E2M1, E4M3, E5M2 };
+// E2M1Ocp is an extension without a counterpart in the reference (see CQ_VALUE_E2M1_OCP in cubek_quant.h).
+enum class QuantValue : uint8_t { Q8F = 0, Q8S, Q4F, Q4S, Q2F, Q2S, E2M1, E4M3, E5M2, E2M1Ocp };
 enum class QuantParam : uint8_t { F32 = 0, F16, BF16 };
 enum class QuantStore : uint8_t { U32 = 0, Native };
 enum class QuantMode : uint8_t { Symmetric = 0 };

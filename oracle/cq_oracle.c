@@ -36,6 +36,11 @@
  *   - abs-max ignores NaN elements (Rust f32::max in the reference's test).
  * Given these decisions, every function below is pinned as listed above.
  *
+ * Extension.  CQ_VALUE_E2M1_OCP (OCP microscaling FP4 without the reference's integer rounding) has no
+ * counterpart in the reference, so there is no parity to speak of; its arm here defines what the kernels must
+ * produce, and it is pinned against the exact-rational model (tests/golden/, cases named ocp_*) and against a
+ * nearest-value search over the eight e2m1 magnitudes.
+ *
  * Build: gcc -O2 -fno-fast-math -ffp-contract=off (see Makefile).
  */
 #include "cq_oracle.h"
@@ -198,7 +203,7 @@ static inline int param_dtype(uint8_t param) {
 uint32_t cqo_value_size_bits(uint8_t value) {
     switch (value) {
         case CQ_VALUE_Q8F: case CQ_VALUE_Q8S: case CQ_VALUE_E4M3: case CQ_VALUE_E5M2: return 8;
-        case CQ_VALUE_Q4F: case CQ_VALUE_Q4S: case CQ_VALUE_E2M1: return 4;
+        case CQ_VALUE_Q4F: case CQ_VALUE_Q4S: case CQ_VALUE_E2M1: case CQ_VALUE_E2M1_OCP: return 4;
         case CQ_VALUE_Q2F: case CQ_VALUE_Q2S: return 2;
         default: return 0;
     }
@@ -211,7 +216,7 @@ uint32_t cqo_num_quants(const cq_scheme* s) {
     uint32_t bits = cqo_value_size_bits(s->value);
     if (bits == 0) return 0;
     if (s->store == CQ_STORE_U32) return 32u / bits;
-    return s->value == CQ_VALUE_E2M1 ? 2u : 1u;
+    return (s->value == CQ_VALUE_E2M1 || s->value == CQ_VALUE_E2M1_OCP) ? 2u : 1u;
 }
 
 int cqo_value_range(uint8_t value, float* lo, float* hi) {
@@ -222,7 +227,7 @@ int cqo_value_range(uint8_t value, float* lo, float* hi) {
         case CQ_VALUE_Q4S: *lo = -7.f; *hi = 7.f; return 0;
         case CQ_VALUE_Q2F: *lo = -2.f; *hi = 1.f; return 0;
         case CQ_VALUE_Q2S: *lo = -1.f; *hi = 1.f; return 0;
-        case CQ_VALUE_E2M1: *lo = -6.f; *hi = 6.f; return 0;
+        case CQ_VALUE_E2M1: case CQ_VALUE_E2M1_OCP: *lo = -6.f; *hi = 6.f; return 0;
         case CQ_VALUE_E4M3: *lo = -448.f; *hi = 448.f; return 0;
         case CQ_VALUE_E5M2: *lo = -57344.f; *hi = 57344.f; return 0;
         default: return -1;
@@ -295,6 +300,13 @@ static inline float quantize_one(float x, float d, int dtype, float lo, float hi
     return fmaxf(lo, fminf(r, hi));   /* Line::clamp */
 }
 
+/* The extension value CQ_VALUE_E2M1_OCP (no counterpart in the reference): the quotient in F, clamped, WITHOUT the
+ * integer rounding; the one rounding is the cast to e2m1 that follows (cqo_f32_to_e2m1: nearest, ties to even). */
+static inline float quantize_one_unrounded(float x, float d, int dtype, float lo, float hi) {
+    float t = round_to(dtype, x / d);
+    return fmaxf(lo, fminf(t, hi));
+}
+
 /* write_scale (src/quantize.rs:83-98): FS(scale_in[idx]); store at block start.
  * Returns the divisor F(FS(scale)) widened to f32. */
 static inline float write_scale(const cq_scheme* s, uint32_t rank, const uint64_t* shape,
@@ -332,8 +344,11 @@ int cqo_quantize_packed(const void* input, int dtype, uint32_t rank, const uint6
         float d = write_scale(s, rank, shape, scale, scale_strides, out_scale, out_scale_strides,
                               dtype, packed_pos);
         int32_t codes[16];
-        for (uint32_t i = 0; i < nq; i++)
-            codes[i] = (int32_t)quantize_one(load_f(input, dtype, packed_pos + i), d, dtype, lo, hi);
+        for (uint32_t i = 0; i < nq; i++) {
+            float x = load_f(input, dtype, packed_pos + i);
+            codes[i] = s->value == CQ_VALUE_E2M1_OCP ? (int32_t)cqo_f32_to_e2m1(quantize_one_unrounded(x, d, dtype, lo, hi))
+                                                      : (int32_t)quantize_one(x, d, dtype, lo, hi);
+        }
         output[p] = cqo_pack_word(codes, bits);
     }
     return 0;
@@ -357,6 +372,7 @@ int cqo_dequantize_packed(const uint32_t* values, uint32_t rank, const uint64_t*
         cqo_unpack_word(values[p], bits, codes);
         for (uint32_t i = 0; i < nq; i++) {
             float v = (float)codes[i]; /* F::cast_from(signed_value), exact */
+            if (s->value == CQ_VALUE_E2M1_OCP) v = cqo_e2m1_to_f32((uint8_t)(codes[i] & 0xf)); /* extension: the nibble decoded */
             store_f(output, dtype, e0 + i, sc * v);
         }
     }
@@ -375,12 +391,13 @@ int cqo_quantize_native(const void* input, int dtype, uint32_t rank, const uint6
     for (uint64_t e = elem_begin; e < elem_end; e++) {
         float d = write_scale(s, rank, shape, scale, scale_strides, out_scale, out_scale_strides,
                               dtype, e);
-        float c = quantize_one(load_f(input, dtype, e), d, dtype, lo, hi);
+        float c = s->value == CQ_VALUE_E2M1_OCP ? quantize_one_unrounded(load_f(input, dtype, e), d, dtype, lo, hi)
+                                                : quantize_one(load_f(input, dtype, e), d, dtype, lo, hi);
         switch (s->value) {
             case CQ_VALUE_Q8F: case CQ_VALUE_Q8S: output[e] = (uint8_t)(int8_t)(int32_t)c; break;
             case CQ_VALUE_E4M3: output[e] = cqo_f32_to_e4m3(c); break;
             case CQ_VALUE_E5M2: output[e] = cqo_f32_to_e5m2(c); break;
-            case CQ_VALUE_E2M1: {
+            case CQ_VALUE_E2M1: case CQ_VALUE_E2M1_OCP: {
                 uint8_t nib = cqo_f32_to_e2m1(c);
                 uint8_t old = (e & 1) ? output[e >> 1] : 0;
                 output[e >> 1] = (e & 1) ? (uint8_t)((old & 0x0f) | (nib << 4)) : nib;
@@ -406,7 +423,7 @@ int cqo_dequantize_native(const uint8_t* values, uint32_t rank, const uint64_t* 
             case CQ_VALUE_Q8F: case CQ_VALUE_Q8S: v = (float)(int8_t)values[e]; break;
             case CQ_VALUE_E4M3: v = cqo_e4m3_to_f32(values[e]); break;
             case CQ_VALUE_E5M2: v = cqo_e5m2_to_f32(values[e]); break;
-            case CQ_VALUE_E2M1: v = cqo_e2m1_to_f32((values[e >> 1] >> ((e & 1) * 4)) & 0xf); break;
+            case CQ_VALUE_E2M1: case CQ_VALUE_E2M1_OCP: v = cqo_e2m1_to_f32((values[e >> 1] >> ((e & 1) * 4)) & 0xf); break;
             default: return -1;
         }
         store_f(output, dtype, e, sc * round_to(dtype, v));

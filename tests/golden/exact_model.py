@@ -88,12 +88,12 @@ def fraction_to_bits(q: Fraction, fmt: str) -> int:
 
 
 def size_bits(value: str) -> int:
-    return {"Q8F": 8, "Q8S": 8, "E4M3": 8, "E5M2": 8, "Q4F": 4, "Q4S": 4, "E2M1": 4,
+    return {"Q8F": 8, "Q8S": 8, "E4M3": 8, "E5M2": 8, "Q4F": 4, "Q4S": 4, "E2M1": 4, "E2M1_OCP": 4,
             "Q2F": 2, "Q2S": 2}[value]
 
 
 RANGES = {"Q8F": (-128, 127), "Q8S": (-127, 127), "Q4F": (-8, 7), "Q4S": (-7, 7),
-          "Q2F": (-2, 1), "Q2S": (-1, 1), "E2M1": (-6, 6), "E4M3": (-448, 448),
+          "Q2F": (-2, 1), "Q2S": (-1, 1), "E2M1": (-6, 6), "E2M1_OCP": (-6, 6), "E4M3": (-448, 448),
           "E5M2": (-57344, 57344)}
 
 
@@ -217,7 +217,9 @@ def scales_from_absmax(x_bits: np.ndarray, fmt: str, shape: Sequence[int],
 # ---------------------------------------------------------------- native store
 # name -> (exponent bits, mantissa bits, bias): OCP 8-bit floating point (E4M3 finite-only
 # with one NaN code, E5M2 IEEE-like) and OCP microscaling FP4 (E2M1, no NaN, no infinity)
-MINIFLOATS = {"E4M3": (4, 3, 7), "E5M2": (5, 2, 15), "E2M1": (2, 1, 1)}
+MINIFLOATS = {"E4M3": (4, 3, 7), "E5M2": (5, 2, 15), "E2M1": (2, 1, 1), "E2M1_OCP": (2, 1, 1)}
+#: values that share a byte in the native store (element 2k in the low nibble)
+NIBBLE_VALUES = ("E2M1", "E2M1_OCP")
 
 
 def minifloat_magnitudes(name: str) -> List[Fraction]:
@@ -266,6 +268,10 @@ def native_code(neg: bool, mag_q: Fraction, fmt: str, value: str) -> int:
     """Stored byte (nibble for E2M1) of one element: ``mag_q`` = |x| / |divisor| exactly,
     ``neg`` the sign of the quotient.  round to F, rint, clamp, cast to Q."""
     lo, hi = RANGES[value]
+    if value == "E2M1_OCP":
+        # the extension: no integer rounding; the quotient in F, clamped, is cast once to the e2m1 grid
+        t = min(round_to_format(mag_q, fmt), Fraction(-lo if neg else hi))
+        return (int(neg) << 3) | minifloat_encode(t, value)
     k = rint_even(round_to_format(mag_q, fmt))  # |rint(t)|: both roundings are sign-symmetric
     k = min(k, -lo) if neg else min(k, hi)
     if value in ("Q8F", "Q8S"):
@@ -296,7 +302,7 @@ def quantize_tensor_native(x_bits: np.ndarray, fmt: str, shape: Sequence[int], s
     nibbles per byte with element 2k in the LOW nibble and element 2k+1 in the high one.
     Returns (bytes uint8, out_scale bit patterns in param_fmt)."""
     n = int(np.prod(shape))
-    per_byte = 2 if value == "E2M1" else 1
+    per_byte = 2 if value in NIBBLE_VALUES else 1
     out = np.zeros(n // per_byte, dtype=np.uint8)
     out_scale = np.zeros(scale_bits.size, dtype=np.uint32 if param_fmt == "f32" else np.uint16)
     blk_vec = None if block is None else (1,) * (len(shape) - len(block)) + tuple(block)
@@ -328,7 +334,7 @@ def dequantize_tensor_native(codes: np.ndarray, fmt: str, shape: Sequence[int], 
         si, _ = _scale_lookup(e, shape, blk_vec, scale_strides)
         s_neg, s_mag = sign_and_magnitude(int(scale_bits.reshape(-1)[si]), param_fmt)
         s = round_to_format(s_mag, fmt)
-        code = int(codes[e // 2] >> (4 * (e % 2))) & 0xF if value == "E2M1" else int(codes[e])
+        code = int(codes[e // 2] >> (4 * (e % 2))) & 0xF if value in NIBBLE_VALUES else int(codes[e])
         q_neg, q_mag = native_decode(code, value)
         out[e] = signed_bits(s_neg != q_neg, round_to_format(s * q_mag, fmt), fmt)
     return out

@@ -17,6 +17,8 @@ Cases
                   pairs for f32/bf16/f16 inputs: every integer quotient of the value
                   range and every half-integer in between, signed zeros, random data
                   with abs-max scales per tensor and per block, f16/bf16 parameters.
+  typed_ocp.npz   the extension value E2M1_OCP (not in the reference): every multiple of 1/8 of
+                  the e2m1 range as a quotient, random data, three float and parameter types.
 """
 from __future__ import annotations
 
@@ -218,8 +220,47 @@ def typed_native():
     return len(store) // 6
 
 
+def typed_ocp():
+    """The extension value E2M1_OCP (no counterpart in the reference): e2m1 nibbles rounded once from the
+    quotient.  Native-store layout; the U32 store holds the same bytes as little-endian words."""
+    rng = np.random.default_rng(20240611)
+    store = {}
+
+    def gauss(n, sigma):
+        return [Fraction(float(v)) for v in rng.normal(0.0, sigma, n)]
+
+    for fmt in ("f32", "bf16", "f16"):
+        # every multiple of 1/8 in [-7, 7] (all seven midpoints of the e2m1 grid, both signs, and the clamp),
+        # sixteenths near zero, signed zeros
+        vals = [Fraction(k, 8) for k in range(-56, 57)]
+        vals += [Fraction(s * k, 16) for k in (1, 3, 5) for s in (-1, 1)]
+        zeros_at = list(range(len(vals), len(vals) + 4))
+        vals += [Fraction(0)] * 4
+        while len(vals) % 64:
+            vals.append(Fraction(0))
+        n = len(vals)
+        sign_bit = 1 << (31 if fmt == "f32" else 15)
+        for tag, s in (("s0.25", Fraction(1, 4)), ("s-0.5", Fraction(-1, 2))):
+            x = to_fmt_bits([v * s for v in vals], fmt)
+            for i in zeros_at[:2]:
+                assert x[i] == 0
+                x[i] = sign_bit
+            run_case(store, f"ocp_ties_{fmt}_{tag}", x, fmt, (n // 64, 64), None, "E2M1_OCP", "f32",
+                     scale_bits=to_fmt_bits([s], fmt), native=True)
+        x = to_fmt_bits(gauss(4 * 128, 0.02), fmt)
+        run_case(store, f"ocp_rand_{fmt}_tensor", x, fmt, (4, 128), None, "E2M1_OCP", "f32", native=True)
+        for param in ("f32", "f16", "bf16"):
+            x = to_fmt_bits(gauss(4 * 128, 0.02), fmt)
+            run_case(store, f"ocp_rand_{fmt}_b32_{param}", x, fmt, (4, 128), (32,), "E2M1_OCP", param, native=True)
+    x = to_fmt_bits(gauss(4 * 6 * 32, 0.5), "f32")
+    run_case(store, "ocp_nd_f32_2x3x16", x, "f32", (4, 6, 32), (2, 3, 16), "E2M1_OCP", "f32", native=True)
+    np.savez_compressed(os.path.join(HERE, "typed_ocp.npz"), **store)
+    return len(store) // 6
+
+
 if __name__ == "__main__":
     a = reference_ramps()
     b = typed_small()
     c = typed_native()
-    print(f"wrote {a} reference ramp cases, {b} typed cases and {c} native-store cases")
+    d = typed_ocp()
+    print(f"wrote {a} reference ramp cases, {b} typed cases, {c} native-store cases and {d} cases of the e2m1 extension")

@@ -22,6 +22,7 @@ CASES = [
     (ElemType.F16, QuantValue.Q4S, [32], QuantParam.F32, 21, 16480, None),        # eight waves per workgroup
     (ElemType.BF16, QuantValue.Q4F, [32], QuantParam.F32, 1, 32768, None),        # one row, the longest it takes
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 9, 32, None),           # one block per row
+    (ElemType.BF16, QuantValue.E2M1_OCP, [32], QuantParam.F32, 37, 2048, None),   # the extension value: e2m1 nibbles in u32 words
     (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 11, 53248, None),       # rows longer than the LDS holds of x
     (ElemType.F16, QuantValue.Q8S, [64], QuantParam.F16, 5, 40000, None),         # ... 8-bit codes, two segments
     (ElemType.F16, QuantValue.Q4S, [128], QuantParam.F16, 33, 4224, None),        # four units under one f16 scale
@@ -122,6 +123,7 @@ NATIVE_CASES = [
     (ElemType.F16, QuantValue.Q8F, [16], QuantParam.BF16, 9, 16, None),             # one unit per row
     (ElemType.F32, QuantValue.E4M3, [32], QuantParam.F32, 37, 2080, None),          # x in f32
     (ElemType.F32, QuantValue.E2M1, [64], QuantParam.F32, 12, 4160, None),
+    (ElemType.BF16, QuantValue.E2M1_OCP, [32], QuantParam.F32, 41, 4160, None),     # the extension value: e2m1 pairs
 ]
 
 

@@ -16,8 +16,8 @@ from cubek_amd import quantize as qz
 pytestmark = pytest.mark.gpu
 
 VALUES_U32 = [QuantValue.Q8F, QuantValue.Q8S, QuantValue.Q4F, QuantValue.Q4S, QuantValue.Q2F, QuantValue.Q2S,
-              QuantValue.E2M1, QuantValue.E4M3, QuantValue.E5M2]
-VALUES_NATIVE = [QuantValue.Q8F, QuantValue.Q8S, QuantValue.E4M3, QuantValue.E5M2, QuantValue.E2M1]
+              QuantValue.E2M1, QuantValue.E4M3, QuantValue.E5M2, QuantValue.E2M1_OCP]
+VALUES_NATIVE = [QuantValue.Q8F, QuantValue.Q8S, QuantValue.E4M3, QuantValue.E5M2, QuantValue.E2M1, QuantValue.E2M1_OCP]
 
 
 @pytest.fixture(scope="module")

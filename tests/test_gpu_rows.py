@@ -23,6 +23,8 @@ CASES = [
     ((96, 256), (16, 128), QuantValue.E4M3, QuantStore.Native),
     ((48, 192), (8, 48), QuantValue.E5M2, QuantStore.Native),
     ((40, 320), (4, 32), QuantValue.E2M1, QuantStore.Native),
+    ((96, 256), (32, 64), QuantValue.E2M1_OCP, QuantStore.U32),      # the extension value, both stores
+    ((48, 320), (8, 32), QuantValue.E2M1_OCP, QuantStore.Native),
     ((7, 4, 3, 64), (4, 3, 32), QuantValue.Q4F, QuantStore.U32),    # block over three dimensions: scales per element
 ]
 

@@ -53,6 +53,8 @@ PIECES = [
     ((77, 1080), (120,), QuantValue.E4M3, QuantStore.Native),
     ((50, 2040), (136,), QuantValue.E5M2, QuantStore.Native),
     ((9, 4960), (248,), QuantValue.E2M1, QuantStore.Native),
+    ((33, 1320), (40,), QuantValue.E2M1_OCP, QuantStore.U32),
+    ((21, 1440), (72,), QuantValue.E2M1_OCP, QuantStore.Native),
     ((2000, 24), (24,), QuantValue.Q8S, QuantStore.Native),
     ((5, 240), (80,), QuantValue.Q2F, QuantStore.U32),
 ]
@@ -213,6 +215,8 @@ TILE_CASES = [
     (5, 4160, 32, QuantValue.Q2S, QuantStore.U32),
     (40, 1280, 128, QuantValue.E4M3, QuantStore.Native),
     (64, 640, 32, QuantValue.E2M1, QuantStore.Native),
+    (45, 1088, 32, QuantValue.E2M1_OCP, QuantStore.U32),
+    (20, 1024, 64, QuantValue.E2M1_OCP, QuantStore.Native),
     (37, 768, 128, QuantValue.Q8F, QuantStore.Native),
 ]
 

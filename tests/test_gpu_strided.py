@@ -108,6 +108,10 @@ SCHEMES = [
     ("e4m3_native_tensor", QuantScheme.default().with_value(QuantValue.E4M3).with_store(QuantStore.Native)),
     ("e2m1_native_block32", QuantScheme.default().with_value(QuantValue.E2M1).with_store(QuantStore.Native)
      .with_level(QuantLevel.block([32]))),
+    # the extension value (e2m1 nibbles rounded once, in either store)
+    ("ocp_u32_block32", QuantScheme.default().with_value(QuantValue.E2M1_OCP).with_level(QuantLevel.block([32]))),
+    ("ocp_native_block16", QuantScheme.default().with_value(QuantValue.E2M1_OCP).with_store(QuantStore.Native)
+     .with_level(QuantLevel.block([16]))),
     # blocks of 64 / 128 columns: on transposed floats, lanes share a block
     ("q8s_block64", QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([64]))),
     ("q4s_block128", QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([128]))),
@@ -285,6 +289,9 @@ LARGE_TRANSPOSED_SCHEMES = {
     "e4m3_native_block32": (QuantScheme.default().with_value(QuantValue.E4M3).with_store(QuantStore.Native)
                             .with_level(QuantLevel.block([32]))),
     "e2m1_block32": QuantScheme.default().with_value(QuantValue.E2M1).with_level(QuantLevel.block([32])),
+    "ocp_u32_block32": QuantScheme.default().with_value(QuantValue.E2M1_OCP).with_level(QuantLevel.block([32])),
+    "ocp_native_block64": (QuantScheme.default().with_value(QuantValue.E2M1_OCP).with_store(QuantStore.Native)
+                           .with_level(QuantLevel.block([64]))),
     "q2s_block32": QuantScheme.default().with_value(QuantValue.Q2S).with_level(QuantLevel.block([32])),
     "q8s_block32": QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.block([32])),
     "q4s_block64": QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block([64])),

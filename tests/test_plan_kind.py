@@ -189,3 +189,10 @@ def test_plan_kind_validates_like_the_entry_points():
     assert e.value.status == _ffi.ERR_BLOCK_NOT_DIVISIBLE
     # an empty tensor launches nothing
     assert _ffi.plan_kind(_ffi.OP_DEQUANTIZE, t((0, 64), 4), t((0, 16), 4), t((0, 2), 4), None, s, F32) == "none"
+
+
+def test_extension_value_runs_on_the_streaming_kernels():
+    """E2M1_OCP (no counterpart in the reference) takes the same families as the native e2m1 encoding, in both stores."""
+    for store in (QuantStore.U32, QuantStore.Native):
+        got = kinds(scheme_of(QuantValue.E2M1_OCP, [32], store=store), BF16, (28672, 8192))
+        assert set(got.values()) == {"flat"}, (store, got)
