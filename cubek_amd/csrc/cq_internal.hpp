@@ -281,6 +281,8 @@ hipError_t gemv_stream_f32_scales(hipStream_t s, const GemvArgs& a);    // the s
 hipError_t gemv_stream_16bit_scales(hipStream_t s, const GemvArgs& a);
 hipError_t gemv_stream_batched(hipStream_t s, const GemvArgs& a);
 hipError_t gemv_stream_f32_x(hipStream_t s, const GemvArgs& a);
+bool gemv_mfma_takes(const GemvArgs& a);  // ... on the matrix cores (4-bit fields, blocks of 32, f32 scales, 1 - 4 vectors)
+hipError_t gemv_mfma(hipStream_t s, const GemvArgs& a);
 hipError_t launch_gemv_quantized(hipStream_t s, const GemvArgs& a);
 
 }  // namespace cq

@@ -580,6 +580,7 @@ bool gemv_streams(const GemvArgs& a) {
 namespace {
 
 hipError_t launch_one(hipStream_t s, const GemvArgs& a) {
+    if (gemv_mfma_takes(a)) return gemv_mfma(s, a);  // two to four vectors of the common 4-bit layout: matrix cores
     if (gemv_streams(a)) {
         if (a.dtype == CQ_F32) return gemv_stream_f32_x(s, a);
         if (a.vectors > 1 || a.cols > kStreamMaxColumns) return gemv_stream_batched(s, a);

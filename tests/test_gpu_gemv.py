@@ -133,6 +133,27 @@ def test_gemv_native_store_matches_oracle_dequantized_weights(oracle, case):
     check_case(oracle, case, rows * 11 + cols, native=True)
 
 
+# 4-bit fields on blocks of 32 with f32 scales, rows of whole groups of 128 values: two to four vectors at once go to
+# the matrix-core kernel (rows in runs of 2048 or 4096 values; a last run cut short; rows not a multiple of 16; pitched
+# rows; more vectors than four in turns, a last single one on the streaming kernel)
+MATRIX_CORE_CASES = [
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 64, 4096, None),
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 77, 4224, None),
+    (ElemType.F16, QuantValue.Q4F, [32], QuantParam.F32, 333, 8192, None),
+    (ElemType.BF16, QuantValue.E2M1, [32], QuantParam.F32, 130, 11008, None),
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 50, 8448, 1060),
+    (ElemType.BF16, QuantValue.Q4S, [32], QuantParam.F32, 21, 16512, None),
+    (ElemType.F16, QuantValue.Q4S, [32], QuantParam.F32, 5, 6144, None),
+    (ElemType.BF16, QuantValue.Q4F, [32], QuantParam.F32, 1, 4096, None),
+]
+
+
+@pytest.mark.parametrize("vectors", [2, 3, 4, 5, 9])
+@pytest.mark.parametrize("case", MATRIX_CORE_CASES, ids=_id)
+def test_gemv_on_the_matrix_cores(oracle, case, vectors):
+    check_case(oracle, case, 3 + vectors, vectors=vectors)
+
+
 @pytest.mark.parametrize("vectors", [2, 3, 4, 7, 8, 11])
 @pytest.mark.parametrize("kind", ["q4-b32", "q8-b64-f16", "e4m3-native", "q4-general", "q4-wide", "e2m1-native-wide",
                                   "e5m2-native", "q2-in-turns"])
