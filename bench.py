@@ -260,12 +260,12 @@ def graph_region(torch, paths, method, launches=32, replays=5):
     return sorted(times)[len(times) // 2]
 
 
-def replicas(torch, w, x, min_footprint=1 << 30, max_sets=8):
+def replicas(torch, w, x, min_footprint=1 << 30, max_sets=8, min_sets=1):
     """Independent buffer sets of one workload, enough of them that a launch never
     finds its operands in the 256 MB Infinity Cache or in L2 from the previous
     launch on the same set (cold, HBM-bound timing).  Set 0 holds the seeded
     input; the others hold copies of it."""
-    n_sets = max(1, min(max_sets, -(-min_footprint // algorithmic_bytes(w))))
+    n_sets = max(min_sets, min(max_sets, -(-min_footprint // algorithmic_bytes(w))))
     paths = [Path(torch, w, x)]
     for _ in range(n_sets - 1):
         paths.append(Path(torch, w, x.clone()))
@@ -397,6 +397,45 @@ def copy_yardstick(torch, x, launches=24):
     return {"what": "torch.Tensor.copy_ of the input tensor, device to device, rotated buffer sets",
             "bytes_read_plus_written": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
             "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+
+
+PROBES_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cubek_amd", "lib", "libcq_bench_probes.so")
+
+
+def memory_yardsticks(torch, nbytes, q_read, q_written):
+    """What this GPU's memory gives kernels that compute nothing, launched like the streaming kernels (bench probes,
+    cubek_amd/csrc/cq_bench_probes.hip): a pure read stream, a pure write stream and a copy of `nbytes`, rotated buffers,
+    median of 50 regions.  `additive_ms_*`: the time the headline kernels' own bytes would take as a pure read stream
+    plus a pure write stream, which is where reads and writes that do not overlap end up."""
+    import ctypes
+
+    if not os.path.exists(PROBES_PATH):
+        return {"skipped": f"{PROBES_PATH} is not built (make -C cubek_amd/csrc)"}
+    L = ctypes.CDLL(PROBES_PATH)
+    L.cq_probe_run.restype = ctypes.c_int
+    L.cq_probe_run.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64,
+                               ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]
+    sets = max(2, min(8, -(-(1 << 30) // nbytes)))
+    bufs = [torch.randint(0, 2 ** 31 - 1, (nbytes // 4,), dtype=torch.int32, device="cuda") for _ in range(sets)]
+    outs = [torch.empty((nbytes // 4,), dtype=torch.int32, device="cuda") for _ in range(sets)]
+    stream = torch.cuda.current_stream().cuda_stream
+    moved = ctypes.c_uint64(0)
+    out = {"what": "read / write / copy kernels that compute nothing (cq_bench_probes.hip), same launch shape as the "
+                   "streaming kernels, rotated buffers, median of 50 regions", "bytes": nbytes}
+    rates = {}
+    for kind, name in ((0, "read_only"), (1, "write_only"), (2, "copy")):
+        def fn(i, kind=kind):
+            rc = L.cq_probe_run(kind, stream, bufs[i % sets].data_ptr(), outs[i % sets].data_ptr(), nbytes, None,
+                                ctypes.byref(moved))
+            assert rc == 0, rc
+        ms = timed_median(torch, fn)["median_ms"]
+        b = moved.value * (2 if kind == 2 else 1)
+        rates[name] = moved.value / (ms * 1e-3) / 1e9  # per direction
+        out[name] = {"ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                     "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+    out["additive_ms_quantize"] = round((q_read / rates["read_only"] + q_written / rates["write_only"]) * 1e-6, 4)
+    out["additive_ms_dequantize"] = round((q_written / rates["read_only"] + q_read / rates["write_only"]) * 1e-6, 4)
+    return out
 
 
 def scheme_matrix(torch):
@@ -829,7 +868,8 @@ def main():
     step_bytes = 2 * q_bytes
     n = x.numel()
 
-    paths = replicas(torch, w, x)
+    # (at least four sets: where the buffers lie in memory moves a launch by up to 2 %, and four placements average it)
+    paths = replicas(torch, w, x, min_sets=4)
     path = paths[0]
     # the process's first launches: what the runtime takes to load the library's code objects is in here
     torch.cuda.synchronize()
@@ -846,6 +886,13 @@ def main():
         p.quantize_dynamic()
         p.dequantize()
 
+    # The clocks of a GPU that has been idle take a few hundred milliseconds of load to settle (the first regions of a
+    # fresh process read 3 - 5 % slower than everything after them): load it for about 0.4 s before anything is timed.
+    settle_until = time.perf_counter() + 0.4
+    while time.perf_counter() < settle_until:
+        for i in range(16):
+            step(i)
+        torch.cuda.synchronize()
     # timed region: exactly K steps between synchronize() calls
     ev_ms, ms_per_step = timed_region(torch, step, args.steps, warmup=args.warmup)
     # the two kernels of the step, each alone: the average over one region of K back-to-back launches (what a
@@ -898,6 +945,13 @@ def main():
     }
 
     result["copy_yardstick"] = yardstick
+    # the headline kernels' bytes: floats on one side, codes + scales on the other
+    float_bytes = n * (2 if w["elem"] != "F32" else 4)
+    result["memory_yardsticks"] = memory_yardsticks(torch, float_bytes, float_bytes, q_bytes - float_bytes)
+    if "additive_ms_quantize" in result["memory_yardsticks"]:
+        y = result["memory_yardsticks"]
+        result["roofline"]["frac_of_read_plus_write_streams"] = round(y["additive_ms_quantize"] / q_med["median_ms"], 4)
+        result["roofline_dequantize"]["frac_of_read_plus_write_streams"] = round(y["additive_ms_dequantize"] / d_med["median_ms"], 4)
     result["first_call_ms"] = {"quantize_dynamic": round(first_ms[0], 2), "dequantize": round(first_ms[1], 2),
                                "library_bytes": os.path.getsize(_ffi.LIB_PATH)}
     if not args.no_cpu:
@@ -910,7 +964,7 @@ def main():
         del path, paths, x
         for name, wk in WORKLOADS.items():
             xi = make_input(torch, wk)
-            ps = replicas(torch, wk, xi)
+            ps = replicas(torch, wk, xi, min_sets=4)
             b = algorithmic_bytes(wk)
             for p in ps:
                 p.compute_scales()

@@ -18,3 +18,19 @@ def test_world_size_from_a_launcher_is_refused_too():
     proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py")], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
                           text=True, timeout=120, env=env)
     assert proc.returncode != 0 and "one GPU" in proc.stderr
+
+
+def test_bench_probe_library_loads():
+    """bench.py's memory yardsticks (cubek_amd/csrc/cq_bench_probes.hip): the library is built, exports its one entry
+    point, and refuses bad arguments before it touches the GPU."""
+    import ctypes
+
+    import bench
+
+    assert os.path.exists(bench.PROBES_PATH), "make -C cubek_amd/csrc builds it"
+    L = ctypes.CDLL(bench.PROBES_PATH)
+    L.cq_probe_run.restype = ctypes.c_int
+    L.cq_probe_run.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64,
+                               ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]
+    assert L.cq_probe_run(0, None, None, None, 100, None, None) == -1      # less than one tile
+    assert L.cq_probe_run(7, None, None, None, 1 << 20, None, None) == -1  # no such probe
