@@ -235,7 +235,7 @@ void launch_float(hipStream_t s, const GemvArgs& a) {
 bool gemv_mfma_takes(const GemvArgs& a) {
     if (a.native != 0 || a.bits != 4 || a.param_dtype != CQ_F32 || a.dtype == CQ_F32) return false;
     if (a.block_rows != 1 || a.block_cols != 32 || a.scale_stride_col != 1) return false;
-    if (a.cols % 128 != 0 || a.cols < 4096 || a.cols >= (1u << 26)) return false;
+    if (a.cols % 128 != 0 || a.cols < 4096 || a.cols >= (1u << 26) || a.rows >= (1u << 31)) return false;
     if (a.word_pitch % 4 != 0 || a.scale_stride_row % 4 != 0 || !a.x_aligned16 || !a.words_aligned16) return false;
     if ((reinterpret_cast<uintptr_t>(a.scales) & 15u) != 0) return false;
     if (a.vectors > 1 && (a.x_stride * 2) % 16 != 0) return false;

@@ -25,7 +25,9 @@ namespace device {
 enum class Float { F32, F16, BF16 };
 
 // How the native store holds one value (QuantStore::Native; the U32 store always holds
-// two's-complement fields, whatever the value type).
+// two's-complement fields, whatever the value type of the reference).  The one exception is this library's
+// extension value CQ_VALUE_E2M1_OCP, whose u32 words hold eight e2m1 nibbles, the same bytes as the native
+// store's pairs: decode them with Native::E2M1x2 (dequantize_symmetric_native_value), not as fields.
 enum class Native { I8, E4M3, E5M2, E2M1x2 };
 
 // ---- scale parameters --------------------------------------------------------------------
