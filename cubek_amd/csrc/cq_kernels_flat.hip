@@ -41,26 +41,46 @@ uint32_t flat_family(const FlatArgs& a, int f_dtype) {
                : CQ_FAMILY_FLAT_LANES;
 }
 
+// the objects of cq_kernels_flat_quantize.hip, by float type, family of scale sources and width of the codes
+#define CQ_QUANTIZE_BY_BITS(f, g)                                              \
+    switch (bits) {                                                            \
+        case 2: return CQ_QUANTIZE_FLAT_TU(f, g, 2)(s, src, a);                \
+        case 4: return CQ_QUANTIZE_FLAT_TU(f, g, 4)(s, src, a);                \
+        case 8: return CQ_QUANTIZE_FLAT_TU(f, g, 8)(s, src, a);                \
+        default: return hipErrorInvalidValue;                                  \
+    }
 hipError_t launch_quantize_flat(hipStream_t s, int dtype, int bits, ScaleSource src, const FlatArgs& a) {
     if (a.num_chunks == 0) return hipSuccess;
     const bool given = src == ScaleSource::Given || src == ScaleSource::Stored;  // the objects that read scales
     switch (dtype) {
-        case CQ_F32: return given ? CQ_QUANTIZE_FLAT_TU(F32, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(F32, 0)(s, bits, src, a);
-        case CQ_BF16: return given ? CQ_QUANTIZE_FLAT_TU(BF16, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(BF16, 0)(s, bits, src, a);
-        case CQ_F16: return given ? CQ_QUANTIZE_FLAT_TU(F16, 1)(s, bits, src, a) : CQ_QUANTIZE_FLAT_TU(F16, 0)(s, bits, src, a);
+        case CQ_F32:
+            if (given) CQ_QUANTIZE_BY_BITS(F32, 1) else CQ_QUANTIZE_BY_BITS(F32, 0)
+        case CQ_BF16:
+            if (given) CQ_QUANTIZE_BY_BITS(BF16, 1) else CQ_QUANTIZE_BY_BITS(BF16, 0)
+        case CQ_F16:
+            if (given) CQ_QUANTIZE_BY_BITS(F16, 1) else CQ_QUANTIZE_BY_BITS(F16, 0)
         default: return hipErrorInvalidValue;
     }
 }
+#undef CQ_QUANTIZE_BY_BITS
 
+#define CQ_DEQUANTIZE_BY_BITS(f)                                               \
+    switch (bits) {                                                            \
+        case 2: return CQ_DEQUANTIZE_FLAT_TU(f, 2)(s, a);                      \
+        case 4: return CQ_DEQUANTIZE_FLAT_TU(f, 4)(s, a);                      \
+        case 8: return CQ_DEQUANTIZE_FLAT_TU(f, 8)(s, a);                      \
+        default: return hipErrorInvalidValue;                                  \
+    }
 hipError_t launch_dequantize_flat(hipStream_t s, int dtype, int bits, const FlatArgs& a) {
     if (a.num_chunks == 0) return hipSuccess;
     switch (dtype) {
-        case CQ_F32: return CQ_DEQUANTIZE_FLAT_TU(F32)(s, bits, a);
-        case CQ_BF16: return CQ_DEQUANTIZE_FLAT_TU(BF16)(s, bits, a);
-        case CQ_F16: return CQ_DEQUANTIZE_FLAT_TU(F16)(s, bits, a);
+        case CQ_F32: CQ_DEQUANTIZE_BY_BITS(F32)
+        case CQ_BF16: CQ_DEQUANTIZE_BY_BITS(BF16)
+        case CQ_F16: CQ_DEQUANTIZE_BY_BITS(F16)
         default: return hipErrorInvalidValue;
     }
 }
+#undef CQ_DEQUANTIZE_BY_BITS
 
 hipError_t launch_scales_flat(hipStream_t s, int dtype, const FlatArgs& a) {
     if (a.num_chunks == 0) return hipSuccess;

@@ -1,10 +1,13 @@
-// Launchers of the flat dequantize kernels of one float type.  The Makefile compiles this file three
-// times (-DCQ_TU_FLOAT=F32|BF16|F16), each into an object of its own: the build runs in parallel, and a
-// process loads the kernels of the float types it uses only.
+// Launchers of the flat dequantize kernels of one float type and one width of codes.  The Makefile compiles this
+// file nine times (-DCQ_TU_FLOAT=F32|BF16|F16, -DCQ_TU_BITS=2|4|8), each into an object of its own: the build runs
+// in parallel, and a process loads the kernels of the float types and widths it uses only.
 #include "cq_kernels_flat_launch.hpp"
 
 #ifndef CQ_TU_FLOAT
 #define CQ_TU_FLOAT F32
+#endif
+#ifndef CQ_TU_BITS
+#define CQ_TU_BITS 4
 #endif
 
 namespace cq {
@@ -82,12 +85,17 @@ hipError_t dequantize_launch(hipStream_t s, const FlatArgs& a) {
 #if CQ_TU_SAME
 hipError_t CQ_DEQUANTIZE_FLAT_SAME_TU(CQ_TU_FLOAT)(hipStream_t s, int bits, const FlatArgs& a) {
 #else
-hipError_t CQ_DEQUANTIZE_FLAT_TU(CQ_TU_FLOAT)(hipStream_t s, int bits, const FlatArgs& a) {
+hipError_t CQ_DEQUANTIZE_FLAT_TU(CQ_TU_FLOAT, CQ_TU_BITS)(hipStream_t s, const FlatArgs& a) {
+    constexpr int bits = CQ_TU_BITS;
 #endif
     int g = group_of(CQ_TU_FLOAT::kDtype, a.block);
     FlatArgs b = a;
     if (g < 0 && (b.any_group = any_group_of(CQ_TU_FLOAT::kDtype, a.block)) != 0) g = shape_group_of(b.any_group);  // lane by lane
+#if CQ_TU_SAME
     CQ_SWITCH_BITS(bits, CQ_SWITCH_GROUP(g, return (dequantize_launch<CQ_TU_FLOAT, kB, kG>(s, b))))
+#else
+    CQ_SWITCH_GROUP(g, return (dequantize_launch<CQ_TU_FLOAT, bits, kG>(s, b)))
+#endif
 }
 
 }  // namespace cq

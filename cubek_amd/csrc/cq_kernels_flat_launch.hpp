@@ -9,17 +9,23 @@
 
 namespace cq {
 
-// The quantize launchers, one per float type and family of scale sources (0: produced in the launch,
-// 1: given), each compiled from cq_kernels_flat_quantize.hip into an object of its own.
-#define CQ_QUANTIZE_FLAT_TU_(f, g) launch_quantize_flat_##f##_##g
-#define CQ_QUANTIZE_FLAT_TU(f, g) CQ_QUANTIZE_FLAT_TU_(f, g)
-hipError_t CQ_QUANTIZE_FLAT_TU(F32, 0)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
-hipError_t CQ_QUANTIZE_FLAT_TU(F32, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
-hipError_t CQ_QUANTIZE_FLAT_TU(BF16, 0)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
-hipError_t CQ_QUANTIZE_FLAT_TU(BF16, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
-hipError_t CQ_QUANTIZE_FLAT_TU(F16, 0)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
-hipError_t CQ_QUANTIZE_FLAT_TU(F16, 1)(hipStream_t s, int bits, ScaleSource src, const FlatArgs& a);
-// the dequantize launchers, one per float type, each compiled from cq_kernels_flat_dequantize.hip
+// The quantize launchers, one per float type, family of scale sources (0: produced in the launch, 1: given) and
+// width of the codes, each compiled from cq_kernels_flat_quantize.hip into an object of its own: the runtime loads
+// an object's code on the first launch out of it, and what a process's first quantize call waits for is the size of
+// that one object.
+#define CQ_QUANTIZE_FLAT_TU_(f, g, b) launch_quantize_flat_##f##_##g##_##b
+#define CQ_QUANTIZE_FLAT_TU(f, g, b) CQ_QUANTIZE_FLAT_TU_(f, g, b)
+#define CQ_DECLARE_QUANTIZE_TU(f, g)                                                             \
+    hipError_t CQ_QUANTIZE_FLAT_TU(f, g, 2)(hipStream_t s, ScaleSource src, const FlatArgs& a); \
+    hipError_t CQ_QUANTIZE_FLAT_TU(f, g, 4)(hipStream_t s, ScaleSource src, const FlatArgs& a); \
+    hipError_t CQ_QUANTIZE_FLAT_TU(f, g, 8)(hipStream_t s, ScaleSource src, const FlatArgs& a);
+CQ_DECLARE_QUANTIZE_TU(F32, 0)
+CQ_DECLARE_QUANTIZE_TU(F32, 1)
+CQ_DECLARE_QUANTIZE_TU(BF16, 0)
+CQ_DECLARE_QUANTIZE_TU(BF16, 1)
+CQ_DECLARE_QUANTIZE_TU(F16, 0)
+CQ_DECLARE_QUANTIZE_TU(F16, 1)
+#undef CQ_DECLARE_QUANTIZE_TU
 // The whole-tile kernels of a contiguous run for parameters typed like the float tensor (bf16 scales of a bf16
 // tensor, f16 of f16) live in objects of their own (-DCQ_TU_SAME=1): the runtime loads an object's code on its
 // first launch, so launches with f32 parameters do not pay for them.  FlatArgs::whole_grid tiles, nothing else.
@@ -55,11 +61,17 @@ hipError_t dequantize_flat_same(hipStream_t s, int bits, const FlatArgs& a) {
         return hipErrorInvalidValue;
 }
 
-#define CQ_DEQUANTIZE_FLAT_TU_(f) launch_dequantize_flat_##f
-#define CQ_DEQUANTIZE_FLAT_TU(f) CQ_DEQUANTIZE_FLAT_TU_(f)
-hipError_t CQ_DEQUANTIZE_FLAT_TU(F32)(hipStream_t s, int bits, const FlatArgs& a);
-hipError_t CQ_DEQUANTIZE_FLAT_TU(BF16)(hipStream_t s, int bits, const FlatArgs& a);
-hipError_t CQ_DEQUANTIZE_FLAT_TU(F16)(hipStream_t s, int bits, const FlatArgs& a);
+// the dequantize launchers, one per float type and width of the codes (cq_kernels_flat_dequantize.hip)
+#define CQ_DEQUANTIZE_FLAT_TU_(f, b) launch_dequantize_flat_##f##_##b
+#define CQ_DEQUANTIZE_FLAT_TU(f, b) CQ_DEQUANTIZE_FLAT_TU_(f, b)
+#define CQ_DECLARE_DEQUANTIZE_TU(f)                                            \
+    hipError_t CQ_DEQUANTIZE_FLAT_TU(f, 2)(hipStream_t s, const FlatArgs& a); \
+    hipError_t CQ_DEQUANTIZE_FLAT_TU(f, 4)(hipStream_t s, const FlatArgs& a); \
+    hipError_t CQ_DEQUANTIZE_FLAT_TU(f, 8)(hipStream_t s, const FlatArgs& a);
+CQ_DECLARE_DEQUANTIZE_TU(F32)
+CQ_DECLARE_DEQUANTIZE_TU(BF16)
+CQ_DECLARE_DEQUANTIZE_TU(F16)
+#undef CQ_DECLARE_DEQUANTIZE_TU
 
 namespace {
 
