@@ -191,6 +191,31 @@ def timed_region(torch, fn, launches, warmup=3):
     return a.elapsed_time(b) / launches, wall * 1e3 / launches
 
 
+def kernels_in_step(torch, paths, steps, warmup=3):
+    """The step's two launches timed where the metric runs them: `steps` steps (quantize, then the dequantize of the
+    same set) with an event before, between and after the two launches of each step, all enqueued first.  Returns
+    the mean and median of each kernel's per-launch times in ms.  An event between two launches adds ~2.5 us to
+    what it brackets, so these read that much longer than a kernel trace of the same launches."""
+    for i in range(warmup):
+        paths[i % len(paths)].quantize_dynamic()
+        paths[i % len(paths)].dequantize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    for i in range(steps):
+        p = paths[i % len(paths)]
+        ev[i][0].record()
+        p.quantize_dynamic()
+        ev[i][1].record()
+        p.dequantize()
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    out = {}
+    for name, k in (("quantize", 0), ("dequantize", 1)):
+        v = sorted(e[k].elapsed_time(e[k + 1]) for e in ev)
+        out[name] = {"avg_launch_ms": sum(v) / len(v), "median_launch_ms": v[len(v) // 2], "launches": len(v)}
+    return out
+
+
 def timed_median(torch, fn, regions=50, warmup=10, region_us=2000.0):
     """The timing protocol of the per-kernel figures: `warmup` untimed launches, then `regions` (>= 50) regions of
     back-to-back launches, each bracketed by HIP events recorded on the launch stream (all regions are enqueued
@@ -903,6 +928,8 @@ def main():
     d_ms, _ = timed_region(torch, lambda i: paths[i % len(paths)].dequantize(), args.steps)
     q_med = timed_median(torch, lambda i: paths[i % len(paths)].quantize_dynamic())
     d_med = timed_median(torch, lambda i: paths[i % len(paths)].dequantize())
+    # and the same two launches inside the step, where the quantize launch runs about a tenth shorter than alone
+    in_step = kernels_in_step(torch, paths, max(args.steps, 50))
 
     yardstick = copy_yardstick(torch, x)
     if args.copy_probe:
@@ -946,6 +973,14 @@ def main():
                                 "frac_at_avg": round(q_bytes / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
     }
 
+    for key, name in (("roofline", "quantize"), ("roofline_dequantize", "dequantize")):
+        t = in_step[name]
+        result[key]["in_step"] = {
+            "avg_launch_ms": round(t["avg_launch_ms"], 4), "median_launch_ms": round(t["median_launch_ms"], 4),
+            "launches": t["launches"],
+            "frac_at_avg": round(q_bytes / (t["avg_launch_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "note": "the launch as the step runs it (quantize, then the dequantize of the same set), one event pair "
+                    "per launch; `achieved` and `frac` above are of the kernel alone, back to back on rotated sets"}
     result["copy_yardstick"] = yardstick
     # the headline kernels' bytes: floats on one side, codes + scales on the other
     float_bytes = n * (2 if w["elem"] != "F32" else 4)
