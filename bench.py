@@ -463,6 +463,44 @@ def memory_yardsticks(torch, nbytes, q_read, q_written):
     return out
 
 
+def same_traffic_probes(torch, w):
+    """Launches with the traffic of configuration `w`'s quantize and dequantize and none of the arithmetic
+    (cq_bench_probes.hip: a workgroup reads 1024 16-byte chunks of floats and writes the share of them that codes and
+    scales take, or the reverse; streaming stores), rotated buffers, median of 50 regions: what a kernel of this shape
+    that computes nothing takes on this GPU at this size."""
+    import ctypes
+
+    if not os.path.exists(PROBES_PATH):
+        return None
+    L = ctypes.CDLL(PROBES_PATH)
+    if not hasattr(L, "cq_probe_shape"):
+        return None
+    L.cq_probe_shape.restype = ctypes.c_int
+    L.cq_probe_shape.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64,
+                                 ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64)]
+    rows, cols = w["shape"]
+    wide = rows * cols * (4 if w["elem"] == "F32" else 2)
+    narrow_chunks = max(1, round((algorithmic_bytes(w) - wide) * 1024 / wide))  # of every 1024 chunks of floats
+    tiles = wide // 16384
+    if tiles == 0:
+        return None
+    narrow = tiles * narrow_chunks * 16
+    sets = max(4, min(16, -(-(1 << 30) // (wide + narrow))))
+    wides = [torch.randint(0, 2 ** 31 - 1, (wide // 4,), dtype=torch.int32, device="cuda") for _ in range(sets)]
+    narrows = [torch.randint(0, 2 ** 31 - 1, (narrow // 4,), dtype=torch.int32, device="cuda") for _ in range(sets)]
+    stream = torch.cuda.current_stream().cuda_stream
+    mw, mn = ctypes.c_uint64(0), ctypes.c_uint64(0)
+    out = {"narrow_chunks_per_1024": narrow_chunks}
+    for widen, name in ((0, "quantize_shaped_ms"), (1, "dequantize_shaped_ms")):
+        def fn(i, widen=widen):
+            rc = L.cq_probe_shape(widen, stream, wides[i % sets].data_ptr(), narrows[i % sets].data_ptr(), wide,
+                                  narrow_chunks, ctypes.byref(mw), ctypes.byref(mn))
+            assert rc == 0, rc
+        out[name] = round(timed_median(torch, fn)["median_ms"], 4)
+    out["bytes_per_launch"] = mw.value + mn.value
+    return out
+
+
 def scheme_matrix(torch):
     """Every float type x value x store on the headline shape, blocks of 32, f32 parameters: the three launches of
     the path, reported only (`--matrix`).  Inputs ~N(0, 0.02) from torch's generator, three rotated buffer sets."""
@@ -1030,8 +1068,14 @@ def main():
             row["step_quantize_dynamic_then_dequantize"] = {
                 "ms": round(step_ms, 4), "GBps": round(2 * b / (step_ms * 1e-3) / 1e9, 1),
                 "sum_of_the_two_alone_ms": round(row["quantize_dynamic"]["ms"] + row["dequantize"]["ms"], 4)}
-            table.append(row)
             del ps, p, xi
+            probes = same_traffic_probes(torch, wk)
+            if probes is not None:
+                row["same_traffic_no_arithmetic"] = probes
+                for label, key in (("quantize_dynamic", "quantize_shaped_ms"), ("quantize_given_scales", "quantize_shaped_ms"),
+                                   ("dequantize", "dequantize_shaped_ms")):
+                    row[label]["frac_of_same_traffic_probe"] = round(probes[key] / row[label]["ms"], 4)
+            table.append(row)
         result["per_config"] = table
         # the same fractions where a reader of `roofline` alone finds them: [fused dynamic quantize, quantize with
         # given scales, dequantize] per configuration, median of 50 regions each, and the smallest cell of the three
@@ -1039,6 +1083,10 @@ def main():
         short = {"quantize_dynamic": "dynamic", "quantize_given_scales": "given", "dequantize": "dequantize"}
         result["roofline"]["per_config"] = {
             row["workload"]: {short[k]: row[k]["frac_hbm_peak"] for k in short} for row in table}
+        if all("same_traffic_no_arithmetic" in row for row in table):
+            # ... and against a launch of the same traffic that computes nothing (probe time / kernel time)
+            result["roofline"]["per_config_vs_same_traffic_probe"] = {
+                row["workload"]: {short[k]: row[k]["frac_of_same_traffic_probe"] for k in short} for row in table}
         result["roofline"]["min_frac_cfg3_5"] = min(
             row[k]["frac_hbm_peak"] for row in table if row["workload"] in ("cfg3", "cfg4", "cfg5") for k in short)
         result["adjacent_kernels"] = adjacent_kernels(torch) + corner_layouts(torch) + per_tensor_passes(torch) + packed_gemv(torch)

@@ -21,8 +21,8 @@ def test_world_size_from_a_launcher_is_refused_too():
 
 
 def test_bench_probe_library_loads():
-    """bench.py's memory yardsticks (cubek_amd/csrc/cq_bench_probes.hip): the library is built, exports its one entry
-    point, and refuses bad arguments before it touches the GPU."""
+    """bench.py's memory yardsticks (cubek_amd/csrc/cq_bench_probes.hip): the library is built, exports its entry
+    points, and refuses bad arguments before it touches the GPU."""
     import ctypes
 
     import bench
@@ -34,3 +34,9 @@ def test_bench_probe_library_loads():
                                ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]
     assert L.cq_probe_run(0, None, None, None, 100, None, None) == -1      # less than one tile
     assert L.cq_probe_run(7, None, None, None, 1 << 20, None, None) == -1  # no such probe
+    L.cq_probe_shape.restype = ctypes.c_int
+    L.cq_probe_shape.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64,
+                                 ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64)]
+    assert L.cq_probe_shape(0, None, None, None, 100, 320, None, None) == -1       # less than one tile
+    assert L.cq_probe_shape(0, None, None, None, 1 << 20, 0, None, None) == -1     # nothing on the narrow side
+    assert L.cq_probe_shape(1, None, None, None, 1 << 20, 1025, None, None) == -1  # narrow side wider than the wide one
