@@ -172,3 +172,20 @@ def test_empty_tensors_are_a_no_op():
     assert status(lambda: qz.launch_ref(CLIENT, x, t((0, 15), 4), sc, sc, Q8_B32, ElemType.F32)) == _ffi.ERR_SHAPE_MISMATCH
     cq_reduce.max_abs(CLIENT, t((0, 8), 4), t((0, 1), 4), 1, ElemType.F32)   # no outputs
     cq_contiguous.into_contiguous_packed_ref(CLIENT, t((0, 4), 4), t((0, 4), 4), (0, 32), 8)
+
+
+def test_argument_checks_walked_over_every_scheme_and_layout():
+    """tests/cpp/plan_walk.cpp: 5.5 million cq_plan_kind calls over operation x float type x value x parameter type
+    x store x block shape x tensor shape x layout, valid, invalid and damaged descriptors alike: no crash, every
+    status a known one, a kernel family named whenever the answer is CQ_OK."""
+    import os
+    import subprocess
+
+    binary = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "plan_walk")
+    assert os.path.exists(binary), "tests/cpp/plan_walk is not built (make -C cubek_amd/csrc)"
+    proc = subprocess.run([binary], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout[-2000:]
+    last = proc.stdout.strip().splitlines()[-1]
+    counts = {int(k): int(v) for k, v in (f[1:].split("]=") for f in last.split()[2:])}
+    assert sum(counts.values()) > 5_000_000 and counts[0] > 100_000, last   # plenty of valid calls among them
+    assert all(counts[k] == 0 for k in (5, 6, 7, 9, 10, 11, 12, 13, 14, 15)), last  # nothing launched, nothing unknown
