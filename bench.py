@@ -515,6 +515,40 @@ def same_traffic_probes(torch, w):
     return out
 
 
+def transposed_tile_probes(torch, widen, floats, codes, scales, rows, cols):
+    """The traffic of the transposed tile kernels without their arithmetic (cq_probe_transposed in cq_bench_probes.hip:
+    tiles of 128 rows x 256 columns, 256-byte runs of floats on one side, 128 bytes of codes and 32 of scales per row
+    on the other), on the buffers of the rows they stand beside: streaming or ordinary stores, tiles in launch order
+    or XCD by XCD; medians of 50 regions each and the best of the four."""
+    import ctypes
+
+    if not os.path.exists(PROBES_PATH):
+        return None
+    L = ctypes.CDLL(PROBES_PATH)
+    if not hasattr(L, "cq_probe_transposed"):
+        return None
+    L.cq_probe_transposed.restype = ctypes.c_int
+    L.cq_probe_transposed.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                      ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32]
+    if rows % 128 or cols % 256:
+        return None
+    assert all(t.numel() * t.element_size() >= rows * cols * 2 for t in floats)
+    assert all(t.numel() * t.element_size() >= rows * cols // 2 for t in codes)
+    assert all(t.numel() * t.element_size() >= rows * cols // 8 for t in scales)
+    stream = torch.cuda.current_stream().cuda_stream
+    # (widen: the probe overwrites `floats`; the caller passes output buffers)
+    out = {}
+    for plain in (0, 1):
+        for xcd in (0, 1):
+            def fn(i, plain=plain, xcd=xcd):
+                rc = L.cq_probe_transposed(int(widen), plain, xcd, stream, floats[i % len(floats)].data_ptr(),
+                                           codes[i % len(codes)].data_ptr(), scales[i % len(scales)].data_ptr(), rows, cols)
+                assert rc == 0, rc
+            name = ("ordinary" if plain else "streaming") + " stores, " + ("tiles XCD by XCD" if xcd else "tiles in launch order")
+            out[name] = round(timed_median(torch, fn)["median_ms"], 4)
+    return {"variants_ms": out, "best_ms": min(out.values())}
+
+
 def scheme_matrix(torch):
     """Every float type x value x store on the headline shape, blocks of 32, f32 parameters: the three launches of
     the path, reported only (`--matrix`).  Inputs ~N(0, 0.02) from torch's generator, three rotated buffer sets."""
@@ -625,6 +659,10 @@ def adjacent_kernels(torch):
         out.append({"kernel": f"{label}, e2m1 blocks of 32, transposed bf16 view [{rows}, {cols}] of a [{cols}, {rows}] buffer",
                     "algorithmic_bytes": b, "ms": round(ms, 4), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+        probe = transposed_tile_probes(torch, label == "dequantize", ys if label == "dequantize" else xs, words, bscales, rows, cols)
+        if probe is not None:
+            out[-1]["same_traffic_no_arithmetic"] = probe
+            out[-1]["frac_of_same_traffic_probe"] = round(probe["best_ms"] / ms, 4)
     # one scale per tensor: two launches, the tensor read twice (pass 1 leaves what it can in the caches for pass 2)
     tensor_scheme = QuantScheme.default().with_value(QuantValue.Q8S).with_level(QuantLevel.Tensor)
     ws_bytes = cq_quantize.workspace_bytes(tensor_scheme, rows * cols)

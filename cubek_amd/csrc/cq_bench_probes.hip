@@ -66,6 +66,57 @@ __global__ __launch_bounds__(kThreads) void probe_widen_kernel(const u32x4* __re
     for (int u = 0; u < kUnroll; u++) __builtin_nontemporal_store(x, out + at + u * kThreads);
 }
 
+// The traffic of the quantize (kWiden false) or dequantize (kWiden true) tile kernels for a bf16 tensor stored
+// transposed, element (r, c) at c * rows + r, without the arithmetic: a workgroup moves a tile of 128 rows x 256
+// columns: 256 runs of 256 bytes of floats `rows` elements apart on one side, 128 bytes of 4-bit codes and 32 bytes of
+// f32 scales (blocks of 32) per row on the other.  kPlain: ordinary stores instead of streaming ones; kXcd: consecutive
+// tiles on one XCD (workgroups go round the eight XCDs).
+template <bool kWiden, bool kPlain, bool kXcd>
+__global__ __launch_bounds__(kThreads) void probe_transposed_tile_kernel(char* __restrict__ floats, char* __restrict__ codes,
+                                                                         char* __restrict__ scales, uint32_t rows, uint32_t cols) {
+    const uint32_t tiles_c = cols / 256u;
+    uint32_t b = blockIdx.x;
+    if (kXcd) {
+        const uint32_t n = gridDim.x / 8u;
+        if (b < n * 8u) b = (b % 8u) * n + b / 8u;
+    }
+    const uint32_t tr = b / tiles_c, tc = b % tiles_c, t = threadIdx.x;
+    char* fbase = floats + static_cast<uint64_t>(tc) * 256u * rows * 2u + static_cast<uint64_t>(tr) * 256u;
+    const auto float_piece = [&](uint32_t p) {  // piece p of the tile: column p / 16, 16 bytes p % 16 of its run
+        return reinterpret_cast<u32x4*>(fbase + static_cast<uint64_t>(p / 16u) * rows * 2u + (p % 16u) * 16u);
+    };
+    const auto code_piece = [&](uint32_t p) {  // row p / 8, 16 bytes p % 8 of its 128
+        return reinterpret_cast<u32x4*>(codes + (static_cast<uint64_t>(tr) * 128u + p / 8u) * (cols / 2u) + static_cast<uint64_t>(tc) * 128u + (p % 8u) * 16u);
+    };
+    u32x4* scale_piece = reinterpret_cast<u32x4*>(scales + (static_cast<uint64_t>(tr) * 128u + t / 2u) * (cols / 8u) + static_cast<uint64_t>(tc) * 32u + (t % 2u) * 16u);
+    const auto put = [](u32x4 v, u32x4* at) {
+        if (kPlain) *at = v; else __builtin_nontemporal_store(v, at);
+    };
+    u32x4 acc = {t, b, 3u, 4u};
+    if (!kWiden) {
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            u32x4 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[j] = __builtin_nontemporal_load(float_piece((s * 4 + j) * kThreads + t));
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc ^= v[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) put(acc, code_piece(j * kThreads + t));
+        put(acc, scale_piece);
+    } else {
+        u32x4 v[5];
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = __builtin_nontemporal_load(code_piece(j * kThreads + t));
+        v[4] = __builtin_nontemporal_load(scale_piece);
+#pragma unroll
+        for (int j = 0; j < 5; j++) acc ^= v[j];
+#pragma unroll
+        for (int j = 0; j < 16; j++) put(acc, float_piece(j * kThreads + t));
+    }
+}
+
 }  // namespace
 
 // kind 0: read `bytes` of `a`; 1: write `bytes` of `b`; 2: copy `bytes` from `a` to `b`.  `bytes` is rounded down to
@@ -104,5 +155,33 @@ extern "C" int cq_probe_shape(int widen, void* stream, void* wide, void* narrow,
         hipLaunchKernelGGL(probe_narrow_kernel, grid, block, 0, s, static_cast<const u32x4*>(wide), static_cast<u32x4*>(narrow), narrow_chunks);
     else
         hipLaunchKernelGGL(probe_widen_kernel, grid, block, 0, s, static_cast<const u32x4*>(narrow), static_cast<u32x4*>(wide), narrow_chunks);
+    return static_cast<int>(hipGetLastError());
+}
+
+// The transposed tile kernels' traffic for a bf16 [rows, cols] tensor stored transposed (`floats`: rows * cols * 2
+// bytes; `codes`: rows * cols / 2; `scales`: rows * cols / 8), rows a multiple of 128 and cols of 256.  widen: 0 reads
+// the floats and writes codes and scales, 1 the reverse; plain_stores / xcd_order pick the variant.
+extern "C" int cq_probe_transposed(int widen, int plain_stores, int xcd_order, void* stream, void* floats, void* codes,
+                                   void* scales, uint32_t rows, uint32_t cols) {
+    if (rows == 0 || cols == 0 || rows % 128u != 0 || cols % 256u != 0) return -1;
+    const uint64_t tiles = static_cast<uint64_t>(rows / 128u) * (cols / 256u);
+    if (tiles >= (1ull << 31)) return -1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid(static_cast<uint32_t>(tiles)), block(kThreads);
+    const int variant = (widen ? 4 : 0) | (plain_stores ? 2 : 0) | (xcd_order ? 1 : 0);
+#define CQ_PROBE_TILE(W, P, X)                                                                                       \
+    hipLaunchKernelGGL((probe_transposed_tile_kernel<W, P, X>), grid, block, 0, s, static_cast<char*>(floats),      \
+                       static_cast<char*>(codes), static_cast<char*>(scales), rows, cols)
+    switch (variant) {
+        case 0: CQ_PROBE_TILE(false, false, false); break;
+        case 1: CQ_PROBE_TILE(false, false, true); break;
+        case 2: CQ_PROBE_TILE(false, true, false); break;
+        case 3: CQ_PROBE_TILE(false, true, true); break;
+        case 4: CQ_PROBE_TILE(true, false, false); break;
+        case 5: CQ_PROBE_TILE(true, false, true); break;
+        case 6: CQ_PROBE_TILE(true, true, false); break;
+        default: CQ_PROBE_TILE(true, true, true); break;
+    }
+#undef CQ_PROBE_TILE
     return static_cast<int>(hipGetLastError());
 }

@@ -40,3 +40,8 @@ def test_bench_probe_library_loads():
     assert L.cq_probe_shape(0, None, None, None, 100, 320, None, None) == -1       # less than one tile
     assert L.cq_probe_shape(0, None, None, None, 1 << 20, 0, None, None) == -1     # nothing on the narrow side
     assert L.cq_probe_shape(1, None, None, None, 1 << 20, 1025, None, None) == -1  # narrow side wider than the wide one
+    L.cq_probe_transposed.restype = ctypes.c_int
+    L.cq_probe_transposed.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                      ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32]
+    assert L.cq_probe_transposed(0, 0, 0, None, None, None, None, 100, 256) == -1   # rows not in whole tiles
+    assert L.cq_probe_transposed(1, 1, 1, None, None, None, None, 128, 0) == -1     # no columns
