@@ -415,6 +415,10 @@ def packed_gemv(torch):
                     "GBps": round(b / (ms * 1e-3) / 1e9, 1), "frac_hbm_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                     "weights_per_s": round(rows * cols / (ms * 1e-3)),
                     "multiply_adds_per_s": round(rows * cols * vectors / (ms * 1e-3))})
+        rs = read_stream_ms(torch, b)
+        if rs is not None:  # the same number of bytes as one plain read stream that computes nothing
+            out[-1]["read_stream_same_bytes_ms"] = round(rs, 4)
+            out[-1]["frac_of_read_stream"] = round(rs / ms, 4)
         if ms < 0.016:  # within four host enqueue times: also as a replayed HIP graph
             one = lambda c, i: matvec.launch_ref(c, hw[i % sets], hs[i % sets], scheme, hx, hy, et, et)
             g_ms = graph_region_of(torch, one, sets)
@@ -513,6 +517,30 @@ def same_traffic_probes(torch, w):
         out[name] = round(timed_median(torch, fn)["median_ms"], 4)
     out["bytes_per_launch"] = mw.value + mn.value
     return out
+
+
+def read_stream_ms(torch, nbytes):
+    """A pure read stream of `nbytes` (probe_read_kernel of cq_bench_probes.hip: 16 KiB per workgroup, consecutive
+    lanes on consecutive 16 bytes), rotated buffers of at least 1 GiB together, median of 50 regions."""
+    import ctypes
+
+    if not os.path.exists(PROBES_PATH):
+        return None
+    L = ctypes.CDLL(PROBES_PATH)
+    L.cq_probe_run.restype = ctypes.c_int
+    L.cq_probe_run.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64,
+                               ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]
+    nbytes = nbytes // 16384 * 16384
+    if nbytes == 0:
+        return None
+    sets = max(4, min(32, -(-(1 << 30) // nbytes)))
+    bufs = [torch.randint(0, 2 ** 31 - 1, (nbytes // 4,), dtype=torch.int32, device="cuda") for _ in range(sets)]
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def fn(i):
+        rc = L.cq_probe_run(0, stream, bufs[i % sets].data_ptr(), None, nbytes, None, None)
+        assert rc == 0, rc
+    return timed_median(torch, fn)["median_ms"]
 
 
 def transposed_tile_probes(torch, widen, floats, codes, scales, rows, cols):
