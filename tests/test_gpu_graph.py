@@ -59,3 +59,50 @@ def test_graph_replays_match_eager(level):
         assert torch.equal(got[0], words) and torch.equal(got[1], scales), (level, it)
         assert torch.equal(got[2].view(torch.int16), y.view(torch.int16)), (level, it)
         assert float(y.float().abs().max()) > 0
+
+
+_COLD_CAPTURE = r"""
+import sys
+import torch
+from cubek_amd import ComputeClient, ElemType, QuantLevel, QuantScheme, QuantValue, TensorHandleRef
+from cubek_amd import dequantize as dq, quantize as qz
+scheme = QuantScheme.default().with_value(QuantValue.Q4S).with_level(QuantLevel.block(BLOCK))
+shape = (512, 1024)
+h = TensorHandleRef.from_torch
+x = torch.randn(shape, device="cuda", dtype=torch.bfloat16)
+words = torch.zeros(scheme.packed_shape(shape), dtype=torch.int32, device="cuda")
+scales = torch.zeros(scheme.scales_shape(shape), dtype=torch.float32, device="cuda")
+y = torch.zeros(shape, device="cuda", dtype=torch.bfloat16)
+torch.cuda.synchronize()
+def run():
+    c = ComputeClient.current()
+    qz.launch_dynamic(c, h(x), h(words), h(scales), scheme, ElemType.BF16, 0, 0)
+    dq.launch_ref(c, h(words), h(y), h(scales), scheme, ElemType.BF16)
+g = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g):
+    run()  # the library's first launches in this process
+g.replay()
+torch.cuda.synchronize()
+got = (words.clone(), scales.clone(), y.clone())
+words.zero_(), scales.zero_(), y.zero_()
+run()
+torch.cuda.synchronize()
+ok = torch.equal(got[0], words) and torch.equal(got[1], scales) and torch.equal(got[2].view(torch.int16), y.view(torch.int16))
+sys.exit(0 if ok and float(y.float().abs().max()) > 0 else 3)
+"""
+
+
+@pytest.mark.parametrize("block", ["[32]", "[64, 64]"])
+def test_a_process_first_calls_can_be_captured(block):
+    """No warm-up: the first launch out of a code object (the streaming kernels' are stored as they are, the 2-D block
+    kernel's compressed) loads it while the stream is capturing; the replay must match the eager result.  Runs in
+    a process of its own, since this one has launched before."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    proc = subprocess.run([sys.executable, "-c", _COLD_CAPTURE.replace("BLOCK", block)], cwd=root, env=env,
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stdout[-2000:]
